@@ -1,0 +1,51 @@
+"""ctypes mirror of include/dsgx.h: constants and structures only (loads nothing)."""
+import ctypes as C
+
+FMT_REF_NVFP4, FMT_REF_INT4, FMT_REF_BF16 = 0, 2, 3
+FMT_FP8, FMT_INT4, FMT_BF16 = 16, 18, 19
+OUT_BF16, OUT_F32, OUT_SWIGLU = 0, 1, 2
+MAX_ROWS, MAX_TOPK, MAX_UNION, SH_SLOT, MAX_EXPERTS, MAX_CHUNK = 16, 8, 128, 128, 512, 8192
+OK, EINVAL, EFORMAT, EUNSUPPORTED, EHIP = 0, 1, 2, 3, 4
+
+
+class MatDesc(C.Structure):
+    _fields_ = [("off", C.c_uint64), ("s2", C.c_float), ("fmt", C.c_uint32), ("rsv", C.c_uint32 * 12)]
+
+
+class SharedW(C.Structure):
+    _fields_ = [(n, C.c_void_p) for n in ("g", "u", "d", "gs", "us", "ds", "bgu", "bd")]
+
+
+class LayerW(C.Structure):
+    _fields_ = [("pool", C.c_void_p), ("desc", C.c_void_p), ("sh", SharedW), ("fmt", C.c_uint32),
+                ("H", C.c_int32), ("I", C.c_int32), ("E", C.c_int32), ("topk", C.c_int32)]
+
+
+class DecodeCfg(C.Structure):
+    _fields_ = [("up", C.c_int32), ("down", C.c_int32), ("parts", C.c_int32), ("ysum", C.c_int32),
+                ("logits", C.c_void_p), ("bias", C.c_void_p), ("route_scale", C.c_float), ("score_fn", C.c_int32),
+                ("post", C.c_void_p)]
+
+
+class PrefillCfg(C.Structure):
+    _fields_ = [("shared", C.c_int32), ("phases", C.c_int32), ("act_fp8", C.c_int32)]
+
+
+class PrefillView(C.Structure):
+    _fields_ = [(n, C.c_void_p) for n in ("rpos", "re", "h", "hsh", "off", "perm")]
+
+
+class GemvSeg(C.Structure):
+    _fields_ = [("fmt", C.c_int32), ("w", C.c_void_p), ("s", C.c_void_p), ("zp", C.c_void_p), ("n", C.c_int32),
+                ("rs", C.c_int32), ("ks", C.c_int32), ("y", C.c_void_p), ("ldy", C.c_int32)]
+
+
+assert C.sizeof(MatDesc) == 64
+
+# every symbol include/dsgx.h declares
+SYMBOLS = [
+    "dsgx_mat_bytes", "dsgx_mat_scale_off", "dsgx_mat_zp_off", "dsgx_route", "dsgx_decode_cfg_default",
+    "dsgx_decode_ws_bytes", "dsgx_moe_decode", "dsgx_finalize", "dsgx_prefill_cfg_default", "dsgx_prefill_ws_bytes",
+    "dsgx_moe_prefill", "dsgx_prefill_view_get", "dsgx_gemv", "dsgx_dequant_int4", "dsgx_probe_dequant_int4",
+    "dsgx_widen_fp8", "dsgx_act_quant", "dsgx_last_error", "dsgx_version", "dsgx_stream_read", "dsgx_stream_copy",
+]

@@ -1,0 +1,190 @@
+// Device helpers shared by the gfx950 kernels: bf16 / e4m3 / INT4 decode in registers, wave64 reductions, the
+// streaming loads, the activation staging layout and the router's row function.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/dsgx.h"
+
+namespace dsgx {
+
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+
+constexpr int kWave = 64;
+
+// ---- scalar codecs ------------------------------------------------------------------------------------------------
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t b) { return __uint_as_float(b << 16); }
+// Round to nearest even, the contract's integer form (engine/experts/formats.cuh:33-37 of the reference): used where
+// a single value is rounded (epilogues); the packed hardware conversion below is used in the streaming loops.
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
+  uint32_t u = __float_as_uint(f);
+  u += 0x7FFFu + ((u >> 16) & 1u);
+  return u >> 16;
+}
+__device__ __forceinline__ float bf16_round(float f) { return __uint_as_float(f32_to_bf16_bits(f) << 16); }
+// two f32 -> packed bf16 (lo = a, hi = b), round to nearest even: v_cvt_pk_bf16_f32
+__device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
+  bf16x2_t v = {(__bf16)a, (__bf16)b};
+  return __builtin_bit_cast(uint32_t, v);
+}
+// acc + a.lo * b.lo + a.hi * b.hi on packed bf16 pairs: v_dot2c_f32_bf16
+__device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float acc) {
+  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, a), __builtin_bit_cast(bf16x2_t, b), acc, false);
+}
+
+// ---- weight decode: 8 consecutive k -> four packed bf16 pairs (k, k+1) ---------------------------------------------------
+// FP8 e4m3fn: two 32-bit words (8 codes) -> exact bf16 values (v_cvt_scalef32_pk_bf16_fp8 with scale 1).
+__device__ __forceinline__ void fp8x8_to_bf16(uint32_t w0, uint32_t w1, uint32_t (&o)[4]) {
+  o[0] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w0, 1.0f, false));
+  o[1] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w0, 1.0f, true));
+  o[2] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w1, 1.0f, false));
+  o[3] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w1, 1.0f, true));
+}
+// INT4-g32: one 32-bit word = 8 stored nibbles u (value i at bits 4i) of one group with scale s (f32 of the bf16) and
+// nzs = -(u_z * s). W = bf16_rne((u - u_z) * s): u * s and u_z * s are exact in f32 (4 x 8 significant bits), so
+// fma(u, s, nzs) is the exact product (u - u_z) * s, and the packed conversion rounds it once to nearest even.
+// (Exact while u_z * s stays finite, i.e. |s| < 2^124; dequant_int4's own kernel uses the subtract-first form.)
+__device__ __forceinline__ void i4x8_to_bf16(uint32_t w, float s, float nzs, uint32_t (&o)[4]) {
+  const uint32_t lo = w & 0x0F0F0F0Fu, hi = (w >> 4) & 0x0F0F0F0Fu;  // lo: values 0,2,4,6; hi: 1,3,5,7
+  o[0] = pack_bf16(fmaf((float)(lo & 0xFFu), s, nzs), fmaf((float)(hi & 0xFFu), s, nzs));
+  o[1] = pack_bf16(fmaf((float)((lo >> 8) & 0xFFu), s, nzs), fmaf((float)((hi >> 8) & 0xFFu), s, nzs));
+  o[2] = pack_bf16(fmaf((float)((lo >> 16) & 0xFFu), s, nzs), fmaf((float)((hi >> 16) & 0xFFu), s, nzs));
+  o[3] = pack_bf16(fmaf((float)(lo >> 24), s, nzs), fmaf((float)(hi >> 24), s, nzs));
+}
+// the contract in its subtract-first form, exact for every finite scale: bf16_rne(float(u - u_z) * s)
+__device__ __forceinline__ uint32_t i4_value_bits(int u, int uz, uint32_t sbits) {
+  return f32_to_bf16_bits((float)(u - uz) * bf16_bits_to_f32(sbits));
+}
+
+// ---- streaming loads (weights are read once: non-temporal) ---------------------------------------------------------------
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ uint4 ldg_stream(const void* p) {
+  const u32x4_t v = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(p));
+  return make_uint4(v.x, v.y, v.z, v.w);
+}
+
+// ---- wave64 sum, result valid in every lane ---------------------------------------------------------------------------------
+template <int CTRL>
+__device__ __forceinline__ float dpp_add(float v) {
+  const int t = __builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, true);
+  return v + __int_as_float(t);
+}
+__device__ __forceinline__ float wave_sum(float v) {
+  v = dpp_add<0xB1>(v);   // quad_perm [1,0,3,2]
+  v = dpp_add<0x4E>(v);   // quad_perm [2,3,0,1]
+  v = dpp_add<0x141>(v);  // row_half_mirror
+  v = dpp_add<0x140>(v);  // row_mirror: every lane of a row of 16 holds the row's sum
+  v += __shfl_xor(v, 16);
+  v += __shfl_xor(v, 32);
+  return v;
+}
+
+// ---- the activation layout in LDS ---------------------------------------------------------------------------------------------
+// A lane of a wavefront that streams a row holds KL consecutive k per segment of 64 * KL k (KL = 16 for FP8: one
+// 16-byte load; 32 for INT4: one 16-byte load; 8, 16 or 32 for BF16: one, two or four 16-byte loads). The activations
+// of row m are staged as 16-byte chunks of 8 k so that the lanes of a wavefront read consecutive chunks (no bank
+// conflicts): chunk c (of KL / 8) of segment s of lane l sits at chunk index ((s * (KL / 8) + c) * 64 + l) of the row.
+template <int KL>
+__device__ __forceinline__ int xchunk_index(int q) {  // q: the row's chunk number in k order (k = 8 q)
+  constexpr int XC = KL / 8;
+  const int seg = q / (64 * XC), r = q % (64 * XC);
+  return (seg * XC + r % XC) * 64 + r / XC;
+}
+// Stage rows x[M][ldx] (bf16, global) into lds [M][K/8 chunks] in the layout above; K a multiple of 8. Chunks past K in
+// the last segment are zero-filled up to Kpad (a multiple of 64 * KL).
+template <int KL>
+__device__ __forceinline__ void stage_x(uint4* lds, const uint16_t* x, size_t ldx, int M, int K, int Kpad) {
+  const int nq = Kpad / 8;
+  for (int i = threadIdx.x; i < M * nq; i += blockDim.x) {
+    const int m = i / nq, q = i % nq;
+    uint4 v = make_uint4(0, 0, 0, 0);
+    if (8 * q < K) v = *reinterpret_cast<const uint4*>(x + (size_t)m * ldx + 8 * q);
+    lds[(size_t)m * nq + xchunk_index<KL>(q)] = v;
+  }
+}
+
+// ---- the router's row function (one wavefront a row) ------------------------------------------------------------------------------
+// s = 1 / (1 + e^-l) from IEEE operations only, so the CPU and the GPU give the same bits: the reference's
+// route_sigmoid (engine/experts/formats.cuh:142-163).
+__device__ __forceinline__ float route_sigmoid(float l) {
+  const float x = -l;
+  if (x > 88.f) return 0.f;
+  if (x < -87.f) return 1.f;
+  const float n = rintf(x * 1.44269504f);
+  float r = fmaf(-n, 0.693145751953125f, x);
+  r = fmaf(-n, 1.428606765330187e-06f, r);
+  float p = 1.f / 5040;
+  p = fmaf(p, r, 1.f / 720);
+  p = fmaf(p, r, 1.f / 120);
+  p = fmaf(p, r, 1.f / 24);
+  p = fmaf(p, r, 1.f / 6);
+  p = fmaf(p, r, 0.5f);
+  p = fmaf(p, r, 1.f);
+  p = fmaf(p, r, 1.f);
+  const float e = ldexpf(p, (int)n);
+  return __fdiv_rn(1.f, __fadd_rn(1.f, e));
+}
+__device__ __forceinline__ float route_score(float l, int score_fn) {
+  if (score_fn == 0) return route_sigmoid(l);
+  return sqrtf(l > 20.f ? l : log1pf(expf(l)));  // DeepSeek's sqrt(softplus): libm-dependent, not promised bit-exact
+}
+// One row by one wavefront: experts e = lane + 64 j, j < 8 (E <= 512). Lane k < topk gets pick k's expert and weight
+// (route_warp of the reference, engine/experts/formats.cuh:207-247, at 64 lanes): descending key, ties to the lower
+// id; the sum in the butterfly order over eight places ((p0+p4)+(p2+p6))+((p1+p5)+(p3+p7)), absent places skipped.
+__device__ __forceinline__ void route_row(const float* __restrict__ logits_row, const float* __restrict__ bias, int E, int topk,
+                                          float scale, int score_fn, int lane, int& id_out, float& w_out) {
+  constexpr int RJ = DSGX_MAX_EXPERTS / kWave;
+  float s[RJ], key[RJ];
+#pragma unroll
+  for (int j = 0; j < RJ; ++j) {
+    const int e = lane + kWave * j;
+    if (e < E) {
+      s[j] = route_score(logits_row[e], score_fn);
+      key[j] = __fadd_rn(s[j], bias ? bias[e] : 0.f);
+    } else {
+      s[j] = 0.f, key[j] = -INFINITY;
+    }
+  }
+  float picked[DSGX_MAX_TOPK];
+  int ids[DSGX_MAX_TOPK];
+#pragma unroll
+  for (int k = 0; k < DSGX_MAX_TOPK; ++k) {
+    picked[k] = 0.f, ids[k] = 0;
+    if (k >= topk) continue;
+    float bv = -INFINITY;
+    int bj = 0;
+#pragma unroll
+    for (int j = 0; j < RJ; ++j)
+      if (key[j] > bv) bv = key[j], bj = j;
+    int be = bv == -INFINITY ? 1 << 30 : lane + kWave * bj;
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      const float ov = __shfl_xor(bv, o);
+      const int oe = __shfl_xor(be, o);
+      if (ov > bv || (ov == bv && oe < be)) bv = ov, be = oe;
+    }
+    ids[k] = be;
+    float sv = 0.f;
+#pragma unroll
+    for (int j = 0; j < RJ; ++j)
+      if (lane + kWave * j == be) sv = s[j], key[j] = -INFINITY;
+    picked[k] = __shfl(sv, be & (kWave - 1));
+  }
+  auto add = [](float a, float b, bool hb) { return hb ? __fadd_rn(a, b) : a; };
+  const float a04 = add(picked[0], picked[4], 4 < topk), a26 = add(picked[2], picked[6], 6 < topk);
+  const float a15 = add(picked[1], picked[5], 5 < topk), a37 = add(picked[3], picked[7], 7 < topk);
+  const float sum = __fadd_rn(add(add(a04, a26, 2 < topk), add(a15, a37, 3 < topk), 1 < topk), 1e-20f);
+  id_out = 0, w_out = 0.f;
+#pragma unroll
+  for (int k = 0; k < DSGX_MAX_TOPK; ++k)
+    if (lane == k && k < topk) id_out = ids[k], w_out = __fmul_rn(__fdiv_rn(picked[k], sum), scale);
+}
+
+// h = bf16(bf16(silu(g)) * u), g and u already bf16 values (engine/experts/decode.cu:110-113 of the reference)
+__device__ __forceinline__ uint32_t swiglu_bits(float g, float u) {
+  const float sl = bf16_round(__fdiv_rn(g, __fadd_rn(1.f, expf(-g))));
+  return f32_to_bf16_bits(__fmul_rn(sl, u));
+}
+
+}  // namespace dsgx

@@ -1,0 +1,227 @@
+// Dense GEMV for 1-16 activation rows over FP8-128x128, INT4-g32 and BF16 weights: the gfx950 counterpart of the
+// reference's glm::gemv (altar1-4xgx10-switchless/engine/attn/gemv.cu:173-333, attn.h:59-123).
+//
+//   y[r][n] = sum_k x[r][k] W[n][k], f32 accumulation, outputs bf16 / f32 / SwiGLU (gemv.cu:138-170).
+//   FP8: per 128-k block the unscaled f32 sum, then acc = fma(S, sum, acc) (gemv.cu:230-244, micro/gemv.cu:512);
+//   INT4: W = bf16_rne((u - u_z) s) per element in registers (attn_common.cuh:65-76), then as BF16.
+//
+// One wavefront owns RB rows of W and the whole of K (rowdot.cuh); the grid is sized to the chip and walks the row
+// batches round-robin. The order of the adds inside a dot product is not the reference's (not part of its contract).
+#include "abi_internal.h"
+#include "rowdot.cuh"
+
+namespace dsgx {
+namespace {
+
+constexpr int kMaxSegs = 4;  // attn.h:94
+struct GemvSegDev {
+  MatDev m;
+  void* y;
+  int n, ldy, row0;
+};
+struct GemvArgs {
+  const uint16_t* x;
+  int ldx, K, nq, nsegk, nsegs, total_rows, out;
+  GemvSegDev sg[kMaxSegs];
+};
+
+template <int FMT, int M, int RB, int D>
+__global__ void __launch_bounds__(256) k_gemv(GemvArgs a) {
+  extern __shared__ uint4 xs[];
+  stage_x<FmtT<FMT>::KL>(xs, a.x, a.ldx, M, a.K, a.nq * 8);
+  __syncthreads();
+  const int lane = threadIdx.x & 63;
+  const int gw = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6), GW = gridDim.x * (blockDim.x >> 6);
+  const int nbatch = a.total_rows / RB;
+  const int nmine = gw < nbatch ? (nbatch - gw + GW - 1) / GW : 0;
+  const int nsteps = nmine * a.nsegk;
+
+  auto locate = [&](int row, int& si) {
+    si = 0;
+#pragma unroll
+    for (int i = 1; i < kMaxSegs; ++i)
+      if (i < a.nsegs && row >= a.sg[i].row0) si = i;
+  };
+  Raw w[D][RB];
+  int lj = 0, lseg = 0;  // the load cursor: batch number of this wave, segment
+  auto load = [&](Raw (&r)[RB]) {
+    const int row = (gw + lj * GW) * RB;
+    int si;
+    locate(row, si);
+#pragma unroll
+    for (int i = 0; i < RB; ++i) load_raw<FMT>(r[i], a.sg[si].m, row - a.sg[si].row0 + i, lseg, lane, a.K);
+    if (++lseg == a.nsegk) lseg = 0, ++lj;
+  };
+#pragma unroll
+  for (int d = 0; d < D; ++d)
+    if (d < nsteps) load(w[d]);
+
+  float acc[RB][M];
+  int cj = 0, cseg = 0;
+  for (int t0 = 0; t0 < nsteps; t0 += D) {
+#pragma unroll
+    for (int d = 0; d < D; ++d) {
+      const int t = t0 + d;
+      if (t >= nsteps) break;
+      if (cseg == 0) {
+#pragma unroll
+        for (int r = 0; r < RB; ++r)
+#pragma unroll
+          for (int m = 0; m < M; ++m) acc[r][m] = 0.f;
+      }
+      step_dot<FMT, M, RB>(w[d], xs, a.nq, cseg, lane, acc);
+      if (t + D < nsteps) load(w[d]);
+      if (++cseg < a.nsegk) continue;
+      cseg = 0;
+      // the batch is complete: add the lanes' partials, lane r * M + m keeps output (row r, activation row m)
+      const int row = (gw + cj * GW) * RB;
+      ++cj;
+      float mine = 0.f, mine2 = 0.f;
+#pragma unroll
+      for (int r = 0; r < RB; ++r)
+#pragma unroll
+        for (int m = 0; m < M; ++m) {
+          const float v = wave_sum(acc[r][m]);
+          if (lane == r * M + m) mine = v;
+          if (lane == (r ^ 1) * M + m) mine2 = v;  // the pair's other row (SwiGLU)
+        }
+      if (lane >= RB * M) continue;
+      int si;
+      locate(row, si);
+      const GemvSegDev& sg = a.sg[si];
+      const int r = lane / M, m = lane % M, n = row - sg.row0 + r;
+      if (a.out == DSGX_OUT_BF16) {
+        static_cast<uint16_t*>(sg.y)[(size_t)m * sg.ldy + n] = (uint16_t)f32_to_bf16_bits(mine);
+      } else if (a.out == DSGX_OUT_F32) {
+        static_cast<float*>(sg.y)[(size_t)m * sg.ldy + n] = mine;
+      } else if ((r & 1) == 0) {  // SwiGLU: row 2i gate, 2i + 1 up -> column i (gemv.cu:164-168)
+        static_cast<uint16_t*>(sg.y)[(size_t)m * sg.ldy + n / 2] = (uint16_t)swiglu_bits(bf16_round(mine), bf16_round(mine2));
+      }
+    }
+  }
+}
+
+
+
+template <int FMT, int M, int RB>
+int launch_gemv(const GemvArgs& a, hipStream_t st) {
+  constexpr int D = 4;
+  const size_t lds = (size_t)M * a.nq * 16;
+  const int nbatch = a.total_rows / RB;
+  // two workgroups of four wavefronts a CU when the activations leave room in LDS, never more workgroups than batches
+  const int per_cu = lds <= 64 * 1024 ? 2 : 1;
+  int grid = num_cus_cached() * per_cu;
+  if (grid > (nbatch + 3) / 4) grid = (nbatch + 3) / 4;
+  if (grid < 1) grid = 1;
+  auto kern = k_gemv<FMT, M, RB, D>;
+  if (lds > 48 * 1024) DSGX_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, st, a);
+  DSGX_HIP(hipGetLastError());
+  return DSGX_OK;
+}
+template <int FMT, int M>
+int launch_gemv_rb(const GemvArgs& a, hipStream_t st) {
+  // few rows: two rows a wavefront so that the whole chip streams
+  if (a.total_rows / 4 < 4 * num_cus_cached()) return launch_gemv<FMT, M, 2>(a, st);
+  return launch_gemv<FMT, M, 4>(a, st);
+}
+template <int FMT>
+int launch_gemv_m(int M, const GemvArgs& a, hipStream_t st) {
+  switch (M) {
+    case 1: return launch_gemv_rb<FMT, 1>(a, st);
+    case 2: return launch_gemv_rb<FMT, 2>(a, st);
+    case 3: return launch_gemv_rb<FMT, 3>(a, st);
+    case 4: return launch_gemv_rb<FMT, 4>(a, st);
+    case 5: return launch_gemv_rb<FMT, 5>(a, st);
+    case 6: return launch_gemv_rb<FMT, 6>(a, st);
+    case 7: return launch_gemv_rb<FMT, 7>(a, st);
+    case 8: return launch_gemv_rb<FMT, 8>(a, st);
+  }
+  return fail(DSGX_EINVAL, "gemv: %d rows a launch", M);
+}
+
+int ilog2_exact(int v) {
+  int l = 0;
+  while ((1 << l) < v) ++l;
+  return (1 << l) == v ? l : -1;
+}
+
+// one launch: the segments of one format (gemv_one of the reference, gemv.cu:459-516)
+int gemv_one(int fmt, const uint16_t* x, int ldx, int rows, int K, const dsgx_gemv_seg* segs, int nseg, int out, hipStream_t st) {
+  GemvArgs a{};
+  a.x = x, a.ldx = ldx, a.K = K, a.out = out, a.nsegs = nseg;
+  const int segk = fmt == DSGX_FMT_FP8_B128 ? 1024 : fmt == DSGX_FMT_INT4_G32 ? 2048 : 512;
+  a.nsegk = (K + segk - 1) / segk;
+  a.nq = a.nsegk * segk / 8;
+  int row0 = 0;
+  for (int i = 0; i < nseg; ++i) {
+    const dsgx_gemv_seg& g = segs[i];
+    GemvSegDev& d = a.sg[i];
+    d.m.w = static_cast<const uint8_t*>(g.w);
+    d.m.s = static_cast<const uint8_t*>(g.s);
+    d.m.zp = static_cast<const uint8_t*>(g.zp);
+    d.m.s2 = 1.f;
+    if (!g.w || !g.y) return fail(DSGX_EINVAL, "gemv: segment %d has a null weight or output", i);
+    if (fmt == DSGX_FMT_FP8_B128) {
+      d.m.lrs = ilog2_exact(g.rs), d.m.lks = ilog2_exact(g.ks);
+      if (!g.s || d.m.lrs < 0 || d.m.lks < 4 || K % g.ks) return fail(DSGX_EINVAL, "gemv: FP8 segment %d scale block %dx%d (powers of two, k >= 16)", i, g.rs, g.ks);
+      if (out == DSGX_OUT_SWIGLU) return fail(DSGX_EUNSUPPORTED, "gemv: SwiGLU output over FP8 weights is not built");
+      d.m.srow = K >> d.m.lks;
+    } else if (fmt == DSGX_FMT_INT4_G32) {
+      if (!g.s || !g.zp) return fail(DSGX_EINVAL, "gemv: INT4 segment %d needs scales and zero points", i);
+    }
+    d.y = g.y, d.n = g.n, d.ldy = g.ldy, d.row0 = row0;
+    row0 += g.n;
+  }
+  a.total_rows = row0;
+  if (rows > 8) return fail(DSGX_EINVAL, "gemv_one: %d rows", rows);
+  switch (fmt) {
+    case DSGX_FMT_FP8_B128: return launch_gemv_m<DSGX_FMT_FP8_B128>(rows, a, st);
+    case DSGX_FMT_INT4_G32: return launch_gemv_m<DSGX_FMT_INT4_G32>(rows, a, st);
+    case DSGX_FMT_BF16: return launch_gemv_m<DSGX_FMT_BF16>(rows, a, st);
+  }
+  return fail(DSGX_EFORMAT, "gemv: format %d", fmt);
+}
+
+}  // namespace
+}  // namespace dsgx
+
+using namespace dsgx;
+
+extern "C" int dsgx_gemv(const uint16_t* x, int ldx, int rows, int K, const dsgx_gemv_seg* segs, int nseg, int out, int splitk,
+                         void* stream) {
+  // argument checks of the reference (gemv.cu:524-543): it dies, this returns an error
+  if (rows < 1 || rows > DSGX_MAX_ROWS) return fail(DSGX_EINVAL, "gemv: %d rows", rows);
+  if (!x || !segs || nseg < 1 || nseg > kMaxSegs) return fail(DSGX_EINVAL, "gemv: K %d, %d segments", K, nseg);
+  if (K < 32 || K % 32 || ldx < K || ldx % 8) return fail(DSGX_EINVAL, "gemv: K %d (a multiple of 32), ldx %d (>= K, a multiple of 8)", K, ldx);
+  if (splitk != 1 && splitk != 2 && splitk != 4) return fail(DSGX_EINVAL, "gemv: splitk %d", splitk);
+  if (out != DSGX_OUT_BF16 && out != DSGX_OUT_F32 && out != DSGX_OUT_SWIGLU) return fail(DSGX_EINVAL, "gemv: output kind %d", out);
+  for (int i = 0; i < nseg; ++i) {
+    const int f = segs[i].fmt;
+    if (f != DSGX_FMT_BF16 && f != DSGX_FMT_INT4_G32 && f != DSGX_FMT_FP8_B128)
+      return fail(DSGX_EFORMAT, "gemv: segment %d has no supported weight format (%d)", i, f);
+    if (segs[i].n < 8 || segs[i].n % 8) return fail(DSGX_EINVAL, "gemv: segment %d has %d rows", i, segs[i].n);
+  }
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  // one launch a format, in the order BF16, INT4, FP8 (outputs do not depend on it); more than 8 activation rows run
+  // as two passes over the weights
+  for (int fmt : {DSGX_FMT_BF16, DSGX_FMT_INT4_G32, DSGX_FMT_FP8_B128}) {
+    dsgx_gemv_seg g[kMaxSegs];
+    int n = 0;
+    for (int i = 0; i < nseg; ++i)
+      if (segs[i].fmt == fmt) g[n++] = segs[i];
+    if (!n) continue;
+    for (int r0 = 0; r0 < rows; r0 += 8) {
+      const int nr = rows - r0 < 8 ? rows - r0 : 8;
+      dsgx_gemv_seg gg[kMaxSegs];
+      for (int i = 0; i < n; ++i) {
+        gg[i] = g[i];
+        const size_t esz = out == DSGX_OUT_F32 ? 4 : 2;
+        gg[i].y = static_cast<uint8_t*>(g[i].y) + (size_t)r0 * g[i].ldy * esz;
+      }
+      const int rc = gemv_one(fmt, x + (size_t)r0 * ldx, ldx, nr, K, gg, n, out, st);
+      if (rc) return rc;
+    }
+  }
+  return DSGX_OK;
+}

@@ -1,0 +1,143 @@
+"""Loader of the C ABI (dsgx10_amd/csrc/libdsgx.so) and the Python mirror of the reference's operators for this path
+(gx::route, gx::moe_decode, gx::moe_prefill, gx::finalize, glm::gemv, glm::dequant_int4): same names, argument
+meaning and error behaviour (the reference dies; these raise DsgxError). torch is used for device memory and
+streams only. There is no CPU path: a missing library raises."""
+import ctypes as C
+import os
+
+from . import abi
+
+_SO = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc", "libdsgx.so")
+_lib = None
+
+
+class DsgxError(RuntimeError):
+    def __init__(self, code, msg):
+        super().__init__("dsgx status %d: %s" % (code, msg))
+        self.code = code
+
+
+def so_path():
+    return _SO
+
+
+def lib():
+    """The loaded C ABI. Raises if the HIP extension has not been built (python -m dsgx10_amd.build)."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_SO):
+            raise RuntimeError("dsgx10_amd: %s is missing; build it with `python -m dsgx10_amd.build` (there is no CPU fallback)" % _SO)
+        L = C.CDLL(_SO)
+        L.dsgx_last_error.restype = C.c_char_p
+        L.dsgx_version.restype = C.c_char_p
+        for f in ("dsgx_mat_bytes", "dsgx_mat_scale_off", "dsgx_mat_zp_off"):
+            getattr(L, f).restype = C.c_size_t
+            getattr(L, f).argtypes = [C.c_uint32, C.c_int, C.c_int]
+        L.dsgx_decode_ws_bytes.restype = C.c_size_t
+        L.dsgx_decode_ws_bytes.argtypes = [C.POINTER(abi.LayerW)]
+        L.dsgx_route.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_float, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]
+        L.dsgx_moe_decode.argtypes = [C.POINTER(abi.LayerW), C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p,
+                                      C.c_void_p, C.c_void_p, C.c_void_p, C.POINTER(abi.DecodeCfg)]
+        L.dsgx_finalize.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p]
+        L.dsgx_gemv.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.POINTER(abi.GemvSeg), C.c_int, C.c_int, C.c_int, C.c_void_p]
+        for f in ("dsgx_dequant_int4", "dsgx_probe_dequant_int4"):
+            getattr(L, f).argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_size_t, C.c_void_p]
+        L.dsgx_widen_fp8.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_size_t, C.c_void_p]
+        L.dsgx_act_quant.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]
+        L.dsgx_stream_read.argtypes = [C.c_void_p, C.c_size_t, C.c_void_p, C.c_void_p]
+        L.dsgx_stream_copy.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]
+        if hasattr(L, "dsgx_moe_prefill"):
+            L.dsgx_prefill_ws_bytes.restype = C.c_size_t
+            L.dsgx_prefill_ws_bytes.argtypes = [C.POINTER(abi.LayerW), C.c_int]
+            L.dsgx_moe_prefill.argtypes = [C.POINTER(abi.LayerW), C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p,
+                                           C.c_void_p, C.c_void_p, C.c_void_p, C.POINTER(abi.PrefillCfg)]
+            L.dsgx_prefill_view_get.argtypes = [C.POINTER(abi.LayerW), C.c_void_p, C.c_int, C.POINTER(abi.PrefillView)]
+        _lib = L
+    return _lib
+
+
+def _check(rc):
+    if rc:
+        raise DsgxError(rc, lib().dsgx_last_error().decode())
+
+
+def _ptr(t):
+    return None if t is None else t.data_ptr()
+
+
+def _stream(stream=None):
+    import torch
+    s = stream if stream is not None else torch.cuda.current_stream()
+    return s.cuda_stream
+
+
+# ---- gx::route ------------------------------------------------------------------------------------------------------
+def route(logits, bias, idx, w, route_scale=2.5, score_fn=0, stream=None):
+    """logits f32 [M][E], bias f32 [E] or None -> idx i32 [M][topk], w f32 [M][topk] (filled)."""
+    M, E = logits.shape
+    topk = idx.shape[1]
+    _check(lib().dsgx_route(_ptr(logits), _ptr(bias), M, E, topk, route_scale, score_fn, _ptr(idx), _ptr(w), _stream(stream)))
+
+
+# ---- gx::moe_decode ---------------------------------------------------------------------------------------------------
+def decode_ws_bytes(layer_w):
+    return lib().dsgx_decode_ws_bytes(C.byref(layer_w))
+
+
+def moe_decode(layer_w, x, idx, w, M, ws, yr, ys, stream=None, parts=3, ysum=False, logits=None, bias=None,
+               route_scale=1.0, score_fn=0, up=0, down=0, post=None):
+    cfg = abi.DecodeCfg(up, down, parts, int(ysum), _ptr(logits), _ptr(bias), route_scale, score_fn, post)
+    _check(lib().dsgx_moe_decode(C.byref(layer_w), _ptr(x), _ptr(idx), _ptr(w), M, _ptr(ws), _ptr(yr), _ptr(ys),
+                                 _stream(stream), C.byref(cfg)))
+
+
+def finalize(R, S, out, stream=None):
+    _check(lib().dsgx_finalize(_ptr(R), _ptr(S), R.numel(), _ptr(out), _stream(stream)))
+
+
+# ---- gx::moe_prefill --------------------------------------------------------------------------------------------------
+def prefill_ws_bytes(layer_w, T):
+    return lib().dsgx_prefill_ws_bytes(C.byref(layer_w), T)
+
+
+def moe_prefill(layer_w, x, idx, w, T, ws, yr, ys, stream=None, shared=True, phases=31, act_fp8=True):
+    cfg = abi.PrefillCfg(int(shared), phases, int(act_fp8))
+    _check(lib().dsgx_moe_prefill(C.byref(layer_w), _ptr(x), _ptr(idx), _ptr(w), T, _ptr(ws), _ptr(yr), _ptr(ys),
+                                  _stream(stream), C.byref(cfg)))
+
+
+def prefill_view(layer_w, ws, T):
+    v = abi.PrefillView()
+    _check(lib().dsgx_prefill_view_get(C.byref(layer_w), _ptr(ws), T, C.byref(v)))
+    return v
+
+
+# ---- glm::gemv ------------------------------------------------------------------------------------------------------------
+def gemv(x, ldx, rows, K, segs, out, splitk=1, stream=None):
+    """segs: list of dict(fmt, w, s, zp, n, y, ldy, rs=128, ks=128) with torch tensors."""
+    arr = (abi.GemvSeg * len(segs))()
+    for i, g in enumerate(segs):
+        arr[i] = abi.GemvSeg(g["fmt"], _ptr(g["w"]), _ptr(g.get("s")), _ptr(g.get("zp")), g["n"], g.get("rs", 128),
+                             g.get("ks", 128), _ptr(g["y"]), g["ldy"])
+    _check(lib().dsgx_gemv(_ptr(x), ldx, rows, K, arr, len(segs), out, splitk, _stream(stream)))
+
+
+def dequant_int4(packed, scale, zp, N, K, out, ld=None, stream=None, probe=False):
+    f = lib().dsgx_probe_dequant_int4 if probe else lib().dsgx_dequant_int4
+    _check(f(_ptr(packed), _ptr(scale), _ptr(zp), N, K, _ptr(out), ld or K, _stream(stream)))
+
+
+def widen_fp8(codes, N, K, out, ld=None, stream=None):
+    _check(lib().dsgx_widen_fp8(_ptr(codes), N, K, _ptr(out), ld or K, _stream(stream)))
+
+
+def act_quant(x, T, K, q, s, stream=None):
+    _check(lib().dsgx_act_quant(_ptr(x), T, K, _ptr(q), _ptr(s), _stream(stream)))
+
+
+def stream_read(buf, nbytes, sink, stream=None):
+    _check(lib().dsgx_stream_read(_ptr(buf), nbytes, _ptr(sink), _stream(stream)))
+
+
+def stream_copy(src, dst, nbytes, stream=None):
+    _check(lib().dsgx_stream_copy(_ptr(src), _ptr(dst), nbytes, _stream(stream)))

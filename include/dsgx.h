@@ -1,0 +1,191 @@
+/* dsgx.h - the C ABI of the MI355X (gfx950) build of dsgx10's quantised-MoE hot path.
+ *
+ * Every entry point is what the reference engine's own C++ operator for this path would bind through an FFI:
+ * plain pointers and sizes, no C++ types, no HIP types (a stream is passed as void*, it is a hipStream_t).
+ * bf16 values are uint16_t bit patterns. All device pointers are caller-owned; every call is asynchronous on
+ * the given stream and allocates nothing.
+ *
+ * Error convention: every function that can fail returns 0 on success and a non-zero dsgx_status otherwise and
+ * leaves a message in a thread-local buffer (dsgx_last_error()). The reference dies (prints and aborts:
+ * altar1-4xgx10-switchless/engine/common/check.h:8-21); the C++ mirror headers under include/gx, include/glm and
+ * include/dsk turn a non-zero status into the same die().
+ *
+ * Weight formats. The reference's formats tags 0 (NVFP4), 2 (INT4) and 3 (BF16) name GB10 lane-map block tilings
+ * (altar1-4xgx10-switchless/engine/experts/experts.h:29-46). Those tilings are not used here: on gfx950 a 64-lane
+ * wavefront reading 16 bytes a lane covers 1 KiB of a K-contiguous row, so the checkpoint's own row-major tensors are
+ * already the coalesced streaming layout. The tags below name them; the reference's tags are refused.
+ */
+#ifndef DSGX_H_
+#define DSGX_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define DSGX_API __attribute__((visibility("default")))
+
+typedef enum dsgx_status {
+  DSGX_OK = 0,
+  DSGX_EINVAL = 1,      /* an argument the reference would die() on */
+  DSGX_EFORMAT = 2,     /* unknown / unsupported weight format tag (never guessed) */
+  DSGX_EUNSUPPORTED = 3,/* a reference feature that has no meaning on one GPU (ring posting) or is not built */
+  DSGX_EHIP = 4         /* a HIP runtime error (message has hipGetErrorString) */
+} dsgx_status;
+
+/* Weight format tags (dsgx_mat_desc::fmt, dsgx_layer_w::fmt, dsgx_gemv_seg::fmt). */
+enum {
+  DSGX_FMT_REF_NVFP4 = 0, /* reference tilings: refused */
+  DSGX_FMT_REF_INT4 = 2,
+  DSGX_FMT_REF_BF16 = 3,
+  /* FP8 e4m3fn codes u8 [N][K] row-major, then (256-byte aligned) f32 scales [ceil(N/128)][K/128]:
+     W(n,k) = e4m3(code) * S[n/128][k/128]   (engine/experts/tests/testdata.h:120-125, attn/tools/pack.py:216-241) */
+  DSGX_FMT_FP8_B128 = 16,
+  /* compressed-tensors pack-quantized INT4, group 32 along K, asymmetric, the checkpoint's three tensors back to
+     back, each 256-byte aligned: weight_packed u32 [N][K/8] (value k at bits 4(k%8) of word k/8), weight_scale
+     bf16 [N][K/32], weight_zero_point u32 [N/8][K/32] (row n at bits 4(n%8)):
+     W(n,k) = bf16_rne((u - u_z) * s)       (engine/experts/layout.h:24-42, docs/model.md:111-195) */
+  DSGX_FMT_INT4_G32 = 18,
+  /* bf16 bits [N][K] row-major */
+  DSGX_FMT_BF16 = 19
+};
+
+/* Bytes of one [N][K] matrix in a format, parts laid as above (0 for an unknown tag or a bad shape).
+   Mirrors gx::mat_bytes (engine/experts/experts.h:47-50). */
+DSGX_API size_t dsgx_mat_bytes(uint32_t fmt, int N, int K);
+/* Byte offsets, from the matrix's start, of its second and third part (scales; zero points). */
+DSGX_API size_t dsgx_mat_scale_off(uint32_t fmt, int N, int K);
+DSGX_API size_t dsgx_mat_zp_off(uint32_t fmt, int N, int K);
+
+/* One routed matrix of one expert. Mirrors gx::MatDesc, 64 bytes (engine/experts/experts.h:58-64). */
+typedef struct dsgx_mat_desc {
+  uint64_t off;     /* byte offset of the matrix in the pool, a multiple of 256 */
+  float s2;         /* per-tensor f32 factor applied in the epilogue; exactly 1 for INT4, BF16 and FP8_B128 */
+  uint32_t fmt;
+  uint32_t rsv[12]; /* zero */
+} dsgx_mat_desc;
+
+/* A shared expert fused into the routed kernels. Mirrors gx::SharedW (engine/experts/experts.h:66-87).
+   FP8: g, u [I][H] and d [H][I] e4m3 row-major with f32 scales gs, us [I/128][H/128], ds [H/128][I/128].
+   BF16: bgu [2I][H] bf16 row-major with rows 2i = gate i, 2i+1 = up i (the reference's interleave), bd [H][I]. */
+typedef struct dsgx_shared_w {
+  const uint8_t *g, *u, *d;
+  const float *gs, *us, *ds;
+  const uint8_t *bgu, *bd;
+} dsgx_shared_w;
+
+/* One MoE layer's weights. Mirrors gx::LayerW (engine/experts/experts.h:91-97); the reference's compile-time shapes
+   (experts.h:18-26) are runtime fields here. desc is a DEVICE array [E][3]: gate [I][H], up [I][H], down [H][I]. */
+typedef struct dsgx_layer_w {
+  const uint8_t* pool;
+  const dsgx_mat_desc* desc;
+  dsgx_shared_w sh;
+  uint32_t fmt;
+  int32_t H, I, E, topk;
+} dsgx_layer_w;
+
+#define DSGX_MAX_ROWS 16   /* decode rows a step (engine/experts/experts.h:24) */
+#define DSGX_MAX_TOPK 8
+#define DSGX_MAX_UNION (DSGX_MAX_ROWS * DSGX_MAX_TOPK) /* 128 (engine/experts/experts.h:25) */
+#define DSGX_SH_SLOT DSGX_MAX_UNION /* the shared expert's slot in the decode h workspace (experts.h:26) */
+#define DSGX_MAX_EXPERTS 512
+#define DSGX_MAX_CHUNK 8192 /* prefill rows a chunk (engine/experts/experts.h:155) */
+
+/* ---- routing: gx::route (engine/experts/experts.h:99-102, route.cu:11-33) --------------------------------------
+   logits f32 [M][E], bias f32 [E] (selection only; may be null = 0) -> idx i32 [M][topk] (descending key, ties to the
+   lower id), w f32 [M][topk] = s / (sum + 1e-20) * route_scale, s = sigmoid(logit). topk <= 8, E <= 512.
+   score_fn 0: sigmoid (GLM / DeepSeek-V3); 1: sqrt(softplus) (ds41f-4xgx10-switchless/engine/kernels/common.cuh:261-315). */
+DSGX_API int dsgx_route(const float* logits, const float* bias, int M, int E, int topk, float route_scale, int score_fn,
+                        int* idx, float* w, void* stream);
+
+/* ---- decode: gx::moe_decode (engine/experts/experts.h:104-147, decode.cu:708-730) ------------------------------- */
+typedef struct dsgx_decode_cfg {
+  int32_t up, down;        /* kernel variants (0 = default) */
+  int32_t parts;           /* 1 up only, 2 down only, 3 both (bench) */
+  int32_t ysum;            /* 1: yr += ys in f32 after the routed experts (experts.h:132-136) */
+  const float* logits;     /* fused routing (experts.h:123-127): with logits (+ optional bias) idx, w are not read */
+  const float* bias;
+  float route_scale;       /* used by fused routing */
+  int32_t score_fn;
+  const void* post;        /* the reference's ring channel (experts.h:128-131): must be null on one GPU */
+} dsgx_decode_cfg;
+DSGX_API void dsgx_decode_cfg_default(dsgx_decode_cfg* cfg);
+/* Workspace bytes of a decode step (gx::decode_ws_bytes; engine/experts/decode.cu:33-35): h bf16
+   [DSGX_MAX_UNION + 1 slots][DSGX_MAX_ROWS][I] plus 256 bytes of counters. Zero it once before the first call. */
+DSGX_API size_t dsgx_decode_ws_bytes(const dsgx_layer_w* L);
+/* x bf16 [M][H]; idx, w from dsgx_route; yr, ys f32 [M][H]. ys is written when the layer has a fused shared expert,
+   otherwise it is an input (only read with ysum). h of the step stays in ws: slot s (the s-th picked expert in
+   expert-id order) at ((s * M + m) * I + c), the shared expert's at slot DSGX_SH_SLOT. */
+DSGX_API int dsgx_moe_decode(const dsgx_layer_w* L, const uint16_t* x, const int* idx, const float* w, int M, void* ws,
+                             float* yr, float* ys, void* stream, const dsgx_decode_cfg* cfg);
+/* out = bf16(bf16(R) + bf16(S)): gx::finalize (engine/experts/experts.h:146-147, decode.cu:591-598) */
+DSGX_API int dsgx_finalize(const float* R, const float* S, int n, uint16_t* out, void* stream);
+
+/* ---- prefill: gx::moe_prefill (engine/experts/experts.h:149-193, prefill.cu:1056-1116) --------------------------- */
+typedef struct dsgx_prefill_cfg {
+  int32_t shared;   /* run the fused shared expert (if the layer has one) */
+  int32_t phases;   /* gx::PrefillPhase bits: 1 bucket, 2 up, 4 down, 8 combine, 16 shared; 31 all */
+  int32_t act_fp8;  /* FP8 layers: 1 = quantise activations per row and 128 k to e4m3 and run the fp8 MFMA
+                       (ds41f-4xgx10-switchless/ref/torchref/kernel.py:56-77, ref/inference/kernel.py:207-274);
+                       0 = bf16 activations, weights widened to bf16 (the altar-1 contract) */
+} dsgx_prefill_cfg;
+DSGX_API void dsgx_prefill_cfg_default(dsgx_prefill_cfg* cfg);
+DSGX_API size_t dsgx_prefill_ws_bytes(const dsgx_layer_w* L, int T);
+DSGX_API int dsgx_moe_prefill(const dsgx_layer_w* L, const uint16_t* x, const int* idx, const float* w, int T, void* ws,
+                              float* yr, float* ys, void* stream, const dsgx_prefill_cfg* cfg);
+/* The workspace's intermediates after a call (gx::prefill_view, experts.h:184-190): device pointers into ws. */
+typedef struct dsgx_prefill_view {
+  const int *rpos, *re;      /* [T][topk]: per row its picks in expert-id order: bucket position, expert */
+  const uint16_t *h, *hsh;   /* h bf16 [position][I]; shared expert's h [T][I] */
+  const int *off;            /* [E+1] bucket offsets */
+  const int *perm;           /* [T*topk] bucket position -> row */
+} dsgx_prefill_view;
+DSGX_API int dsgx_prefill_view_get(const dsgx_layer_w* L, void* ws, int T, dsgx_prefill_view* out);
+
+/* ---- dense GEMV: glm::gemv (engine/attn/attn.h:59-123, gemv.cu:522-543) ------------------------------------------ */
+enum { DSGX_OUT_BF16 = 0, DSGX_OUT_F32 = 1, DSGX_OUT_SWIGLU = 2 };
+typedef struct dsgx_gemv_seg {
+  int32_t fmt;        /* DSGX_FMT_BF16, DSGX_FMT_INT4_G32, DSGX_FMT_FP8_B128 */
+  const void* w;      /* the matrix in its format; INT4: weight_packed */
+  const void* s;      /* FP8: f32 scales [ceil(N/rs)][K/ks]; INT4: bf16 scales [N][K/32] */
+  const void* zp;     /* INT4: weight_zero_point u32 [N/8][K/32] */
+  int32_t n;          /* rows of W (outputs), a multiple of 8 */
+  int32_t rs, ks;     /* FP8 scale block (rows, k): 128, 128 */
+  void* y;
+  int32_t ldy;        /* y's row stride in elements */
+} dsgx_gemv_seg;
+/* y[r][n] = sum_k x[r][k] W[n][k]; x bf16 [rows][ldx], rows 1..16, K a multiple of 128 (INT4: of 256).
+   out: DSGX_OUT_*; SwiGLU: rows interleaved gate/up in pairs. splitk is accepted for signature parity and ignored
+   (K is always split over the 64 lanes of a wavefront and reduced by cross-lane shuffles). */
+DSGX_API int dsgx_gemv(const uint16_t* x, int ldx, int rows, int K, const dsgx_gemv_seg* segs, int nseg, int out,
+                       int splitk, void* stream);
+/* glm::dequant_int4 (engine/attn/attn.h:154-158): the contract's bf16 weight [N][ld] from the canonical tensors */
+DSGX_API int dsgx_dequant_int4(const void* packed, const void* scale, const void* zp, int N, int K, uint16_t* out,
+                               size_t ld, void* stream);
+/* The same through the streaming kernels' own in-register decode: the probe that pins the hot loops' INT4 arithmetic to
+   the contract bit for bit, as the reference's k_deq does (engine/experts/tests/test_experts.cu:217-235). Exact for
+   |scale| < 2^124 (the checkpoint's scales are 2^-15 .. 2^-4); dsgx_dequant_int4 is exact for every finite scale. */
+DSGX_API int dsgx_probe_dequant_int4(const void* packed, const void* scale, const void* zp, int N, int K, uint16_t* out,
+                                     size_t ld, void* stream);
+/* FP8 codes -> bf16 bits of the exact e4m3 values [N][ld] (the widening the GEMV and MoE kernels use;
+   engine/experts/formats.cuh:121-128, tests/test_experts.cu:124-134) */
+DSGX_API int dsgx_widen_fp8(const void* codes, int N, int K, uint16_t* out, size_t ld, void* stream);
+/* act_quant(x, 128): x bf16 [T][K] -> e4m3 codes [T][K], f32 scales [T][K/128]
+   (ds41f-4xgx10-switchless/ref/torchref/kernel.py:56-77) */
+DSGX_API int dsgx_act_quant(const uint16_t* x, int T, int K, uint8_t* q, float* s, void* stream);
+
+/* ---- misc ---------------------------------------------------------------------------------------------------- */
+DSGX_API const char* dsgx_last_error(void);
+DSGX_API const char* dsgx_version(void);
+/* A plain streaming-read kernel over n bytes (the bandwidth baseline the bench prints beside the kernels,
+   as engine/experts/tests/bench_experts.cu:102-130 does); sink: 4 bytes of device memory. */
+DSGX_API int dsgx_stream_read(const void* p, size_t n, void* sink, void* stream);
+/* A plain copy kernel (the reference for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE counters). */
+DSGX_API int dsgx_stream_copy(const void* src, void* dst, size_t n, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DSGX_H_ */

@@ -1,0 +1,615 @@
+// oracle.cpp - TEST INFRASTRUCTURE, NOT PRODUCT CODE.
+//
+// A CPU restatement (C++17, OpenMP) of the arithmetic contract of dsgx10's quantised-MoE hot path, used only as the
+// checker in tests/, in __graft_entry__.smoke() and as the timed CPU baseline of bench.py. Nothing in the product
+// (dsgx10_amd/, include/) links, loads or calls it, and the product has no CPU fallback.
+//
+// Each function names the reference lines it restates (paths relative to the reference tree; A/ =
+// altar1-4xgx10-switchless/, D/ = ds41f-4xgx10-switchless/). The reference's own implementation of this path is CUDA
+// for sm_121a with inline PTX and cannot be compiled here, so there is no oracle/_ref build; the functions below are
+// pinned by closed forms, exhaustive checks, torch-CPU library routines and brute force in tests/test_oracle_*.py.
+//
+// Pinned: bf16 RNE, e4m3 decode/encode, INT4 dequant, FP8 quantiser and dequant, act_quant, router, union,
+// GEMV and MoE sums (f32 contract order, f64 and sum of |terms|). Parity unpinned: none of the functions here; the
+// INT4 *quantiser* (orc_int4_quantize_sym) has no reference counterpart at all (the reference never quantises INT4)
+// and is this build's own definition.
+//
+// Build: make -C oracle   (gcc -O3 -march=x86-64-v3 -fopenmp -ffp-contract=off)
+#include <algorithm>
+#include <cmath>
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <vector>
+#include <omp.h>
+
+#include "../include/dsgx.h"
+
+#define ORC extern "C" __attribute__((visibility("default")))
+
+// ---- codecs ------------------------------------------------------------------------------------------------------
+// A/engine/experts/formats.cuh:32-38
+static inline float bf2f(uint16_t b) { uint32_t u = (uint32_t)b << 16; float f; memcpy(&f, &u, 4); return f; }
+static inline uint16_t f2bf(float f) {  // round to nearest even (finite f, subnormals included)
+  uint32_t u; memcpy(&u, &f, 4);
+  u += 0x7FFFu + ((u >> 16) & 1u);
+  return (uint16_t)(u >> 16);
+}
+static inline float bfr(float f) { return bf2f(f2bf(f)); }
+// OCP e4m3fn, closed form (A/engine/attn/tests/attn_tests.cu:33-37): e ? 2^(e-7)(1+m/8) : 2^-6 m/8; 0x7F/0xFF NaN
+static inline float e4m3f(uint8_t b) {
+  const int e = (b >> 3) & 15, m = b & 7;
+  float v;
+  if (e == 15 && m == 7) v = NAN;
+  else v = e ? ldexpf(1.f + m / 8.f, e - 7) : ldexpf(m / 8.f, -6);
+  return (b & 0x80) ? -v : v;
+}
+// f32 -> e4m3fn, round to nearest even, what torch's Tensor.to(torch.float8_e4m3fn) computes (PyTorch
+// c10/util/Float8_e4m3fn.h fp8e4m3fn_from_fp32_value, the cast inside A/engine/attn/tools/pack.py:229 and
+// D/ref/torchref/kernel.py:29-30): magnitudes >= 480 and NaN give the NaN code, no saturation.
+static inline uint8_t f2e4m3(float f) {
+  uint32_t u; memcpy(&u, &f, 4);
+  const uint32_t sign = u & 0x80000000u;
+  u ^= sign;
+  uint8_t r;
+  if (u >= (1087u << 20)) r = 0x7F;
+  else if (u < (121u << 23)) {  // below 2^-6: the subnormal range, rounded by the float adder
+    const uint32_t dm = 141u << 23;
+    float a, d; memcpy(&a, &u, 4); memcpy(&d, &dm, 4);
+    const float s = a + d;
+    uint32_t sb; memcpy(&sb, &s, 4);
+    r = (uint8_t)(sb - dm);
+  } else {
+    const uint32_t odd = (u >> 20) & 1u;
+    u += ((uint32_t)(7 - 127) << 23) + 0x7FFFFu;
+    u += odd;
+    r = (uint8_t)(u >> 20);
+  }
+  return r | (uint8_t)(sign >> 24);
+}
+
+ORC uint16_t orc_f32_to_bf16(float f) { return f2bf(f); }
+ORC float orc_bf16_to_f32(uint16_t b) { return bf2f(b); }
+ORC float orc_e4m3_to_f32(uint8_t b) { return e4m3f(b); }
+ORC uint8_t orc_f32_to_e4m3(float f) { return f2e4m3(f); }
+ORC void orc_f32_to_bf16_n(const float* f, size_t n, uint16_t* o) {
+#pragma omp parallel for
+  for (size_t i = 0; i < n; ++i) o[i] = f2bf(f[i]);
+}
+ORC void orc_f32_to_e4m3_n(const float* f, size_t n, uint8_t* o) {
+#pragma omp parallel for
+  for (size_t i = 0; i < n; ++i) o[i] = f2e4m3(f[i]);
+}
+
+// ---- seeded data: splitmix64 (A/engine/experts/formats.cuh:131-136) -> Box-Muller ------------------------------------
+static inline uint64_t mix64(uint64_t x) {
+  x += 0x9E3779B97F4A7C15ull;
+  x = (x ^ (x >> 30)) * 0xBF58476D1CE4E5B9ull;
+  x = (x ^ (x >> 27)) * 0x94D049BB133111EBull;
+  return x ^ (x >> 31);
+}
+ORC uint64_t orc_mix64(uint64_t x) { return mix64(x); }
+// N(0,1) number i of tensor `tid` under `seed`: a = mix64(seed * 0x100000001B3 + tid); h1 = mix64(a + 2i),
+// h2 = mix64(a + 2i + 1); u1 = ((h1 >> 11) + 1) 2^-53 in (0, 1], u2 = (h2 >> 11) 2^-53 in [0, 1);
+// z = sqrt(-2 ln u1) cos(2 pi u2), all in f64.
+static inline double normal_at(uint64_t a, uint64_t i) {
+  const uint64_t h1 = mix64(a + 2 * i), h2 = mix64(a + 2 * i + 1);
+  const double u1 = (double)((h1 >> 11) + 1) * 0x1p-53, u2 = (double)(h2 >> 11) * 0x1p-53;
+  return sqrt(-2.0 * log(u1)) * cos(6.283185307179586476925286766559 * u2);
+}
+static inline uint64_t stream_key(uint64_t seed, uint64_t tid) { return mix64(seed * 0x100000001B3ull + tid); }
+ORC double orc_normal(uint64_t seed, uint64_t tid, uint64_t i) { return normal_at(stream_key(seed, tid), i); }
+ORC void orc_fill_normal_f32(uint64_t seed, uint64_t tid, size_t n, double sigma, float* out) {
+  const uint64_t a = stream_key(seed, tid);
+#pragma omp parallel for
+  for (size_t i = 0; i < n; ++i) out[i] = (float)(sigma * normal_at(a, i));
+}
+ORC void orc_fill_normal_bf16(uint64_t seed, uint64_t tid, size_t n, double sigma, uint16_t* out) {
+  const uint64_t a = stream_key(seed, tid);
+#pragma omp parallel for
+  for (size_t i = 0; i < n; ++i) out[i] = f2bf((float)(sigma * normal_at(a, i)));
+}
+
+// ---- INT4-g32 (compressed-tensors pack-quantized) ----------------------------------------------------------------------
+// canonical readers: A/engine/experts/layout.h:33-34 and docs/model.md:111-114,136-139
+static inline int i4_nib(const uint32_t* packed, int K, int n, int k) { return (packed[(size_t)n * (K / 8) + k / 8] >> (4 * (k & 7))) & 15; }
+static inline int i4_zp(const uint32_t* zp, int K, int n, int g) { return (zp[(size_t)(n / 8) * (K / 32) + g] >> (4 * (n & 7))) & 15; }
+// the contract: A/engine/experts/formats.cuh:117-119
+static inline uint16_t i4_bits(int u, int uz, uint16_t s) { return f2bf((float)(u - uz) * bf2f(s)); }
+ORC uint16_t orc_int4_value_bits(int u, int uz, uint16_t s) { return i4_bits(u, uz, s); }
+// A/engine/experts/layout.h:40-42 (canon_i4) over a whole matrix; A/engine/attn/tools/pack.py:76-83
+ORC void orc_int4_dequant(const uint32_t* packed, const uint16_t* scale, const uint32_t* zp, int N, int K, uint16_t* out) {
+#pragma omp parallel for
+  for (int n = 0; n < N; ++n)
+    for (int k = 0; k < K; ++k)
+      out[(size_t)n * K + k] = i4_bits(i4_nib(packed, K, n, k), i4_zp(zp, K, n, k / 32), scale[(size_t)n * (K / 32) + k / 32]);
+}
+// This build's own symmetric quantiser (the reference has none: its INT4 weights are the checkpoint's bytes):
+// per group of 32: s = bf16_rne(amax / 7) (1.0 for an all-zero group), q = clamp(rint(w / s), -8, 7), stored
+// u = q + 8, stored zero point 8.
+ORC void orc_int4_quantize_sym(const float* w, int N, int K, uint32_t* packed, uint16_t* scale, uint32_t* zp) {
+  const int G = K / 32;
+  memset(packed, 0, (size_t)N * (K / 8) * 4);
+#pragma omp parallel for
+  for (int n = 0; n < N; ++n)
+    for (int g = 0; g < G; ++g) {
+      const float* p = w + (size_t)n * K + 32 * g;
+      float amax = 0.f;
+      for (int i = 0; i < 32; ++i) amax = std::max(amax, fabsf(p[i]));
+      uint16_t sb = amax > 0.f ? f2bf(amax / 7.f) : (uint16_t)0x3F80;
+      if (bf2f(sb) == 0.f) sb = 0x0080;  // never a zero scale
+      const float s = bf2f(sb);
+      scale[(size_t)n * G + g] = sb;
+      for (int i = 0; i < 32; ++i) {
+        int q = (int)nearbyintf(p[i] / s);
+        q = std::min(7, std::max(-8, q));
+        packed[(size_t)n * (K / 8) + (32 * g + i) / 8] |= (uint32_t)(q + 8) << (4 * (i & 7));
+      }
+    }
+  for (size_t i = 0; i < (size_t)(N / 8) * G; ++i) zp[i] = 0x88888888u;
+}
+// Random asymmetric INT4 tensors as the reference's tests make them (A/engine/experts/tests/testdata.h:45-48,70-82):
+// every nibble and zero point value, scales positive bf16 in [2^-9, 2^-5) with a random mantissa.
+ORC void orc_int4_random(uint64_t seed, int N, int K, uint32_t* packed, uint16_t* scale, uint32_t* zp) {
+  uint8_t* pb = reinterpret_cast<uint8_t*>(packed);
+  const size_t nb = (size_t)N * K / 2, ns = (size_t)N * K / 32, nz = (size_t)N / 8 * K / 32;
+#pragma omp parallel for
+  for (size_t i = 0; i < nb; ++i) pb[i] = (uint8_t)mix64(seed * 1000003 + i);
+#pragma omp parallel for
+  for (size_t i = 0; i < ns; ++i) {
+    const uint64_t h = mix64(seed * 7919 + i + (1ull << 40));
+    scale[i] = (uint16_t)(((118 + h % 4) << 7) | ((h >> 8) & 0x7F));
+  }
+#pragma omp parallel for
+  for (size_t i = 0; i < nz; ++i) zp[i] = (uint32_t)mix64(seed * 104729 + i + (1ull << 41));
+}
+
+// ---- FP8 e4m3, one f32 scale per 128x128 block --------------------------------------------------------------------------
+// the quantiser: A/engine/attn/tools/pack.py:216-232 (fp8_from_master): per block amax over the zero-padded block,
+// scale = max(f32(amax) * f32(1/448), 1e-12), code = e4m3_rne(f32(w) / scale). scales [ceil(N/128)][K/128].
+ORC void orc_fp8_quantize(const float* w, int N, int K, uint8_t* codes, float* scales) {
+  const int NB = (N + 127) / 128, KB = K / 128;
+  const float r448 = 1.0f / 448.0f;
+#pragma omp parallel for collapse(2)
+  for (int nb = 0; nb < NB; ++nb)
+    for (int kb = 0; kb < KB; ++kb) {
+      float amax = 0.f;
+      const int n1 = std::min(N, 128 * nb + 128);
+      for (int n = 128 * nb; n < n1; ++n)
+        for (int k = 128 * kb; k < 128 * kb + 128; ++k) amax = std::max(amax, fabsf(w[(size_t)n * K + k]));
+      float s = amax * r448;
+      if (s < 1e-12f) s = 1e-12f;
+      scales[(size_t)nb * KB + kb] = s;
+      for (int n = 128 * nb; n < n1; ++n)
+        for (int k = 128 * kb; k < 128 * kb + 128; ++k) codes[(size_t)n * K + k] = f2e4m3(w[(size_t)n * K + k] / s);
+    }
+}
+// W = e4m3 * S: A/engine/experts/tests/testdata.h:120-125, A/engine/attn/tools/pack.py:235-241
+ORC void orc_fp8_dequant(const uint8_t* codes, const float* scales, int N, int K, float* out) {
+  const int KB = K / 128;
+#pragma omp parallel for
+  for (int n = 0; n < N; ++n)
+    for (int k = 0; k < K; ++k) out[(size_t)n * K + k] = e4m3f(codes[(size_t)n * K + k]) * scales[(size_t)(n / 128) * KB + k / 128];
+}
+// Random FP8 tensors as the reference's tests make them (A/engine/experts/tests/testdata.h:126-140): random bytes
+// with the top magnitudes and the NaN codes removed, scales = scale * (0.5 + (hash % 1000) / 1000).
+ORC void orc_fp8_random(uint64_t seed, int N, int K, float scale, uint8_t* codes, float* scales) {
+  const size_t nw = (size_t)N * K, ns = (size_t)((N + 127) / 128) * (K / 128);
+#pragma omp parallel for
+  for (size_t i = 0; i < nw; ++i) {
+    uint8_t v = (uint8_t)mix64(seed * 1000003 + i);
+    if ((v & 0x78) > 0x48) v &= 0xC7;
+    codes[i] = v;
+  }
+  for (size_t i = 0; i < ns; ++i) scales[i] = scale * (0.5f + (float)(mix64(seed + i) % 1000) / 1000.f);
+}
+// act_quant(x, 128) on bf16 rows: D/ref/torchref/kernel.py:56-77 (scale_fmt None): amax per 128 clamped to >= 1e-4,
+// s = amax * f32(1/448), q = e4m3_rne(clamp(x / s, -448, 448)).
+ORC void orc_act_quant(const uint16_t* x, int T, int K, uint8_t* q, float* s) {
+  const int KB = K / 128;
+  const float r448 = 1.0f / 448.0f;
+#pragma omp parallel for
+  for (int t = 0; t < T; ++t)
+    for (int b = 0; b < KB; ++b) {
+      const uint16_t* p = x + (size_t)t * K + 128 * b;
+      float amax = 0.f;
+      for (int i = 0; i < 128; ++i) amax = std::max(amax, fabsf(bf2f(p[i])));
+      if (amax < 1e-4f) amax = 1e-4f;
+      const float sc = amax * r448;
+      s[(size_t)t * KB + b] = sc;
+      for (int i = 0; i < 128; ++i) {
+        float v = bf2f(p[i]) / sc;
+        v = std::min(448.f, std::max(-448.f, v));
+        q[(size_t)t * K + 128 * b + i] = f2e4m3(v);
+      }
+    }
+}
+
+// ---- router ---------------------------------------------------------------------------------------------------------------
+// A/engine/experts/formats.cuh:142-163, IEEE operations only (compile with -ffp-contract=off)
+static inline float route_sigmoid(float l) {
+  const float x = -l;
+  if (x > 88.f) return 0.f;
+  if (x < -87.f) return 1.f;
+  const float n = rintf(x * 1.44269504f);
+  float r = fmaf(-n, 0.693145751953125f, x);
+  r = fmaf(-n, 1.428606765330187e-06f, r);
+  float p = 1.f / 5040;
+  p = fmaf(p, r, 1.f / 720);
+  p = fmaf(p, r, 1.f / 120);
+  p = fmaf(p, r, 1.f / 24);
+  p = fmaf(p, r, 1.f / 6);
+  p = fmaf(p, r, 0.5f);
+  p = fmaf(p, r, 1.f);
+  p = fmaf(p, r, 1.f);
+  const float e = ldexpf(p, (int)n);
+  return 1.f / (1.f + e);
+}
+ORC float orc_route_sigmoid(float l) { return route_sigmoid(l); }
+// The sum of the picked scores in the butterfly order over eight places, absent places skipped:
+// 8 picks ((p0+p4)+(p2+p6))+((p1+p5)+(p3+p7)) (A/engine/experts/formats.cuh:166-168),
+// 6 picks ((p0+p4)+p2)+((p1+p5)+p3) (D/engine/kernels/common.cuh:310).
+static inline float route_sum(const float* p, int k) {
+  float q[8];
+  for (int i = 0; i < 8; ++i) q[i] = i < k ? p[i] : 0.f;
+  auto add = [](float a, float b, bool hb) { return hb ? a + b : a; };
+  const float a04 = add(q[0], q[4], 4 < k), a26 = add(q[2], q[6], 6 < k), a15 = add(q[1], q[5], 5 < k), a37 = add(q[3], q[7], 7 < k);
+  const float l = add(a04, a26, 2 < k), r = add(a15, a37, 3 < k);
+  return add(l, r, 1 < k);
+}
+// A/engine/experts/tests/testdata.h:339-355 (route_ref) with E, top-k and the scale as arguments; bias may be null.
+// score_fn 1: sqrt(softplus(l)), softplus as torch's (l > 20 ? l : log1p(exp(l))): D/engine/kernels/common.cuh:261-315.
+ORC void orc_route(const float* l, const float* bias, int M, int E, int topk, float scale, int score_fn, int* idx, float* w) {
+  std::vector<float> s(E), key(E);
+  for (int m = 0; m < M; ++m) {
+    for (int e = 0; e < E; ++e) {
+      const float v = l[(size_t)m * E + e];
+      s[e] = score_fn == 0 ? route_sigmoid(v) : sqrtf(v > 20.f ? v : log1pf(expf(v)));
+      key[e] = s[e] + (bias ? bias[e] : 0.f);
+    }
+    float p[8];
+    for (int k = 0; k < topk; ++k) {
+      int b = -1;
+      for (int e = 0; e < E; ++e)
+        if (key[e] != -INFINITY && (b < 0 || key[e] > key[b])) b = e;
+      idx[m * topk + k] = b;
+      p[k] = s[b];
+      key[b] = -INFINITY;
+    }
+    const float sum = route_sum(p, topk) + 1e-20f;
+    for (int k = 0; k < topk; ++k) w[m * topk + k] = p[k] / sum * scale;
+  }
+}
+
+// ---- matrices in the pool formats (include/dsgx.h) ----------------------------------------------------------------------------
+static inline size_t al256(size_t b) { return (b + 255) / 256 * 256; }
+struct Mat {
+  uint32_t fmt; int N, K; float s2;
+  const uint8_t* codes = nullptr; const float* fs = nullptr;                               // FP8
+  const uint32_t* packed = nullptr; const uint16_t* bs = nullptr; const uint32_t* zp = nullptr;  // INT4
+  const uint16_t* b16 = nullptr;                                                          // BF16
+};
+static Mat mat_at(const uint8_t* base, uint32_t fmt, int N, int K, float s2) {
+  Mat m; m.fmt = fmt; m.N = N; m.K = K; m.s2 = s2;
+  if (fmt == DSGX_FMT_FP8_B128) {
+    m.codes = base; m.fs = reinterpret_cast<const float*>(base + al256((size_t)N * K));
+  } else if (fmt == DSGX_FMT_INT4_G32) {
+    m.packed = reinterpret_cast<const uint32_t*>(base);
+    m.bs = reinterpret_cast<const uint16_t*>(base + al256((size_t)N * K / 2));
+    m.zp = reinterpret_cast<const uint32_t*>(base + al256((size_t)N * K / 2) + al256((size_t)N * (K / 32) * 2));
+  } else if (fmt == DSGX_FMT_BF16) {
+    m.b16 = reinterpret_cast<const uint16_t*>(base);
+  } else {
+    fprintf(stderr, "oracle: format %u\n", fmt); abort();
+  }
+  return m;
+}
+// the exact value of one weight as f32, FP8 without its block scale
+static inline float mat_raw(const Mat& m, int n, int k) {
+  if (m.fmt == DSGX_FMT_FP8_B128) return e4m3f(m.codes[(size_t)n * m.K + k]);
+  if (m.fmt == DSGX_FMT_INT4_G32) return bf2f(i4_bits(i4_nib(m.packed, m.K, n, k), i4_zp(m.zp, m.K, n, k / 32), m.bs[(size_t)n * (m.K / 32) + k / 32]));
+  return bf2f(m.b16[(size_t)n * m.K + k]);
+}
+static inline void mat_row_raw(const Mat& m, int n, float* out) {
+  for (int k = 0; k < m.K; ++k) out[k] = mat_raw(m, n, k);
+}
+struct Dot { float f; double d, mag; };
+// One output: the f32 sum in the contract's order and the f64 sum with the sum of |terms|.
+// FP8 (A/engine/experts/decode.cu:283-303, A/micro/gemv.cu:512): per 128-k unit c from zero, acc = fmaf(S, c, acc).
+// INT4, BF16 (A/engine/attn/gemv.cu:246, 315): straight f32 accumulation in k order; bf16 x bf16 products are exact.
+static inline Dot dot_row(const Mat& m, int n, const float* wrow, const float* x) {
+  Dot r{0.f, 0.0, 0.0};
+  if (m.fmt == DSGX_FMT_FP8_B128) {
+    const float* sr = m.fs + (size_t)(n / 128) * (m.K / 128);
+    for (int b = 0; b < m.K / 128; ++b) {
+      float c = 0.f; double cd = 0, cm = 0;
+      for (int k = 128 * b; k < 128 * b + 128; ++k) {
+        const float t = x[k] * wrow[k];
+        c += t; cd += (double)x[k] * wrow[k]; cm += fabs((double)x[k] * wrow[k]);
+      }
+      r.f = fmaf(sr[b], c, r.f);
+      r.d += (double)sr[b] * cd; r.mag += fabs((double)sr[b]) * cm;
+    }
+  } else {
+    for (int k = 0; k < m.K; ++k) {
+      r.f += x[k] * wrow[k];
+      const double t = (double)x[k] * wrow[k];
+      r.d += t; r.mag += fabs(t);
+    }
+  }
+  return r;
+}
+// h = bf16(bf16(silu(g)) * u): A/engine/experts/decode.cu:110-113, tests/test_experts.cu:350
+static inline float silu_mul(float g, float u) { return bfr(bfr(g / (1.f + expf(-g))) * u); }
+
+// ---- dense GEMV: glm::gemv's contract (A/engine/attn/gemv.cu:138-170,173-333; A/engine/attn/attn.h:80-92) -----------------------
+// x bf16 [M][ldx]; base: the matrix in a pool format (FP8: scales and INT4: scale/zp tensors given apart, as the C ABI's
+// segment carries them). out_kind DSGX_OUT_*: y16 (bf16, SwiGLU: [M][N/2]) and/or yf (the f32 sums [M][N]), yd / ymag
+// the f64 sums and sums of |terms| [M][N]. Any output pointer may be null.
+ORC void orc_gemv(const uint16_t* x, int ldx, int M, int K, uint32_t fmt, const void* w, const void* s, const void* zp, int N,
+                  int out_kind, uint16_t* y16, float* yf, double* yd, double* ymag) {
+  Mat m; m.fmt = fmt; m.N = N; m.K = K; m.s2 = 1.f;
+  if (fmt == DSGX_FMT_FP8_B128) m.codes = (const uint8_t*)w, m.fs = (const float*)s;
+  else if (fmt == DSGX_FMT_INT4_G32) m.packed = (const uint32_t*)w, m.bs = (const uint16_t*)s, m.zp = (const uint32_t*)zp;
+  else m.b16 = (const uint16_t*)w;
+  std::vector<float> xf((size_t)M * K);
+  for (int r = 0; r < M; ++r)
+    for (int k = 0; k < K; ++k) xf[(size_t)r * K + k] = bf2f(x[(size_t)r * ldx + k]);
+  std::vector<float> sums((size_t)M * N);
+#pragma omp parallel
+  {
+    std::vector<float> row(K);
+#pragma omp for schedule(static)
+    for (int n = 0; n < N; ++n) {
+      mat_row_raw(m, n, row.data());
+      for (int r = 0; r < M; ++r) {
+        const Dot d = dot_row(m, n, row.data(), &xf[(size_t)r * K]);
+        sums[(size_t)r * N + n] = d.f;
+        if (yf) yf[(size_t)r * N + n] = d.f;
+        if (yd) yd[(size_t)r * N + n] = d.d;
+        if (ymag) ymag[(size_t)r * N + n] = d.mag;
+      }
+    }
+  }
+  if (!y16) return;
+  for (int r = 0; r < M; ++r) {
+    if (out_kind == DSGX_OUT_SWIGLU) {
+      for (int i = 0; i < N / 2; ++i)
+        y16[(size_t)r * (N / 2) + i] = f2bf(silu_mul(bfr(sums[(size_t)r * N + 2 * i]), bfr(sums[(size_t)r * N + 2 * i + 1])));
+    } else {
+      for (int n = 0; n < N; ++n) y16[(size_t)r * N + n] = f2bf(sums[(size_t)r * N + n]);
+    }
+  }
+}
+
+// ---- the MoE layer ---------------------------------------------------------------------------------------------------------------
+// The union of the rows' picks in expert-id order (A/engine/experts/decode.cu:57-106). Returns its size.
+ORC int orc_union(const int* idx, int n, int E, int* uni) {
+  std::vector<char> hit(E, 0);
+  for (int i = 0; i < n; ++i) hit[idx[i]] = 1;
+  int u = 0;
+  for (int e = 0; e < E; ++e)
+    if (hit[e]) uni[u++] = e;
+  return u;
+}
+static Mat expert_mat(const dsgx_layer_w* L, const dsgx_mat_desc* desc, int e, int j) {
+  const dsgx_mat_desc& d = desc[e * 3 + j];
+  const int N = j < 2 ? L->I : L->H, K = j < 2 ? L->H : L->I;
+  if (d.fmt != L->fmt) { fprintf(stderr, "oracle: expert %d matrix %d format %u, layer %u\n", e, j, d.fmt, L->fmt); abort(); }
+  return mat_at(L->pool + d.off, d.fmt, N, K, d.s2);
+}
+static bool sh_fp8(const dsgx_layer_w* L) { return L->sh.g != nullptr; }
+static bool sh_b16(const dsgx_layer_w* L) { return L->sh.bgu != nullptr; }
+static Mat shared_mat(const dsgx_layer_w* L, int j) {  // 0 gate, 1 up, 2 down (FP8); BF16: 0 = interleaved gate/up, 2 = down
+  Mat m; m.s2 = 1.f;
+  if (sh_fp8(L)) {
+    m.fmt = DSGX_FMT_FP8_B128; m.N = j < 2 ? L->I : L->H; m.K = j < 2 ? L->H : L->I;
+    m.codes = j == 0 ? L->sh.g : j == 1 ? L->sh.u : L->sh.d;
+    m.fs = j == 0 ? L->sh.gs : j == 1 ? L->sh.us : L->sh.ds;
+  } else {
+    m.fmt = DSGX_FMT_BF16; m.N = j < 2 ? 2 * L->I : L->H; m.K = j < 2 ? L->H : L->I;
+    m.b16 = reinterpret_cast<const uint16_t*>(j < 2 ? L->sh.bgu : L->sh.bd);
+  }
+  return m;
+}
+
+// Gate/up + SwiGLU for M rows (A/engine/experts/decode.cu:307-343,366-400; tests/test_experts.cu:363-407):
+// h [U (+1 with a fused shared expert, last)][M][I]: h32 from the f32 sums in the contract's order, h64 from the f64
+// sums rounded as the kernel rounds, lo/hi the range h can take when each of the two sums moves by sum_tol * its sum
+// of |terms| (test_experts.cu:395-404). All as bf16 bit patterns / f32 values; any output may be null.
+// L and desc are HOST copies (pool, shared-expert pointers and desc in host memory).
+ORC void orc_moe_up(const dsgx_layer_w* L, const dsgx_mat_desc* desc, const uint16_t* x, int M, const int* uni, int U,
+                    double sum_tol, uint16_t* h32, uint16_t* h64, float* lo, float* hi) {
+  const int H = L->H, I = L->I, US = U + ((sh_fp8(L) || sh_b16(L)) ? 1 : 0);
+  std::vector<float> xf((size_t)M * H);
+  for (size_t i = 0; i < xf.size(); ++i) xf[i] = bf2f(x[i]);
+  for (int u = 0; u < US; ++u) {
+    const bool sh = u == U;
+    const bool inter = sh && sh_b16(L);  // interleaved gate/up rows
+    const Mat G = sh ? shared_mat(L, 0) : expert_mat(L, desc, uni[u], 0);
+    const Mat Uw = sh ? (inter ? G : shared_mat(L, 1)) : expert_mat(L, desc, uni[u], 1);
+#pragma omp parallel
+    {
+      std::vector<float> gr(H), ur(H);
+#pragma omp for schedule(static)
+      for (int c = 0; c < I; ++c) {
+        mat_row_raw(G, inter ? 2 * c : c, gr.data());
+        mat_row_raw(Uw, inter ? 2 * c + 1 : c, ur.data());
+        for (int m = 0; m < M; ++m) {
+          const Dot dg = dot_row(G, inter ? 2 * c : c, gr.data(), &xf[(size_t)m * H]);
+          const Dot du = dot_row(Uw, inter ? 2 * c + 1 : c, ur.data(), &xf[(size_t)m * H]);
+          const size_t i = ((size_t)u * M + m) * I + c;
+          const float kg = G.s2, ku = Uw.s2;
+          if (h32) h32[i] = f2bf(silu_mul(bfr(dg.f * kg), bfr(du.f * ku)));
+          const float hv = silu_mul(bfr((float)(dg.d * kg)), bfr((float)(du.d * ku)));
+          if (h64) h64[i] = f2bf(hv);
+          if (lo || hi) {
+            float l = hv, hh = hv;
+            const double g0 = (dg.d - sum_tol * dg.mag) * kg, g1 = (dg.d + sum_tol * dg.mag) * kg;
+            const double u0 = (du.d - sum_tol * du.mag) * ku, u1 = (du.d + sum_tol * du.mag) * ku;
+            const double gs[3] = {g0, g1, std::min(std::max(-1.2785, g0), g1)};
+            for (double gg : gs)
+              for (double uu : {u0, u1}) {
+                const float v = silu_mul(bfr((float)gg), bfr((float)uu));
+                l = std::min(l, v), hh = std::max(hh, v);
+              }
+            if (lo) lo[i] = l;
+            if (hi) hi[i] = hh;
+          }
+        }
+      }
+    }
+  }
+}
+
+// Down + weighted sum in expert-id order from a given h [US][M][I] (A/engine/experts/decode.cu:526-587;
+// tests/test_experts.cu:502-524): yr32 = the f32 contract (per slot d = f32 sum, acc = fmaf(k0, d, acc),
+// k0 = s2 * w_row; rows that did not pick a slot skip it, which equals adding 0 * d), ys32 the shared expert's
+// f32 sums; yr64 / ys64 the f64 sums and yrmag / ysmag the sums of |terms|. ysum: yr32 += ys32 (one f32 add,
+// decode.cu:569-581), yr64 += ys64, yrmag += ysmag. Any output may be null.
+ORC void orc_moe_down(const dsgx_layer_w* L, const dsgx_mat_desc* desc, const uint16_t* h, int M, const int* idx,
+                      const float* w, const int* uni, int U, int ysum, const float* ys_in, float* yr32, float* ys32,
+                      double* yr64, double* ys64, double* yrmag, double* ysmag) {
+  const int H = L->H, I = L->I, topk = L->topk;
+  const bool shf = sh_fp8(L) || sh_b16(L);
+  std::vector<float> hf((size_t)(U + shf) * M * I);
+  for (size_t i = 0; i < hf.size(); ++i) hf[i] = bf2f(h[i]);
+  std::vector<float> rw((size_t)U * M, 0.f);
+  std::vector<char> picked((size_t)U * M, 0);
+  for (int u = 0; u < U; ++u)
+    for (int m = 0; m < M; ++m)
+      for (int k = 0; k < topk; ++k)
+        if (idx[m * topk + k] == uni[u]) rw[(size_t)u * M + m] = w[m * topk + k], picked[(size_t)u * M + m] = 1;
+  std::vector<Mat> D(U);
+  for (int u = 0; u < U; ++u) D[u] = expert_mat(L, desc, uni[u], 2);
+  Mat SD{};
+  if (shf) SD = shared_mat(L, 2);
+#pragma omp parallel
+  {
+    std::vector<float> row(I);
+#pragma omp for schedule(static)
+    for (int n = 0; n < H; ++n) {
+      std::vector<float> acc(M, 0.f);
+      std::vector<double> a64(M, 0.0), am(M, 0.0);
+      for (int u = 0; u < U; ++u) {
+        mat_row_raw(D[u], n, row.data());
+        for (int m = 0; m < M; ++m) {
+          if (!picked[(size_t)u * M + m]) continue;
+          const Dot d = dot_row(D[u], n, row.data(), &hf[((size_t)u * M + m) * I]);
+          const float k0 = D[u].s2 * rw[(size_t)u * M + m];
+          acc[m] = fmaf(k0, d.f, acc[m]);
+          a64[m] += (double)k0 * d.d;
+          am[m] += fabs((double)k0) * d.mag;
+        }
+      }
+      for (int m = 0; m < M; ++m) {
+        float s32 = ys_in ? ys_in[(size_t)m * H + n] : 0.f;
+        double s64 = s32, sm = fabs((double)s32);
+        if (shf) {
+          if (m == 0) mat_row_raw(SD, n, row.data());
+          const Dot d = dot_row(SD, n, row.data(), &hf[((size_t)U * M + m) * I]);
+          s32 = d.f, s64 = d.d, sm = d.mag;
+          if (ys32) ys32[(size_t)m * H + n] = s32;
+          if (ys64) ys64[(size_t)m * H + n] = s64;
+          if (ysmag) ysmag[(size_t)m * H + n] = sm;
+        }
+        if (ysum) acc[m] = acc[m] + s32, a64[m] += s64, am[m] += sm;
+        if (yr32) yr32[(size_t)m * H + n] = acc[m];
+        if (yr64) yr64[(size_t)m * H + n] = a64[m];
+        if (yrmag) yrmag[(size_t)m * H + n] = am[m];
+      }
+    }
+  }
+}
+
+// out = bf16(bf16(R) + bf16(S)): A/engine/experts/decode.cu:591-598
+ORC void orc_finalize(const float* R, const float* S, size_t n, uint16_t* out) {
+  for (size_t i = 0; i < n; ++i) out[i] = f2bf(bfr(R[i]) + bfr(S[i]));
+}
+
+// ---- prefill with FP8 activations (D/ref/torchref/kernel.py:56-77,105-125; D/ref/inference/kernel.py:207-274) -----------------
+// One token row through one FP8 expert with the activations quantised per 128 k: xq/xs = act_quant(x); per 128-k
+// block the f32 sum of the exact e4m3 x e4m3 products, scaled by xs * ws and added in block order (fp8_gemm_kernel's
+// accumulation, kernel.py:266-270); g, u rounded to bf16, h = bf16(bf16(silu(g)) * u); h quantised the same way for
+// the down projection. Outputs: h bf16 [I] and d f32 [H] (the pick's down sums before the routing weight).
+static void fp8_row_qdot(const Mat& m, const uint8_t* xq, const float* xs, std::vector<float>& out, std::vector<double>* out64,
+                         std::vector<double>* mag) {
+  const int KB = m.K / 128;
+  out.assign(m.N, 0.f);
+  if (out64) out64->assign(m.N, 0.0);
+  if (mag) mag->assign(m.N, 0.0);
+  std::vector<float> xv(m.K);
+  for (int k = 0; k < m.K; ++k) xv[k] = e4m3f(xq[k]);
+#pragma omp parallel for schedule(static)
+  for (int n = 0; n < m.N; ++n) {
+    const float* sr = m.fs + (size_t)(n / 128) * KB;
+    float acc = 0.f; double a64 = 0, am = 0;
+    for (int b = 0; b < KB; ++b) {
+      float c = 0.f; double cd = 0, cm = 0;
+      for (int k = 128 * b; k < 128 * b + 128; ++k) {
+        const float wv = e4m3f(m.codes[(size_t)n * m.K + k]);
+        c += xv[k] * wv;
+        cd += (double)xv[k] * wv; cm += fabs((double)xv[k] * wv);
+      }
+      const float sc = xs[b] * sr[b];
+      acc = fmaf(sc, c, acc);
+      a64 += (double)sc * cd; am += fabs((double)sc) * cm;
+    }
+    out[n] = acc;
+    if (out64) (*out64)[n] = a64;
+    if (mag) (*mag)[n] = am;
+  }
+}
+// One row of the chunk: picks idx[topk], w[topk] of token row x bf16 [H]. hq_out (optional) h bf16 [topk sorted by
+// expert id][I]; yr f32 [H] (sum in expert-id order, acc = fmaf(w_e, d_e, acc)), yr64 / yrmag from the same quantised
+// operands in f64. With a fused FP8 shared expert ys f32 [H] likewise (null allowed).
+ORC void orc_moe_prefill_fp8_row(const dsgx_layer_w* L, const dsgx_mat_desc* desc, const uint16_t* x, const int* idx,
+                                 const float* w, uint16_t* h_out, float* yr, double* yr64, double* yrmag, float* ys,
+                                 double* ys64, double* ysmag) {
+  const int H = L->H, I = L->I, topk = L->topk;
+  std::vector<uint8_t> xq(H), hq(I);
+  std::vector<float> xs(H / 128), hs(I / 128);
+  orc_act_quant(x, 1, H, xq.data(), xs.data());
+  int ord[8];
+  for (int k = 0; k < topk; ++k) ord[k] = k;
+  std::sort(ord, ord + topk, [&](int a, int b) { return idx[a] < idx[b]; });
+  std::vector<float> acc(H, 0.f), g, u, d;
+  std::vector<double> a64(H, 0.0), am(H, 0.0), d64, dm;
+  std::vector<uint16_t> hb(I);
+  const int nsl = topk + (sh_fp8(L) ? 1 : 0);
+  for (int s = 0; s < nsl; ++s) {
+    const bool sh = s == topk;
+    const int e = sh ? -1 : idx[ord[s]];
+    const Mat G = sh ? shared_mat(L, 0) : expert_mat(L, desc, e, 0);
+    const Mat Uw = sh ? shared_mat(L, 1) : expert_mat(L, desc, e, 1);
+    const Mat Dn = sh ? shared_mat(L, 2) : expert_mat(L, desc, e, 2);
+    fp8_row_qdot(G, xq.data(), xs.data(), g, nullptr, nullptr);
+    fp8_row_qdot(Uw, xq.data(), xs.data(), u, nullptr, nullptr);
+    for (int c = 0; c < I; ++c) hb[c] = f2bf(silu_mul(bfr(g[c] * G.s2), bfr(u[c] * Uw.s2)));
+    if (h_out && !sh) memcpy(h_out + (size_t)s * I, hb.data(), (size_t)I * 2);
+    orc_act_quant(hb.data(), 1, I, hq.data(), hs.data());
+    fp8_row_qdot(Dn, hq.data(), hs.data(), d, &d64, &dm);
+    if (sh) {
+      for (int n = 0; n < H; ++n) {
+        if (ys) ys[n] = d[n];
+        if (ys64) ys64[n] = d64[n];
+        if (ysmag) ysmag[n] = dm[n];
+      }
+    } else {
+      const float k0 = Dn.s2 * w[ord[s]];
+      for (int n = 0; n < H; ++n) {
+        acc[n] = fmaf(k0, d[n], acc[n]);
+        a64[n] += (double)k0 * d64[n];
+        am[n] += fabs((double)k0) * dm[n];
+      }
+    }
+  }
+  for (int n = 0; n < H; ++n) {
+    if (yr) yr[n] = acc[n];
+    if (yr64) yr64[n] = a64[n];
+    if (yrmag) yrmag[n] = am[n];
+  }
+}
+
+ORC int orc_threads() { return omp_get_max_threads(); }

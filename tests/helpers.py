@@ -1,0 +1,61 @@
+"""Shared builders for the tests: seeded synthetic layers in the pool formats and tolerance checks."""
+import numpy as np
+
+from dsgx10_amd import abi
+from dsgx10_amd.layer import HostLayer
+from tests import orc
+
+
+def quant_fp8(seed, tid, N, K, sigma=0.02):
+    """W ~ N(0, sigma) quantised to e4m3 with 128x128 block scales (the reference's quantiser)."""
+    return orc.fp8_quantize(orc.normal_f32(seed, tid, (N, K), sigma))
+
+
+def quant_int4(seed, tid, N, K, sigma=0.02):
+    return orc.int4_quantize_sym(orc.normal_f32(seed, tid, (N, K), sigma))
+
+
+def make_layer(fmt, H, I, E, topk, NS, seed=0, shared=None, random_codes=False):
+    """NS stored experts; expert id e uses stored expert mix64(seed + 99 + e) % NS (testdata.h:197).
+    shared: None | 'fp8' | 'bf16'. random_codes: the reference's random-byte tensors (asymmetric INT4 with every zero
+    point; random FP8 codes) instead of quantised normal weights."""
+    experts = []
+    for e in range(NS):
+        mats = []
+        for j in range(3):
+            N, K = (I, H) if j < 2 else (H, I)
+            tid = 1000 + e * 3 + j
+            if fmt == abi.FMT_FP8:
+                mats.append(orc.fp8_random(seed * 131 + tid, N, K, 1.0 / 1024 if j < 2 else 1.0 / 256) if random_codes
+                            else quant_fp8(seed, tid, N, K))
+            elif fmt == abi.FMT_INT4:
+                mats.append(orc.int4_random(seed * 131 + tid, N, K) if random_codes else quant_int4(seed, tid, N, K))
+            else:
+                mats.append((orc.normal_bf16(seed, tid, (N, K), 0.02),))
+        experts.append(tuple(mats))
+    emap = np.array([orc.lib().orc_mix64(seed + 99 + e) % NS for e in range(E)], np.int64)
+    sh8 = sh16 = None
+    if shared == "fp8":
+        sh8 = (quant_fp8(seed, 17, I, H), quant_fp8(seed, 18, I, H), quant_fp8(seed, 19, H, I))
+    elif shared == "bf16":
+        sh16 = (orc.normal_bf16(seed, 27, (2 * I, H), 0.02), orc.normal_bf16(seed, 28, (H, I), 0.02))
+    return HostLayer(fmt, H, I, E, topk, experts, emap, shared_fp8=sh8, shared_bf16=sh16)
+
+
+def rows_and_routing(seed, M, H, E, topk, scale, bias=None):
+    x = orc.normal_bf16(seed, 1, (M, H), 1.0)
+    logits = orc.normal_f32(seed, 2, (M, E), 1.0)
+    idx, w = orc.route(logits, bias, topk, scale)
+    return x, logits, idx, w
+
+
+def rel_l2(got, ref):
+    got, ref = np.asarray(got, np.float64), np.asarray(ref, np.float64)
+    return float(np.sqrt(((got - ref) ** 2).sum() / max((ref ** 2).sum(), 1e-300)))
+
+
+def check_sums(got, ref64, mag, tol=1e-4):
+    """the reference's rule for GEMV / down outputs: |got - ref| <= tol * sum|terms| (test_experts.cu:352-361,525)"""
+    got, ref64, mag = np.asarray(got, np.float64), np.asarray(ref64), np.asarray(mag)
+    e = np.abs(got - ref64) / np.where(mag > 0, mag, 1.0)
+    return float(e.max()), int((~(e <= tol)).sum())

@@ -1,0 +1,238 @@
+"""ctypes binding of the CPU oracle (oracle/liboracle.so). Test infrastructure: only tests/, smoke() and the
+cpu_baseline leg of bench.py import this."""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+_SO = os.path.join(ROOT, "oracle", "liboracle.so")
+
+
+def build(force=False):
+    if force or not os.path.exists(_SO):
+        subprocess.check_call(["make", "-C", os.path.join(ROOT, "oracle"), "-B" if force else "-s"])
+    return _SO
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        _lib = C.CDLL(build())
+        L = _lib
+        L.orc_f32_to_bf16.restype = C.c_uint16
+        L.orc_f32_to_bf16.argtypes = [C.c_float]
+        L.orc_bf16_to_f32.restype = C.c_float
+        L.orc_bf16_to_f32.argtypes = [C.c_uint16]
+        L.orc_e4m3_to_f32.restype = C.c_float
+        L.orc_e4m3_to_f32.argtypes = [C.c_uint8]
+        L.orc_f32_to_e4m3.restype = C.c_uint8
+        L.orc_f32_to_e4m3.argtypes = [C.c_float]
+        L.orc_mix64.restype = C.c_uint64
+        L.orc_mix64.argtypes = [C.c_uint64]
+        L.orc_normal.restype = C.c_double
+        L.orc_normal.argtypes = [C.c_uint64, C.c_uint64, C.c_uint64]
+        L.orc_int4_value_bits.restype = C.c_uint16
+        L.orc_int4_value_bits.argtypes = [C.c_int, C.c_int, C.c_uint16]
+        L.orc_route_sigmoid.restype = C.c_float
+        L.orc_route_sigmoid.argtypes = [C.c_float]
+        L.orc_union.restype = C.c_int
+        L.orc_threads.restype = C.c_int
+    return _lib
+
+
+def _p(a):
+    if a is None:
+        return None
+    assert isinstance(a, np.ndarray) and a.flags["C_CONTIGUOUS"], "contiguous numpy array expected"
+    return a.ctypes.data_as(C.c_void_p)
+
+
+# ---- ctypes mirrors of include/dsgx.h ------------------------------------------------------------------------
+from dsgx10_amd.abi import FMT_BF16, FMT_FP8, FMT_INT4, OUT_BF16, OUT_F32, OUT_SWIGLU, LayerW, MatDesc, SharedW  # noqa: E402,F401
+
+
+# ---- codecs and data ------------------------------------------------------------------------------------------
+def f32_to_bf16(f):
+    f = np.ascontiguousarray(f, np.float32)
+    o = np.empty(f.shape, np.uint16)
+    lib().orc_f32_to_bf16_n(_p(f), C.c_size_t(f.size), _p(o))
+    return o
+
+
+def bf16_to_f32(b):
+    return (np.asarray(b, np.uint16).astype(np.uint32) << 16).view(np.float32)
+
+
+def f32_to_e4m3(f):
+    f = np.ascontiguousarray(f, np.float32)
+    o = np.empty(f.shape, np.uint8)
+    lib().orc_f32_to_e4m3_n(_p(f), C.c_size_t(f.size), _p(o))
+    return o
+
+
+def e4m3_table():
+    return np.array([lib().orc_e4m3_to_f32(i) for i in range(256)], np.float32)
+
+
+def normal_f32(seed, tid, shape, sigma=1.0):
+    o = np.empty(shape, np.float32)
+    lib().orc_fill_normal_f32(C.c_uint64(seed), C.c_uint64(tid), C.c_size_t(o.size), C.c_double(sigma), _p(o))
+    return o
+
+
+def normal_bf16(seed, tid, shape, sigma=1.0):
+    o = np.empty(shape, np.uint16)
+    lib().orc_fill_normal_bf16(C.c_uint64(seed), C.c_uint64(tid), C.c_size_t(o.size), C.c_double(sigma), _p(o))
+    return o
+
+
+# ---- formats --------------------------------------------------------------------------------------------------
+def int4_dequant(packed, scale, zp):
+    N, K = packed.shape[0], packed.shape[1] * 8
+    o = np.empty((N, K), np.uint16)
+    lib().orc_int4_dequant(_p(packed), _p(scale), _p(zp), N, K, _p(o))
+    return o
+
+
+def int4_quantize_sym(w):
+    w = np.ascontiguousarray(w, np.float32)
+    N, K = w.shape
+    packed = np.empty((N, K // 8), np.uint32)
+    scale = np.empty((N, K // 32), np.uint16)
+    zp = np.empty((N // 8, K // 32), np.uint32)
+    lib().orc_int4_quantize_sym(_p(w), N, K, _p(packed), _p(scale), _p(zp))
+    return packed, scale, zp
+
+
+def int4_random(seed, N, K):
+    packed = np.empty((N, K // 8), np.uint32)
+    scale = np.empty((N, K // 32), np.uint16)
+    zp = np.empty((N // 8, K // 32), np.uint32)
+    lib().orc_int4_random(C.c_uint64(seed), N, K, _p(packed), _p(scale), _p(zp))
+    return packed, scale, zp
+
+
+def fp8_quantize(w):
+    w = np.ascontiguousarray(w, np.float32)
+    N, K = w.shape
+    codes = np.empty((N, K), np.uint8)
+    scales = np.empty(((N + 127) // 128, K // 128), np.float32)
+    lib().orc_fp8_quantize(_p(w), N, K, _p(codes), _p(scales))
+    return codes, scales
+
+
+def fp8_dequant(codes, scales):
+    N, K = codes.shape
+    o = np.empty((N, K), np.float32)
+    lib().orc_fp8_dequant(_p(codes), _p(scales), N, K, _p(o))
+    return o
+
+
+def fp8_random(seed, N, K, scale):
+    codes = np.empty((N, K), np.uint8)
+    scales = np.empty(((N + 127) // 128, K // 128), np.float32)
+    lib().orc_fp8_random(C.c_uint64(seed), N, K, C.c_float(scale), _p(codes), _p(scales))
+    return codes, scales
+
+
+def act_quant(x):
+    x = np.ascontiguousarray(x, np.uint16)
+    T, K = x.shape
+    q = np.empty((T, K), np.uint8)
+    s = np.empty((T, K // 128), np.float32)
+    lib().orc_act_quant(_p(x), T, K, _p(q), _p(s))
+    return q, s
+
+
+# ---- router ---------------------------------------------------------------------------------------------------
+def route(logits, bias, topk, scale, score_fn=0):
+    logits = np.ascontiguousarray(logits, np.float32)
+    M, E = logits.shape
+    idx = np.empty((M, topk), np.int32)
+    w = np.empty((M, topk), np.float32)
+    b = None if bias is None else np.ascontiguousarray(bias, np.float32)
+    lib().orc_route(_p(logits), _p(b), M, E, topk, C.c_float(scale), score_fn, _p(idx), _p(w))
+    return idx, w
+
+
+def union(idx, E):
+    idx = np.ascontiguousarray(idx, np.int32)
+    u = np.empty(idx.size, np.int32)
+    n = lib().orc_union(_p(idx), idx.size, E, _p(u))
+    return u[:n].copy()
+
+
+# ---- GEMV -----------------------------------------------------------------------------------------------------
+def gemv(x, fmt, w, s, zp, N, K, out_kind=OUT_BF16, want64=True):
+    """x bf16 bits [M][K]. Returns dict(y16, yf, yd, ymag)."""
+    x = np.ascontiguousarray(x, np.uint16)
+    M = x.shape[0]
+    y16 = np.empty((M, N // 2 if out_kind == OUT_SWIGLU else N), np.uint16)
+    yf = np.empty((M, N), np.float32)
+    yd = np.empty((M, N), np.float64) if want64 else None
+    ym = np.empty((M, N), np.float64) if want64 else None
+    lib().orc_gemv(_p(x), x.shape[1], M, K, fmt, _p(w), _p(s), _p(zp), N, out_kind, _p(y16), _p(yf), _p(yd), _p(ym))
+    return dict(y16=y16, yf=yf, yd=yd, ymag=ym)
+
+
+# ---- MoE ------------------------------------------------------------------------------------------------------
+def moe_up(hl, x, uni, sum_tol=2e-5, want_range=True):
+    """hl: a host layer (dsgx10_amd.layer.HostLayer). Returns dict(h32, h64, lo, hi) [US][M][I]."""
+    x = np.ascontiguousarray(x, np.uint16)
+    M = x.shape[0]
+    uni = np.ascontiguousarray(uni, np.int32)
+    US = len(uni) + (1 if hl.has_shared else 0)
+    shp = (US, M, hl.I)
+    h32, h64 = np.empty(shp, np.uint16), np.empty(shp, np.uint16)
+    lo = np.empty(shp, np.float32) if want_range else None
+    hi = np.empty(shp, np.float32) if want_range else None
+    Lw, desc = hl.host_layer_w()
+    lib().orc_moe_up(C.byref(Lw), _p(desc), _p(x), M, _p(uni), len(uni), C.c_double(sum_tol), _p(h32), _p(h64), _p(lo), _p(hi))
+    return dict(h32=h32, h64=h64, lo=lo, hi=hi)
+
+
+def moe_down(hl, h, idx, w, uni, ysum=False, ys_in=None):
+    h = np.ascontiguousarray(h, np.uint16)
+    M = h.shape[1]
+    idx = np.ascontiguousarray(idx, np.int32)
+    w = np.ascontiguousarray(w, np.float32)
+    uni = np.ascontiguousarray(uni, np.int32)
+    H = hl.H
+    out = {k: np.zeros((M, H), np.float32 if k.endswith("32") else np.float64)
+           for k in ("yr32", "ys32", "yr64", "ys64", "yrmag", "ysmag")}
+    Lw, desc = hl.host_layer_w()
+    ysi = None if ys_in is None else np.ascontiguousarray(ys_in, np.float32)
+    lib().orc_moe_down(C.byref(Lw), _p(desc), _p(h), M, _p(idx), _p(w), _p(uni), len(uni), int(ysum), _p(ysi),
+                       _p(out["yr32"]), _p(out["ys32"]), _p(out["yr64"]), _p(out["ys64"]), _p(out["yrmag"]), _p(out["ysmag"]))
+    return out
+
+
+def moe_prefill_fp8_row(hl, xrow, idx, w):
+    xrow = np.ascontiguousarray(xrow, np.uint16)
+    idx = np.ascontiguousarray(idx, np.int32)
+    w = np.ascontiguousarray(w, np.float32)
+    H, I, topk = hl.H, hl.I, hl.topk
+    h = np.empty((topk, I), np.uint16)
+    out = dict(h=h, yr=np.empty(H, np.float32), yr64=np.empty(H, np.float64), yrmag=np.empty(H, np.float64),
+               ys=np.zeros(H, np.float32), ys64=np.zeros(H, np.float64), ysmag=np.zeros(H, np.float64))
+    Lw, desc = hl.host_layer_w()
+    lib().orc_moe_prefill_fp8_row(C.byref(Lw), _p(desc), _p(xrow), _p(idx), _p(w), _p(h), _p(out["yr"]), _p(out["yr64"]),
+                                  _p(out["yrmag"]), _p(out["ys"]), _p(out["ys64"]), _p(out["ysmag"]))
+    return out
+
+
+def finalize(R, S):
+    R = np.ascontiguousarray(R, np.float32)
+    S = np.ascontiguousarray(S, np.float32)
+    o = np.empty(R.shape, np.uint16)
+    lib().orc_finalize(_p(R), _p(S), C.c_size_t(R.size), _p(o))
+    return o
+
+
+def threads():
+    return lib().orc_threads()

@@ -1,0 +1,128 @@
+"""GPU parity of the decode expert step (dsgx_moe_decode = gx::moe_decode of the reference) against the CPU oracle,
+shaped after the reference's test_decode (altar1-4xgx10-switchless/engine/experts/tests/test_experts.cu:466-578):
+h against the f64 reference (bit-exact share and the f32-sum range), the outputs against f64 from the GPU's own h
+(|err| <= 1e-4 sum|terms|) and against the f32 oracle (max-abs <= 2e-2, relative L2 <= 1e-3 on the bf16 outputs),
+batch invariance, determinism, ys untouched without a fused shared expert, fused routing, ysum."""
+import numpy as np
+import pytest
+
+from dsgx10_amd import abi, lib
+from tests import gpu, orc
+from tests.helpers import check_sums, make_layer, rel_l2, rows_and_routing
+
+pytestmark = pytest.mark.gpu
+
+_cache = {}
+
+
+def _layer(fmt, H, I, E, topk, NS, shared, random_codes=False, seed=1):
+    key = (fmt, H, I, E, topk, NS, shared, random_codes, seed)
+    if key not in _cache:
+        hl = make_layer(fmt, H, I, E, topk, NS, seed=seed, shared=shared, random_codes=random_codes)
+        _cache[key] = (hl, hl.upload())
+    return _cache[key]
+
+
+def _check_step(hl, dl, x, idx, w, M, scale_note=""):
+    E = hl.E
+    yr, ys, ws = gpu.decode_layer(dl, x[:M], idx[:M], w[:M], M)
+    uni = orc.union(idx[:M], E)
+    U = len(uni)
+    hg = gpu.h_of(ws, dl, M, U)
+    up = orc.moe_up(hl, x[:M], uni)
+    hv = orc.bf16_to_f32(hg)
+    exact = (hg == up["h64"]) | ((hv == 0) & (orc.bf16_to_f32(up["h64"]) == 0))
+    far = ~((hv >= up["lo"]) & (hv <= up["hi"]))
+    assert far.sum() == 0, "%d of %d h outside the range of f32 sums" % (far.sum(), far.size)
+    assert exact.mean() >= 0.995, exact.mean()
+    # down from the GPU's own h, in f64
+    dn = orc.moe_down(hl, hg, idx[:M], w[:M], uni)
+    worst, bad = check_sums(yr, dn["yr64"], dn["yrmag"], 1e-4)
+    assert bad == 0, worst
+    if hl.has_shared:
+        worst, bad = check_sums(ys, dn["ys64"], dn["ysmag"], 1e-4)
+        assert bad == 0, worst
+    else:
+        assert np.all(ys.view(np.uint32) == 0xFFFFFFFF)  # ys is an input then: left as it was
+    # end to end against the f32-accumulated oracle: bf16 outputs
+    full = orc.moe_down(hl, up["h32"], idx[:M], w[:M], uni)
+    for got, ref in ((yr, full["yr32"]),) + (((ys, full["ys32"]),) if hl.has_shared else ()):
+        g16, r16 = orc.bf16_to_f32(orc.f32_to_bf16(got)), orc.bf16_to_f32(orc.f32_to_bf16(ref))
+        assert np.abs(g16 - r16).max() <= 2e-2 and rel_l2(g16, r16) <= 1e-3
+    return yr, ys, hg
+
+
+CASES = [
+    # fmt, H, I, E, topk, NS, shared, scale
+    (abi.FMT_FP8, 2048, 1024, 32, 8, 6, "fp8", 1.0),
+    (abi.FMT_FP8, 1024, 2048, 256, 8, 4, None, 1.0),
+    (abi.FMT_INT4, 2048, 2048, 168, 8, 5, "bf16", 2.5),
+    (abi.FMT_INT4, 4096, 2048, 168, 8, 3, None, 2.5),
+    (abi.FMT_BF16, 1024, 512, 16, 4, 4, None, 2.5),
+]
+
+
+@pytest.mark.parametrize("case", CASES, ids=lambda c: "fmt%d-H%d-I%d-E%d-%s" % (c[0], c[1], c[2], c[3], c[6]))
+def test_decode_rows(case):
+    fmt, H, I, E, topk, NS, shared, scale = case
+    hl, dl = _layer(fmt, H, I, E, topk, NS, shared)
+    x, logits, idx, w = rows_and_routing(21, 8, H, E, topk, scale)
+    runs = {}
+    for M in (1, 3, 5, 8):
+        runs[M] = _check_step(hl, dl, x, idx, w, M)
+    # a row's bits do not depend on the other rows: each row alone against the 8-row step
+    for m in range(8):
+        yr1, ys1, _ = gpu.decode_layer(dl, x[m:m + 1], idx[m:m + 1], w[m:m + 1], 1)
+        assert np.array_equal(yr1[0].view(np.uint32), runs[8][0][m].view(np.uint32)), m
+        if hl.has_shared:
+            assert np.array_equal(ys1[0].view(np.uint32), runs[8][1][m].view(np.uint32)), m
+    # deterministic
+    yr2, ys2, _ = gpu.decode_layer(dl, x, idx, w, 8)
+    assert np.array_equal(yr2.view(np.uint32), runs[8][0].view(np.uint32))
+
+
+def test_decode_random_codes_asymmetric_int4_and_fp8():
+    """the reference's random-byte tensors: every INT4 nibble and zero point, random FP8 codes"""
+    for fmt, shared in ((abi.FMT_INT4, None), (abi.FMT_FP8, None)):
+        hl, dl = _layer(fmt, 2048, 2048, 64, 8, 3, shared, random_codes=True, seed=3)
+        x, logits, idx, w = rows_and_routing(5, 4, 2048, 64, 8, 2.5)
+        _check_step(hl, dl, x, idx, w, 4)
+
+
+def test_decode_fused_routing_and_ysum():
+    fmt, H, I, E, topk, NS, shared, scale = CASES[0]
+    hl, dl = _layer(fmt, H, I, E, topk, NS, shared)
+    x, logits, idx, w = rows_and_routing(33, 4, H, E, topk, scale)
+    bias = orc.normal_f32(33, 3, (E,), 0.3)
+    idx, w = orc.route(logits, bias, topk, scale)
+    base_yr, base_ys, _ = gpu.decode_layer(dl, x, idx, w, 4)
+    dl_, db = gpu.dev(logits), gpu.dev(bias)
+    yr, ys, _ = gpu.decode_layer(dl, x, None, None, 4, logits=dl_, bias=db, route_scale=scale)
+    assert np.array_equal(yr.view(np.uint32), base_yr.view(np.uint32)) and np.array_equal(ys.view(np.uint32), base_ys.view(np.uint32))
+    yr, ys, _ = gpu.decode_layer(dl, x, idx, w, 4, ysum=True)
+    assert np.array_equal(ys.view(np.uint32), base_ys.view(np.uint32))
+    assert np.array_equal(yr, base_yr + base_ys)  # one f32 add a value, after the routed experts
+    # without a fused shared expert ysum adds the caller's ys
+    hl2, dl2 = _layer(abi.FMT_FP8, 1024, 2048, 256, 8, 4, None)
+    x2, l2, i2, w2 = rows_and_routing(34, 2, 1024, 256, 8, 1.0)
+    ysin = orc.normal_f32(1, 9, (2, 1024), 1.0)
+    b_yr, _, _ = gpu.decode_layer(dl2, x2, i2, w2, 2)
+    yr, ys, _ = gpu.decode_layer(dl2, x2, i2, w2, 2, ysum=True, ys_in=ysin)
+    assert np.array_equal(yr, b_yr + ysin) and np.array_equal(ys, ysin)
+
+
+def test_decode_parts_and_duplicate_experts_across_rows():
+    # rows that share every expert (a union of exactly top-k slots) and the up-only / down-only bench switches
+    fmt, H, I, E, topk, NS, shared, scale = CASES[1]
+    hl, dl = _layer(fmt, H, I, E, topk, NS, shared)
+    x, logits, idx, w = rows_and_routing(40, 4, H, E, topk, scale)
+    idx[:] = idx[0]
+    yr, ys, ws = gpu.decode_layer(dl, x, idx, w, 4)
+    assert len(orc.union(idx, E)) == topk
+    _check_step(hl, dl, x, idx, w, 4)
+    H_ = hl.H
+    yr1 = gpu.empty(4 * H_ * 4, 0xFF)
+    lib.moe_decode(dl.w, gpu.dev(x), gpu.dev(idx), gpu.dev(w), 4, ws, yr1, None, parts=1)   # up only: yr untouched
+    assert np.all(gpu.host(yr1, np.uint32, (-1,)) == 0xFFFFFFFF)
+    lib.moe_decode(dl.w, gpu.dev(x), gpu.dev(idx), gpu.dev(w), 4, ws, yr1, None, parts=2)   # down only, from ws's h
+    assert np.array_equal(gpu.host(yr1, np.float32, (4, H_)).view(np.uint32), yr.view(np.uint32))

@@ -1,0 +1,166 @@
+"""Pins the oracle's GEMV and MoE-layer sums: special cases with exact answers (one-hot rows), numpy float64 matrix
+products on independently dequantised weights, the INT4 = BF16(dequantised) identity, batch invariance, and the
+expert-id order of the weighted sum."""
+import numpy as np
+import torch
+
+from dsgx10_amd import abi
+from dsgx10_amd.layer import HostLayer
+from tests import orc
+from tests.helpers import check_sums, make_layer, quant_fp8, quant_int4, rel_l2, rows_and_routing
+
+
+def _deq_fp8(c, s):
+    N, K = c.shape
+    v = torch.from_numpy(c).view(torch.float8_e4m3fn).double().numpy()
+    return v * np.repeat(np.repeat(s.astype(np.float64), 128, 0)[:N], 128, 1)
+
+
+def _deq_int4_np(packed, scale, zp):
+    """numpy restatement of pack.py int4_dequant, independent of the C++ reader"""
+    N, K = packed.shape[0], packed.shape[1] * 8
+    sh = np.arange(8, dtype=np.uint32) * 4
+    q = ((packed[:, :, None] >> sh) & 0xF).astype(np.int32).reshape(N, K)
+    z = ((zp[:, None, :] >> sh[None, :, None]) & 0xF).astype(np.int32).reshape(-1, zp.shape[1])[:N]
+    d = (q.reshape(N, K // 32, 32) - z[:, :, None]).astype(np.float32) * orc.bf16_to_f32(scale)[:, :, None]
+    return torch.from_numpy(d.reshape(N, K)).to(torch.bfloat16).double().numpy()
+
+
+def test_int4_dequant_matches_numpy_reader():
+    packed, scale, zp = orc.int4_random(3, 24, 1024)
+    got = orc.bf16_to_f32(orc.int4_dequant(packed, scale, zp)).astype(np.float64)
+    assert np.array_equal(got, _deq_int4_np(packed, scale, zp))
+
+
+def test_gemv_one_hot_rows_give_the_weights():
+    K, N = 256, 64
+    x = np.zeros((4, K), np.uint16)
+    ks = [0, 31, 128, 255]
+    for r, k in enumerate(ks):
+        x[r, k] = 0x3F80
+    c, s = quant_fp8(0, 1, N, K)
+    out = orc.gemv(x, abi.FMT_FP8, c, s, None, N, K, abi.OUT_F32)
+    W = _deq_fp8(c, s)
+    for r, k in enumerate(ks):
+        assert np.array_equal(out["yf"][r].astype(np.float64), W[:, k].astype(np.float32).astype(np.float64))
+    p, sc, zp = orc.int4_random(5, N, K)
+    out = orc.gemv(x, abi.FMT_INT4, p, sc, zp, N, K, abi.OUT_F32)
+    W4 = _deq_int4_np(p, sc, zp)
+    for r, k in enumerate(ks):
+        assert np.array_equal(out["yf"][r].astype(np.float64), W4[:, k])
+
+
+def test_gemv_vs_float64_matmul_and_int4_equals_bf16():
+    M, K, N = 3, 1024, 96
+    x16 = orc.normal_bf16(0, 9, (M, K), 1.0)
+    x = orc.bf16_to_f32(x16).astype(np.float64)
+    c, s = quant_fp8(0, 2, N, K)
+    o = orc.gemv(x16, abi.FMT_FP8, c, s, None, N, K, abi.OUT_BF16)
+    W = _deq_fp8(c, s)
+    ref = x @ W.T
+    assert np.allclose(o["yd"], ref, rtol=0, atol=1e-12 * np.abs(ref).max() + 1e-15)
+    assert np.allclose(o["ymag"], np.abs(x)[:, None, :].__mul__(np.abs(W)[None]).sum(-1), rtol=1e-12)
+    worst, bad = check_sums(o["yf"], ref, o["ymag"], 2e-6)
+    assert bad == 0
+    assert np.array_equal(o["y16"], orc.f32_to_bf16(o["yf"]))
+    p, sc, zp = quant_int4(0, 3, N, K)
+    o4 = orc.gemv(x16, abi.FMT_INT4, p, sc, zp, N, K, abi.OUT_BF16)
+    W4 = _deq_int4_np(p, sc, zp)
+    assert np.allclose(o4["yd"], x @ W4.T, rtol=0, atol=1e-12)
+    wb = orc.int4_dequant(p, sc, zp)
+    ob = orc.gemv(x16, abi.FMT_BF16, wb, None, None, N, K, abi.OUT_BF16)
+    assert np.array_equal(o4["yf"].view(np.uint32), ob["yf"].view(np.uint32))  # INT4 == BF16 of its dequantised values
+    # SwiGLU output: rows 2i gate, 2i + 1 up
+    osw = orc.gemv(x16, abi.FMT_BF16, wb, None, None, N, K, abi.OUT_SWIGLU)
+    g = torch.from_numpy(ob["yf"][:, 0::2]).to(torch.bfloat16).float()
+    u = torch.from_numpy(ob["yf"][:, 1::2]).to(torch.bfloat16).float()
+    sl = (g / (1 + torch.exp(-g))).to(torch.bfloat16).float()
+    want = (sl * u).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+    assert (osw["y16"] != want).mean() < 0.01  # expf differs between libms by an ulp at most, rarely visible in bf16
+
+
+def _dense_moe_f64(hl, x16, idx, w, uni, h16):
+    """float64 restatement from the given h: yr[m] = sum over the row's picks of w * Wd_e h_e"""
+    H, I, M = hl.H, hl.I, x16.shape[0]
+    yr = np.zeros((M, H))
+    for u, e in enumerate(uni):
+        parts = hl.experts[int(hl.emap[e])][2]
+        W = _deq_fp8(*parts) if hl.fmt == abi.FMT_FP8 else _deq_int4_np(*parts)
+        for m in range(M):
+            k = np.where(idx[m] == e)[0]
+            if len(k):
+                yr[m] += float(w[m, k[0]]) * (W @ orc.bf16_to_f32(h16[u, m]).astype(np.float64))
+    return yr
+
+
+def _check_layer(fmt, shared):
+    H, I, E, topk, M = 1024, 1024, 16, 4, 3
+    if fmt == abi.FMT_INT4:
+        H = I = 2048
+    hl = make_layer(fmt, H, I, E, topk, NS=3, seed=1, shared=shared)
+    x, logits, idx, w = rows_and_routing(1, M, H, E, topk, 2.5)
+    uni = orc.union(idx, E)
+    up = orc.moe_up(hl, x, uni)
+    # h: gate/up sums in float64 on independently dequantised weights, rounded with torch's bf16
+    xf = orc.bf16_to_f32(x).astype(np.float64)
+    for u, e in enumerate(uni[:2]):
+        gp, upp, _ = hl.experts[int(hl.emap[e])]
+        G = _deq_fp8(*gp) if fmt == abi.FMT_FP8 else _deq_int4_np(*gp)
+        U = _deq_fp8(*upp) if fmt == abi.FMT_FP8 else _deq_int4_np(*upp)
+        g = torch.from_numpy((xf @ G.T).astype(np.float32)).to(torch.bfloat16).float()
+        uu = torch.from_numpy((xf @ U.T).astype(np.float32)).to(torch.bfloat16).float()
+        sl = (g / (1 + torch.exp(-g))).to(torch.bfloat16).float()
+        want = (sl * uu).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+        assert (up["h64"][u] != want).mean() < 0.01
+        hv = orc.bf16_to_f32(up["h32"][u])
+        assert np.all(hv >= up["lo"][u]) and np.all(hv <= up["hi"][u])
+        assert (up["h32"][u] != up["h64"][u]).mean() < 0.01
+    dn = orc.moe_down(hl, up["h32"], idx, w, uni)
+    ref = _dense_moe_f64(hl, x, idx, w, uni, up["h32"][:len(uni)])
+    assert np.allclose(dn["yr64"], ref, rtol=0, atol=1e-11 * max(1.0, np.abs(ref).max()))
+    worst, bad = check_sums(dn["yr32"], dn["yr64"], dn["yrmag"], 2e-6)
+    assert bad == 0, worst
+    # batch invariance: each row alone gives the row's bits in the batch
+    for m in range(M):
+        uni1 = orc.union(idx[m:m + 1], E)
+        up1 = orc.moe_up(hl, x[m:m + 1], uni1, want_range=False)
+        d1 = orc.moe_down(hl, up1["h32"], idx[m:m + 1], w[m:m + 1], uni1)
+        assert np.array_equal(d1["yr32"][0].view(np.uint32), dn["yr32"][m].view(np.uint32))
+    if shared:
+        assert np.any(dn["ys32"] != 0)
+        ds = orc.moe_down(hl, up["h32"], idx, w, uni, ysum=True)
+        assert np.array_equal(ds["yr32"], dn["yr32"] + dn["ys32"])  # one f32 add after the routed experts
+    return hl, x, idx, w, uni, up, dn
+
+
+def test_moe_fp8_layer_with_fused_shared():
+    _check_layer(abi.FMT_FP8, "fp8")
+
+
+def test_moe_int4_layer_with_bf16_shared():
+    _check_layer(abi.FMT_INT4, "bf16")
+
+
+def test_moe_expert_order_matters_and_is_ascending():
+    # the f32 sum over a row's experts runs in ascending expert id: reversing the order changes some bits
+    hl, x, idx, w, uni, up, dn = _check_layer(abi.FMT_FP8, None)
+    M, H = x.shape[0], hl.H
+    contrib = np.zeros((len(uni), M, H), np.float32)
+    for u, e in enumerate(uni):
+        one = orc.moe_down(hl, up["h32"], np.where(idx == e, idx, -1).astype(np.int32), w, uni)
+        contrib[u] = one["yr32"]
+    fwd = np.zeros((M, H), np.float32)
+    rev = np.zeros((M, H), np.float32)
+    for u in range(len(uni)):
+        fwd = (fwd + contrib[u]).astype(np.float32)
+        rev = (rev + contrib[len(uni) - 1 - u]).astype(np.float32)
+    # fma(k0, d, acc) and acc + k0 * d differ by at most the product's rounding: compare loosely, but order strictly
+    assert np.allclose(fwd, dn["yr32"], rtol=1e-5, atol=1e-7)
+    assert np.any(fwd != rev)
+
+
+def test_finalize():
+    R = orc.normal_f32(0, 1, (64,), 1.0)
+    S = orc.normal_f32(0, 2, (64,), 1.0)
+    want = (torch.from_numpy(R).to(torch.bfloat16) + torch.from_numpy(S).to(torch.bfloat16)).view(torch.int16).numpy().view(np.uint16)
+    assert np.array_equal(orc.finalize(R, S), want)
