@@ -1,0 +1,152 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantised-MoE hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extra] [--no-cpu]
+
+A step is one MoE layer: the router kernel plus the decode expert step (gate/up + SwiGLU, down + weighted sum) for M
+rows, inputs resident in HBM. The headline workload is the FP8 MoE decode layer at M = 1 (hidden 4096, 256 routed
+experts + 1 shared, intermediate 2048, e4m3 weights with 128 x 128 block scales, sigmoid top-8 renormalised). Every
+step routes a different seeded logits row, so its experts come from a 6.4 GB pool and not from the caches; the shared
+expert rotates over copies that together exceed the 256 MB Infinity Cache.
+
+Prints ONE JSON line: metric us_per_moe_layer (lower is better), the roofline of the dominant kernel (the gate/up
+kernel, timed alone with HIP events on its launch stream), the CPU baseline (the C++ oracle on the host cores over
+the same step) and, unless --no-extra, the other benchmark configurations.
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=512)
+    ap.add_argument("--warmup", type=int, default=64)
+    ap.add_argument("--no-extra", action="store_true", help="only the headline workload")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--workload", default="fp8_m1", help="headline workload: fp8_m1 | int4_m1")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build runs on one GPU (the whole layer is resident; no collectives are built); "
+              "--gpus %d is not supported" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from dsgx10_amd import abi, lib
+    from dsgx10_amd.benchdata import DecodeBench, Fp8LayerGen, Int4LayerGen
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU", file=sys.stderr)
+        sys.exit(2)
+    lib.lib()  # fails loudly when the HIP extension is not built
+    torch.cuda.set_device(0)
+    K, W = args.steps, args.warmup
+    t_start = time.time()
+
+    def run_decode(gen, M, steps, warmup):
+        b = DecodeBench(gen, M, steps)
+        r = b.time_layer(warmup)
+        r.update(b.time_up_kernel())
+        log("  %s M=%d: %.2f us/layer (%.1f%% of 8 TB/s), gate/up kernel %.2f us (%.1f%%)" %
+            (gen.name, M, r["us_per_layer"], 100 * r["layer_hbm_frac"], r["up_us"], 100 * r["up_frac"]))
+        return b, r
+
+    def cpu_baseline(b, budget_s):
+        """The C++ oracle on the host cores over step 0 of the same workload (f32 contract sums only), repeated for about
+        budget_s seconds; its result is also the checker of the GPU's outputs for that step."""
+        from tests import orc   # the oracle: test infrastructure, used here as baseline and checker only
+        d = b.run_step_and_download(0)
+        hl, uni = d["layer"], np.arange(len(d["experts"]), dtype=np.int32)
+        orc.set_f32_only(True)
+        ts = []
+        while (sum(ts) < budget_s and len(ts) < 200) or len(ts) < 3:
+            t0 = time.perf_counter()
+            up = orc.moe_up(hl, d["x"], uni, want_range=False)
+            dn = orc.moe_down(hl, up["h32"], d["idx"], d["w"], uni)
+            ts.append(time.perf_counter() - t0)
+        orc.set_f32_only(False)
+        def err(got, ref):
+            return dict(max_abs_err=float(np.abs(got - ref).max()),
+                        rel_l2=float(np.sqrt(((got - ref).astype(np.float64) ** 2).sum() / max((ref.astype(np.float64) ** 2).sum(), 1e-300))))
+        par = {"yr": err(d["yr"], dn["yr32"])}
+        if hl.has_shared:
+            par["ys"] = err(d["ys"], dn["ys32"])
+        return dict(value=float(np.mean(ts[1:]) * 1e6), unit="us", cores=orc.threads(), kind="port",
+                    sample="step 0 of the same workload (M=%d, %d routed experts + shared), %d repetitions after one warm-up, "
+                           "C++ oracle, OpenMP, f32 sums" % (b.M, len(d["experts"]), len(ts) - 1),
+                    gpu_vs_oracle=par)
+
+    head_fp8 = args.workload == "fp8_m1"
+    log("generating the %s layer ..." % ("FP8 256-expert" if head_fp8 else "INT4 168-expert"))
+    gen = Fp8LayerGen(seed=0) if head_fp8 else Int4LayerGen(seed=0)
+    log("  %.1f s, pool %.2f GB" % (time.time() - t_start, gen.pool.numel() / 1e9))
+    stream_gbs = gen.stream_read_gbs()
+    b, r = run_decode(gen, 1, K, W)
+    cpu = None
+    if not args.no_cpu:
+        cpu = cpu_baseline(b, 10.0)
+        log("  cpu baseline: %.0f us on %d cores; gpu vs oracle %s" % (cpu["value"], cpu["cores"], cpu["gpu_vs_oracle"]))
+    extra = []
+    if not args.no_extra:
+        ks = min(K, 128)
+        for M in (4, 8):
+            _, e = run_decode(gen, M, ks, min(W, 16))
+            extra.append(dict(workload=gen.name, M=M, us_per_layer=e["us_per_layer"], bytes=e["bytes_per_layer"],
+                              hbm_frac=e["layer_hbm_frac"], up_kernel_us=e["up_us"], up_hbm_frac=e["up_frac"]))
+        del b
+        other = Int4LayerGen(seed=0) if head_fp8 else Fp8LayerGen(seed=0)
+        for M in (1, 8):
+            ob, e = run_decode(other, M, ks if M > 1 else K, min(W, 16))
+            d = dict(workload=other.name, M=M, us_per_layer=e["us_per_layer"], bytes=e["bytes_per_layer"],
+                     hbm_frac=e["layer_hbm_frac"], up_kernel_us=e["up_us"], up_hbm_frac=e["up_frac"])
+            if M == 1 and not args.no_cpu:
+                d["cpu_baseline"] = cpu_baseline(ob, 5.0)
+            extra.append(d)
+            del ob
+        del other
+        from dsgx10_amd.benchdata import gemv_bench
+        extra += gemv_bench()
+
+    out = {
+        "metric": "us_per_moe_layer",
+        "value": r["us_per_layer"],
+        "unit": "us",
+        "n_gpus": 1,
+        "steps": K,
+        "warmup": W,
+        "ms_per_step": r["us_per_layer"] / 1000.0,
+        "higher_is_better": False,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32 accumulate over e4m3 weights x bf16 activations" if head_fp8 else "f32 accumulate over int4-g32 weights x bf16 activations",
+        "data": "synthetic (torch-seeded N(0,0.02) weights quantised on the GPU, N(0,1) bf16 rows and f32 logits)",
+        "config": {"workload": gen.describe(1), "rows_M": 1, "steps_route_different_experts": True,
+                   "bytes_per_layer": r["bytes_per_layer"], "layer_hbm_frac_of_8TBs": r["layer_hbm_frac"],
+                   "kernels_per_step": ["k_route", "k_up", "k_down"], "timed_as": "one HIP graph of all steps, one replay"},
+        "roofline": {"bound": "hbm", "kernel": "k_up (gate/up + SwiGLU)", "achieved": r["up_gbs"], "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": r["up_frac"], "traffic": None, "bytes_per_launch": r["up_bytes"],
+                     "avg_launch_us": r["up_us"], "measured_stream_read_gbs": stream_gbs},
+        "cpu_baseline": cpu,
+        "extra": extra,
+        "wall_s": round(time.time() - t_start, 1),
+    }
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,325 @@
+"""Synthetic layers and timing loops for bench.py (GPU side only; torch is the allocator and RNG).
+
+The layers have the benchmark's full shapes: weights ~ N(0, 0.02) quantised on the GPU with the reference's FP8
+quantiser (per 128 x 128 block: scale = amax * f32(1/448), e4m3 round-to-nearest-even;
+altar1-4xgx10-switchless/engine/attn/tools/pack.py:216-232) or this build's symmetric INT4-g32 quantiser (scale =
+bf16(amax / 7), stored zero point 8), laid out in the pool formats of include/dsgx.h."""
+import ctypes as C
+
+import numpy as np
+import torch
+
+from . import abi, lib
+from .layer import DESC_DTYPE, HostLayer, mat_bytes
+
+HBM_PEAK = 8.0e12
+
+
+def _al256(n):
+    return (n + 255) // 256 * 256
+
+
+def fp8_quantize_gpu(w):
+    """w f32 [N][K] on the GPU -> (codes u8 [N][K], scales f32 [N/128][K/128])"""
+    N, K = w.shape
+    blk = w.view(N // 128, 128, K // 128, 128)
+    amax = blk.abs().amax(dim=(1, 3))
+    scale = (amax * torch.tensor(1.0 / 448.0, dtype=torch.float32, device=w.device)).clamp_min(1e-12)
+    q = (blk / scale[:, None, :, None]).to(torch.float8_e4m3fn)
+    return q.view(torch.uint8).reshape(N, K), scale
+
+
+def int4_quantize_gpu(w):
+    """w f32 [N][K] -> (packed i32 [N][K/8], scale bf16 [N][K/32], zp i32 [N/8][K/32]) symmetric, stored zero point 8"""
+    N, K = w.shape
+    g = w.view(N, K // 32, 32)
+    amax = g.abs().amax(-1)
+    s = torch.where(amax > 0, amax / 7.0, torch.ones_like(amax)).to(torch.bfloat16)
+    q = torch.clamp(torch.round(g / s.float()[..., None]), -8, 7).to(torch.int64) + 8
+    sh = torch.arange(8, device=w.device, dtype=torch.int64) * 4
+    words = (q.view(N, K // 8, 8) << sh).sum(-1)
+    words = torch.where(words >= 2 ** 31, words - 2 ** 32, words).to(torch.int32)
+    zp = torch.full((N // 8, K // 32), -0x77777778, dtype=torch.int32, device=w.device)  # 0x88888888
+    return words, s, zp
+
+
+def _put(pool, off, t):
+    b = t.contiguous().view(torch.uint8).reshape(-1)
+    pool[off:off + b.numel()] = b
+    return _al256(b.numel())
+
+
+class _LayerGen:
+    """A full layer on the GPU: pool + descriptors + NSH rotating copies of the shared expert."""
+
+    def layer_w(self, shared_copy):
+        L = abi.LayerW()
+        L.pool, L.desc = self.pool.data_ptr(), self.desc.data_ptr()
+        L.fmt, L.H, L.I, L.E, L.topk = self.fmt, self.H, self.I, self.E, self.topk
+        self._set_shared(L, shared_copy % self.NSH)
+        return L
+
+    def stream_read_gbs(self):
+        sink = torch.zeros(4, dtype=torch.uint8, device="cuda")
+        n = self.pool.numel() // 16 * 16
+        lib.stream_read(self.pool, n, sink)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        lib.stream_read(self.pool, n, sink)
+        e1.record()
+        torch.cuda.synchronize()
+        return n / (e0.elapsed_time(e1) * 1e-3) / 1e9
+
+
+class Fp8LayerGen(_LayerGen):
+    name = "fp8_moe_decode"
+    fmt, H, I, E, topk, route_scale, NSH = abi.FMT_FP8, 4096, 2048, 256, 8, 1.0, 16
+
+    def __init__(self, seed=0):
+        g = torch.Generator(device="cuda")
+        g.manual_seed(seed)
+        H, I, E = self.H, self.I, self.E
+        per = [mat_bytes(self.fmt, I, H), mat_bytes(self.fmt, I, H), mat_bytes(self.fmt, H, I)]
+        self.expert_bytes = sum(per)
+        self.pool = torch.zeros(E * self.expert_bytes, dtype=torch.uint8, device="cuda")
+        desc = np.zeros(E * 3, DESC_DTYPE)
+        o = 0
+        for e in range(E):
+            for j in range(3):
+                N, K = (I, H) if j < 2 else (H, I)
+                codes, scale = fp8_quantize_gpu(torch.randn(N, K, generator=g, device="cuda") * 0.02)
+                d = desc[e * 3 + j]
+                d["off"], d["s2"], d["fmt"] = o, 1.0, self.fmt
+                _put(self.pool, o, codes)
+                _put(self.pool, o + _al256(N * K), scale)
+                o += per[j]
+        self.desc = torch.from_numpy(desc.view(np.uint8).reshape(-1)).cuda()
+        self.shared = []
+        for c in range(self.NSH):
+            mats = []
+            for j in range(3):
+                N, K = (I, H) if j < 2 else (H, I)
+                mats.append(fp8_quantize_gpu(torch.randn(N, K, generator=g, device="cuda") * 0.02))
+            self.shared.append(mats)
+        self.shared_bytes = self.expert_bytes
+
+    def _set_shared(self, L, c):
+        (gc, gs), (uc, us), (dc, ds) = self.shared[c]
+        L.sh.g, L.sh.u, L.sh.d = gc.data_ptr(), uc.data_ptr(), dc.data_ptr()
+        L.sh.gs, L.sh.us, L.sh.ds = gs.data_ptr(), us.data_ptr(), ds.data_ptr()
+
+    def describe(self, M):
+        return ("FP8 MoE decode layer: hidden 4096, 256 routed experts + 1 fused shared, intermediate 2048, e4m3 weights with "
+                "128x128 f32 block scales, sigmoid top-8 renormalised (scale 1, no bias), M=%d bf16 rows" % M)
+
+    def up_bytes(self, U):
+        return (U + 1) * 2 * mat_bytes(self.fmt, self.I, self.H)
+
+    def layer_bytes(self, U):
+        return (U + 1) * self.expert_bytes
+
+    def host_sublayer(self, experts, shared_copy):
+        """the picked experts (ascending ids) and the shared copy as a HostLayer whose expert ids are 0..len-1"""
+        H, I = self.H, self.I
+        desc = np.frombuffer(self.desc.cpu().numpy().tobytes(), DESC_DTYPE)
+        ex = []
+        for e in experts:
+            mats = []
+            for j in range(3):
+                N, K = (I, H) if j < 2 else (H, I)
+                o = int(desc[e * 3 + j]["off"])
+                codes = self.pool[o:o + N * K].cpu().numpy().reshape(N, K)
+                so = o + _al256(N * K)
+                sc = self.pool[so:so + (N // 128) * (K // 128) * 4].cpu().numpy().view(np.float32).reshape(N // 128, K // 128)
+                mats.append((codes, sc))
+            ex.append(tuple(mats))
+        sh = tuple((c.cpu().numpy(), s.cpu().numpy()) for c, s in self.shared[shared_copy % self.NSH])
+        return HostLayer(self.fmt, H, I, len(experts), self.topk, ex, emap=np.arange(len(experts)), shared_fp8=sh)
+
+
+class Int4LayerGen(_LayerGen):
+    name = "int4_moe_decode"
+    fmt, H, I, E, topk, route_scale, NSH = abi.FMT_INT4, 6144, 2048, 168, 8, 2.5, 8
+
+    def __init__(self, seed=0):
+        g = torch.Generator(device="cuda")
+        g.manual_seed(seed + 1)
+        H, I, E = self.H, self.I, self.E
+        per = [mat_bytes(self.fmt, I, H), mat_bytes(self.fmt, I, H), mat_bytes(self.fmt, H, I)]
+        self.expert_bytes = sum(per)
+        self.pool = torch.zeros(E * self.expert_bytes, dtype=torch.uint8, device="cuda")
+        desc = np.zeros(E * 3, DESC_DTYPE)
+        o = 0
+        for e in range(E):
+            for j in range(3):
+                N, K = (I, H) if j < 2 else (H, I)
+                words, s, zp = int4_quantize_gpu(torch.randn(N, K, generator=g, device="cuda") * 0.02)
+                d = desc[e * 3 + j]
+                d["off"], d["s2"], d["fmt"] = o, 1.0, self.fmt
+                _put(self.pool, o, words)
+                _put(self.pool, o + _al256(N * K // 2), s)
+                _put(self.pool, o + _al256(N * K // 2) + _al256(N * (K // 32) * 2), zp)
+                o += per[j]
+        self.desc = torch.from_numpy(desc.view(np.uint8).reshape(-1)).cuda()
+        self.shared = []
+        for c in range(self.NSH):
+            bgu = (torch.randn(2 * I, H, generator=g, device="cuda") * 0.02).to(torch.bfloat16)
+            bd = (torch.randn(H, I, generator=g, device="cuda") * 0.02).to(torch.bfloat16)
+            self.shared.append((bgu, bd))
+        self.shared_bytes = 3 * H * I * 2
+
+    def _set_shared(self, L, c):
+        bgu, bd = self.shared[c]
+        L.sh.bgu, L.sh.bd = bgu.data_ptr(), bd.data_ptr()
+
+    def describe(self, M):
+        return ("INT4-g32 MoE decode layer (GLM-style): hidden 6144, 168 routed experts (compressed-tensors int4, bf16 group scales, "
+                "stored zero points) + 1 fused bf16 shared expert, intermediate 2048, sigmoid top-8 x 2.5, M=%d bf16 rows" % M)
+
+    def up_bytes(self, U):
+        return U * 2 * mat_bytes(self.fmt, self.I, self.H) + 2 * self.I * self.H * 2
+
+    def layer_bytes(self, U):
+        return U * self.expert_bytes + self.shared_bytes
+
+    def host_sublayer(self, experts, shared_copy):
+        H, I = self.H, self.I
+        desc = np.frombuffer(self.desc.cpu().numpy().tobytes(), DESC_DTYPE)
+        ex = []
+        for e in experts:
+            mats = []
+            for j in range(3):
+                N, K = (I, H) if j < 2 else (H, I)
+                o = int(desc[e * 3 + j]["off"])
+                a, b = _al256(N * K // 2), _al256(N * (K // 32) * 2)
+                p = self.pool[o:o + N * K // 2].cpu().numpy().view(np.uint32).reshape(N, K // 8)
+                s = self.pool[o + a:o + a + N * (K // 32) * 2].cpu().numpy().view(np.uint16).reshape(N, K // 32)
+                z = self.pool[o + a + b:o + a + b + (N // 8) * (K // 32) * 4].cpu().numpy().view(np.uint32).reshape(N // 8, K // 32)
+                mats.append((p, s, z))
+            ex.append(tuple(mats))
+        bgu, bd = self.shared[shared_copy % self.NSH]
+        sh = (bgu.view(torch.int16).cpu().numpy().view(np.uint16), bd.view(torch.int16).cpu().numpy().view(np.uint16))
+        return HostLayer(self.fmt, H, I, len(experts), self.topk, ex, emap=np.arange(len(experts)), shared_bf16=sh)
+
+
+class DecodeBench:
+    """`steps` decode steps of M rows over a generated layer; step s routes logits[s] (seeded N(0,1))."""
+
+    def __init__(self, gen, M, steps, seed=1234):
+        self.gen, self.M, self.steps = gen, M, steps
+        g = torch.Generator(device="cuda")
+        g.manual_seed(seed)
+        self.x = torch.randn(M, gen.H, generator=g, device="cuda").to(torch.bfloat16)
+        self.logits = torch.randn(steps, M, gen.E, generator=g, device="cuda")
+        self.idx = torch.zeros(steps, M, gen.topk, dtype=torch.int32, device="cuda")
+        self.w = torch.zeros(steps, M, gen.topk, dtype=torch.float32, device="cuda")
+        self.layers = [gen.layer_w(c) for c in range(gen.NSH)]
+        self.ws = torch.zeros(lib.decode_ws_bytes(self.layers[0]), dtype=torch.uint8, device="cuda")
+        self.yr = torch.zeros(M, gen.H, dtype=torch.float32, device="cuda")
+        self.ys = torch.zeros(M, gen.H, dtype=torch.float32, device="cuda")
+        for s in range(steps):
+            lib.route(self.logits[s], None, self.idx[s], self.w[s], gen.route_scale)
+        torch.cuda.synchronize()
+        idx = self.idx.cpu().numpy()
+        self.union_sizes = np.array([len(np.unique(idx[s])) for s in range(steps)])
+
+    def step(self, s, parts=3, route=True):
+        g = self.gen
+        if route:
+            lib.route(self.logits[s], None, self.idx[s], self.w[s], g.route_scale)
+        lib.moe_decode(self.layers[s % g.NSH], self.x, self.idx[s], self.w[s], self.M, self.ws, self.yr, self.ys, parts=parts)
+
+    def _graph(self, fn):
+        gr = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(gr):
+            fn()
+        return gr
+
+    def _time_graph(self, gr, reps=1):
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            gr.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e-3 / reps
+
+    def time_layer(self, warmup):
+        for s in range(warmup):
+            self.step(s % self.steps)
+        torch.cuda.synchronize()
+        gr = self._graph(lambda: [self.step(s) for s in range(self.steps)])
+        gr.replay()  # untimed: uploads the graph
+        sec = self._time_graph(gr)
+        us = sec / self.steps * 1e6
+        bytes_ = float(np.mean([self.gen.layer_bytes(u) for u in self.union_sizes]))
+        return dict(us_per_layer=us, bytes_per_layer=bytes_, layer_hbm_frac=bytes_ / (us * 1e-6) / HBM_PEAK,
+                    mean_union=float(self.union_sizes.mean()))
+
+    def time_up_kernel(self):
+        """the dominant kernel alone: `steps` launches of the gate/up kernel back to back in one graph"""
+        gr = self._graph(lambda: [self.step(s, parts=1, route=False) for s in range(self.steps)])
+        gr.replay()
+        sec = self._time_graph(gr)
+        us = sec / self.steps * 1e6
+        b = float(np.mean([self.gen.up_bytes(u) for u in self.union_sizes]))
+        gbs = b / (us * 1e-6) / 1e9
+        return dict(up_us=us, up_bytes=b, up_gbs=gbs, up_frac=gbs * 1e9 / HBM_PEAK)
+
+    def run_step_and_download(self, s):
+        """runs step s eagerly; returns the host copies the CPU oracle needs and the GPU's outputs"""
+        self.step(s)
+        torch.cuda.synchronize()
+        idx = self.idx[s].cpu().numpy()
+        w = self.w[s].cpu().numpy()
+        experts = sorted(set(int(e) for e in idx.reshape(-1)))
+        remap = {e: i for i, e in enumerate(experts)}
+        idx_local = np.vectorize(remap.get)(idx).astype(np.int32)
+        hl = self.gen.host_sublayer(experts, s)
+        x = self.x.view(torch.int16).cpu().numpy().view(np.uint16)
+        return dict(layer=hl, x=x, idx=idx_local, w=w, yr=self.yr.cpu().numpy().copy(), ys=self.ys.cpu().numpy().copy(),
+                    experts=experts)
+
+
+def gemv_bench(reps=64):
+    """the two dense GEMV configurations: FP8 [2048 x 4096] at 1 row, INT4 [1536 x 6144] at 1, 2, 4, 6 rows; weights rotate
+    over copies that exceed the caches"""
+    out = []
+    g = torch.Generator(device="cuda")
+    g.manual_seed(7)
+    for name, fmt, N, K, rows in (("dense_fp8_gemv_2048x4096", abi.FMT_FP8, 2048, 4096, (1,)),
+                                  ("dense_int4_gemv_1536x6144", abi.FMT_INT4, 1536, 6144, (1, 2, 4, 6))):
+        per = mat_bytes(fmt, N, K)
+        copies = max(8, int(600e6 // per))
+        mats = []
+        for c in range(copies):
+            w = torch.randn(N, K, generator=g, device="cuda") * 0.02
+            mats.append(fp8_quantize_gpu(w) if fmt == abi.FMT_FP8 else int4_quantize_gpu(w))
+        for M in rows:
+            x = torch.randn(M, K, generator=g, device="cuda").to(torch.bfloat16)
+            y = torch.zeros(M, N, dtype=torch.bfloat16, device="cuda")
+
+            def one(c):
+                m = mats[c % copies]
+                seg = dict(fmt=fmt, w=m[0], s=m[1], zp=m[2] if len(m) > 2 else None, n=N, y=y, ldy=N)
+                lib.gemv(x, K, M, K, [seg], abi.OUT_BF16)
+            for c in range(4):
+                one(c)
+            torch.cuda.synchronize()
+            gr = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(gr):
+                for c in range(reps):
+                    one(c)
+            gr.replay()
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            gr.replay()
+            e1.record()
+            torch.cuda.synchronize()
+            us = e0.elapsed_time(e1) * 1e3 / reps
+            b = per + M * K * 2 + M * N * 2
+            out.append(dict(workload=name, M=M, us_per_call=us, bytes=b, hbm_frac=b / (us * 1e-6) / HBM_PEAK))
+    return out

@@ -2,6 +2,8 @@
 // baselines, finalize, the dequantisation probes and act_quant.
 #include <cstdarg>
 #include <cstdio>
+#include <mutex>
+#include <unordered_map>
 
 #include "abi_internal.h"
 #include "common.cuh"
@@ -27,6 +29,18 @@ int num_cus_cached() {
     if (n <= 0) n = 256;
   }
   return n;
+}
+
+int allow_dynamic_lds(const void* kern, size_t lds) {
+  if (lds <= 48 * 1024) return DSGX_OK;
+  static std::mutex mu;
+  static std::unordered_map<const void*, size_t> seen;
+  std::lock_guard<std::mutex> lk(mu);
+  auto it = seen.find(kern);
+  if (it != seen.end() && it->second >= lds) return DSGX_OK;
+  DSGX_HIP(hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+  seen[kern] = lds;
+  return DSGX_OK;
 }
 
 namespace {

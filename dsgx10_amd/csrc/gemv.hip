@@ -114,7 +114,7 @@ int launch_gemv(const GemvArgs& a, hipStream_t st) {
   if (grid > (nbatch + 3) / 4) grid = (nbatch + 3) / 4;
   if (grid < 1) grid = 1;
   auto kern = k_gemv<FMT, M, RB, D>;
-  if (lds > 48 * 1024) DSGX_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+  if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds)) return rc;
   hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, st, a);
   DSGX_HIP(hipGetLastError());
   return DSGX_OK;

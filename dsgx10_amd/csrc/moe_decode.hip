@@ -340,10 +340,7 @@ __global__ void __launch_bounds__(256) k_down(DecodeArgs a, int slots_per_chunk)
 
 // ---------------------------------------------------------------------------------------------------------------------
 template <class K>
-int set_lds(K kern, size_t lds) {
-  if (lds > 48 * 1024) DSGX_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-  return DSGX_OK;
-}
+int set_lds(K kern, size_t lds) { return allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds); }
 
 template <int FMT, int SHFMT, int M>
 int launch_decode(const DecodeArgs& a, int parts, hipStream_t st) {

@@ -91,8 +91,9 @@ def moe_decode(layer_w, x, idx, w, M, ws, yr, ys, stream=None, parts=3, ysum=Fal
                                  _stream(stream), C.byref(cfg)))
 
 
-def finalize(R, S, out, stream=None):
-    _check(lib().dsgx_finalize(_ptr(R), _ptr(S), R.numel(), _ptr(out), _stream(stream)))
+def finalize(R, S, n, out, stream=None):
+    """out[i] = bf16(bf16(R[i]) + bf16(S[i])) for n = M * H values"""
+    _check(lib().dsgx_finalize(_ptr(R), _ptr(S), n, _ptr(out), _stream(stream)))
 
 
 # ---- gx::moe_prefill --------------------------------------------------------------------------------------------------

@@ -165,8 +165,9 @@ DSGX_API int dsgx_gemv(const uint16_t* x, int ldx, int rows, int K, const dsgx_g
 DSGX_API int dsgx_dequant_int4(const void* packed, const void* scale, const void* zp, int N, int K, uint16_t* out,
                                size_t ld, void* stream);
 /* The same through the streaming kernels' own in-register decode: the probe that pins the hot loops' INT4 arithmetic to
-   the contract bit for bit, as the reference's k_deq does (engine/experts/tests/test_experts.cu:217-235). Exact for
-   |scale| < 2^124 (the checkpoint's scales are 2^-15 .. 2^-4); dsgx_dequant_int4 is exact for every finite scale. */
+   the contract bit for bit, as the reference's k_deq does (engine/experts/tests/test_experts.cu:217-235). Bit-exact for
+   positive scales below 2^124 (the checkpoint's are 2^-15 .. 2^-4; a negative scale, which the format forbids, gives
+   +0 instead of -0 where u = u_z); dsgx_dequant_int4 is exact for every finite scale. */
 DSGX_API int dsgx_probe_dequant_int4(const void* packed, const void* scale, const void* zp, int N, int K, uint16_t* out,
                                      size_t ld, void* stream);
 /* FP8 codes -> bf16 bits of the exact e4m3 values [N][ld] (the widening the GEMV and MoE kernels use;

@@ -1,0 +1,140 @@
+// gx:: - the routed-expert operators with the reference engine's names and argument order
+// (altar1-4xgx10-switchless/engine/experts/experts.h:15-195), forwarding to the C ABI in dsgx.h.
+//
+// What differs from the reference header, and why:
+//  * cudaStream_t -> a hipStream_t passed as void*; __nv_bfloat16 -> uint16_t bit patterns.
+//  * the per-rank shape constants (kH, kI, kE, kTopK: experts.h:18-26) are fields of LayerW, defaulting to the
+//    reference's values, so the whole-layer shapes of one GPU (intermediate 2048) and the DeepSeek-shaped layer fit.
+//  * Fmt gains the tags of the MI355X layouts (the checkpoint's row-major tensors); the reference's tags name GB10
+//    block tilings and are refused by every operator.
+//  * DecodeCfg::post (ring posting) must stay null; pdl is accepted and ignored (HIP has no programmatic dependent launch).
+#pragma once
+#include <cstddef>
+#include <cstdint>
+
+#include "check.h"
+
+namespace gx {
+
+constexpr int kH = 6144, kI = 512, kE = 168, kTopK = 8;  // the reference's per-rank defaults (experts.h:18-22)
+constexpr float kRouteScale = 2.5f;
+constexpr int kMaxRows = DSGX_MAX_ROWS, kMaxUnion = DSGX_MAX_UNION, kShSlot = DSGX_SH_SLOT, kMaxChunk = DSGX_MAX_CHUNK;
+
+enum Fmt : uint32_t {
+  kNVFP4 = DSGX_FMT_REF_NVFP4, kINT4 = DSGX_FMT_REF_INT4, kBF16 = DSGX_FMT_REF_BF16,  // GB10 tilings: refused
+  kFP8B128 = DSGX_FMT_FP8_B128, kINT4G32 = DSGX_FMT_INT4_G32, kBF16Rows = DSGX_FMT_BF16
+};
+constexpr bool fmt_known(uint32_t f) { return f == kFP8B128 || f == kINT4G32 || f == kBF16Rows; }
+inline size_t mat_bytes(uint32_t fmt, int N, int K) { return dsgx_mat_bytes(fmt, N, K); }
+constexpr const char* fmt_name(uint32_t f) {
+  return f == kFP8B128 ? "FP8_B128" : f == kINT4G32 ? "INT4_G32" : f == kBF16Rows ? "BF16" : "unknown";
+}
+
+using MatDesc = dsgx_mat_desc;
+static_assert(sizeof(MatDesc) == 64, "MatDesc is 64 B");
+// make_desc / desc_ok of the reference (engine/experts/layout.h:165-183)
+inline MatDesc make_desc(uint64_t off, float s2, uint32_t fmt) {
+  if (!fmt_known(fmt)) die("make_desc: expert format %u is not FP8_B128 (16), INT4_G32 (18) or BF16 (19)", fmt);
+  MatDesc d{};
+  d.off = off, d.s2 = s2, d.fmt = fmt;
+  return d;
+}
+inline bool desc_ok(const MatDesc& d, uint32_t fmt) {
+  if (d.fmt != fmt || !fmt_known(fmt) || d.off % 256) return false;
+  if (!(d.s2 > 0.f) || d.s2 != d.s2 || d.s2 > 3.4e38f || d.s2 != 1.f) return false;
+  for (uint32_t r : d.rsv)
+    if (r) return false;
+  return true;
+}
+
+struct SharedW : dsgx_shared_w {
+  SharedW() : dsgx_shared_w{} {}
+  bool fused() const { return g != nullptr; }
+  bool bf16() const { return bgu != nullptr; }
+};
+
+struct LayerW {
+  const uint8_t* pool = nullptr;
+  const MatDesc* desc = nullptr;  // [E][3]: gate, up, down (device memory)
+  SharedW sh;
+  uint32_t fmt = kINT4G32;
+  int H = kH, I = kI, E = kE, topk = kTopK;
+  dsgx_layer_w c() const { return dsgx_layer_w{pool, desc, sh, fmt, H, I, E, topk}; }
+};
+
+// ---- routing (experts.h:99-102) -----------------------------------------------------------------------------------
+inline void route(const float* logits, const float* bias, int M, int* idx, float* w, void* st, bool pdl = true, int E = kE,
+                  int topk = kTopK, float scale = kRouteScale) {
+  (void)pdl;
+  DSGX_DIE_ON(dsgx_route(logits, bias, M, E, topk, scale, 0, idx, w, st));
+}
+
+// ---- decode (experts.h:104-147) -----------------------------------------------------------------------------------
+struct DecodeCfg {
+  int up = 0, down = 0;
+  int up_ctas_per_sm = 0;  // accepted, unused: the grid is sized to the chip
+  bool pdl = true;         // accepted, unused
+  bool dyn = true;         // accepted, unused: batches are walked round-robin, no task counter
+  bool xpf = true;         // accepted, unused
+  int parts = 3;
+  const float* logits = nullptr;
+  const float* bias = nullptr;
+  float route_scale = kRouteScale;  // fused routing's scale (the reference's is the constant 2.5)
+  const void* post = nullptr;       // must be null
+  bool ysum = false;
+};
+inline size_t decode_ws_bytes(const LayerW& L) { const dsgx_layer_w c = L.c(); return dsgx_decode_ws_bytes(&c); }
+inline void moe_decode(const LayerW& L, const uint16_t* x, const int* idx, const float* w, int M, void* ws, float* yr, float* ys,
+                       void* st, const DecodeCfg& cfg = DecodeCfg()) {
+  const dsgx_layer_w c = L.c();
+  dsgx_decode_cfg d;
+  dsgx_decode_cfg_default(&d);
+  d.up = cfg.up, d.down = cfg.down, d.parts = cfg.parts, d.ysum = cfg.ysum, d.logits = cfg.logits, d.bias = cfg.bias;
+  d.route_scale = cfg.route_scale, d.post = cfg.post;
+  DSGX_DIE_ON(dsgx_moe_decode(&c, x, idx, w, M, ws, yr, ys, st, &d));
+}
+inline int decode_up_variants() { return 1; }
+inline int decode_down_variants() { return 1; }
+inline const char* decode_up_name(int) { return "rows4 lanes64"; }
+inline const char* decode_down_name(int) { return "rows2 lanes64"; }
+inline void finalize(const float* R, const float* S, int M, uint16_t* out, void* st, bool pdl = true, int H = kH) {
+  (void)pdl;
+  DSGX_DIE_ON(dsgx_finalize(R, S, M * H, out, st));
+}
+
+// ---- prefill (experts.h:149-193) ----------------------------------------------------------------------------------
+enum PrefillPhase { kPhBucket = 1, kPhUp = 2, kPhDown = 4, kPhCombine = 8, kPhShared = 16, kPhAll = 31 };
+struct PrefillCfg {
+  bool shared = true;
+  int diag = 0, ddiag = 0;  // accepted, must be 0
+  int down = 1, up = 1;     // accepted, unused (one implementation of each)
+  int sh_rows = 128, yr_kb = 0, chain_q = 4;
+  void* side = nullptr;     // accepted, unused
+  bool act_fp8 = true;      // FP8 layers: e4m3 activations on the fp8 MFMA (see dsgx_prefill_cfg)
+};
+inline size_t prefill_ws_bytes(const LayerW& L, int T) { const dsgx_layer_w c = L.c(); return dsgx_prefill_ws_bytes(&c, T); }
+inline void moe_prefill_phases(const LayerW& L, const uint16_t* x, const int* idx, const float* w, int T, void* ws, float* yr,
+                               float* ys, void* st, const PrefillCfg& cfg, int phases) {
+  if (cfg.diag || cfg.ddiag) die("moe_prefill: bench diagnostics are not built");
+  const dsgx_layer_w c = L.c();
+  dsgx_prefill_cfg p;
+  dsgx_prefill_cfg_default(&p);
+  p.shared = cfg.shared, p.phases = phases, p.act_fp8 = cfg.act_fp8;
+  DSGX_DIE_ON(dsgx_moe_prefill(&c, x, idx, w, T, ws, yr, ys, st, &p));
+}
+inline void moe_prefill(const LayerW& L, const uint16_t* x, const int* idx, const float* w, int T, void* ws, float* yr, float* ys,
+                        void* st, const PrefillCfg& cfg = PrefillCfg()) {
+  moe_prefill_phases(L, x, idx, w, T, ws, yr, ys, st, cfg, kPhAll);
+}
+struct PrefillView {
+  const int *rpos, *re;
+  const uint16_t *h, *hsh;
+};
+inline PrefillView prefill_view(const LayerW& L, void* ws, int T) {
+  const dsgx_layer_w c = L.c();
+  dsgx_prefill_view v;
+  DSGX_DIE_ON(dsgx_prefill_view_get(&c, ws, T, &v));
+  return PrefillView{v.rpos, v.re, v.h, v.hsh};
+}
+
+}  // namespace gx

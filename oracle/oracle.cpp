@@ -315,11 +315,27 @@ static inline void mat_row_raw(const Mat& m, int n, float* out) {
   for (int k = 0; k < m.K; ++k) out[k] = mat_raw(m, n, k);
 }
 struct Dot { float f; double d, mag; };
+// f32 sums only (the timed CPU baseline): the f64 sums and sums of |terms| come back as 0
+static int g_f32_only = 0;
+ORC void orc_set_f32_only(int on) { g_f32_only = on; }
 // One output: the f32 sum in the contract's order and the f64 sum with the sum of |terms|.
 // FP8 (A/engine/experts/decode.cu:283-303, A/micro/gemv.cu:512): per 128-k unit c from zero, acc = fmaf(S, c, acc).
 // INT4, BF16 (A/engine/attn/gemv.cu:246, 315): straight f32 accumulation in k order; bf16 x bf16 products are exact.
 static inline Dot dot_row(const Mat& m, int n, const float* wrow, const float* x) {
   Dot r{0.f, 0.0, 0.0};
+  if (g_f32_only) {
+    if (m.fmt == DSGX_FMT_FP8_B128) {
+      const float* sr = m.fs + (size_t)(n / 128) * (m.K / 128);
+      for (int b = 0; b < m.K / 128; ++b) {
+        float c = 0.f;
+        for (int k = 128 * b; k < 128 * b + 128; ++k) c += x[k] * wrow[k];
+        r.f = fmaf(sr[b], c, r.f);
+      }
+    } else {
+      for (int k = 0; k < m.K; ++k) r.f += x[k] * wrow[k];
+    }
+    return r;
+  }
   if (m.fmt == DSGX_FMT_FP8_B128) {
     const float* sr = m.fs + (size_t)(n / 128) * (m.K / 128);
     for (int b = 0; b < m.K / 128; ++b) {

@@ -234,5 +234,10 @@ def finalize(R, S):
     return o
 
 
+def set_f32_only(on):
+    """the timed CPU baseline computes the f32 contract sums only"""
+    lib().orc_set_f32_only(int(on))
+
+
 def threads():
     return lib().orc_threads()
