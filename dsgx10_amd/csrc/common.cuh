@@ -64,19 +64,47 @@ __device__ __forceinline__ uint4 ldg_stream(const void* p) {
   return make_uint4(v.x, v.y, v.z, v.w);
 }
 
-// ---- wave64 sum, result valid in every lane ---------------------------------------------------------------------------------
+// ---- wave64 reductions, result valid in every lane -------------------------------------------------------------------------
+// Steps 1, 2, 4, 8 run inside a row of 16 lanes with DPP (quad permutes and mirrors); rows are joined with gfx950's
+// v_permlane16_swap / v_permlane32_swap: with both operands v, the two results hold each lane's own half and the other
+// half, so their sum (or max) is the xor-16 / xor-32 butterfly step without a trip through LDS.
 template <int CTRL>
-__device__ __forceinline__ float dpp_add(float v) {
-  const int t = __builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, true);
-  return v + __int_as_float(t);
+__device__ __forceinline__ uint32_t dpp_mov(uint32_t v) {
+  return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, 0xF, 0xF, true);
 }
+template <int CTRL>
+__device__ __forceinline__ float dpp_add(float v) { return v + __uint_as_float(dpp_mov<CTRL>(__float_as_uint(v))); }
 __device__ __forceinline__ float wave_sum(float v) {
   v = dpp_add<0xB1>(v);   // quad_perm [1,0,3,2]
   v = dpp_add<0x4E>(v);   // quad_perm [2,3,0,1]
   v = dpp_add<0x141>(v);  // row_half_mirror
   v = dpp_add<0x140>(v);  // row_mirror: every lane of a row of 16 holds the row's sum
-  v += __shfl_xor(v, 16);
-  v += __shfl_xor(v, 32);
+  auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  v = __uint_as_float(r[0]) + __uint_as_float(r[1]);
+  r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+__device__ __forceinline__ uint64_t wave_max_u64(uint64_t v) {
+  auto step = [](uint64_t x, uint32_t olo, uint32_t ohi) {
+    const uint64_t o = ((uint64_t)ohi << 32) | olo;
+    return o > x ? o : x;
+  };
+  v = step(v, dpp_mov<0xB1>((uint32_t)v), dpp_mov<0xB1>((uint32_t)(v >> 32)));
+  v = step(v, dpp_mov<0x4E>((uint32_t)v), dpp_mov<0x4E>((uint32_t)(v >> 32)));
+  v = step(v, dpp_mov<0x141>((uint32_t)v), dpp_mov<0x141>((uint32_t)(v >> 32)));
+  v = step(v, dpp_mov<0x140>((uint32_t)v), dpp_mov<0x140>((uint32_t)(v >> 32)));
+  {
+    auto lo = __builtin_amdgcn_permlane16_swap((uint32_t)v, (uint32_t)v, false, false);
+    auto hi = __builtin_amdgcn_permlane16_swap((uint32_t)(v >> 32), (uint32_t)(v >> 32), false, false);
+    const uint64_t a = ((uint64_t)hi[0] << 32) | lo[0], b = ((uint64_t)hi[1] << 32) | lo[1];
+    v = a > b ? a : b;
+  }
+  {
+    auto lo = __builtin_amdgcn_permlane32_swap((uint32_t)v, (uint32_t)v, false, false);
+    auto hi = __builtin_amdgcn_permlane32_swap((uint32_t)(v >> 32), (uint32_t)(v >> 32), false, false);
+    const uint64_t a = ((uint64_t)hi[0] << 32) | lo[0], b = ((uint64_t)hi[1] << 32) | lo[1];
+    v = a > b ? a : b;
+  }
   return v;
 }
 
@@ -132,18 +160,23 @@ __device__ __forceinline__ float route_score(float l, int score_fn) {
 // One row by one wavefront: experts e = lane + 64 j, j < 8 (E <= 512). Lane k < topk gets pick k's expert and weight
 // (route_warp of the reference, engine/experts/formats.cuh:207-247, at 64 lanes): descending key, ties to the lower
 // id; the sum in the butterfly order over eight places ((p0+p4)+(p2+p6))+((p1+p5)+(p3+p7)), absent places skipped.
+// The (key, id) order is one unsigned 64-bit order: the key's bits made monotone (sign flipped for positive, all
+// flipped for negative floats) above the complemented id, so each pick is one wave-wide integer maximum.
 __device__ __forceinline__ void route_row(const float* __restrict__ logits_row, const float* __restrict__ bias, int E, int topk,
                                           float scale, int score_fn, int lane, int& id_out, float& w_out) {
   constexpr int RJ = DSGX_MAX_EXPERTS / kWave;
-  float s[RJ], key[RJ];
+  float s[RJ];
+  uint64_t key[RJ];
+  const int nj = (E + kWave - 1) / kWave;
 #pragma unroll
   for (int j = 0; j < RJ; ++j) {
     const int e = lane + kWave * j;
-    if (e < E) {
+    s[j] = 0.f, key[j] = 0;  // an empty place: below every real key
+    if (j < nj && e < E) {
       s[j] = route_score(logits_row[e], score_fn);
-      key[j] = __fadd_rn(s[j], bias ? bias[e] : 0.f);
-    } else {
-      s[j] = 0.f, key[j] = -INFINITY;
+      const uint32_t kb = __float_as_uint(__fadd_rn(s[j], bias ? bias[e] : 0.f));
+      const uint32_t mono = kb ^ ((kb >> 31) ? 0xFFFFFFFFu : 0x80000000u);
+      key[j] = ((uint64_t)mono << 32) | (uint32_t)(~e);
     }
   }
   float picked[DSGX_MAX_TOPK];
@@ -152,24 +185,18 @@ __device__ __forceinline__ void route_row(const float* __restrict__ logits_row, 
   for (int k = 0; k < DSGX_MAX_TOPK; ++k) {
     picked[k] = 0.f, ids[k] = 0;
     if (k >= topk) continue;
-    float bv = -INFINITY;
-    int bj = 0;
+    uint64_t best = 0;
 #pragma unroll
     for (int j = 0; j < RJ; ++j)
-      if (key[j] > bv) bv = key[j], bj = j;
-    int be = bv == -INFINITY ? 1 << 30 : lane + kWave * bj;
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) {
-      const float ov = __shfl_xor(bv, o);
-      const int oe = __shfl_xor(be, o);
-      if (ov > bv || (ov == bv && oe < be)) bv = ov, be = oe;
-    }
+      if (j < nj && key[j] > best) best = key[j];
+    best = wave_max_u64(best);
+    const int be = (int)(~(uint32_t)best);
     ids[k] = be;
     float sv = 0.f;
 #pragma unroll
     for (int j = 0; j < RJ; ++j)
-      if (lane + kWave * j == be) sv = s[j], key[j] = -INFINITY;
-    picked[k] = __shfl(sv, be & (kWave - 1));
+      if (j < nj && lane + kWave * j == be) sv = s[j], key[j] = 0;
+    picked[k] = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(sv), __builtin_amdgcn_readfirstlane(be & (kWave - 1))));
   }
   auto add = [](float a, float b, bool hb) { return hb ? __fadd_rn(a, b) : a; };
   const float a04 = add(picked[0], picked[4], 4 < topk), a26 = add(picked[2], picked[6], 6 < topk);

@@ -1,0 +1,506 @@
+// The decode expert step for 1-8 rows: the gfx950 counterpart of the reference's gx::moe_decode
+// (altar1-4xgx10-switchless/engine/experts/decode.cu; contract in engine/experts/experts.h:104-147).
+//
+// The arithmetic of the reference's two kernels:
+//  up    every (slot, channel pair) of the union of the rows' picks (expert-id order; a fused shared expert first) is a
+//        batch of four weight rows (gate c, gate c+1, up c, up c+1) owned by one wavefront, which streams them once,
+//        K split over its 64 lanes, dequantises in registers, sums against the M activation rows staged in LDS, adds
+//        the lanes' partials with cross-lane shuffles, and writes h = bf16(bf16(silu(bf16 g)) * bf16 u) (decode.cu:366-400).
+//  down  a wavefront owns output rows and walks every slot in expert-id order: per lane acc = fma(s2 * w_row, partial,
+//        acc), the routing weight 0 for rows that did not pick the expert, so a row's bits do not depend on the other
+//        rows (decode.cu:526-566); the lanes are added once at the end. The fused shared expert's rows go to ys, and
+//        with ysum yr += ys (decode.cu:569-581).
+// Default: ONE persistent kernel runs both phases (k_decode): the grid is sized so that every workgroup is resident,
+// each wavefront issues the first loads of its down rows, then the grid meets at a barrier in device memory (h is
+// complete), then the down phase runs. This is what the reference gets from programmatic dependent launch
+// (decode.cu:170-172, 448-452): the second phase's weights are already in flight while the first one drains. With
+// DecodeCfg::logits the routing runs inside the kernel too (experts.h:123-127), so a layer is a single launch.
+// The two phases are also built as two kernels (k_up, k_down) for the bench's `parts` switch.
+// No atomics touch the results: they are deterministic and batch-invariant. The order of the f32 adds inside a dot
+// product differs from the reference's (not part of its contract).
+#pragma once
+#include <algorithm>
+
+#include "abi_internal.h"
+#include "rowdot.cuh"
+
+namespace dsgx {
+
+struct DecodeArgs {
+  const uint16_t* x;
+  int M;
+  const int* idx;
+  const float* w;
+  const float* logits;  // fused routing (DecodeCfg::logits): idx, w unused
+  const float* bias;
+  float route_scale;
+  int score_fn;
+  dsgx_layer_w L;
+  uint16_t* h;  // [slot][M][I]
+  float* yr;
+  float* ys;
+  int ysum;
+  int* bar;     // the grid barrier's words in the workspace: arrivals, generation, error flag
+  int spin_limit;
+};
+
+int launch_decode_fp8(const DecodeArgs& a, int parts, bool shared, hipStream_t st);
+int launch_decode_int4(const DecodeArgs& a, int parts, bool shared_bf16, hipStream_t st);
+int launch_decode_bf16(const DecodeArgs& a, int parts, hipStream_t st);
+
+// ---- what a workgroup knows about the step -------------------------------------------------------------------------
+struct MatRef {
+  const uint8_t* w;  // codes / weight_packed / bf16 rows
+  const uint8_t* s;  // scales (FP8 f32, INT4 bf16); INT4's zero points follow at a fixed offset
+  float s2;
+  int pad;
+};
+struct Slot {
+  MatRef g, u, d;
+  int hslot, shared;
+};
+template <int M>
+struct Step {
+  int n;                               // distinct picked experts
+  uint32_t mask[DSGX_MAX_EXPERTS / 32];
+  int ri[M * DSGX_MAX_TOPK];
+  float rw[M * DSGX_MAX_TOPK];
+  int id[M * DSGX_MAX_TOPK];
+  float wslot[M * DSGX_MAX_TOPK][M];   // per slot the rows' routing weights (0: the row did not pick it)
+  Slot slots[M * DSGX_MAX_TOPK + 1];
+  int gen;                             // the grid barrier's generation at kernel start
+};
+
+// The union of the rows' picks in expert-id order (build_union of the reference, decode.cu:57-106), by every
+// workgroup for itself; with logits the rows are routed here first (a wavefront a row, route()'s code and bits).
+template <int M>
+__device__ void build_union(Step<M>& S, const DecodeArgs& a) {
+  const int tid = threadIdx.x, E = a.L.E, topk = a.L.topk, ne = M * topk;
+  if (tid < DSGX_MAX_EXPERTS / 32) S.mask[tid] = 0;
+  for (int i = tid; i < M * DSGX_MAX_TOPK * M; i += blockDim.x) (&S.wslot[0][0])[i] = 0.f;
+  if (a.logits) {
+    for (int row = tid >> 6; row < M; row += blockDim.x >> 6) {
+      int id;
+      float w;
+      route_row(a.logits + (size_t)row * E, a.bias, E, topk, a.route_scale, a.score_fn, tid & 63, id, w);
+      if ((tid & 63) < topk) S.ri[row * topk + (tid & 63)] = id, S.rw[row * topk + (tid & 63)] = w;
+    }
+  } else {
+    for (int i = tid; i < ne; i += blockDim.x) S.ri[i] = a.idx[i], S.rw[i] = a.w[i];
+  }
+  __syncthreads();
+  for (int i = tid; i < ne; i += blockDim.x) atomicOr(&S.mask[S.ri[i] >> 5], 1u << (S.ri[i] & 31));
+  __syncthreads();
+  for (int i = tid; i < ne; i += blockDim.x) {
+    const int e = S.ri[i];
+    int r = __popc(S.mask[e >> 5] & ((1u << (e & 31)) - 1));
+    for (int j = 0; j < (e >> 5); ++j) r += __popc(S.mask[j]);
+    S.id[r] = e;
+    S.wslot[r][i / topk] = S.rw[i];
+  }
+  if (tid == 0) {
+    int n = 0;
+    for (int j = 0; j < DSGX_MAX_EXPERTS / 32; ++j) n += __popc(S.mask[j]);
+    S.n = n;
+  }
+  __syncthreads();
+}
+
+__device__ __forceinline__ size_t al256d(size_t b) { return (b + 255) / 256 * 256; }
+template <int FMT>
+__device__ __forceinline__ MatRef mat_ref(const uint8_t* base, int N, int K, float s2) {
+  MatRef m;
+  m.w = base, m.s = nullptr, m.s2 = s2, m.pad = 0;
+  if (FMT == DSGX_FMT_FP8_B128) m.s = base + al256d((size_t)N * K);
+  else if (FMT == DSGX_FMT_INT4_G32) m.s = base + al256d((size_t)N * K / 2);
+  return m;
+}
+template <int FMT>
+__device__ __forceinline__ MatDev mat_dev(const MatRef& r, int N, int K) {
+  MatDev m;
+  m.w = r.w, m.s = r.s, m.zp = nullptr, m.lrs = m.lks = 7, m.srow = K >> 7, m.s2 = r.s2;
+  if (FMT == DSGX_FMT_INT4_G32) m.zp = r.s + al256d((size_t)N * (K / 32) * 2);
+  return m;
+}
+// slots: a fused shared expert first (slot 0), then the union in expert-id order
+template <int FMT, int SHFMT, int M>
+__device__ void fill_slots(Step<M>& S, const DecodeArgs& a) {
+  const int H = a.L.H, I = a.L.I, nsh = SHFMT != 0 ? 1 : 0;
+  for (int s = threadIdx.x; s < nsh + S.n; s += blockDim.x) {
+    Slot t;
+    if (s < nsh) {
+      if (SHFMT == DSGX_FMT_BF16) {
+        t.g = MatRef{a.L.sh.bgu, nullptr, 1.f, 0};
+        t.u = t.g;
+        t.d = MatRef{a.L.sh.bd, nullptr, 1.f, 0};
+      } else {
+        t.g = MatRef{a.L.sh.g, reinterpret_cast<const uint8_t*>(a.L.sh.gs), 1.f, 0};
+        t.u = MatRef{a.L.sh.u, reinterpret_cast<const uint8_t*>(a.L.sh.us), 1.f, 0};
+        t.d = MatRef{a.L.sh.d, reinterpret_cast<const uint8_t*>(a.L.sh.ds), 1.f, 0};
+      }
+      t.hslot = DSGX_SH_SLOT, t.shared = 1;
+    } else {
+      const dsgx_mat_desc* d = a.L.desc + (size_t)S.id[s - nsh] * 3;
+      t.g = mat_ref<FMT>(a.L.pool + d[0].off, I, H, d[0].s2);
+      t.u = mat_ref<FMT>(a.L.pool + d[1].off, I, H, d[1].s2);
+      t.d = mat_ref<FMT>(a.L.pool + d[2].off, H, I, d[2].s2);
+      t.hslot = s - nsh, t.shared = 0;
+    }
+    S.slots[s] = t;
+  }
+  __syncthreads();
+}
+
+// ---- gate/up ------------------------------------------------------------------------------------------------------------
+// Walks slots [s0, s0 + nsl) in format F. INTER: the slot's gate matrix is the BF16 shared expert's interleaved gate/up
+// (rows 2c gate, 2c + 1 up). The wave is number gw of GW; batches go round-robin.
+template <int FMT, int M, bool INTER, int D>
+__device__ __forceinline__ void up_body(const DecodeArgs& a, const uint4* xs, const Slot* slots, int nsl, int gw, int GW) {
+  constexpr int RB = 4;
+  const int lane = threadIdx.x & 63, H = a.L.H, I = a.L.I;
+  const int nsegk = num_segs<FMT>(H), nq = nsegk * FmtT<FMT>::SEGK / 8;
+  const int nb_e = I / 2, nbatch = nsl * nb_e;
+  const int nmine = gw < nbatch ? (nbatch - gw + GW - 1) / GW : 0;
+  const int nsteps = nmine * nsegk;
+  Raw w[D][RB];
+  int lj = 0, lseg = 0;
+  auto load = [&](Raw (&r)[RB]) {
+    const int b = gw + lj * GW, sl = b / nb_e, p = b % nb_e;
+    const Slot& S = slots[sl];
+    const MatDev g = mat_dev<FMT>(S.g, INTER ? 2 * I : I, H), u = mat_dev<FMT>(S.u, I, H);
+#pragma unroll
+    for (int i = 0; i < RB; ++i) {
+      if (INTER) load_raw<FMT>(r[i], g, 4 * p + i, lseg, lane, H);
+      else load_raw<FMT>(r[i], i < 2 ? g : u, 2 * p + (i & 1), lseg, lane, H);
+    }
+    if (++lseg == nsegk) lseg = 0, ++lj;
+  };
+#pragma unroll
+  for (int d = 0; d < D; ++d)
+    if (d < nsteps) load(w[d]);
+  float acc[RB][M];
+  int cj = 0, cseg = 0;
+  for (int t0 = 0; t0 < nsteps; t0 += D) {
+#pragma unroll
+    for (int d = 0; d < D; ++d) {
+      const int t = t0 + d;
+      if (t >= nsteps) break;
+      if (cseg == 0) {
+#pragma unroll
+        for (int r = 0; r < RB; ++r)
+#pragma unroll
+          for (int m = 0; m < M; ++m) acc[r][m] = 0.f;
+      }
+      step_dot<FMT, M, RB>(w[d], xs, nq, cseg, lane, acc);
+      if (t + D < nsteps) load(w[d]);
+      if (++cseg < nsegk) continue;
+      cseg = 0;
+      const int b = gw + cj * GW, sl = b / nb_e, p = b % nb_e;
+      ++cj;
+      // lane i * M + m (i: the batch's channel 0 or 1) finishes channel 2p + i of activation row m
+      float gv = 0.f, uv = 0.f;
+#pragma unroll
+      for (int r = 0; r < RB; ++r)
+#pragma unroll
+        for (int m = 0; m < M; ++m) {
+          const float v = wave_sum(acc[r][m]);
+          const int ch = INTER ? r >> 1 : r & 1;
+          const bool up = INTER ? (r & 1) : (r >> 1);
+          if (lane == ch * M + m) {
+            if (up) uv = v;
+            else gv = v;
+          }
+        }
+      if (lane < 2 * M) {
+        const Slot& S = slots[sl];
+        const int i = lane / M, m = lane % M;
+        const float gt = bf16_round(__fmul_rn(gv, S.g.s2)), ut = bf16_round(__fmul_rn(uv, S.u.s2));
+        a.h[((size_t)S.hslot * M + m) * I + 2 * p + i] = (uint16_t)swiglu_bits(gt, ut);
+      }
+    }
+  }
+}
+
+// x staged for format F, then the up phase of this workgroup. With a shared expert of another format (INT4 experts,
+// BF16 shared expert) the first `shared_wgs` workgroups do the shared expert's gate/up and the others the routed slots.
+template <int FMT, int SHFMT, int M>
+__device__ __forceinline__ void up_phase(const DecodeArgs& a, uint4* xs, Step<M>& S, int shared_wgs) {
+  constexpr bool kMixed = SHFMT != 0 && SHFMT != FMT;
+  const int H = a.L.H, wpb = blockDim.x >> 6, wave = threadIdx.x >> 6;
+  const int nsh = SHFMT != 0 ? 1 : 0;
+  if (kMixed) {
+    if ((int)blockIdx.x < shared_wgs) {
+      stage_x<FmtT<DSGX_FMT_BF16>::KL>(xs, a.x, H, M, H, num_segs<DSGX_FMT_BF16>(H) * 512);
+      __syncthreads();
+      up_body<kMixed ? DSGX_FMT_BF16 : FMT, M, kMixed, 4>(a, xs, S.slots, 1, blockIdx.x * wpb + wave, shared_wgs * wpb);
+    } else {
+      stage_x<FmtT<FMT>::KL>(xs, a.x, H, M, H, num_segs<FMT>(H) * FmtT<FMT>::SEGK);
+      __syncthreads();
+      up_body<FMT, M, false, 4>(a, xs, S.slots + nsh, S.n, ((int)blockIdx.x - shared_wgs) * wpb + wave, ((int)gridDim.x - shared_wgs) * wpb);
+    }
+  } else {
+    stage_x<FmtT<FMT>::KL>(xs, a.x, H, M, H, num_segs<FMT>(H) * FmtT<FMT>::SEGK);
+    __syncthreads();
+    up_body<FMT, M, false, 4>(a, xs, S.slots, nsh + S.n, blockIdx.x * wpb + wave, gridDim.x * wpb);
+  }
+}
+
+// ---- down ------------------------------------------------------------------------------------------------------------------
+// The wave's rows [n_lo, n_hi) in sub-batches of RB; per sub-batch every slot in order. hs: LDS for `spc` slots' h.
+// `between` runs after the first loads are issued and before any h is read (the fused kernel's grid barrier).
+template <int FMT, int SHFMT, int M, int D, class Between>
+__device__ __forceinline__ void down_phase(const DecodeArgs& a, uint4* hs, Step<M>& S, int spc, int n_lo, int n_hi, Between&& between) {
+  constexpr int RB = 2;
+  constexpr bool kMixed = SHFMT != 0 && SHFMT != FMT;
+  constexpr int SF = SHFMT == 0 ? FMT : SHFMT;  // the shared slot's format
+  const int H = a.L.H, I = a.L.I, lane = threadIdx.x & 63;
+  const int nsh = SHFMT != 0 ? 1 : 0, nsl = nsh + S.n;
+  const int nq = I / 8;
+  const int segs_r = num_segs<FMT>(I), segs_s = nsh ? num_segs<SF>(I) : 0;
+  const int nsub = n_hi > n_lo ? (n_hi - n_lo + RB - 1) / RB : 0;
+  const int steps_sub = segs_s + S.n * segs_r;
+  const int nsteps = nsub * steps_sub;
+  // every wave of the workgroup must make the same number of passes over the chunks (the barriers)
+  __shared__ int s_maxsub;
+  if (threadIdx.x == 0) s_maxsub = 0;
+  __syncthreads();
+  if (lane == 0) atomicMax(&s_maxsub, nsub);
+
+  Raw w[D][RB];
+  int lsub = 0, ls = 0, lseg = 0;
+  auto load = [&](Raw (&r)[RB]) {
+    const Slot& T = S.slots[ls];
+    const bool sh = kMixed && ls < nsh;
+    const int n0 = n_lo + lsub * RB;
+#pragma unroll
+    for (int i = 0; i < RB; ++i) {
+      const int n = n0 + i < n_hi ? n0 + i : n_hi - 1;  // a row past the end re-reads the last one (its result is dropped)
+      if (sh) load_raw<SF>(r[i], mat_dev<SF>(T.d, H, I), n, lseg, lane, I);
+      else load_raw<FMT>(r[i], mat_dev<FMT>(T.d, H, I), n, lseg, lane, I);
+    }
+    if (++lseg == (ls < nsh ? segs_s : segs_r)) {
+      lseg = 0;
+      if (++ls == nsl) ls = 0, ++lsub;
+    }
+  };
+#pragma unroll
+  for (int d = 0; d < D; ++d)
+    if (d < nsteps) load(w[d]);
+
+  between();
+  __syncthreads();
+  const int maxsub = s_maxsub;
+  const bool one_chunk = nsl <= spc;
+
+  int t = 0;
+  for (int sub = 0; sub < maxsub; ++sub) {
+    const bool live = sub < nsub;
+    const int n0 = n_lo + sub * RB;
+    float yacc[RB][M], sacc[RB][M], acc[RB][M];
+#pragma unroll
+    for (int r = 0; r < RB; ++r)
+#pragma unroll
+      for (int m = 0; m < M; ++m) yacc[r][m] = sacc[r][m] = 0.f;
+    for (int c0 = 0; c0 < nsl; c0 += spc) {
+      const int c1 = min(nsl, c0 + spc);
+      if (!(one_chunk && sub > 0)) {
+        // stage the chunk's h rows, each slot in its format's lane order
+        __syncthreads();
+        for (int s = c0; s < c1; ++s) {
+          const uint16_t* hp = a.h + (size_t)S.slots[s].hslot * M * I;
+          uint4* dst = hs + (size_t)(s - c0) * M * nq;
+          if (kMixed && s < nsh) stage_x<FmtT<SF>::KL>(dst, hp, I, M, I, I);
+          else stage_x<FmtT<FMT>::KL>(dst, hp, I, M, I, I);
+        }
+        __syncthreads();
+      }
+      if (!live) continue;
+      for (int s = c0; s < c1; ++s) {
+        const bool sh = s < nsh;
+        const int nseg = sh ? segs_s : segs_r;
+        const uint4* xs = hs + (size_t)(s - c0) * M * nq;
+#pragma unroll
+        for (int r = 0; r < RB; ++r)
+#pragma unroll
+          for (int m = 0; m < M; ++m) acc[r][m] = 0.f;
+        for (int seg = 0; seg < nseg; ++seg, ++t) {
+          // the ring place of step t is t % D: dispatched so that the register index is a constant
+          bool done = false;
+#pragma unroll
+          for (int d = 0; d < D; ++d) {
+            if (done || (t % D) != d) continue;
+            if (kMixed && sh) step_dot<SF, M, RB>(w[d], xs, nq, seg, lane, acc);
+            else step_dot<FMT, M, RB>(w[d], xs, nq, seg, lane, acc);
+            if (t + D < nsteps) load(w[d]);
+            done = true;
+          }
+        }
+        const float s2 = S.slots[s].d.s2;
+#pragma unroll
+        for (int r = 0; r < RB; ++r)
+#pragma unroll
+          for (int m = 0; m < M; ++m) {
+            if (sh) sacc[r][m] = acc[r][m];
+            else yacc[r][m] = fmaf(__fmul_rn(s2, S.wslot[s - nsh][m]), acc[r][m], yacc[r][m]);
+          }
+      }
+    }
+    if (!live) continue;
+    // add the lanes; lane r * M + m keeps output (row n0 + r, activation row m)
+    float yv = 0.f, sv = 0.f;
+#pragma unroll
+    for (int r = 0; r < RB; ++r)
+#pragma unroll
+      for (int m = 0; m < M; ++m) {
+        const float v = wave_sum(yacc[r][m]);
+        if (lane == r * M + m) yv = v;
+        if (SHFMT != 0) {
+          const float s = wave_sum(sacc[r][m]);
+          if (lane == r * M + m) sv = s;
+        }
+      }
+    if (lane < RB * M) {
+      const int r = lane / M, m = lane % M;
+      if (n0 + r < n_hi) {
+        const size_t o = (size_t)m * H + n0 + r;
+        if (SHFMT != 0) a.ys[o] = sv;
+        else if (a.ysum) sv = a.ys[o];
+        if (a.ysum) yv = __fadd_rn(yv, sv);
+        a.yr[o] = yv;
+      }
+    }
+  }
+}
+
+// ---- the grid barrier ---------------------------------------------------------------------------------------------------------
+// bar[0] arrivals, bar[1] generation, bar[2] error flag; all zero before the first launch, and left with arrivals 0.
+// Every workgroup of the grid must be resident (the launch sizes the grid from the occupancy query). The wait is
+// bounded: past spin_limit polls the workgroup raises the error flag and goes on (wrong results, never a hang).
+__device__ __forceinline__ void grid_barrier(int* bar, int my_gen, int spin_limit) {
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+    const int old = __hip_atomic_fetch_add(&bar[0], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (old == (int)gridDim.x - 1) {
+      __hip_atomic_store(&bar[0], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_fetch_add(&bar[1], 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+    } else {
+      int spins = 0;
+      while (__hip_atomic_load(&bar[1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == my_gen) {
+        __builtin_amdgcn_s_sleep(1);
+        if (++spins > spin_limit) {
+          __hip_atomic_store(&bar[2], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          break;
+        }
+      }
+    }
+  }
+  __syncthreads();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+}
+
+// ---- kernels ----------------------------------------------------------------------------------------------------------------
+template <int FMT, int SHFMT, int M>
+__global__ void __launch_bounds__(256) k_decode(DecodeArgs a, int shared_wgs, int spc) {
+  extern __shared__ uint4 lds[];
+  __shared__ Step<M> S;
+  if (threadIdx.x == 0) S.gen = __hip_atomic_load(&a.bar[1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  build_union(S, a);
+  fill_slots<FMT, SHFMT, M>(S, a);
+  up_phase<FMT, SHFMT, M>(a, lds, S, shared_wgs);
+  const int H = a.L.H, GW = gridDim.x * (blockDim.x >> 6), gw = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  const int rpw = (H + GW - 1) / GW;
+  const int n_lo = min(H, gw * rpw), n_hi = min(H, n_lo + rpw);
+  down_phase<FMT, SHFMT, M, 4>(a, lds, S, spc, n_lo, n_hi, [&] { grid_barrier(a.bar, S.gen, a.spin_limit); });
+}
+template <int FMT, int SHFMT, int M>
+__global__ void __launch_bounds__(256) k_up(DecodeArgs a, int shared_wgs) {
+  extern __shared__ uint4 lds[];
+  __shared__ Step<M> S;
+  build_union(S, a);
+  fill_slots<FMT, SHFMT, M>(S, a);
+  up_phase<FMT, SHFMT, M>(a, lds, S, shared_wgs);
+}
+template <int FMT, int SHFMT, int M>
+__global__ void __launch_bounds__(256) k_down(DecodeArgs a, int spc) {
+  extern __shared__ uint4 lds[];
+  __shared__ Step<M> S;
+  build_union(S, a);
+  fill_slots<FMT, SHFMT, M>(S, a);
+  const int H = a.L.H, gw = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  const int n_lo = min(H, gw * 2), n_hi = min(H, n_lo + 2);
+  down_phase<FMT, SHFMT, M, 4>(a, lds, S, spc, n_lo, n_hi, [] {});
+}
+
+// ---- launches ---------------------------------------------------------------------------------------------------------------
+template <int FMT, int SHFMT, int M>
+int launch_decode(const DecodeArgs& a, int parts, hipStream_t st) {
+  const int H = a.L.H, I = a.L.I, cus = num_cus_cached();
+  constexpr bool kMixed = SHFMT != 0 && SHFMT != FMT;
+  constexpr int SF = SHFMT == 0 ? FMT : SHFMT;
+  const int nsl_max = std::min(a.M * a.L.topk, a.L.E) + (SHFMT != 0 ? 1 : 0);
+  // x in LDS for the up phase
+  const int segk = FmtT<FMT>::SEGK;
+  size_t lds_up = (size_t)M * ((H + segk - 1) / segk * segk) * 2;
+  if (kMixed) lds_up = std::max(lds_up, (size_t)M * ((H + 511) / 512 * 512) * 2);
+  // h of a chunk of slots in LDS for the down phase: all of them when they fit in 64 KiB
+  const size_t slot_bytes = (size_t)M * I * 2;
+  int spc = std::max(1, (int)((64 * 1024) / slot_bytes));
+  spc = std::min(spc, nsl_max);
+  const size_t lds_down = (size_t)spc * slot_bytes;
+  auto shared_split = [&](int grid) {
+    if (!kMixed) return 0;
+    // the workgroups split between the BF16 shared expert and the routed experts by their bytes
+    const double bsh = 2.0 * I * H * 2, bro = (double)std::min(a.M * a.L.topk, a.L.E) * 2.0 * (double)dsgx_mat_bytes(FMT, I, H);
+    return std::max(1, std::min(grid - 1, (int)(grid * bsh / (bsh + bro) + 0.5)));
+  };
+  (void)SF;
+  if (parts == 3) {
+    auto kern = k_decode<FMT, SHFMT, M>;
+    const size_t lds = std::max(lds_up, lds_down);
+    if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds)) return rc;
+    // every workgroup must be resident: the grid comes from the occupancy of this kernel with this much LDS
+    int per_cu = 0;
+    DSGX_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kern, 256, lds));
+    if (per_cu >= 1) {
+      per_cu = std::min(per_cu, 2);
+      const int grid = cus * per_cu;
+      hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, st, a, shared_split(grid), spc);
+      DSGX_HIP(hipGetLastError());
+      return DSGX_OK;
+    }
+    // (no resident grid possible: fall through to the two kernels)
+  }
+  if (parts & 1) {
+    auto kern = k_up<FMT, SHFMT, M>;
+    if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds_up)) return rc;
+    const int grid = cus * (lds_up <= 56 * 1024 ? 2 : 1);
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds_up, st, a, shared_split(grid));
+    DSGX_HIP(hipGetLastError());
+  }
+  if (parts & 2) {
+    auto kern = k_down<FMT, SHFMT, M>;
+    if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds_down)) return rc;
+    const int waves = (H + 1) / 2, grid = (waves + 3) / 4;
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds_down, st, a, spc);
+    DSGX_HIP(hipGetLastError());
+  }
+  return DSGX_OK;
+}
+
+template <int FMT, int SHFMT>
+int launch_decode_m(const DecodeArgs& a, int parts, hipStream_t st) {
+  switch (a.M) {
+    case 1: return launch_decode<FMT, SHFMT, 1>(a, parts, st);
+    case 2: return launch_decode<FMT, SHFMT, 2>(a, parts, st);
+    case 3: return launch_decode<FMT, SHFMT, 3>(a, parts, st);
+    case 4: return launch_decode<FMT, SHFMT, 4>(a, parts, st);
+    case 5: return launch_decode<FMT, SHFMT, 5>(a, parts, st);
+    case 6: return launch_decode<FMT, SHFMT, 6>(a, parts, st);
+    case 7: return launch_decode<FMT, SHFMT, 7>(a, parts, st);
+    case 8: return launch_decode<FMT, SHFMT, 8>(a, parts, st);
+  }
+  return fail(DSGX_EUNSUPPORTED, "moe_decode: %d rows (1..8 are built; the reference takes up to 16)", a.M);
+}
+
+}  // namespace dsgx

@@ -25,6 +25,7 @@ def lib():
     """The loaded C ABI. Raises if the HIP extension has not been built (python -m dsgx10_amd.build)."""
     global _lib
     if _lib is None:
+        import torch  # noqa: F401  first: the library must bind to the HIP runtime torch's streams and buffers belong to
         if not os.path.exists(_SO):
             raise RuntimeError("dsgx10_amd: %s is missing; build it with `python -m dsgx10_amd.build` (there is no CPU fallback)" % _SO)
         L = C.CDLL(_SO)
@@ -33,8 +34,9 @@ def lib():
         for f in ("dsgx_mat_bytes", "dsgx_mat_scale_off", "dsgx_mat_zp_off"):
             getattr(L, f).restype = C.c_size_t
             getattr(L, f).argtypes = [C.c_uint32, C.c_int, C.c_int]
-        L.dsgx_decode_ws_bytes.restype = C.c_size_t
-        L.dsgx_decode_ws_bytes.argtypes = [C.POINTER(abi.LayerW)]
+        for f in ("dsgx_decode_ws_bytes", "dsgx_decode_ws_flag_offset"):
+            getattr(L, f).restype = C.c_size_t
+            getattr(L, f).argtypes = [C.POINTER(abi.LayerW)]
         L.dsgx_route.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_float, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]
         L.dsgx_moe_decode.argtypes = [C.POINTER(abi.LayerW), C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p,
                                       C.c_void_p, C.c_void_p, C.c_void_p, C.POINTER(abi.DecodeCfg)]
@@ -82,6 +84,10 @@ def route(logits, bias, idx, w, route_scale=2.5, score_fn=0, stream=None):
 # ---- gx::moe_decode ---------------------------------------------------------------------------------------------------
 def decode_ws_bytes(layer_w):
     return lib().dsgx_decode_ws_bytes(C.byref(layer_w))
+
+
+def decode_ws_flag_offset(layer_w):
+    return lib().dsgx_decode_ws_flag_offset(C.byref(layer_w))
 
 
 def moe_decode(layer_w, x, idx, w, M, ws, yr, ys, stream=None, parts=3, ysum=False, logits=None, bias=None,

@@ -102,7 +102,7 @@ DSGX_API int dsgx_route(const float* logits, const float* bias, int M, int E, in
 
 /* ---- decode: gx::moe_decode (engine/experts/experts.h:104-147, decode.cu:708-730) ------------------------------- */
 typedef struct dsgx_decode_cfg {
-  int32_t up, down;        /* kernel variants (0 = default) */
+  int32_t up, down;        /* kernel variants: up 0 only; down 0 = both phases in one persistent kernel, 1 = two launches */
   int32_t parts;           /* 1 up only, 2 down only, 3 both (bench) */
   int32_t ysum;            /* 1: yr += ys in f32 after the routed experts (experts.h:132-136) */
   const float* logits;     /* fused routing (experts.h:123-127): with logits (+ optional bias) idx, w are not read */
@@ -115,6 +115,11 @@ DSGX_API void dsgx_decode_cfg_default(dsgx_decode_cfg* cfg);
 /* Workspace bytes of a decode step (gx::decode_ws_bytes; engine/experts/decode.cu:33-35): h bf16
    [DSGX_MAX_UNION + 1 slots][DSGX_MAX_ROWS][I] plus 256 bytes of counters. Zero it once before the first call. */
 DSGX_API size_t dsgx_decode_ws_bytes(const dsgx_layer_w* L);
+/* Byte offset in ws of a 32-bit error flag. The default decode step is one persistent kernel whose workgroups meet at a
+   barrier in device memory between the two phases; the wait is bounded, and a workgroup that gives up (it can only
+   happen when the grid is not resident, e.g. the GPU is shared with another process) sets this flag to 1 and the step's
+   outputs are invalid. No counterpart in the reference (its two kernels are ordered by the stream). */
+DSGX_API size_t dsgx_decode_ws_flag_offset(const dsgx_layer_w* L);
 /* x bf16 [M][H]; idx, w from dsgx_route; yr, ys f32 [M][H]. ys is written when the layer has a fused shared expert,
    otherwise it is an input (only read with ysum). h of the step stays in ws: slot s (the s-th picked expert in
    expert-id order) at ((s * M + m) * I + c), the shared expert's at slot DSGX_SH_SLOT. */

@@ -8,7 +8,7 @@ import pytest
 
 from dsgx10_amd import abi, lib
 from tests import gpu, orc
-from tests.helpers import check_sums, make_layer, rel_l2, rows_and_routing
+from tests.helpers import check_outputs, check_sums, make_layer, rel_l2, rows_and_routing
 
 pytestmark = pytest.mark.gpu
 
@@ -47,8 +47,7 @@ def _check_step(hl, dl, x, idx, w, M, scale_note=""):
     # end to end against the f32-accumulated oracle: bf16 outputs
     full = orc.moe_down(hl, up["h32"], idx[:M], w[:M], uni)
     for got, ref in ((yr, full["yr32"]),) + (((ys, full["ys32"]),) if hl.has_shared else ()):
-        g16, r16 = orc.bf16_to_f32(orc.f32_to_bf16(got)), orc.bf16_to_f32(orc.f32_to_bf16(ref))
-        assert np.abs(g16 - r16).max() <= 2e-2 and rel_l2(g16, r16) <= 1e-3
+        check_outputs(got, ref)
     return yr, ys, hg
 
 
@@ -109,6 +108,24 @@ def test_decode_fused_routing_and_ysum():
     b_yr, _, _ = gpu.decode_layer(dl2, x2, i2, w2, 2)
     yr, ys, _ = gpu.decode_layer(dl2, x2, i2, w2, 2, ysum=True, ys_in=ysin)
     assert np.array_equal(yr, b_yr + ysin) and np.array_equal(ys, ysin)
+
+
+def test_decode_two_launch_variant_equals_default_and_flag_clear():
+    """down variant 1 (gate/up and down as two launches) gives the default's bits (one persistent kernel with a grid
+    barrier); the barrier's error flag in the workspace stays 0"""
+    for case in (CASES[0], CASES[2]):
+        fmt, H, I, E, topk, NS, shared, scale = case
+        hl, dl = _layer(fmt, H, I, E, topk, NS, shared)
+        x, logits, idx, w = rows_and_routing(51, 6, H, E, topk, scale)
+        for M in (1, 2, 6):
+            yr, ys, ws = gpu.decode_layer(dl, x[:M], idx[:M], w[:M], M)
+            yr2, ys2, _ = gpu.decode_layer(dl, x[:M], idx[:M], w[:M], M, down=1)
+            assert np.array_equal(yr.view(np.uint32), yr2.view(np.uint32)) and np.array_equal(ys.view(np.uint32), ys2.view(np.uint32))
+            off = lib.decode_ws_flag_offset(dl.w)
+            assert gpu.host(ws[off:off + 4], np.int32, (1,))[0] == 0
+            # the same workspace again: the barrier's counters reset themselves
+            yr3, ys3, _ = gpu.decode_layer(dl, x[:M], idx[:M], w[:M], M, ws=ws)
+            assert np.array_equal(yr.view(np.uint32), yr3.view(np.uint32))
 
 
 def test_decode_parts_and_duplicate_experts_across_rows():
