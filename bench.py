@@ -137,7 +137,7 @@ def main():
         "data": "synthetic (torch-seeded N(0,0.02) weights quantised on the GPU, N(0,1) bf16 rows and f32 logits)",
         "config": {"workload": gen.describe(1), "rows_M": 1, "steps_route_different_experts": True,
                    "bytes_per_layer": r["bytes_per_layer"], "layer_hbm_frac_of_8TBs": r["layer_hbm_frac"],
-                   "kernels_per_step": ["k_route", "k_up", "k_down"], "timed_as": "one HIP graph of all steps, one replay"},
+                   "kernels_per_step": ["k_decode (routing + gate/up + SwiGLU + down + weighted sum, one persistent launch)"], "timed_as": "one HIP graph of all steps, one replay"},
         "roofline": {"bound": "hbm", "kernel": "k_up (gate/up + SwiGLU)", "achieved": r["up_gbs"], "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": r["up_frac"], "traffic": None, "bytes_per_launch": r["up_bytes"],
                      "avg_launch_us": r["up_us"], "measured_stream_read_gbs": stream_gbs},

@@ -224,8 +224,14 @@ class DecodeBench:
         idx = self.idx.cpu().numpy()
         self.union_sizes = np.array([len(np.unique(idx[s])) for s in range(steps)])
 
-    def step(self, s, parts=3, route=True):
+    def step(self, s, parts=3, route=True, fused_routing=True):
+        """one layer: with fused_routing the router runs inside the expert kernel (the reference runner's default,
+        DecodeCfg::logits), else as its own launch before it"""
         g = self.gen
+        if fused_routing:
+            lib.moe_decode(self.layers[s % g.NSH], self.x, None, None, self.M, self.ws, self.yr, self.ys, parts=parts,
+                           logits=self.logits[s], route_scale=g.route_scale)
+            return
         if route:
             lib.route(self.logits[s], None, self.idx[s], self.w[s], g.route_scale)
         lib.moe_decode(self.layers[s % g.NSH], self.x, self.idx[s], self.w[s], self.M, self.ws, self.yr, self.ys, parts=parts)

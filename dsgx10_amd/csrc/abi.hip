@@ -45,17 +45,20 @@ int allow_dynamic_lds(const void* kern, size_t lds) {
 
 namespace {
 
+// U 16-byte loads in flight a lane; a block walks contiguous tiles of 256 * U * 16 bytes, blocks round-robin
+template <int U>
 __global__ void __launch_bounds__(256) k_stream_read(const uint4* __restrict__ p, size_t n16, uint32_t* sink) {
   uint32_t acc = 0;
-  const size_t stride = (size_t)gridDim.x * blockDim.x;
-  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-  for (; i + 3 * stride < n16; i += 4 * stride) {
-    const uint4 a = ldg_stream(p + i), b = ldg_stream(p + i + stride), c = ldg_stream(p + i + 2 * stride), d = ldg_stream(p + i + 3 * stride);
-    acc ^= a.x ^ a.y ^ a.z ^ a.w ^ b.x ^ b.y ^ b.z ^ b.w ^ c.x ^ c.y ^ c.z ^ c.w ^ d.x ^ d.y ^ d.z ^ d.w;
-  }
-  for (; i < n16; i += stride) {
-    const uint4 a = ldg_stream(p + i);
-    acc ^= a.x ^ a.y ^ a.z ^ a.w;
+  const size_t tile = (size_t)256 * U;
+  for (size_t t0 = (size_t)blockIdx.x * tile; t0 < n16; t0 += (size_t)gridDim.x * tile) {
+    u32x4_t v[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const size_t i = t0 + (size_t)u * 256 + threadIdx.x;
+      v[u] = i < n16 ? ldg_stream(p + i) : u32x4_t{0, 0, 0, 0};
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) acc ^= v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
   }
   if (acc == 0x9E3779B9u) *sink = acc;  // keeps the loads alive; practically never taken
 }
@@ -165,13 +168,24 @@ size_t dsgx_mat_bytes(uint32_t fmt, int N, int K) {
   return 0;
 }
 
-int dsgx_stream_read(const void* p, size_t n, void* sink, void* stream) {
+int dsgx_stream_read_cfg(const void* p, size_t n, void* sink, int wgs_per_cu, int unroll, void* stream) {
   if (!p || !sink || n % 16 || ((uintptr_t)p & 15)) return fail(DSGX_EINVAL, "stream_read: %zu bytes at %p (16-byte units)", n, p);
-  hipLaunchKernelGGL(k_stream_read, dim3(num_cus_cached() * 8), dim3(256), 0, static_cast<hipStream_t>(stream),
-                     static_cast<const uint4*>(p), n / 16, static_cast<uint32_t*>(sink));
+  if (wgs_per_cu < 1 || wgs_per_cu > 16) return fail(DSGX_EINVAL, "stream_read: %d workgroups a CU", wgs_per_cu);
+  const dim3 grid(num_cus_cached() * wgs_per_cu), block(256);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const uint4* q = static_cast<const uint4*>(p);
+  uint32_t* sk = static_cast<uint32_t*>(sink);
+  switch (unroll) {
+    case 2: hipLaunchKernelGGL(k_stream_read<2>, grid, block, 0, st, q, n / 16, sk); break;
+    case 4: hipLaunchKernelGGL(k_stream_read<4>, grid, block, 0, st, q, n / 16, sk); break;
+    case 8: hipLaunchKernelGGL(k_stream_read<8>, grid, block, 0, st, q, n / 16, sk); break;
+    case 16: hipLaunchKernelGGL(k_stream_read<16>, grid, block, 0, st, q, n / 16, sk); break;
+    default: return fail(DSGX_EINVAL, "stream_read: %d loads in flight (2, 4, 8 or 16)", unroll);
+  }
   DSGX_HIP(hipGetLastError());
   return DSGX_OK;
 }
+int dsgx_stream_read(const void* p, size_t n, void* sink, void* stream) { return dsgx_stream_read_cfg(p, n, sink, 8, 4, stream); }
 int dsgx_stream_copy(const void* src, void* dst, size_t n, void* stream) {
   if (!src || !dst || n % 16 || (((uintptr_t)src | (uintptr_t)dst) & 15)) return fail(DSGX_EINVAL, "stream_copy: %zu bytes (16-byte units)", n);
   hipLaunchKernelGGL(k_stream_copy, dim3(num_cus_cached() * 8), dim3(256), 0, static_cast<hipStream_t>(stream),

@@ -58,11 +58,30 @@ __device__ __forceinline__ uint32_t i4_value_bits(int u, int uz, uint32_t sbits)
 }
 
 // ---- streaming loads (weights are read once: non-temporal) ---------------------------------------------------------------
+// Pointers that come out of LDS tables (the slot descriptors) have lost their address space: the loads below cast
+// them back to the global address space, so that they are global_load (vmcnt only) and not flat_load instructions.
+#define DSGX_GLOBAL __attribute__((address_space(1)))
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
-__device__ __forceinline__ uint4 ldg_stream(const void* p) {
-  const u32x4_t v = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(p));
-  return make_uint4(v.x, v.y, v.z, v.w);
+__device__ __forceinline__ u32x4_t ldg_stream(const void* p) {
+  return __builtin_nontemporal_load((const DSGX_GLOBAL u32x4_t*)(uintptr_t)p);
 }
+// The software pipelines below keep D steps of loads in flight in a ring of registers: step t is computed, then the
+// load of step t + D is issued into the same registers. Two empty asm statements keep the compiler from undoing that:
+// pin_after() makes a load's address depend on a value the preceding compute produced, so the load is not hoisted
+// above the compute (which would need a second set of registers and copies that wait for the new data); keep_whole()
+// passes a loaded 16-byte value through as one register tuple, so the loop-carried value is not split into scalars
+// that no longer line up with the load's destination.
+__device__ __forceinline__ const uint8_t* pin_after(const uint8_t* p, float dep) {
+  uint64_t a = (uint64_t)p;
+  asm volatile("" : "+v"(a) : "v"(dep));
+  return (const uint8_t*)a;
+}
+__device__ __forceinline__ u32x4_t keep_whole(u32x4_t v) {
+  asm volatile("" : "+v"(v));
+  return v;
+}
+__device__ __forceinline__ uint32_t ldg_u32(const void* p) { return *(const DSGX_GLOBAL uint32_t*)(uintptr_t)p; }
+__device__ __forceinline__ uint32_t ldg_u16(const void* p) { return *(const DSGX_GLOBAL uint16_t*)(uintptr_t)p; }
 
 // ---- wave64 reductions, result valid in every lane -------------------------------------------------------------------------
 // Steps 1, 2, 4, 8 run inside a row of 16 lanes with DPP (quad permutes and mirrors); rows are joined with gfx950's
@@ -121,13 +140,23 @@ __device__ __forceinline__ int xchunk_index(int q) {  // q: the row's chunk numb
 }
 // Stage rows x[M][ldx] (bf16, global) into lds [M][K/8 chunks] in the layout above; K a multiple of 8. Chunks past K in
 // the last segment are zero-filled up to Kpad (a multiple of 64 * KL).
-template <int KL>
+// COHERENT: read with device-scope coherent loads (data written by other workgroups of the same kernel).
+template <int KL, bool COHERENT = false>
 __device__ __forceinline__ void stage_x(uint4* lds, const uint16_t* x, size_t ldx, int M, int K, int Kpad) {
   const int nq = Kpad / 8;
   for (int i = threadIdx.x; i < M * nq; i += blockDim.x) {
     const int m = i / nq, q = i % nq;
     uint4 v = make_uint4(0, 0, 0, 0);
-    if (8 * q < K) v = *reinterpret_cast<const uint4*>(x + (size_t)m * ldx + 8 * q);
+    if (8 * q < K) {
+      if (COHERENT) {
+        const uint64_t* p = reinterpret_cast<const uint64_t*>(x + (size_t)m * ldx + 8 * q);
+        const uint64_t a = __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const uint64_t b = __hip_atomic_load(p + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        v = make_uint4((uint32_t)a, (uint32_t)(a >> 32), (uint32_t)b, (uint32_t)(b >> 32));
+      } else {
+        v = *reinterpret_cast<const uint4*>(x + (size_t)m * ldx + 8 * q);
+      }
+    }
     lds[(size_t)m * nq + xchunk_index<KL>(q)] = v;
   }
 }

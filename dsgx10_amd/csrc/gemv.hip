@@ -43,65 +43,66 @@ __global__ void __launch_bounds__(256) k_gemv(GemvArgs a) {
       if (i < a.nsegs && row >= a.sg[i].row0) si = i;
   };
   Raw w[D][RB];
-  int lj = 0, lseg = 0;  // the load cursor: batch number of this wave, segment
+  float acc[RB][M];
+#pragma unroll
+  for (int r = 0; r < RB; ++r)
+#pragma unroll
+    for (int m = 0; m < M; ++m) acc[r][m] = 0.f;
+  const uint8_t* dummy = reinterpret_cast<const uint8_t*>(a.x);  // where the loads past the last step go
+  int lt = 0, lj = 0, lseg = 0;  // the load cursor: step, batch number of this wave, segment
   auto load = [&](Raw (&r)[RB]) {
-    const int row = (gw + lj * GW) * RB;
+    const bool ok = lt < nsteps;
+    ++lt;
+    const int row = ok ? (gw + lj * GW) * RB : 0;
     int si;
     locate(row, si);
 #pragma unroll
-    for (int i = 0; i < RB; ++i) load_raw<FMT>(r[i], a.sg[si].m, row - a.sg[si].row0 + i, lseg, lane, a.K);
-    if (++lseg == a.nsegk) lseg = 0, ++lj;
+    for (int i = 0; i < RB; ++i)
+      load_raw<FMT, true>(r[i], a.sg[si].m, row - a.sg[si].row0 + i, lseg, lane, a.K, acc[i][0], ok ? nullptr : dummy);
+    if (ok && ++lseg == a.nsegk) lseg = 0, ++lj;
   };
-#pragma unroll
-  for (int d = 0; d < D; ++d)
-    if (d < nsteps) load(w[d]);
-
-  float acc[RB][M];
   int cj = 0, cseg = 0;
-  for (int t0 = 0; t0 < nsteps; t0 += D) {
+  auto compute = [&](const Raw (&raw)[RB]) {
+    step_dot<FMT, M, RB, true>(raw, xs, a.nq, cseg, lane, acc, a.K);
+    if (++cseg < a.nsegk) return;
+    cseg = 0;
+    // the batch is complete: add the lanes' partials, lane r * M + m keeps output (row r, activation row m)
+    const int row = (gw + cj * GW) * RB;
+    ++cj;
+    float mine = 0.f, mine2 = 0.f;
+#pragma unroll
+    for (int i = 0; i < RB; ++i)
+#pragma unroll
+      for (int m = 0; m < M; ++m) {
+        const float v = wave_sum(acc[i][m]);
+        acc[i][m] = 0.f;
+        if (lane == i * M + m) mine = v;
+        if (lane == (i ^ 1) * M + m) mine2 = v;  // the pair's other row (SwiGLU)
+      }
+    if (lane >= RB * M) return;
+    int si;
+    locate(row, si);
+    const GemvSegDev& sg = a.sg[si];
+    const int r = lane / M, m = lane % M, n = row - sg.row0 + r;
+    if (a.out == DSGX_OUT_BF16) {
+      static_cast<uint16_t*>(sg.y)[(size_t)m * sg.ldy + n] = (uint16_t)f32_to_bf16_bits(mine);
+    } else if (a.out == DSGX_OUT_F32) {
+      static_cast<float*>(sg.y)[(size_t)m * sg.ldy + n] = mine;
+    } else if ((r & 1) == 0) {  // SwiGLU: row 2i gate, 2i + 1 up -> column i (gemv.cu:164-168)
+      static_cast<uint16_t*>(sg.y)[(size_t)m * sg.ldy + n / 2] = (uint16_t)swiglu_bits(bf16_round(mine), bf16_round(mine2));
+    }
+  };
+  if (nsteps == 0) return;
+#pragma unroll
+  for (int d = 0; d < D; ++d) load(w[d]);
+  for (int t = 0; t < nsteps; t += D) {
 #pragma unroll
     for (int d = 0; d < D; ++d) {
-      const int t = t0 + d;
-      if (t >= nsteps) break;
-      if (cseg == 0) {
-#pragma unroll
-        for (int r = 0; r < RB; ++r)
-#pragma unroll
-          for (int m = 0; m < M; ++m) acc[r][m] = 0.f;
-      }
-      step_dot<FMT, M, RB>(w[d], xs, a.nq, cseg, lane, acc);
-      if (t + D < nsteps) load(w[d]);
-      if (++cseg < a.nsegk) continue;
-      cseg = 0;
-      // the batch is complete: add the lanes' partials, lane r * M + m keeps output (row r, activation row m)
-      const int row = (gw + cj * GW) * RB;
-      ++cj;
-      float mine = 0.f, mine2 = 0.f;
-#pragma unroll
-      for (int r = 0; r < RB; ++r)
-#pragma unroll
-        for (int m = 0; m < M; ++m) {
-          const float v = wave_sum(acc[r][m]);
-          if (lane == r * M + m) mine = v;
-          if (lane == (r ^ 1) * M + m) mine2 = v;  // the pair's other row (SwiGLU)
-        }
-      if (lane >= RB * M) continue;
-      int si;
-      locate(row, si);
-      const GemvSegDev& sg = a.sg[si];
-      const int r = lane / M, m = lane % M, n = row - sg.row0 + r;
-      if (a.out == DSGX_OUT_BF16) {
-        static_cast<uint16_t*>(sg.y)[(size_t)m * sg.ldy + n] = (uint16_t)f32_to_bf16_bits(mine);
-      } else if (a.out == DSGX_OUT_F32) {
-        static_cast<float*>(sg.y)[(size_t)m * sg.ldy + n] = mine;
-      } else if ((r & 1) == 0) {  // SwiGLU: row 2i gate, 2i + 1 up -> column i (gemv.cu:164-168)
-        static_cast<uint16_t*>(sg.y)[(size_t)m * sg.ldy + n / 2] = (uint16_t)swiglu_bits(bf16_round(mine), bf16_round(mine2));
-      }
+      if (t + d < nsteps) compute(w[d]);
+      load(w[d]);
     }
   }
 }
-
-
 
 template <int FMT, int M, int RB>
 int launch_gemv(const GemvArgs& a, hipStream_t st) {

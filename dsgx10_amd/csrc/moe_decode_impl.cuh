@@ -162,61 +162,75 @@ __device__ __forceinline__ void up_body(const DecodeArgs& a, const uint4* xs, co
   const int nb_e = I / 2, nbatch = nsl * nb_e;
   const int nmine = gw < nbatch ? (nbatch - gw + GW - 1) / GW : 0;
   const int nsteps = nmine * nsegk;
+  // the batch cursors advance by GW batches: (slot, pair) += (GW / nb_e, GW % nb_e) with carry
+  const int dsl = GW / nb_e, dp = GW % nb_e;
+  int lsl = gw / nb_e, lp = gw % nb_e, lseg = 0;   // the load cursor
+  int csl = lsl, cp = lp, cseg = 0;                 // the compute cursor
   Raw w[D][RB];
-  int lj = 0, lseg = 0;
+  float acc[RB][M];
+#pragma unroll
+  for (int i = 0; i < RB; ++i)
+#pragma unroll
+    for (int m = 0; m < M; ++m) acc[i][m] = 0.f;
+  const uint8_t* dummy = reinterpret_cast<const uint8_t*>(a.x);  // where the loads past the last step go (cached)
+  int lt = 0;
   auto load = [&](Raw (&r)[RB]) {
-    const int b = gw + lj * GW, sl = b / nb_e, p = b % nb_e;
-    const Slot& S = slots[sl];
+    const bool ok = lt < nsteps;
+    ++lt;
+    const Slot& S = slots[ok ? lsl : 0];
     const MatDev g = mat_dev<FMT>(S.g, INTER ? 2 * I : I, H), u = mat_dev<FMT>(S.u, I, H);
 #pragma unroll
     for (int i = 0; i < RB; ++i) {
-      if (INTER) load_raw<FMT>(r[i], g, 4 * p + i, lseg, lane, H);
-      else load_raw<FMT>(r[i], i < 2 ? g : u, 2 * p + (i & 1), lseg, lane, H);
+      if (INTER) load_raw<FMT, false>(r[i], g, 4 * lp + i, lseg, lane, H, acc[i][0], ok ? nullptr : dummy);
+      else load_raw<FMT, false>(r[i], i < 2 ? g : u, 2 * lp + (i & 1), lseg, lane, H, acc[i][0], ok ? nullptr : dummy);
     }
-    if (++lseg == nsegk) lseg = 0, ++lj;
+    if (ok && ++lseg == nsegk) {
+      lseg = 0, lsl += dsl, lp += dp;
+      if (lp >= nb_e) lp -= nb_e, ++lsl;
+      if (lsl >= nsl) lsl = 0, lp = 0;  // past the wave's last batch: any valid place (these loads go to `dummy`)
+    }
   };
+  auto compute = [&](const Raw (&r)[RB]) {
+    step_dot<FMT, M, RB>(r, xs, nq, cseg, lane, acc);
+    if (++cseg < nsegk) return;
+    cseg = 0;
+    // lane m < M finishes the batch's two channels of activation row m and stores them as one 32-bit word. The
+    // store is coherent at device scope (it bypasses the XCD-local L2): the down phase of the same kernel reads h on
+    // other XCDs right after the grid barrier.
+    float g0 = 0.f, g1 = 0.f, u0 = 0.f, u1 = 0.f;
 #pragma unroll
-  for (int d = 0; d < D; ++d)
-    if (d < nsteps) load(w[d]);
-  float acc[RB][M];
-  int cj = 0, cseg = 0;
-  for (int t0 = 0; t0 < nsteps; t0 += D) {
+    for (int i = 0; i < RB; ++i)
+#pragma unroll
+      for (int m = 0; m < M; ++m) {
+        const float v = wave_sum(acc[i][m]);
+        acc[i][m] = 0.f;
+        const int ch = INTER ? i >> 1 : i & 1;
+        const bool up = INTER ? (i & 1) : (i >> 1);
+        if (lane == m) {
+          if (up) (ch ? u1 : u0) = v;
+          else (ch ? g1 : g0) = v;
+        }
+      }
+    if (lane < M) {
+      const Slot& S = slots[csl];
+      const float sg = S.g.s2, su = S.u.s2;
+      const uint32_t h0 = swiglu_bits(bf16_round(__fmul_rn(g0, sg)), bf16_round(__fmul_rn(u0, su)));
+      const uint32_t h1 = swiglu_bits(bf16_round(__fmul_rn(g1, sg)), bf16_round(__fmul_rn(u1, su)));
+      uint32_t* dst = reinterpret_cast<uint32_t*>(a.h + ((size_t)S.hslot * M + lane) * I + 2 * cp);
+      __hip_atomic_store((DSGX_GLOBAL uint32_t*)(uintptr_t)dst, h0 | (h1 << 16), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    csl += dsl, cp += dp;
+    if (cp >= nb_e) cp -= nb_e, ++csl;
+  };
+  // software pipeline: D steps in flight; every iteration computes a step (while there is one) and issues a load
+  if (nsteps == 0) return;
+#pragma unroll
+  for (int d = 0; d < D; ++d) load(w[d]);
+  for (int t = 0; t < nsteps; t += D) {
 #pragma unroll
     for (int d = 0; d < D; ++d) {
-      const int t = t0 + d;
-      if (t >= nsteps) break;
-      if (cseg == 0) {
-#pragma unroll
-        for (int r = 0; r < RB; ++r)
-#pragma unroll
-          for (int m = 0; m < M; ++m) acc[r][m] = 0.f;
-      }
-      step_dot<FMT, M, RB>(w[d], xs, nq, cseg, lane, acc);
-      if (t + D < nsteps) load(w[d]);
-      if (++cseg < nsegk) continue;
-      cseg = 0;
-      const int b = gw + cj * GW, sl = b / nb_e, p = b % nb_e;
-      ++cj;
-      // lane i * M + m (i: the batch's channel 0 or 1) finishes channel 2p + i of activation row m
-      float gv = 0.f, uv = 0.f;
-#pragma unroll
-      for (int r = 0; r < RB; ++r)
-#pragma unroll
-        for (int m = 0; m < M; ++m) {
-          const float v = wave_sum(acc[r][m]);
-          const int ch = INTER ? r >> 1 : r & 1;
-          const bool up = INTER ? (r & 1) : (r >> 1);
-          if (lane == ch * M + m) {
-            if (up) uv = v;
-            else gv = v;
-          }
-        }
-      if (lane < 2 * M) {
-        const Slot& S = slots[sl];
-        const int i = lane / M, m = lane % M;
-        const float gt = bf16_round(__fmul_rn(gv, S.g.s2)), ut = bf16_round(__fmul_rn(uv, S.u.s2));
-        a.h[((size_t)S.hslot * M + m) * I + 2 * p + i] = (uint16_t)swiglu_bits(gt, ut);
-      }
+      if (t + d < nsteps) compute(w[d]);
+      load(w[d]);
     }
   }
 }
@@ -259,115 +273,115 @@ __device__ __forceinline__ void down_phase(const DecodeArgs& a, uint4* hs, Step<
   const int segs_r = num_segs<FMT>(I), segs_s = nsh ? num_segs<SF>(I) : 0;
   const int nsub = n_hi > n_lo ? (n_hi - n_lo + RB - 1) / RB : 0;
   const int steps_sub = segs_s + S.n * segs_r;
-  const int nsteps = nsub * steps_sub;
-  // every wave of the workgroup must make the same number of passes over the chunks (the barriers)
+  const int nsteps = nsub * steps_sub;  // this wave's steps with real loads
+  // every wave of the workgroup walks the same number of steps (the barriers around the h chunks)
   __shared__ int s_maxsub;
   if (threadIdx.x == 0) s_maxsub = 0;
   __syncthreads();
   if (lane == 0) atomicMax(&s_maxsub, nsub);
 
   Raw w[D][RB];
-  int lsub = 0, ls = 0, lseg = 0;
+  float yacc[RB][M], sacc[RB][M], acc[RB][M];
+#pragma unroll
+  for (int r = 0; r < RB; ++r)
+#pragma unroll
+    for (int m = 0; m < M; ++m) yacc[r][m] = sacc[r][m] = acc[r][m] = 0.f;
+  const uint8_t* dummy = reinterpret_cast<const uint8_t*>(a.x);
+  int lt = 0, lsub = 0, ls = 0, lseg = 0;  // the load cursor
   auto load = [&](Raw (&r)[RB]) {
-    const Slot& T = S.slots[ls];
+    const bool ok = lt < nsteps;
+    ++lt;
+    const Slot& T = S.slots[ok ? ls : 0];
     const bool sh = kMixed && ls < nsh;
     const int n0 = n_lo + lsub * RB;
 #pragma unroll
     for (int i = 0; i < RB; ++i) {
-      const int n = n0 + i < n_hi ? n0 + i : n_hi - 1;  // a row past the end re-reads the last one (its result is dropped)
-      if (sh) load_raw<SF>(r[i], mat_dev<SF>(T.d, H, I), n, lseg, lane, I);
-      else load_raw<FMT>(r[i], mat_dev<FMT>(T.d, H, I), n, lseg, lane, I);
+      const int n = ok ? (n0 + i < n_hi ? n0 + i : n_hi - 1) : 0;  // a row past the end re-reads the last one (its result is dropped)
+      if (sh) load_raw<SF, false>(r[i], mat_dev<SF>(T.d, H, I), n, lseg, lane, I, acc[i][0], ok ? nullptr : dummy);
+      else load_raw<FMT, false>(r[i], mat_dev<FMT>(T.d, H, I), n, lseg, lane, I, acc[i][0], ok ? nullptr : dummy);
     }
-    if (++lseg == (ls < nsh ? segs_s : segs_r)) {
+    if (ok && ++lseg == (ls < nsh ? segs_s : segs_r)) {
       lseg = 0;
       if (++ls == nsl) ls = 0, ++lsub;
     }
   };
 #pragma unroll
-  for (int d = 0; d < D; ++d)
-    if (d < nsteps) load(w[d]);
+  for (int d = 0; d < D; ++d) load(w[d]);
 
   between();
   __syncthreads();
   const int maxsub = s_maxsub;
   const bool one_chunk = nsl <= spc;
+  const int wg_steps = maxsub * steps_sub;
 
-  int t = 0;
-  for (int sub = 0; sub < maxsub; ++sub) {
-    const bool live = sub < nsub;
-    const int n0 = n_lo + sub * RB;
-    float yacc[RB][M], sacc[RB][M], acc[RB][M];
-#pragma unroll
-    for (int r = 0; r < RB; ++r)
-#pragma unroll
-      for (int m = 0; m < M; ++m) yacc[r][m] = sacc[r][m] = 0.f;
-    for (int c0 = 0; c0 < nsl; c0 += spc) {
+  int csub = 0, cs = 0, cseg = 0;  // the compute cursor
+  auto compute = [&](const Raw (&r)[RB]) {
+    const bool live = csub < nsub;
+    const bool sh = cs < nsh;
+    const int c0 = cs / spc * spc;
+    if (cseg == 0 && cs == c0 && !(one_chunk && csub > 0)) {
+      // entering a chunk of slots: stage their h rows, each slot in its format's lane order
       const int c1 = min(nsl, c0 + spc);
-      if (!(one_chunk && sub > 0)) {
-        // stage the chunk's h rows, each slot in its format's lane order
-        __syncthreads();
-        for (int s = c0; s < c1; ++s) {
-          const uint16_t* hp = a.h + (size_t)S.slots[s].hslot * M * I;
-          uint4* dst = hs + (size_t)(s - c0) * M * nq;
-          if (kMixed && s < nsh) stage_x<FmtT<SF>::KL>(dst, hp, I, M, I, I);
-          else stage_x<FmtT<FMT>::KL>(dst, hp, I, M, I, I);
-        }
-        __syncthreads();
-      }
-      if (!live) continue;
+      __syncthreads();
       for (int s = c0; s < c1; ++s) {
-        const bool sh = s < nsh;
-        const int nseg = sh ? segs_s : segs_r;
-        const uint4* xs = hs + (size_t)(s - c0) * M * nq;
-#pragma unroll
-        for (int r = 0; r < RB; ++r)
-#pragma unroll
-          for (int m = 0; m < M; ++m) acc[r][m] = 0.f;
-        for (int seg = 0; seg < nseg; ++seg, ++t) {
-          // the ring place of step t is t % D: dispatched so that the register index is a constant
-          bool done = false;
-#pragma unroll
-          for (int d = 0; d < D; ++d) {
-            if (done || (t % D) != d) continue;
-            if (kMixed && sh) step_dot<SF, M, RB>(w[d], xs, nq, seg, lane, acc);
-            else step_dot<FMT, M, RB>(w[d], xs, nq, seg, lane, acc);
-            if (t + D < nsteps) load(w[d]);
-            done = true;
-          }
-        }
-        const float s2 = S.slots[s].d.s2;
-#pragma unroll
-        for (int r = 0; r < RB; ++r)
-#pragma unroll
-          for (int m = 0; m < M; ++m) {
-            if (sh) sacc[r][m] = acc[r][m];
-            else yacc[r][m] = fmaf(__fmul_rn(s2, S.wslot[s - nsh][m]), acc[r][m], yacc[r][m]);
-          }
+        const uint16_t* hp = a.h + (size_t)S.slots[s].hslot * M * I;
+        uint4* dst = hs + (size_t)(s - c0) * M * nq;
+        if (kMixed && s < nsh) stage_x<FmtT<SF>::KL, true>(dst, hp, I, M, I, I);
+        else stage_x<FmtT<FMT>::KL, true>(dst, hp, I, M, I, I);
       }
+      __syncthreads();
     }
-    if (!live) continue;
-    // add the lanes; lane r * M + m keeps output (row n0 + r, activation row m)
-    float yv = 0.f, sv = 0.f;
+    const uint4* xs = hs + (size_t)(cs - c0) * M * nq;
+    if (live) {
+      if (kMixed && sh) step_dot<SF, M, RB>(r, xs, nq, cseg, lane, acc);
+      else step_dot<FMT, M, RB>(r, xs, nq, cseg, lane, acc);
+    }
+    if (++cseg < (sh ? segs_s : segs_r)) return;
+    cseg = 0;
+    // the slot is complete: into the rows' running sums, in slot (= expert id) order
+    const float s2 = S.slots[cs].d.s2;
 #pragma unroll
-    for (int r = 0; r < RB; ++r)
+    for (int i = 0; i < RB; ++i)
 #pragma unroll
       for (int m = 0; m < M; ++m) {
-        const float v = wave_sum(yacc[r][m]);
-        if (lane == r * M + m) yv = v;
-        if (SHFMT != 0) {
-          const float s = wave_sum(sacc[r][m]);
-          if (lane == r * M + m) sv = s;
-        }
+        if (sh) sacc[i][m] = acc[i][m];
+        else yacc[i][m] = fmaf(__fmul_rn(s2, S.wslot[cs - nsh][m]), acc[i][m], yacc[i][m]);
+        acc[i][m] = 0.f;
       }
-    if (lane < RB * M) {
-      const int r = lane / M, m = lane % M;
-      if (n0 + r < n_hi) {
-        const size_t o = (size_t)m * H + n0 + r;
+    if (++cs < nsl) return;
+    cs = 0;
+    // the sub-batch is complete: add the lanes; lane i * M + m keeps output (row n0 + i, activation row m)
+    const int n0 = n_lo + csub * RB;
+    ++csub;
+    float yv = 0.f, sv = 0.f;
+#pragma unroll
+    for (int i = 0; i < RB; ++i)
+#pragma unroll
+      for (int m = 0; m < M; ++m) {
+        const float v = wave_sum(yacc[i][m]);
+        if (lane == i * M + m) yv = v;
+        if (SHFMT != 0) {
+          const float s = wave_sum(sacc[i][m]);
+          if (lane == i * M + m) sv = s;
+        }
+        yacc[i][m] = sacc[i][m] = 0.f;
+      }
+    if (live && lane < RB * M) {
+      const int i = lane / M, m = lane % M;
+      if (n0 + i < n_hi) {
+        const size_t o = (size_t)m * H + n0 + i;
         if (SHFMT != 0) a.ys[o] = sv;
         else if (a.ysum) sv = a.ys[o];
         if (a.ysum) yv = __fadd_rn(yv, sv);
         a.yr[o] = yv;
       }
+    }
+  };
+  for (int t = 0; t < wg_steps; t += D) {
+#pragma unroll
+    for (int d = 0; d < D; ++d) {
+      if (t + d < wg_steps) compute(w[d]);
+      load(w[d]);
     }
   }
 }
@@ -377,17 +391,18 @@ __device__ __forceinline__ void down_phase(const DecodeArgs& a, uint4* hs, Step<
 // Every workgroup of the grid must be resident (the launch sizes the grid from the occupancy query). The wait is
 // bounded: past spin_limit polls the workgroup raises the error flag and goes on (wrong results, never a hang).
 __device__ __forceinline__ void grid_barrier(int* bar, int my_gen, int spin_limit) {
+  // h was stored with device-scope coherent stores; __syncthreads() waits for every wave's stores to complete, so no
+  // cache write-back or invalidate is needed around the counter (a device-scope fence would flush the whole L2 here)
   __syncthreads();
   if (threadIdx.x == 0) {
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
     const int old = __hip_atomic_fetch_add(&bar[0], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     if (old == (int)gridDim.x - 1) {
       __hip_atomic_store(&bar[0], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      __hip_atomic_fetch_add(&bar[1], 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_fetch_add(&bar[1], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     } else {
       int spins = 0;
       while (__hip_atomic_load(&bar[1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == my_gen) {
-        __builtin_amdgcn_s_sleep(1);
+        __builtin_amdgcn_s_sleep(4);
         if (++spins > spin_limit) {
           __hip_atomic_store(&bar[2], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
           break;
@@ -396,7 +411,6 @@ __device__ __forceinline__ void grid_barrier(int* bar, int my_gen, int spin_limi
     }
   }
   __syncthreads();
-  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
 }
 
 // ---- kernels ----------------------------------------------------------------------------------------------------------------

@@ -12,7 +12,7 @@
 namespace dsgx {
 
 struct Raw {
-  uint4 v;       // 16 bytes of the row
+  u32x4_t v;     // 16 bytes of the row
   uint32_t aux;  // FP8: the lane's block scale (f32 bits); INT4: bf16 scale bits | zero-point nibble << 16
 };
 
@@ -40,32 +40,47 @@ template <> struct FmtT<DSGX_FMT_BF16> {
   __device__ static __forceinline__ size_t row_bytes(int K) { return (size_t)K * 2; }
 };
 
-// the lane's 16 bytes of (row n, segment seg) and what it needs to decode them
-template <int FMT>
-__device__ __forceinline__ void load_raw(Raw& r, const MatDev& m, int n, int seg, int lane, int K) {
+// The lane's 16 bytes of (row n, segment seg) and what it needs to decode them. The loads are unconditional: a lane
+// past the end of K (TAIL: the dense GEMV's partial last segment) reads the row's first bytes instead and step_dot
+// drops them; with `dummy` set (the pipeline's loads past the wave's last step) every lane reads there instead.
+// `pin`: a value of the preceding compute, see pin_after().
+template <int FMT, bool TAIL>
+__device__ __forceinline__ void load_raw(Raw& r, const MatDev& m, int n, int seg, int lane, int K, float pin, const uint8_t* dummy) {
   using F = FmtT<FMT>;
-  const int k0 = seg * F::SEGK + lane * F::KL;
-  r.v = make_uint4(0, 0, 0, 0);
-  r.aux = 0;
-  if (k0 >= K) return;  // the partial last segment: zeros (INT4: scale +0, so every value decodes to 0)
-  r.v = ldg_stream(m.w + (size_t)n * F::row_bytes(K) + (size_t)seg * 1024 + lane * 16);
+  int k0 = seg * F::SEGK + lane * F::KL;
+  if (TAIL && k0 >= K) k0 = 0;
+  const uint8_t* wp = m.w + (size_t)n * F::row_bytes(K) + F::row_bytes(k0);
+  const uint8_t* ap = nullptr;
+  if constexpr (FMT == DSGX_FMT_FP8_B128) ap = m.s + ((size_t)(n >> m.lrs) * m.srow + (k0 >> m.lks)) * 4;
+  if (dummy) wp = dummy + lane * 16, ap = dummy;
+  r.v = ldg_stream(pin_after(wp, pin));
   if constexpr (FMT == DSGX_FMT_FP8_B128) {
-    r.aux = reinterpret_cast<const uint32_t*>(m.s)[(size_t)(n >> m.lrs) * m.srow + (k0 >> m.lks)];
+    r.aux = ldg_u32(ap);
   } else if constexpr (FMT == DSGX_FMT_INT4_G32) {
     const int g = k0 >> 5, G = K >> 5;
-    const uint32_t sb = reinterpret_cast<const uint16_t*>(m.s)[(size_t)n * G + g];
-    const uint32_t zw = reinterpret_cast<const uint32_t*>(m.zp)[(size_t)(n >> 3) * G + g];
-    r.aux = sb | (((zw >> (4 * (n & 7))) & 15u) << 16);
+    const uint8_t* sp = m.s + ((size_t)n * G + g) * 2;
+    const uint8_t* zp = m.zp + ((size_t)(n >> 3) * G + g) * 4;
+    if (dummy) sp = zp = dummy;
+    r.aux = ldg_u16(sp) | (((ldg_u32(zp) >> (4 * (n & 7))) & 15u) << 16);
+  } else {
+    r.aux = 0;
   }
 }
 
 // RB rows of one segment against M activation rows. xs: the workgroup's staged activations, row m at xs + m * nq
 // (nq chunks a row); acc[r][m] are the lanes' running sums.
-template <int FMT, int M, int RB>
-__device__ __forceinline__ void step_dot(const Raw (&raw)[RB], const uint4* __restrict__ xs, int nq, int seg, int lane,
-                                         float (&acc)[RB][M]) {
+template <int FMT, int M, int RB, bool TAIL = false>
+__device__ __forceinline__ void step_dot(const Raw (&raw_in)[RB], const uint4* __restrict__ xs, int nq, int seg, int lane,
+                                         float (&acc)[RB][M], int K = 0) {
   using F = FmtT<FMT>;
   const uint4* xl = xs + (size_t)seg * F::XC * 64 + lane;
+  Raw raw[RB];
+#pragma unroll
+  for (int r = 0; r < RB; ++r) {
+    raw[r].v = keep_whole(raw_in[r].v);
+    raw[r].aux = raw_in[r].aux;
+    if (TAIL && seg * F::SEGK + lane * F::KL >= K) raw[r].v = u32x4_t{0, 0, 0, 0}, raw[r].aux = 0;  // INT4: scale +0
+  }
   if constexpr (FMT == DSGX_FMT_FP8_B128) {
     // per (row, 128-k block): the unscaled sum from zero, then acc = fma(S, sum, acc); a lane's 16 k lie in one block
     float p[RB][M];

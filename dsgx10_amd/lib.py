@@ -47,6 +47,7 @@ def lib():
         L.dsgx_widen_fp8.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_size_t, C.c_void_p]
         L.dsgx_act_quant.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]
         L.dsgx_stream_read.argtypes = [C.c_void_p, C.c_size_t, C.c_void_p, C.c_void_p]
+        L.dsgx_stream_read_cfg.argtypes = [C.c_void_p, C.c_size_t, C.c_void_p, C.c_int, C.c_int, C.c_void_p]
         L.dsgx_stream_copy.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]
         if hasattr(L, "dsgx_moe_prefill"):
             L.dsgx_prefill_ws_bytes.restype = C.c_size_t
@@ -144,6 +145,10 @@ def act_quant(x, T, K, q, s, stream=None):
 
 def stream_read(buf, nbytes, sink, stream=None):
     _check(lib().dsgx_stream_read(_ptr(buf), nbytes, _ptr(sink), _stream(stream)))
+
+
+def stream_read_cfg(buf, nbytes, sink, wgs_per_cu, unroll, stream=None):
+    _check(lib().dsgx_stream_read_cfg(_ptr(buf), nbytes, _ptr(sink), wgs_per_cu, unroll, _stream(stream)))
 
 
 def stream_copy(src, dst, nbytes, stream=None):

@@ -188,6 +188,8 @@ DSGX_API const char* dsgx_version(void);
 /* A plain streaming-read kernel over n bytes (the bandwidth baseline the bench prints beside the kernels,
    as engine/experts/tests/bench_experts.cu:102-130 does); sink: 4 bytes of device memory. */
 DSGX_API int dsgx_stream_read(const void* p, size_t n, void* sink, void* stream);
+/* The same with the launch shape given: workgroups (of 256 threads) a CU and 16-byte loads in flight a lane (2, 4, 8, 16). */
+DSGX_API int dsgx_stream_read_cfg(const void* p, size_t n, void* sink, int wgs_per_cu, int unroll, void* stream);
 /* A plain copy kernel (the reference for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE counters). */
 DSGX_API int dsgx_stream_copy(const void* src, void* dst, size_t n, void* stream);
 
