@@ -30,11 +30,11 @@ def _stale(out, srcs):
     return any(os.path.getmtime(s) > t for s in srcs)
 
 
-def _compile(src, force):
-    obj = os.path.join(CSRC, os.path.splitext(src)[0] + ".o")
+def _compile(src, force, extra=(), suffix=""):
+    obj = os.path.join(CSRC, os.path.splitext(src)[0] + suffix + ".o")
     path = os.path.join(CSRC, src)
     if force or _stale(obj, [path] + _deps()):
-        cmd = ["hipcc"] + FLAGS + ["-c", path, "-o", obj]
+        cmd = ["hipcc"] + FLAGS + list(extra) + ["-c", path, "-o", obj]
         r = subprocess.run(cmd, capture_output=True, text=True)
         err = "\n".join(l for l in r.stderr.splitlines() if "packed-fp32-ops" not in l)
         if r.returncode:
@@ -44,20 +44,23 @@ def _compile(src, force):
     return obj
 
 
-def build(jobs=None, force=False):
+def build(jobs=None, force=False, extra=(), suffix=""):
+    """extra / suffix: a diagnostic variant (e.g. extra=["-DDSGX_TRACE"], suffix="_trace" -> libdsgx_trace.so)"""
     srcs = [s for s in SOURCES if os.path.exists(os.path.join(CSRC, s))]
     jobs = jobs or min(len(srcs), os.cpu_count() or 4)
+    so = SO.replace(".so", suffix + ".so")
     with cf.ThreadPoolExecutor(jobs) as ex:
-        objs = list(ex.map(lambda s: _compile(s, force), srcs))
-    if force or _stale(SO, objs):
-        cmd = ["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", "-o", SO] + objs
+        objs = list(ex.map(lambda s: _compile(s, force, extra, suffix), srcs))
+    if force or _stale(so, objs):
+        cmd = ["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", "-o", so] + objs
         subprocess.check_call(cmd)
-    return SO
+    return so
 
 
 if __name__ == "__main__":
     ap = argparse.ArgumentParser()
     ap.add_argument("-j", type=int, default=None)
     ap.add_argument("--force", action="store_true")
+    ap.add_argument("--trace", action="store_true", help="the diagnostic variant libdsgx_trace.so (phase time stamps)")
     a = ap.parse_args()
-    print(build(a.j, a.force))
+    print(build(a.j, a.force, ["-DDSGX_TRACE"], "_trace") if a.trace else build(a.j, a.force))

@@ -141,23 +141,65 @@ __device__ __forceinline__ int xchunk_index(int q) {  // q: the row's chunk numb
 // Stage rows x[M][ldx] (bf16, global) into lds [M][K/8 chunks] in the layout above; K a multiple of 8. Chunks past K in
 // the last segment are zero-filled up to Kpad (a multiple of 64 * KL).
 // COHERENT: read with device-scope coherent loads (data written by other workgroups of the same kernel).
+// Eight chunks a thread are loaded before any is written to LDS, so their latencies overlap.
+template <bool COHERENT>
+__device__ __forceinline__ uint4 load_chunk(const uint16_t* p) {
+  if (COHERENT) {
+    const uint64_t* q = reinterpret_cast<const uint64_t*>(p);
+    const uint64_t a = __hip_atomic_load((const DSGX_GLOBAL uint64_t*)(uintptr_t)q, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const uint64_t b = __hip_atomic_load((const DSGX_GLOBAL uint64_t*)(uintptr_t)(q + 1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return make_uint4((uint32_t)a, (uint32_t)(a >> 32), (uint32_t)b, (uint32_t)(b >> 32));
+  }
+  const u32x4_t v = *(const DSGX_GLOBAL u32x4_t*)(uintptr_t)p;
+  return make_uint4(v.x, v.y, v.z, v.w);
+}
 template <int KL, bool COHERENT = false>
 __device__ __forceinline__ void stage_x(uint4* lds, const uint16_t* x, size_t ldx, int M, int K, int Kpad) {
-  const int nq = Kpad / 8;
-  for (int i = threadIdx.x; i < M * nq; i += blockDim.x) {
-    const int m = i / nq, q = i % nq;
-    uint4 v = make_uint4(0, 0, 0, 0);
-    if (8 * q < K) {
-      if (COHERENT) {
-        const uint64_t* p = reinterpret_cast<const uint64_t*>(x + (size_t)m * ldx + 8 * q);
-        const uint64_t a = __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        const uint64_t b = __hip_atomic_load(p + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        v = make_uint4((uint32_t)a, (uint32_t)(a >> 32), (uint32_t)b, (uint32_t)(b >> 32));
-      } else {
-        v = *reinterpret_cast<const uint4*>(x + (size_t)m * ldx + 8 * q);
+  const int nq = Kpad / 8, total = M * nq;
+  constexpr int U = 8;
+  for (int i0 = threadIdx.x; i0 < total; i0 += U * blockDim.x) {
+    uint4 v[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int i = i0 + u * blockDim.x;
+      v[u] = make_uint4(0, 0, 0, 0);
+      if (i < total) {
+        const int m = i / nq, q = i % nq;
+        if (8 * q < K) v[u] = load_chunk<COHERENT>(x + (size_t)m * ldx + 8 * q);
       }
     }
-    lds[(size_t)m * nq + xchunk_index<KL>(q)] = v;
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int i = i0 + u * blockDim.x;
+      if (i < total) lds[(size_t)(i / nq) * nq + xchunk_index<KL>(i % nq)] = v[u];
+    }
+  }
+}
+// The same for `ns` consecutive slots of h (each M rows of K = ldx values) staged back to back: one pass over all of
+// them, so that a chunk of slots costs one round trip and not one a slot. base(s) gives slot s's rows.
+template <int KL, bool COHERENT, class Base>
+__device__ __forceinline__ void stage_slots(uint4* lds, int ns, int M, int K, Base&& base) {
+  const int nq = K / 8, per = M * nq, total = ns * per;
+  constexpr int U = 8;
+  for (int i0 = threadIdx.x; i0 < total; i0 += U * blockDim.x) {
+    uint4 v[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int i = i0 + u * blockDim.x;
+      v[u] = make_uint4(0, 0, 0, 0);
+      if (i < total) {
+        const int s = i / per, r = i % per;
+        v[u] = load_chunk<COHERENT>(base(s) + (size_t)(r / nq) * K + 8 * (r % nq));
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int i = i0 + u * blockDim.x;
+      if (i < total) {
+        const int s = i / per, r = i % per;
+        lds[(size_t)s * per + (size_t)(r / nq) * nq + xchunk_index<KL>(r % nq)] = v[u];
+      }
+    }
   }
 }
 

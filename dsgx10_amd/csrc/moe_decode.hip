@@ -5,6 +5,11 @@
 
 using namespace dsgx;
 
+#ifdef DSGX_TRACE
+static unsigned long long* g_trace_buf = nullptr;  // device memory, [workgroups][16]
+extern "C" __attribute__((visibility("default"))) void dsgx_trace_set(void* dev) { g_trace_buf = static_cast<unsigned long long*>(dev); }
+#endif
+
 extern "C" {
 
 void dsgx_decode_cfg_default(dsgx_decode_cfg* c) {
@@ -21,11 +26,11 @@ void dsgx_decode_cfg_default(dsgx_decode_cfg* c) {
 static size_t ws_h_bytes(const dsgx_layer_w* L) { return (size_t)(DSGX_MAX_UNION + 1) * DSGX_MAX_ROWS * L->I * 2; }
 size_t dsgx_decode_ws_bytes(const dsgx_layer_w* L) {
   if (!L || L->I <= 0) return 0;
-  return ws_h_bytes(L) + 256;
+  return ws_h_bytes(L) + kBarBytes;
 }
 size_t dsgx_decode_ws_flag_offset(const dsgx_layer_w* L) {
   if (!L || L->I <= 0) return 0;
-  return ws_h_bytes(L) + 8;
+  return ws_h_bytes(L) + (size_t)(2 * kBarGroups + 1) * kBarLine * 4;
 }
 
 int dsgx_moe_decode(const dsgx_layer_w* L, const uint16_t* x, const int* idx, const float* w, int M, void* ws, float* yr, float* ys,
@@ -66,6 +71,9 @@ int dsgx_moe_decode(const dsgx_layer_w* L, const uint16_t* x, const int* idx, co
   a.L = *L, a.h = static_cast<uint16_t*>(ws), a.yr = yr, a.ys = ys, a.ysum = c.ysum;
   a.bar = reinterpret_cast<int*>(static_cast<uint8_t*>(ws) + ws_h_bytes(L));
   a.spin_limit = 1 << 22;
+#ifdef DSGX_TRACE
+  a.trace = g_trace_buf;
+#endif
   hipStream_t st = static_cast<hipStream_t>(stream);
   const uint32_t f = L->fmt;
   if (f == DSGX_FMT_FP8_B128) {

@@ -26,6 +26,16 @@
 
 namespace dsgx {
 
+// Diagnostic build only (-DDSGX_TRACE): thread 0 of every workgroup stamps the 100 MHz wall clock at phase marks.
+#ifdef DSGX_TRACE
+#define DSGX_MARK(k)                                                                        \
+  do {                                                                                      \
+    if (a.trace && threadIdx.x == 0) a.trace[blockIdx.x * 16 + (k)] = wall_clock64();       \
+  } while (0)
+#else
+#define DSGX_MARK(k) do { } while (0)
+#endif
+
 struct DecodeArgs {
   const uint16_t* x;
   int M;
@@ -40,7 +50,10 @@ struct DecodeArgs {
   float* yr;
   float* ys;
   int ysum;
-  int* bar;     // the grid barrier's words in the workspace: arrivals, generation, error flag
+  int* bar;     // the grid barrier's words in the workspace (grid_barrier)
+#ifdef DSGX_TRACE
+  unsigned long long* trace;
+#endif
   int spin_limit;
 };
 
@@ -154,12 +167,14 @@ __device__ void fill_slots(Step<M>& S, const DecodeArgs& a) {
 // ---- gate/up ------------------------------------------------------------------------------------------------------------
 // Walks slots [s0, s0 + nsl) in format F. INTER: the slot's gate matrix is the BF16 shared expert's interleaved gate/up
 // (rows 2c gate, 2c + 1 up). The wave is number gw of GW; batches go round-robin.
-template <int FMT, int M, bool INTER, int D>
+// CH channels a batch (RB = 2 CH weight rows a step): one channel at few activation rows, where an even split of the
+// batches over the waves matters most (the benchmark's 9 slots x 2048 channels over 2048 waves: nine each).
+template <int FMT, int M, bool INTER, int CH, int D>
 __device__ __forceinline__ void up_body(const DecodeArgs& a, const uint4* xs, const Slot* slots, int nsl, int gw, int GW) {
-  constexpr int RB = 4;
+  constexpr int RB = 2 * CH;
   const int lane = threadIdx.x & 63, H = a.L.H, I = a.L.I;
   const int nsegk = num_segs<FMT>(H), nq = nsegk * FmtT<FMT>::SEGK / 8;
-  const int nb_e = I / 2, nbatch = nsl * nb_e;
+  const int nb_e = I / CH, nbatch = nsl * nb_e;
   const int nmine = gw < nbatch ? (nbatch - gw + GW - 1) / GW : 0;
   const int nsteps = nmine * nsegk;
   // the batch cursors advance by GW batches: (slot, pair) += (GW / nb_e, GW % nb_e) with carry
@@ -181,8 +196,8 @@ __device__ __forceinline__ void up_body(const DecodeArgs& a, const uint4* xs, co
     const MatDev g = mat_dev<FMT>(S.g, INTER ? 2 * I : I, H), u = mat_dev<FMT>(S.u, I, H);
 #pragma unroll
     for (int i = 0; i < RB; ++i) {
-      if (INTER) load_raw<FMT, false>(r[i], g, 4 * lp + i, lseg, lane, H, acc[i][0], ok ? nullptr : dummy);
-      else load_raw<FMT, false>(r[i], i < 2 ? g : u, 2 * lp + (i & 1), lseg, lane, H, acc[i][0], ok ? nullptr : dummy);
+      if (INTER) load_raw<FMT, false>(r[i], g, RB * lp + i, lseg, lane, H, acc[i][0], ok ? nullptr : dummy);
+      else load_raw<FMT, false>(r[i], i < CH ? g : u, CH * lp + i % CH, lseg, lane, H, acc[i][0], ok ? nullptr : dummy);
     }
     if (ok && ++lseg == nsegk) {
       lseg = 0, lsl += dsl, lp += dp;
@@ -194,30 +209,34 @@ __device__ __forceinline__ void up_body(const DecodeArgs& a, const uint4* xs, co
     step_dot<FMT, M, RB>(r, xs, nq, cseg, lane, acc);
     if (++cseg < nsegk) return;
     cseg = 0;
-    // lane m < M finishes the batch's two channels of activation row m and stores them as one 32-bit word. The
+    // lane m < M finishes the batch's channel(s) of activation row m and stores them as one 16- or 32-bit word. The
     // store is coherent at device scope (it bypasses the XCD-local L2): the down phase of the same kernel reads h on
     // other XCDs right after the grid barrier.
-    float g0 = 0.f, g1 = 0.f, u0 = 0.f, u1 = 0.f;
+    float gv[CH], uv[CH];
+#pragma unroll
+    for (int c = 0; c < CH; ++c) gv[c] = uv[c] = 0.f;
 #pragma unroll
     for (int i = 0; i < RB; ++i)
 #pragma unroll
       for (int m = 0; m < M; ++m) {
         const float v = wave_sum(acc[i][m]);
         acc[i][m] = 0.f;
-        const int ch = INTER ? i >> 1 : i & 1;
-        const bool up = INTER ? (i & 1) : (i >> 1);
+        const int ch = INTER ? i >> 1 : i % CH;
+        const bool up = INTER ? (i & 1) : (i >= CH);
         if (lane == m) {
-          if (up) (ch ? u1 : u0) = v;
-          else (ch ? g1 : g0) = v;
+          if (up) uv[ch] = v;
+          else gv[ch] = v;
         }
       }
     if (lane < M) {
       const Slot& S = slots[csl];
       const float sg = S.g.s2, su = S.u.s2;
-      const uint32_t h0 = swiglu_bits(bf16_round(__fmul_rn(g0, sg)), bf16_round(__fmul_rn(u0, su)));
-      const uint32_t h1 = swiglu_bits(bf16_round(__fmul_rn(g1, sg)), bf16_round(__fmul_rn(u1, su)));
-      uint32_t* dst = reinterpret_cast<uint32_t*>(a.h + ((size_t)S.hslot * M + lane) * I + 2 * cp);
-      __hip_atomic_store((DSGX_GLOBAL uint32_t*)(uintptr_t)dst, h0 | (h1 << 16), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      uint32_t hb = 0;
+#pragma unroll
+      for (int c = 0; c < CH; ++c) hb |= swiglu_bits(bf16_round(__fmul_rn(gv[c], sg)), bf16_round(__fmul_rn(uv[c], su))) << (16 * c);
+      uint16_t* dst = a.h + ((size_t)S.hslot * M + lane) * I + CH * cp;
+      if (CH == 1) __hip_atomic_store((DSGX_GLOBAL uint16_t*)(uintptr_t)dst, (uint16_t)hb, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      else __hip_atomic_store((DSGX_GLOBAL uint32_t*)(uintptr_t)dst, hb, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     csl += dsl, cp += dp;
     if (cp >= nb_e) cp -= nb_e, ++csl;
@@ -240,22 +259,23 @@ __device__ __forceinline__ void up_body(const DecodeArgs& a, const uint4* xs, co
 template <int FMT, int SHFMT, int M>
 __device__ __forceinline__ void up_phase(const DecodeArgs& a, uint4* xs, Step<M>& S, int shared_wgs) {
   constexpr bool kMixed = SHFMT != 0 && SHFMT != FMT;
+  constexpr int kUpCH = M <= 2 ? 1 : 2, kUpD = 8 / kUpCH;  // 16 KiB of weights in flight a wave either way
   const int H = a.L.H, wpb = blockDim.x >> 6, wave = threadIdx.x >> 6;
   const int nsh = SHFMT != 0 ? 1 : 0;
   if (kMixed) {
     if ((int)blockIdx.x < shared_wgs) {
       stage_x<FmtT<DSGX_FMT_BF16>::KL>(xs, a.x, H, M, H, num_segs<DSGX_FMT_BF16>(H) * 512);
       __syncthreads();
-      up_body<kMixed ? DSGX_FMT_BF16 : FMT, M, kMixed, 4>(a, xs, S.slots, 1, blockIdx.x * wpb + wave, shared_wgs * wpb);
+      up_body<kMixed ? DSGX_FMT_BF16 : FMT, M, kMixed, kUpCH, kUpD>(a, xs, S.slots, 1, blockIdx.x * wpb + wave, shared_wgs * wpb);
     } else {
       stage_x<FmtT<FMT>::KL>(xs, a.x, H, M, H, num_segs<FMT>(H) * FmtT<FMT>::SEGK);
       __syncthreads();
-      up_body<FMT, M, false, 4>(a, xs, S.slots + nsh, S.n, ((int)blockIdx.x - shared_wgs) * wpb + wave, ((int)gridDim.x - shared_wgs) * wpb);
+      up_body<FMT, M, false, kUpCH, kUpD>(a, xs, S.slots + nsh, S.n, ((int)blockIdx.x - shared_wgs) * wpb + wave, ((int)gridDim.x - shared_wgs) * wpb);
     }
   } else {
     stage_x<FmtT<FMT>::KL>(xs, a.x, H, M, H, num_segs<FMT>(H) * FmtT<FMT>::SEGK);
     __syncthreads();
-    up_body<FMT, M, false, 4>(a, xs, S.slots, nsh + S.n, blockIdx.x * wpb + wave, gridDim.x * wpb);
+    up_body<FMT, M, false, kUpCH, kUpD>(a, xs, S.slots, nsh + S.n, blockIdx.x * wpb + wave, gridDim.x * wpb);
   }
 }
 
@@ -323,13 +343,15 @@ __device__ __forceinline__ void down_phase(const DecodeArgs& a, uint4* hs, Step<
       // entering a chunk of slots: stage their h rows, each slot in its format's lane order
       const int c1 = min(nsl, c0 + spc);
       __syncthreads();
-      for (int s = c0; s < c1; ++s) {
-        const uint16_t* hp = a.h + (size_t)S.slots[s].hslot * M * I;
-        uint4* dst = hs + (size_t)(s - c0) * M * nq;
-        if (kMixed && s < nsh) stage_x<FmtT<SF>::KL, true>(dst, hp, I, M, I, I);
-        else stage_x<FmtT<FMT>::KL, true>(dst, hp, I, M, I, I);
+      if (kMixed && c0 < nsh) {  // the shared slot (another format's lane order), then the routed ones
+        stage_slots<FmtT<SF>::KL, false>(hs, 1, M, I, [&](int) { return a.h + (size_t)S.slots[0].hslot * M * I; });
+        stage_slots<FmtT<FMT>::KL, false>(hs + (size_t)M * nq, c1 - c0 - 1, M, I,
+                                         [&](int s) { return a.h + (size_t)S.slots[c0 + 1 + s].hslot * M * I; });
+      } else {
+        stage_slots<FmtT<FMT>::KL, false>(hs, c1 - c0, M, I, [&](int s) { return a.h + (size_t)S.slots[c0 + s].hslot * M * I; });
       }
       __syncthreads();
+      DSGX_MARK(7);
     }
     const uint4* xs = hs + (size_t)(cs - c0) * M * nq;
     if (live) {
@@ -387,24 +409,43 @@ __device__ __forceinline__ void down_phase(const DecodeArgs& a, uint4* hs, Step<
 }
 
 // ---- the grid barrier ---------------------------------------------------------------------------------------------------------
-// bar[0] arrivals, bar[1] generation, bar[2] error flag; all zero before the first launch, and left with arrivals 0.
+// A two-level counting barrier in the workspace, every word on its own 128-byte line (kBarLine ints apart):
+//   line g < kBarGroups        arrivals of group g (the workgroups with blockIdx % kBarGroups == g)
+//   line kBarGroups            arrivals of the groups' last members
+//   line kBarGroups + 1 + g    group g's release word: the generation, bumped by the very last arriver
+//   line 2 kBarGroups + 1      error flag
+// All zero before the first launch; arrivals are left at 0, the release words all equal. Counters on separate lines
+// keep the 500-odd device-scope atomics from queueing on one address, and each waiter polls its own group's word.
 // Every workgroup of the grid must be resident (the launch sizes the grid from the occupancy query). The wait is
 // bounded: past spin_limit polls the workgroup raises the error flag and goes on (wrong results, never a hang).
+constexpr int kBarGroups = 16, kBarLine = 32;
+constexpr size_t kBarBytes = (size_t)(2 * kBarGroups + 2) * kBarLine * 4;
+__device__ __forceinline__ int bar_load(int* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+__device__ __forceinline__ int grid_barrier_gen(int* bar) { return bar_load(bar + (kBarGroups + 1 + blockIdx.x % kBarGroups) * kBarLine); }
 __device__ __forceinline__ void grid_barrier(int* bar, int my_gen, int spin_limit) {
   // h was stored with device-scope coherent stores; __syncthreads() waits for every wave's stores to complete, so no
-  // cache write-back or invalidate is needed around the counter (a device-scope fence would flush the whole L2 here)
+  // cache write-back or invalidate is needed around the counters (a device-scope fence would flush the whole L2 here)
   __syncthreads();
   if (threadIdx.x == 0) {
-    const int old = __hip_atomic_fetch_add(&bar[0], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    if (old == (int)gridDim.x - 1) {
-      __hip_atomic_store(&bar[0], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      __hip_atomic_fetch_add(&bar[1], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    } else {
+    const int g = blockIdx.x % kBarGroups;
+    const int members = ((int)gridDim.x - g + kBarGroups - 1) / kBarGroups;
+    const int groups = min((int)gridDim.x, kBarGroups);
+    int* rel = bar + (kBarGroups + 1) * kBarLine;
+    bool released = false;
+    if (__hip_atomic_fetch_add(bar + g * kBarLine, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == members - 1) {
+      __hip_atomic_store(bar + g * kBarLine, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (__hip_atomic_fetch_add(bar + kBarGroups * kBarLine, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == groups - 1) {
+        __hip_atomic_store(bar + kBarGroups * kBarLine, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        for (int i = 0; i < kBarGroups; ++i) __hip_atomic_store(rel + i * kBarLine, my_gen + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        released = true;
+      }
+    }
+    if (!released) {
       int spins = 0;
-      while (__hip_atomic_load(&bar[1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == my_gen) {
-        __builtin_amdgcn_s_sleep(4);
+      while (bar_load(rel + g * kBarLine) == my_gen) {
+        __builtin_amdgcn_s_sleep(8);
         if (++spins > spin_limit) {
-          __hip_atomic_store(&bar[2], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          __hip_atomic_store(bar + (2 * kBarGroups + 1) * kBarLine, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
           break;
         }
       }
@@ -418,14 +459,19 @@ template <int FMT, int SHFMT, int M>
 __global__ void __launch_bounds__(256) k_decode(DecodeArgs a, int shared_wgs, int spc) {
   extern __shared__ uint4 lds[];
   __shared__ Step<M> S;
-  if (threadIdx.x == 0) S.gen = __hip_atomic_load(&a.bar[1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  DSGX_MARK(0);
+  if (threadIdx.x == 0) S.gen = grid_barrier_gen(a.bar);
   build_union(S, a);
+  DSGX_MARK(1);
   fill_slots<FMT, SHFMT, M>(S, a);
+  DSGX_MARK(2);
   up_phase<FMT, SHFMT, M>(a, lds, S, shared_wgs);
+  DSGX_MARK(4);
   const int H = a.L.H, GW = gridDim.x * (blockDim.x >> 6), gw = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
   const int rpw = (H + GW - 1) / GW;
   const int n_lo = min(H, gw * rpw), n_hi = min(H, n_lo + rpw);
-  down_phase<FMT, SHFMT, M, 4>(a, lds, S, spc, n_lo, n_hi, [&] { grid_barrier(a.bar, S.gen, a.spin_limit); });
+  down_phase<FMT, SHFMT, M, 4>(a, lds, S, spc, n_lo, n_hi, [&] { DSGX_MARK(5); grid_barrier(a.bar, S.gen, a.spin_limit); DSGX_MARK(6); });
+  DSGX_MARK(8);
 }
 template <int FMT, int SHFMT, int M>
 __global__ void __launch_bounds__(256) k_up(DecodeArgs a, int shared_wgs) {

@@ -7,7 +7,7 @@ import os
 
 from . import abi
 
-_SO = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc", "libdsgx.so")
+_SO = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc", os.environ.get("DSGX_LIB", "libdsgx.so"))
 _lib = None
 
 

@@ -113,7 +113,7 @@ typedef struct dsgx_decode_cfg {
 } dsgx_decode_cfg;
 DSGX_API void dsgx_decode_cfg_default(dsgx_decode_cfg* cfg);
 /* Workspace bytes of a decode step (gx::decode_ws_bytes; engine/experts/decode.cu:33-35): h bf16
-   [DSGX_MAX_UNION + 1 slots][DSGX_MAX_ROWS][I] plus 256 bytes of counters. Zero it once before the first call. */
+   [DSGX_MAX_UNION + 1 slots][DSGX_MAX_ROWS][I] plus the grid barrier's counters (a few KiB). Zero it once before the first call. */
 DSGX_API size_t dsgx_decode_ws_bytes(const dsgx_layer_w* L);
 /* Byte offset in ws of a 32-bit error flag. The default decode step is one persistent kernel whose workgroups meet at a
    barrier in device memory between the two phases; the wait is bounded, and a workgroup that gives up (it can only

@@ -38,7 +38,7 @@ int main() {
   glm::GemvSeg seg;
   dsk::MoeWeights mw;
   bad += dc.parts != 3 || !pc.shared || seg.rs != 128 || mw.fp8 != nullptr, ++n;
-  bad += gx::decode_ws_bytes(L) != (size_t)(128 + 1) * 16 * 512 * 2 + 256, ++n;  // decode.cu:33-35
+  bad += gx::decode_ws_bytes(L) < (size_t)(128 + 1) * 16 * 512 * 2 + 256, ++n;  // h as decode.cu:33-35, then the counters
   std::printf("CHECK mirror headers %s  %d wrong of %d\n", bad ? "FAIL" : "ok", bad, n);
   return bad != 0;
 }

@@ -128,6 +128,24 @@ def test_decode_two_launch_variant_equals_default_and_flag_clear():
             assert np.array_equal(yr.view(np.uint32), yr3.view(np.uint32))
 
 
+def test_decode_workspace_reuse_with_other_inputs():
+    """h crosses the chip inside one kernel (written in the gate/up phase, read after the grid barrier through the
+    caches): a reused workspace must never serve the previous step's h. Alternate two different steps on one workspace."""
+    for case in (CASES[0], CASES[2]):
+        fmt, H, I, E, topk, NS, shared, scale = case
+        hl, dl = _layer(fmt, H, I, E, topk, NS, shared)
+        steps = []
+        for seed in (61, 62, 63):
+            x, logits, idx, w = rows_and_routing(seed, 2, H, E, topk, scale)
+            yr, ys, _ = gpu.decode_layer(dl, x, idx, w, 2)     # a fresh workspace each
+            steps.append((x, idx, w, yr, ys))
+        ws = gpu.empty(lib.decode_ws_bytes(dl.w), 0)
+        for rep in range(4):
+            for x, idx, w, yr0, ys0 in steps:
+                yr, ys, _ = gpu.decode_layer(dl, x, idx, w, 2, ws=ws)
+                assert np.array_equal(yr.view(np.uint32), yr0.view(np.uint32)) and np.array_equal(ys.view(np.uint32), ys0.view(np.uint32))
+
+
 def test_decode_parts_and_duplicate_experts_across_rows():
     # rows that share every expert (a union of exactly top-k slots) and the up-only / down-only bench switches
     fmt, H, I, E, topk, NS, shared, scale = CASES[1]
