@@ -80,6 +80,31 @@ __device__ __forceinline__ u32x4_t keep_whole(u32x4_t v) {
   asm volatile("" : "+v"(v));
   return v;
 }
+// Wave-uniform values. The compiler cannot know that a value read from LDS or derived from the wave's index is the
+// same in every lane; uni() says so (v_readfirstlane), which moves the value and all arithmetic on it (row bases,
+// cursors, loop bounds, branches) to the scalar unit and lets loads use the "scalar base + lane offset" addressing.
+__device__ __forceinline__ int uni(int v) { return __builtin_amdgcn_readfirstlane(v); }
+__device__ __forceinline__ uint32_t uni(uint32_t v) { return (uint32_t)__builtin_amdgcn_readfirstlane((int)v); }
+__device__ __forceinline__ float uni(float v) { return __uint_as_float(uni(__float_as_uint(v))); }
+__device__ __forceinline__ const uint8_t* uni(const uint8_t* p) {
+  const uint64_t a = (uint64_t)p;
+  return (const uint8_t*)(((uint64_t)uni((uint32_t)(a >> 32)) << 32) | uni((uint32_t)a));
+}
+// loads at (wave-uniform base) + (32-bit lane offset)
+__device__ __forceinline__ u32x4_t ldg_stream(const uint8_t* base, uint32_t voff) {
+  return __builtin_nontemporal_load((const DSGX_GLOBAL u32x4_t*)((const DSGX_GLOBAL uint8_t*)(uintptr_t)base + voff));
+}
+__device__ __forceinline__ uint32_t ldg_u32(const uint8_t* base, uint32_t voff) {
+  return *(const DSGX_GLOBAL uint32_t*)((const DSGX_GLOBAL uint8_t*)(uintptr_t)base + voff);
+}
+__device__ __forceinline__ uint32_t ldg_u16(const uint8_t* base, uint32_t voff) {
+  return *(const DSGX_GLOBAL uint16_t*)((const DSGX_GLOBAL uint8_t*)(uintptr_t)base + voff);
+}
+// pin_after() for a lane offset
+__device__ __forceinline__ uint32_t pin_after(uint32_t voff, float dep) {
+  asm volatile("" : "+v"(voff) : "v"(dep));
+  return voff;
+}
 __device__ __forceinline__ uint32_t ldg_u32(const void* p) { return *(const DSGX_GLOBAL uint32_t*)(uintptr_t)p; }
 __device__ __forceinline__ uint32_t ldg_u16(const void* p) { return *(const DSGX_GLOBAL uint16_t*)(uintptr_t)p; }
 
@@ -228,55 +253,106 @@ __device__ __forceinline__ float route_score(float l, int score_fn) {
   if (score_fn == 0) return route_sigmoid(l);
   return sqrtf(l > 20.f ? l : log1pf(expf(l)));  // DeepSeek's sqrt(softplus): libm-dependent, not promised bit-exact
 }
-// One row by one wavefront: experts e = lane + 64 j, j < 8 (E <= 512). Lane k < topk gets pick k's expert and weight
-// (route_warp of the reference, engine/experts/formats.cuh:207-247, at 64 lanes): descending key, ties to the lower
-// id; the sum in the butterfly order over eight places ((p0+p4)+(p2+p6))+((p1+p5)+(p3+p7)), absent places skipped.
-// The (key, id) order is one unsigned 64-bit order: the key's bits made monotone (sign flipped for positive, all
-// flipped for negative floats) above the complemented id, so each pick is one wave-wide integer maximum.
-__device__ __forceinline__ void route_row(const float* __restrict__ logits_row, const float* __restrict__ bias, int E, int topk,
-                                          float scale, int score_fn, int lane, int& id_out, float& w_out) {
-  constexpr int RJ = DSGX_MAX_EXPERTS / kWave;
-  float s[RJ];
-  uint64_t key[RJ];
+// wave-wide maximum of floats (no NaNs), valid in every lane
+template <int CTRL>
+__device__ __forceinline__ float dpp_max(float v) { return fmaxf(v, __uint_as_float(dpp_mov<CTRL>(__float_as_uint(v)))); }
+__device__ __forceinline__ float wave_max_f32(float v) {
+  v = dpp_max<0xB1>(v);
+  v = dpp_max<0x4E>(v);
+  v = dpp_max<0x141>(v);
+  v = dpp_max<0x140>(v);
+  auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  v = fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+  r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+
+// wave-wide minimum of unsigned ints, valid in every lane
+__device__ __forceinline__ uint32_t wave_min_u32(uint32_t v) {
+  v = min(v, dpp_mov<0xB1>(v));
+  v = min(v, dpp_mov<0x4E>(v));
+  v = min(v, dpp_mov<0x141>(v));
+  v = min(v, dpp_mov<0x140>(v));
+  auto r = __builtin_amdgcn_permlane16_swap(v, v, false, false);
+  v = min(r[0], r[1]);
+  r = __builtin_amdgcn_permlane32_swap(v, v, false, false);
+  return min(r[0], r[1]);
+}
+
+// One row by one wavefront: experts e = lane + 64 j, j < NJ (E <= 64 NJ). Lane k < topk gets pick k's expert and
+// weight (route_warp of the reference, engine/experts/formats.cuh:207-247, at 64 lanes): descending key (float
+// compares), ties to the lower id; the sum in the butterfly order ((p0+p4)+(p2+p6))+((p1+p5)+(p3+p7)), absent places
+// skipped. The code runs once a launch on a single wavefront, so its instruction count is its latency:
+//  - every lane first sorts its NJ places by (key descending, j ascending) with adjacent exchanges (stable);
+//  - a pick is the wave-wide maximum of the lanes' heads; the lane holding it (on a tie, rare, the lowest expert id
+//    among the heads that hold it: a lane's own ties are already in id order) pops its list.
+constexpr int kRouteRJ = DSGX_MAX_EXPERTS / kWave;
+// a row's logits (or the bias; null: zeros) in the lanes' places; E wave-uniform
+__device__ __forceinline__ void route_fetch(const float* __restrict__ row, int E, int lane, float (&v)[kRouteRJ]) {
   const int nj = (E + kWave - 1) / kWave;
 #pragma unroll
-  for (int j = 0; j < RJ; ++j) {
+  for (int j = 0; j < kRouteRJ; ++j) {
     const int e = lane + kWave * j;
-    s[j] = 0.f, key[j] = 0;  // an empty place: below every real key
-    if (j < nj && e < E) {
-      s[j] = route_score(logits_row[e], score_fn);
-      const uint32_t kb = __float_as_uint(__fadd_rn(s[j], bias ? bias[e] : 0.f));
-      const uint32_t mono = kb ^ ((kb >> 31) ? 0xFFFFFFFFu : 0x80000000u);
-      key[j] = ((uint64_t)mono << 32) | (uint32_t)(~e);
+    v[j] = 0.f;
+    if (row && j < nj && e < E) v[j] = row[e];
+  }
+}
+template <int NJ>
+__device__ __forceinline__ void route_row_nj(const float (&logit)[kRouteRJ], const float (&bias)[kRouteRJ], int E, int topk, float scale,
+                                             int score_fn, int lane, int& id_out, float& w_out) {
+  constexpr float kDead = -__builtin_inff();
+  float s[NJ], key[NJ];
+  int jj[NJ];
+#pragma unroll
+  for (int j = 0; j < NJ; ++j) {
+    s[j] = 0.f, key[j] = kDead, jj[j] = j;  // an empty place never wins
+    if (lane + kWave * j < E) {
+      s[j] = route_score(logit[j], score_fn);
+      key[j] = __fadd_rn(s[j], bias[j]);
     }
   }
-  float picked[DSGX_MAX_TOPK];
-  int ids[DSGX_MAX_TOPK];
+  // odd-even transposition: NJ passes of adjacent exchanges, strictly-greater only (equal keys keep their j order)
 #pragma unroll
-  for (int k = 0; k < DSGX_MAX_TOPK; ++k) {
-    picked[k] = 0.f, ids[k] = 0;
-    if (k >= topk) continue;
-    uint64_t best = 0;
+  for (int pass = 0; pass < NJ; ++pass)
 #pragma unroll
-    for (int j = 0; j < RJ; ++j)
-      if (j < nj && key[j] > best) best = key[j];
-    best = wave_max_u64(best);
-    const int be = (int)(~(uint32_t)best);
-    ids[k] = be;
-    float sv = 0.f;
+    for (int j = pass & 1; j + 1 < NJ; j += 2) {
+      const bool sw = key[j + 1] > key[j];
+      const float k0 = key[j], s0 = s[j];
+      const int j0 = jj[j];
+      key[j] = sw ? key[j + 1] : k0, s[j] = sw ? s[j + 1] : s0, jj[j] = sw ? jj[j + 1] : j0;
+      key[j + 1] = sw ? k0 : key[j + 1], s[j + 1] = sw ? s0 : s[j + 1], jj[j + 1] = sw ? j0 : jj[j + 1];
+    }
+  // lane k keeps pick k; the loop is not unrolled
+  float my_s = 0.f;
+  int my_id = 0;
+#pragma unroll 1
+  for (int k = 0; k < topk; ++k) {
+    const float top = wave_max_f32(key[0]);
+    const uint64_t hit = __ballot(key[0] == top);
+    int wl = __builtin_ctzll(hit);
+    if (hit & (hit - 1)) wl = wave_min_u32(key[0] == top ? (uint32_t)(lane + kWave * jj[0]) : 0xFFFFFFFFu) & (kWave - 1);
+    const int id = wl + kWave * __builtin_amdgcn_readlane(jj[0], wl);
+    const float sv = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(s[0]), wl));
+    if (lane == wl) {
 #pragma unroll
-    for (int j = 0; j < RJ; ++j)
-      if (j < nj && lane + kWave * j == be) sv = s[j], key[j] = 0;
-    picked[k] = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(sv), __builtin_amdgcn_readfirstlane(be & (kWave - 1))));
+      for (int j = 0; j + 1 < NJ; ++j) key[j] = key[j + 1], s[j] = s[j + 1], jj[j] = jj[j + 1];
+      key[NJ - 1] = kDead;
+    }
+    if (lane == k) my_s = sv, my_id = id;
   }
-  auto add = [](float a, float b, bool hb) { return hb ? __fadd_rn(a, b) : a; };
-  const float a04 = add(picked[0], picked[4], 4 < topk), a26 = add(picked[2], picked[6], 6 < topk);
-  const float a15 = add(picked[1], picked[5], 5 < topk), a37 = add(picked[3], picked[7], 7 < topk);
-  const float sum = __fadd_rn(add(add(a04, a26, 2 < topk), add(a15, a37, 3 < topk), 1 < topk), 1e-20f);
-  id_out = 0, w_out = 0.f;
-#pragma unroll
-  for (int k = 0; k < DSGX_MAX_TOPK; ++k)
-    if (lane == k && k < topk) id_out = ids[k], w_out = __fmul_rn(__fdiv_rn(picked[k], sum), scale);
+  // lanes 0..7 hold p0..p7 (0 past topk: x + 0 = x): three xor steps are the reference's order of adds
+  float sum = my_s;
+  sum = __fadd_rn(sum, __shfl_xor(sum, 4));
+  sum = __fadd_rn(sum, __shfl_xor(sum, 2));
+  sum = __fadd_rn(sum, __shfl_xor(sum, 1));
+  sum = __fadd_rn(sum, 1e-20f);
+  id_out = my_id, w_out = lane < topk ? __fmul_rn(__fdiv_rn(my_s, sum), scale) : 0.f;
+}
+__device__ __forceinline__ void route_row(const float (&logit)[kRouteRJ], const float (&bias)[kRouteRJ], int E, int topk, float scale,
+                                          int score_fn, int lane, int& id_out, float& w_out) {
+  if (E <= 2 * kWave) route_row_nj<2>(logit, bias, E, topk, scale, score_fn, lane, id_out, w_out);
+  else if (E <= 4 * kWave) route_row_nj<4>(logit, bias, E, topk, scale, score_fn, lane, id_out, w_out);
+  else route_row_nj<kRouteRJ>(logit, bias, E, topk, scale, score_fn, lane, id_out, w_out);
 }
 
 // h = bf16(bf16(silu(g)) * u), g and u already bf16 values (engine/experts/decode.cu:110-113 of the reference)

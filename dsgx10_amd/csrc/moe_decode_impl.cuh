@@ -20,10 +20,24 @@
 // product differs from the reference's (not part of its contract).
 #pragma once
 #include <algorithm>
+#include <type_traits>
 
 #include "abi_internal.h"
 #include "rowdot.cuh"
 
+#ifndef DSGX_UPD
+#define DSGX_UPD 4
+#endif
+#ifndef DSGX_WGS
+#define DSGX_WGS 1
+#endif
+// threads of a decode workgroup (one workgroup a CU)
+#ifndef DSGX_DECODE_THREADS
+#define DSGX_DECODE_THREADS 512
+#endif
+#ifndef DSGX_DOWND
+#define DSGX_DOWND 4
+#endif
 namespace dsgx {
 
 // Diagnostic build only (-DDSGX_TRACE): thread 0 of every workgroup stamps the 100 MHz wall clock at phase marks.
@@ -32,8 +46,14 @@ namespace dsgx {
   do {                                                                                      \
     if (a.trace && threadIdx.x == 0) a.trace[blockIdx.x * 16 + (k)] = wall_clock64();       \
   } while (0)
+// (by lane 0 of whichever wave runs the code)
+#define DSGX_MARKW(k)                                                                       \
+  do {                                                                                      \
+    if (a.trace && (threadIdx.x & 63) == 0) a.trace[blockIdx.x * 16 + (k)] = wall_clock64(); \
+  } while (0)
 #else
 #define DSGX_MARK(k) do { } while (0)
+#define DSGX_MARKW(k) do { } while (0)
 #endif
 
 struct DecodeArgs {
@@ -78,47 +98,61 @@ struct Step {
   uint32_t mask[DSGX_MAX_EXPERTS / 32];
   int ri[M * DSGX_MAX_TOPK];
   float rw[M * DSGX_MAX_TOPK];
-  int id[M * DSGX_MAX_TOPK];
   float wslot[M * DSGX_MAX_TOPK][M];   // per slot the rows' routing weights (0: the row did not pick it)
   Slot slots[M * DSGX_MAX_TOPK + 1];
   int gen;                             // the grid barrier's generation at kernel start
+  int next_up;                         // the gate/up phase's batch counter (up_body)
+  int rdone, ready;                    // rows routed so far; the slots are complete (resolve)
+  uint4 dtab[DSGX_MAX_EXPERTS * 3];    // the descriptors' first 16 bytes (off, s2, fmt), fetched before the routing is known
 };
 
-// The union of the rows' picks in expert-id order (build_union of the reference, decode.cu:57-106), by every
-// workgroup for itself; with logits the rows are routed here first (a wavefront a row, route()'s code and bits).
-template <int M>
-__device__ void build_union(Step<M>& S, const DecodeArgs& a) {
-  const int tid = threadIdx.x, E = a.L.E, topk = a.L.topk, ne = M * topk;
+// The step's set-up comes in two parts, so that the weights that do not depend on the routing (the fused shared
+// expert's, slot 0) stream while the routing's dependent memory round trips are under way:
+//   prep()     by all threads: clears the tables, fills slot 0 and copies every expert's descriptor into LDS (a load
+//              that depends on the routing would take a memory round trip under the weight streams' load: several
+//              microseconds); a __syncthreads() follows it;
+//   resolve()  by the workgroup's last few wavefronts only ("resolvers", resolver_waves()), without workgroup
+//              barriers: with logits routes the rows (a wavefront a row at a time, route()'s code and bits), builds
+//              the union of the rows' picks in expert-id order (build_union of the reference, decode.cu:57-106) and
+//              the routed slots, then raises S.ready. The other wavefronts stream slot 0 meanwhile and look at
+//              S.ready when they need a routed slot (wait_slots()).
+// Every workgroup does both for itself.
+template <int M> __device__ __forceinline__ constexpr int resolver_waves() { return M < 4 ? M : 4; }
+template <int FMT, int SHFMT, int M>
+__device__ __forceinline__ void prep(Step<M>& S, const DecodeArgs& a) {
+  const int tid = threadIdx.x;
+  // every expert's descriptors into S.dtab (their first 16 of 64 bytes), three loads in flight a thread
+  const uint4* d = reinterpret_cast<const uint4*>(a.L.desc);
+  const int nd = a.L.E * 3, bd = blockDim.x;
+  for (int i0 = tid; i0 < nd; i0 += 3 * bd) {
+    uint4 v[3];
+#pragma unroll
+    for (int u = 0; u < 3; ++u)
+      if (i0 + u * bd < nd) v[u] = d[(size_t)(i0 + u * bd) * 4];
+#pragma unroll
+    for (int u = 0; u < 3; ++u)
+      if (i0 + u * bd < nd) S.dtab[i0 + u * bd] = v[u];
+  }
   if (tid < DSGX_MAX_EXPERTS / 32) S.mask[tid] = 0;
   for (int i = tid; i < M * DSGX_MAX_TOPK * M; i += blockDim.x) (&S.wslot[0][0])[i] = 0.f;
-  if (a.logits) {
-    for (int row = tid >> 6; row < M; row += blockDim.x >> 6) {
-      int id;
-      float w;
-      route_row(a.logits + (size_t)row * E, a.bias, E, topk, a.route_scale, a.score_fn, tid & 63, id, w);
-      if ((tid & 63) < topk) S.ri[row * topk + (tid & 63)] = id, S.rw[row * topk + (tid & 63)] = w;
-    }
-  } else {
-    for (int i = tid; i < ne; i += blockDim.x) S.ri[i] = a.idx[i], S.rw[i] = a.w[i];
-  }
-  __syncthreads();
-  for (int i = tid; i < ne; i += blockDim.x) atomicOr(&S.mask[S.ri[i] >> 5], 1u << (S.ri[i] & 31));
-  __syncthreads();
-  for (int i = tid; i < ne; i += blockDim.x) {
-    const int e = S.ri[i];
-    int r = __popc(S.mask[e >> 5] & ((1u << (e & 31)) - 1));
-    for (int j = 0; j < (e >> 5); ++j) r += __popc(S.mask[j]);
-    S.id[r] = e;
-    S.wslot[r][i / topk] = S.rw[i];
-  }
   if (tid == 0) {
-    int n = 0;
-    for (int j = 0; j < DSGX_MAX_EXPERTS / 32; ++j) n += __popc(S.mask[j]);
-    S.n = n;
+    S.next_up = 0, S.ready = 0, S.rdone = 0;
+    if (SHFMT != 0) {
+      Slot t;
+      if (SHFMT == DSGX_FMT_BF16) {
+        t.g = MatRef{a.L.sh.bgu, nullptr, 1.f, 0};
+        t.u = t.g;
+        t.d = MatRef{a.L.sh.bd, nullptr, 1.f, 0};
+      } else {
+        t.g = MatRef{a.L.sh.g, reinterpret_cast<const uint8_t*>(a.L.sh.gs), 1.f, 0};
+        t.u = MatRef{a.L.sh.u, reinterpret_cast<const uint8_t*>(a.L.sh.us), 1.f, 0};
+        t.d = MatRef{a.L.sh.d, reinterpret_cast<const uint8_t*>(a.L.sh.ds), 1.f, 0};
+      }
+      t.hslot = DSGX_SH_SLOT, t.shared = 1;
+      S.slots[0] = t;
+    }
   }
-  __syncthreads();
 }
-
 __device__ __forceinline__ size_t al256d(size_t b) { return (b + 255) / 256 * 256; }
 template <int FMT>
 __device__ __forceinline__ MatRef mat_ref(const uint8_t* base, int N, int K, float s2) {
@@ -135,80 +169,152 @@ __device__ __forceinline__ MatDev mat_dev(const MatRef& r, int N, int K) {
   if (FMT == DSGX_FMT_INT4_G32) m.zp = r.s + al256d((size_t)N * (K / 32) * 2);
   return m;
 }
-// slots: a fused shared expert first (slot 0), then the union in expert-id order
-template <int FMT, int SHFMT, int M>
-__device__ void fill_slots(Step<M>& S, const DecodeArgs& a) {
-  const int H = a.L.H, I = a.L.I, nsh = SHFMT != 0 ? 1 : 0;
-  for (int s = threadIdx.x; s < nsh + S.n; s += blockDim.x) {
-    Slot t;
-    if (s < nsh) {
-      if (SHFMT == DSGX_FMT_BF16) {
-        t.g = MatRef{a.L.sh.bgu, nullptr, 1.f, 0};
-        t.u = t.g;
-        t.d = MatRef{a.L.sh.bd, nullptr, 1.f, 0};
-      } else {
-        t.g = MatRef{a.L.sh.g, reinterpret_cast<const uint8_t*>(a.L.sh.gs), 1.f, 0};
-        t.u = MatRef{a.L.sh.u, reinterpret_cast<const uint8_t*>(a.L.sh.us), 1.f, 0};
-        t.d = MatRef{a.L.sh.d, reinterpret_cast<const uint8_t*>(a.L.sh.ds), 1.f, 0};
-      }
-      t.hslot = DSGX_SH_SLOT, t.shared = 1;
-    } else {
-      const dsgx_mat_desc* d = a.L.desc + (size_t)S.id[s - nsh] * 3;
-      t.g = mat_ref<FMT>(a.L.pool + d[0].off, I, H, d[0].s2);
-      t.u = mat_ref<FMT>(a.L.pool + d[1].off, I, H, d[1].s2);
-      t.d = mat_ref<FMT>(a.L.pool + d[2].off, H, I, d[2].s2);
-      t.hslot = s - nsh, t.shared = 0;
-    }
-    S.slots[s] = t;
+// rw: this resolver's number, nr: how many there are. What a resolver can load before the routing is known it loads
+// first, in resolve_fetch() at the start of the kernel (under the weight streams' load a dependent memory round trip
+// takes several microseconds): its first row's logits and the bias.
+// resolve() follows the workgroup's barrier after prep(). LDS operations of a wavefront complete in program order,
+// and the release fences order them before the counter and the flag.
+struct ResolveRegs {
+  float lg[kRouteRJ], bs[kRouteRJ];
+};
+template <int M>
+__device__ __forceinline__ void resolve_fetch(Step<M>& S, const DecodeArgs& a, int rw, int nr, ResolveRegs& R) {
+  const int lane = threadIdx.x & 63, E = a.L.E;
+  if (a.logits) {
+    route_fetch(rw < M ? a.logits + (size_t)rw * E : nullptr, E, lane, R.lg);
+    route_fetch(a.bias, E, lane, R.bs);
   }
-  __syncthreads();
+}
+template <int FMT, int SHFMT, int M>
+__device__ __forceinline__ void resolve(Step<M>& S, const DecodeArgs& a, int rw, int nr, ResolveRegs& R) {
+  const int lane = threadIdx.x & 63, E = a.L.E, topk = a.L.topk, ne = M * topk;
+  const int H = a.L.H, I = a.L.I, nsh = SHFMT != 0 ? 1 : 0;
+  __builtin_amdgcn_s_setprio(3);
+  int mine = 0;
+  for (int row = rw; row < M; row += nr, ++mine) {
+    int id = 0;
+    float w = 0.f;
+    if (a.logits) {
+      if (row != rw) route_fetch(a.logits + (size_t)row * E, E, lane, R.lg);
+      route_row(R.lg, R.bs, E, topk, a.route_scale, a.score_fn, lane, id, w);
+    } else if (lane < topk) {
+      id = a.idx[row * topk + lane], w = a.w[row * topk + lane];
+    }
+    if (lane < topk) {
+      S.ri[row * topk + lane] = id, S.rw[row * topk + lane] = w;
+      atomicOr(&S.mask[id >> 5], 1u << (id & 31));
+    }
+  }
+  DSGX_MARKW(9);
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+  int before = 0;
+  if (lane == 0) before = __hip_atomic_fetch_add(&S.rdone, mine, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+  if (uni(before) + mine < M) {  // another resolver finishes later: it does the rest
+    __builtin_amdgcn_s_setprio(0);
+    return;
+  }
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+  for (int i = lane; i < ne; i += kWave) {
+    const int e = S.ri[i];
+    int r = __popc(S.mask[e >> 5] & ((1u << (e & 31)) - 1));
+    for (int j = 0; j < (e >> 5); ++j) r += __popc(S.mask[j]);
+    S.wslot[r][i / topk] = S.rw[i];
+    // the routed slot (rows that picked the same expert write the same values)
+    Slot t;
+    auto ref = [&](int which, int N, int K) {
+      const uint4 d = S.dtab[e * 3 + which];
+      return mat_ref<FMT>(a.L.pool + (((uint64_t)d.y << 32) | d.x), N, K, __uint_as_float(d.z));
+    };
+    t.g = ref(0, I, H), t.u = ref(1, I, H), t.d = ref(2, H, I);
+    t.hslot = r, t.shared = 0;
+    S.slots[nsh + r] = t;
+  }
+  if (lane == 0) {
+    int n = 0;
+    for (int j = 0; j < DSGX_MAX_EXPERTS / 32; ++j) n += __popc(S.mask[j]);
+    S.n = n;
+  }
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+  if (lane == 0) __hip_atomic_store(&S.ready, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+  __builtin_amdgcn_s_setprio(0);
+  DSGX_MARKW(2);
+}
+// The number of routed slots, once the resolvers have raised S.ready. No fence after the flag: a wavefront's LDS reads
+// are served in order, the compiler barrier keeps them in program order, and a fence would also wait for every
+// weight load the caller has in flight.
+template <int M>
+__device__ __forceinline__ int wait_slots(Step<M>& S) {
+  while (__hip_atomic_load(&S.ready, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) == 0) __builtin_amdgcn_s_sleep(2);
+  asm volatile("" ::: "memory");
+  return uni(*(volatile int*)&S.n);
 }
 
 // ---- gate/up ------------------------------------------------------------------------------------------------------------
 // Walks slots [s0, s0 + nsl) in format F. INTER: the slot's gate matrix is the BF16 shared expert's interleaved gate/up
-// (rows 2c gate, 2c + 1 up). The wave is number gw of GW; batches go round-robin.
-// CH channels a batch (RB = 2 CH weight rows a step): one channel at few activation rows, where an even split of the
-// batches over the waves matters most (the benchmark's 9 slots x 2048 channels over 2048 waves: nine each).
-template <int FMT, int M, bool INTER, int CH, int D>
-__device__ __forceinline__ void up_body(const DecodeArgs& a, const uint4* xs, const Slot* slots, int nsl, int gw, int GW) {
+// (rows 2c gate, 2c + 1 up). A batch is CH channels of one slot (RB = 2 CH weight rows); batch b is (slot b / nb_e,
+// channels CH (b % nb_e)...). Workgroup g of G owns the batches g, g + G, g + 2 G, ... (spread over the slots and the
+// memory channels); its waves take them one at a time from a counter in LDS, so that a wave that is served faster
+// by the memory system (on a busy CU the older waves are) simply takes more batches, and all waves finish together.
+// The claim for the batch after the next is issued a batch ahead: its latency is never waited for.
+// The routing is resolved late: the workgroup's batches of slot 0 (nsl0 = 1: a fused shared expert; 0: none) need no
+// routing; a wave whose next batch lies beyond them calls wait_nsl(), which waits for the resolvers (wait_slots())
+// and returns the number of slots. Every wave calls it before it leaves (its last claim lies beyond any count).
+template <int FMT, int M, bool INTER, int CH, int D, class WaitNsl>
+__device__ __forceinline__ void up_body(const DecodeArgs& a, const uint4* xs, const Slot* slots, int nsl0, int* counter, int g, int G,
+                                        WaitNsl&& wait_nsl) {
+  // g, G are wave-uniform (uni()): the cursors below live on the scalar unit
   constexpr int RB = 2 * CH;
-  const int lane = threadIdx.x & 63, H = a.L.H, I = a.L.I;
+  const uint32_t lane = threadIdx.x & 63;
+  const int H = a.L.H, I = a.L.I;
   const int nsegk = num_segs<FMT>(H), nq = nsegk * FmtT<FMT>::SEGK / 8;
-  const int nb_e = I / CH, nbatch = nsl * nb_e;
-  const int nmine = gw < nbatch ? (nbatch - gw + GW - 1) / GW : 0;
-  const int nsteps = nmine * nsegk;
-  // the batch cursors advance by GW batches: (slot, pair) += (GW / nb_e, GW % nb_e) with carry
-  const int dsl = GW / nb_e, dp = GW % nb_e;
-  int lsl = gw / nb_e, lp = gw % nb_e, lseg = 0;   // the load cursor
-  int csl = lsl, cp = lp, cseg = 0;                 // the compute cursor
+  const int nb_e = I / CH;
+  // (integer division runs on the vector unit: its results are declared uniform again)
+  auto batches_of = [&](int nslots) { return uni(g < nslots * nb_e ? (nslots * nb_e - g + G - 1) / G : 0); };
+  int nk = batches_of(nsl0);  // the workgroup's batches that can be opened: slot 0's until the routing is resolved
+  bool resolved = false;
   Raw w[D][RB];
+  int rsl[D], rp[D], rseg[D];  // what each ring entry holds: slot, pair, segment; rseg < 0: nothing
   float acc[RB][M];
 #pragma unroll
   for (int i = 0; i < RB; ++i)
 #pragma unroll
     for (int m = 0; m < M; ++m) acc[i][m] = 0.f;
-  const uint8_t* dummy = reinterpret_cast<const uint8_t*>(a.x);  // where the loads past the last step go (cached)
-  int lt = 0;
-  auto load = [&](Raw (&r)[RB]) {
-    const bool ok = lt < nsteps;
-    ++lt;
-    const Slot& S = slots[ok ? lsl : 0];
-    const MatDev g = mat_dev<FMT>(S.g, INTER ? 2 * I : I, H), u = mat_dev<FMT>(S.u, I, H);
-#pragma unroll
-    for (int i = 0; i < RB; ++i) {
-      if (INTER) load_raw<FMT, false>(r[i], g, RB * lp + i, lseg, lane, H, acc[i][0], ok ? nullptr : dummy);
-      else load_raw<FMT, false>(r[i], i < CH ? g : u, CH * lp + i % CH, lseg, lane, H, acc[i][0], ok ? nullptr : dummy);
-    }
-    if (ok && ++lseg == nsegk) {
-      lseg = 0, lsl += dsl, lp += dp;
-      if (lp >= nb_e) lp -= nb_e, ++lsl;
-      if (lsl >= nsl) lsl = 0, lp = 0;  // past the wave's last batch: any valid place (these loads go to `dummy`)
-    }
+  int pending = 0;  // lane 0: the claim in flight
+  auto claim = [&]() {
+    if (lane == 0) pending = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
   };
-  auto compute = [&](const Raw (&r)[RB]) {
+  RowSrc src[RB];
+  int lsl = 0, lp = 0, lseg = 0;
+  bool lvalid = true;
+  auto open = [&]() {  // the next batch of this wave: the claim issued a batch ago; then claims the one after
+    const int k = uni(pending);
+    claim();
+    if (k >= nk && !resolved) nk = batches_of(wait_nsl()), resolved = true;
+    lvalid = k < nk;
+    const int b = lvalid ? g + k * G : 0;  // past the end the ring keeps loading: the first rows of the first slot (cached)
+    lsl = uni(b / nb_e), lp = b - lsl * nb_e, lseg = 0;
+    const Slot& S = slots[lsl];
+    MatRef gr{}, ur{};
+    gr.w = uni(S.g.w), gr.s = uni(S.g.s), ur.w = uni(S.u.w), ur.s = uni(S.u.s);
+    const MatDev gm = mat_dev<FMT>(gr, INTER ? 2 * I : I, H), um = mat_dev<FMT>(ur, I, H);
+#pragma unroll
+    for (int i = 0; i < RB; ++i) src[i] = INTER ? row_src<FMT>(gm, RB * lp + i, H) : row_src<FMT>(i < CH ? gm : um, CH * lp + i % CH, H);
+  };
+  claim();
+  open();
+  auto load = [&](Raw (&r)[RB], int& sl, int& p, int& seg) {
+    if (lseg == nsegk) {  // the batch's loads are all issued: the next batch (opened only now, when it is needed)
+      if (lvalid) open();
+      else lseg = 0;
+    }
+#pragma unroll
+    for (int i = 0; i < RB; ++i) load_row<FMT>(r[i], src[i], lseg, lane, 7, acc[i][0]);
+    sl = lsl, p = lp, seg = lvalid ? lseg : -1;
+    ++lseg;
+  };
+  auto compute = [&](const Raw (&r)[RB], int csl, int cp, int cseg) {
     step_dot<FMT, M, RB>(r, xs, nq, cseg, lane, acc);
-    if (++cseg < nsegk) return;
-    cseg = 0;
+    if (cseg + 1 < nsegk) return;
     // lane m < M finishes the batch's channel(s) of activation row m and stores them as one 16- or 32-bit word. The
     // store is coherent at device scope (it bypasses the XCD-local L2): the down phase of the same kernel reads h on
     // other XCDs right after the grid barrier.
@@ -238,44 +344,50 @@ __device__ __forceinline__ void up_body(const DecodeArgs& a, const uint4* xs, co
       if (CH == 1) __hip_atomic_store((DSGX_GLOBAL uint16_t*)(uintptr_t)dst, (uint16_t)hb, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       else __hip_atomic_store((DSGX_GLOBAL uint32_t*)(uintptr_t)dst, hb, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
-    csl += dsl, cp += dp;
-    if (cp >= nb_e) cp -= nb_e, ++csl;
   };
-  // software pipeline: D steps in flight; every iteration computes a step (while there is one) and issues a load
-  if (nsteps == 0) return;
+  // software pipeline: a ring of D steps in flight; every turn computes the oldest step and issues a load in its place
 #pragma unroll
-  for (int d = 0; d < D; ++d) load(w[d]);
-  for (int t = 0; t < nsteps; t += D) {
+  for (int d = 0; d < D; ++d) load(w[d], rsl[d], rp[d], rseg[d]);
+  for (;;) {
+    bool any = lvalid;
 #pragma unroll
     for (int d = 0; d < D; ++d) {
-      if (t + d < nsteps) compute(w[d]);
-      load(w[d]);
+      if (rseg[d] >= 0) compute(w[d], rsl[d], rp[d], rseg[d]), any = true;
+      load(w[d], rsl[d], rp[d], rseg[d]);
     }
+    if (!any) break;
   }
 }
 
 // x staged for format F, then the up phase of this workgroup. With a shared expert of another format (INT4 experts,
 // BF16 shared expert) the first `shared_wgs` workgroups do the shared expert's gate/up and the others the routed slots.
+// prep() has run; resolve() runs inside (up_body).
 template <int FMT, int SHFMT, int M>
 __device__ __forceinline__ void up_phase(const DecodeArgs& a, uint4* xs, Step<M>& S, int shared_wgs) {
   constexpr bool kMixed = SHFMT != 0 && SHFMT != FMT;
-  constexpr int kUpCH = M <= 2 ? 1 : 2, kUpD = 8 / kUpCH;  // 16 KiB of weights in flight a wave either way
-  const int H = a.L.H, wpb = blockDim.x >> 6, wave = threadIdx.x >> 6;
-  const int nsh = SHFMT != 0 ? 1 : 0;
-  if (kMixed) {
-    if ((int)blockIdx.x < shared_wgs) {
-      stage_x<FmtT<DSGX_FMT_BF16>::KL>(xs, a.x, H, M, H, num_segs<DSGX_FMT_BF16>(H) * 512);
-      __syncthreads();
-      up_body<kMixed ? DSGX_FMT_BF16 : FMT, M, kMixed, kUpCH, kUpD>(a, xs, S.slots, 1, blockIdx.x * wpb + wave, shared_wgs * wpb);
-    } else {
-      stage_x<FmtT<FMT>::KL>(xs, a.x, H, M, H, num_segs<FMT>(H) * FmtT<FMT>::SEGK);
-      __syncthreads();
-      up_body<FMT, M, false, kUpCH, kUpD>(a, xs, S.slots + nsh, S.n, ((int)blockIdx.x - shared_wgs) * wpb + wave, ((int)gridDim.x - shared_wgs) * wpb);
-    }
+  constexpr int kUpCH = M <= 2 ? 1 : 2, kUpD = DSGX_UPD / kUpCH;
+  constexpr int nsh = SHFMT != 0 ? 1 : 0, NR = resolver_waves<M>();
+  const int H = a.L.H, wave = uni((int)(threadIdx.x >> 6)), nw = blockDim.x >> 6;
+  const bool shared_wg = kMixed && (int)blockIdx.x < shared_wgs;
+  const bool resolver = wave >= nw - NR;
+  ResolveRegs rr;
+  if (resolver) resolve_fetch(S, a, wave - (nw - NR), NR, rr);
+  prep<FMT, SHFMT, M>(S, a);
+  if (shared_wg) stage_x<FmtT<DSGX_FMT_BF16>::KL>(xs, a.x, H, M, H, num_segs<DSGX_FMT_BF16>(H) * 512);
+  else stage_x<FmtT<FMT>::KL>(xs, a.x, H, M, H, num_segs<FMT>(H) * FmtT<FMT>::SEGK);
+  __syncthreads();
+  DSGX_MARK(1);
+  if (resolver) resolve<FMT, SHFMT, M>(S, a, wave - (nw - NR), NR, rr);
+  if (shared_wg) {
+    up_body<kMixed ? DSGX_FMT_BF16 : FMT, M, kMixed, kUpCH, kUpD>(a, xs, S.slots, 1, &S.next_up, blockIdx.x, shared_wgs, [&] {
+      wait_slots(S);
+      return 1;
+    });
+  } else if (kMixed) {
+    up_body<FMT, M, false, kUpCH, kUpD>(a, xs, S.slots + nsh, 0, &S.next_up, (int)blockIdx.x - shared_wgs, (int)gridDim.x - shared_wgs,
+                                        [&] { return wait_slots(S); });
   } else {
-    stage_x<FmtT<FMT>::KL>(xs, a.x, H, M, H, num_segs<FMT>(H) * FmtT<FMT>::SEGK);
-    __syncthreads();
-    up_body<FMT, M, false, kUpCH, kUpD>(a, xs, S.slots, nsh + S.n, blockIdx.x * wpb + wave, gridDim.x * wpb);
+    up_body<FMT, M, false, kUpCH, kUpD>(a, xs, S.slots, nsh, &S.next_up, blockIdx.x, gridDim.x, [&] { return nsh + wait_slots(S); });
   }
 }
 
@@ -287,13 +399,13 @@ __device__ __forceinline__ void down_phase(const DecodeArgs& a, uint4* hs, Step<
   constexpr int RB = 2;
   constexpr bool kMixed = SHFMT != 0 && SHFMT != FMT;
   constexpr int SF = SHFMT == 0 ? FMT : SHFMT;  // the shared slot's format
-  const int H = a.L.H, I = a.L.I, lane = threadIdx.x & 63;
-  const int nsh = SHFMT != 0 ? 1 : 0, nsl = nsh + S.n;
+  const int H = a.L.H, I = a.L.I;
+  const uint32_t lane = threadIdx.x & 63;
+  const int nsh = SHFMT != 0 ? 1 : 0, nrouted = uni(S.n), nsl = nsh + nrouted;
   const int nq = I / 8;
   const int segs_r = num_segs<FMT>(I), segs_s = nsh ? num_segs<SF>(I) : 0;
-  const int nsub = n_hi > n_lo ? (n_hi - n_lo + RB - 1) / RB : 0;
-  const int steps_sub = segs_s + S.n * segs_r;
-  const int nsteps = nsub * steps_sub;  // this wave's steps with real loads
+  const int nsub = uni(n_hi > n_lo ? (n_hi - n_lo + RB - 1) / RB : 0);
+  const int steps_sub = segs_s + nrouted * segs_r;
   // every wave of the workgroup walks the same number of steps (the barriers around the h chunks)
   __shared__ int s_maxsub;
   if (threadIdx.x == 0) s_maxsub = 0;
@@ -306,23 +418,35 @@ __device__ __forceinline__ void down_phase(const DecodeArgs& a, uint4* hs, Step<
   for (int r = 0; r < RB; ++r)
 #pragma unroll
     for (int m = 0; m < M; ++m) yacc[r][m] = sacc[r][m] = acc[r][m] = 0.f;
-  const uint8_t* dummy = reinterpret_cast<const uint8_t*>(a.x);
-  int lt = 0, lsub = 0, ls = 0, lseg = 0;  // the load cursor
-  auto load = [&](Raw (&r)[RB]) {
-    const bool ok = lt < nsteps;
-    ++lt;
-    const Slot& T = S.slots[ok ? ls : 0];
-    const bool sh = kMixed && ls < nsh;
-    const int n0 = n_lo + lsub * RB;
+  int lsub = 0, ls = 0, lseg = 0;  // the load cursor (scalar): sub-batch, slot, segment
+  bool lsh = kMixed && nsh > 0;    // the slot under the load cursor is the shared one in another format
+  RowSrc src[RB];
+  auto open = [&](int sub, int sl) {  // the RB rows of sub-batch `sub` in slot sl's down matrix
+    const Slot& T = S.slots[sl];
+    MatRef dr{};
+    dr.w = uni(T.d.w), dr.s = uni(T.d.s);
+    const int n0 = n_lo + sub * RB;
 #pragma unroll
     for (int i = 0; i < RB; ++i) {
-      const int n = ok ? (n0 + i < n_hi ? n0 + i : n_hi - 1) : 0;  // a row past the end re-reads the last one (its result is dropped)
-      if (sh) load_raw<SF, false>(r[i], mat_dev<SF>(T.d, H, I), n, lseg, lane, I, acc[i][0], ok ? nullptr : dummy);
-      else load_raw<FMT, false>(r[i], mat_dev<FMT>(T.d, H, I), n, lseg, lane, I, acc[i][0], ok ? nullptr : dummy);
+      // a row past the wave's end re-reads its last one (the result is dropped); sub < 0: the matrix's first rows
+      const int n = sub < 0 ? min(i, H - 1) : n0 + i < n_hi ? n0 + i : n_hi - 1;
+      if (kMixed && sl < nsh) src[i] = row_src<SF>(mat_dev<SF>(dr, H, I), n, I);
+      else src[i] = row_src<FMT>(mat_dev<FMT>(dr, H, I), n, I);
     }
-    if (ok && ++lseg == (ls < nsh ? segs_s : segs_r)) {
+  };
+  open(nsub > 0 ? 0 : -1, 0);
+  auto load = [&](Raw (&r)[RB]) {
+#pragma unroll
+    for (int i = 0; i < RB; ++i) {
+      if (lsh) load_row<SF>(r[i], src[i], lseg, lane, 7, acc[i][0]);
+      else load_row<FMT>(r[i], src[i], lseg, lane, 7, acc[i][0]);
+    }
+    if (++lseg == (ls < nsh ? segs_s : segs_r)) {
       lseg = 0;
       if (++ls == nsl) ls = 0, ++lsub;
+      // past the wave's last step the ring keeps loading: the first rows of every slot in turn (the same for all waves)
+      open(lsub < nsub ? lsub : -1, ls);
+      lsh = kMixed && ls < nsh;
     }
   };
 #pragma unroll
@@ -330,28 +454,30 @@ __device__ __forceinline__ void down_phase(const DecodeArgs& a, uint4* hs, Step<
 
   between();
   __syncthreads();
-  const int maxsub = s_maxsub;
+  const int maxsub = uni(s_maxsub);
   const bool one_chunk = nsl <= spc;
   const int wg_steps = maxsub * steps_sub;
 
-  int csub = 0, cs = 0, cseg = 0;  // the compute cursor
-  auto compute = [&](const Raw (&r)[RB]) {
+  int csub = 0, cs = 0, cseg = 0, c0 = 0;  // the compute cursor; c0: first slot of the chunk of h in LDS
+  auto stage_chunk = [&]() {  // h of the slots [c0, c0 + spc) into LDS, each slot in its format's lane order
+    const int c1 = min(nsl, c0 + spc);
+    __syncthreads();
+    if (kMixed && c0 < nsh) {  // the shared slot (another format's lane order), then the routed ones
+      stage_slots<FmtT<SF>::KL, false>(hs, 1, M, I, [&](int) { return a.h + (size_t)S.slots[0].hslot * M * I; });
+      stage_slots<FmtT<FMT>::KL, false>(hs + (size_t)M * nq, c1 - c0 - 1, M, I,
+                                       [&](int s) { return a.h + (size_t)S.slots[c0 + 1 + s].hslot * M * I; });
+    } else {
+      stage_slots<FmtT<FMT>::KL, false>(hs, c1 - c0, M, I, [&](int s) { return a.h + (size_t)S.slots[c0 + s].hslot * M * I; });
+    }
+    __syncthreads();
+    DSGX_MARK(7);
+  };
+  // restage: the step may enter a new chunk of slots (the variant without it is for h that fits LDS whole)
+  auto compute = [&](const Raw (&r)[RB], auto restage) {
     const bool live = csub < nsub;
     const bool sh = cs < nsh;
-    const int c0 = cs / spc * spc;
-    if (cseg == 0 && cs == c0 && !(one_chunk && csub > 0)) {
-      // entering a chunk of slots: stage their h rows, each slot in its format's lane order
-      const int c1 = min(nsl, c0 + spc);
-      __syncthreads();
-      if (kMixed && c0 < nsh) {  // the shared slot (another format's lane order), then the routed ones
-        stage_slots<FmtT<SF>::KL, false>(hs, 1, M, I, [&](int) { return a.h + (size_t)S.slots[0].hslot * M * I; });
-        stage_slots<FmtT<FMT>::KL, false>(hs + (size_t)M * nq, c1 - c0 - 1, M, I,
-                                         [&](int s) { return a.h + (size_t)S.slots[c0 + 1 + s].hslot * M * I; });
-      } else {
-        stage_slots<FmtT<FMT>::KL, false>(hs, c1 - c0, M, I, [&](int s) { return a.h + (size_t)S.slots[c0 + s].hslot * M * I; });
-      }
-      __syncthreads();
-      DSGX_MARK(7);
+    if constexpr (decltype(restage)::value) {
+      if (cseg == 0 && cs == c0) stage_chunk();
     }
     const uint4* xs = hs + (size_t)(cs - c0) * M * nq;
     if (live) {
@@ -370,8 +496,11 @@ __device__ __forceinline__ void down_phase(const DecodeArgs& a, uint4* hs, Step<
         else yacc[i][m] = fmaf(__fmul_rn(s2, S.wslot[cs - nsh][m]), acc[i][m], yacc[i][m]);
         acc[i][m] = 0.f;
       }
-    if (++cs < nsl) return;
-    cs = 0;
+    if (++cs < nsl) {
+      if (cs == c0 + spc) c0 += spc;
+      return;
+    }
+    cs = 0, c0 = 0;
     // the sub-batch is complete: add the lanes; lane i * M + m keeps output (row n0 + i, activation row m)
     const int n0 = n_lo + csub * RB;
     ++csub;
@@ -399,11 +528,22 @@ __device__ __forceinline__ void down_phase(const DecodeArgs& a, uint4* hs, Step<
       }
     }
   };
-  for (int t = 0; t < wg_steps; t += D) {
+  if (one_chunk) {
+    if (wg_steps > 0) stage_chunk();
+    for (int t = 0; t < wg_steps; t += D) {
 #pragma unroll
-    for (int d = 0; d < D; ++d) {
-      if (t + d < wg_steps) compute(w[d]);
-      load(w[d]);
+      for (int d = 0; d < D; ++d) {
+        if (t + d < wg_steps) compute(w[d], std::false_type{});
+        load(w[d]);
+      }
+    }
+  } else {
+    for (int t = 0; t < wg_steps; t += D) {
+#pragma unroll
+      for (int d = 0; d < D; ++d) {
+        if (t + d < wg_steps) compute(w[d], std::true_type{});
+        load(w[d]);
+      }
     }
   }
 }
@@ -456,38 +596,40 @@ __device__ __forceinline__ void grid_barrier(int* bar, int my_gen, int spin_limi
 
 // ---- kernels ----------------------------------------------------------------------------------------------------------------
 template <int FMT, int SHFMT, int M>
-__global__ void __launch_bounds__(256) k_decode(DecodeArgs a, int shared_wgs, int spc) {
+__global__ void __launch_bounds__(DSGX_DECODE_THREADS) k_decode(DecodeArgs a, int shared_wgs, int spc) {
   extern __shared__ uint4 lds[];
   __shared__ Step<M> S;
   DSGX_MARK(0);
   if (threadIdx.x == 0) S.gen = grid_barrier_gen(a.bar);
-  build_union(S, a);
-  DSGX_MARK(1);
-  fill_slots<FMT, SHFMT, M>(S, a);
-  DSGX_MARK(2);
   up_phase<FMT, SHFMT, M>(a, lds, S, shared_wgs);
   DSGX_MARK(4);
-  const int H = a.L.H, GW = gridDim.x * (blockDim.x >> 6), gw = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
-  const int rpw = (H + GW - 1) / GW;
+  const int H = a.L.H, GW = gridDim.x * (blockDim.x >> 6), gw = uni((int)(blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)));
+  const int rpw = uni((H + GW - 1) / GW);
   const int n_lo = min(H, gw * rpw), n_hi = min(H, n_lo + rpw);
-  down_phase<FMT, SHFMT, M, 4>(a, lds, S, spc, n_lo, n_hi, [&] { DSGX_MARK(5); grid_barrier(a.bar, S.gen, a.spin_limit); DSGX_MARK(6); });
+  down_phase<FMT, SHFMT, M, DSGX_DOWND>(a, lds, S, spc, n_lo, n_hi, [&] { DSGX_MARK(5); grid_barrier(a.bar, S.gen, a.spin_limit); DSGX_MARK(6); });
   DSGX_MARK(8);
 }
 template <int FMT, int SHFMT, int M>
-__global__ void __launch_bounds__(256) k_up(DecodeArgs a, int shared_wgs) {
+__global__ void __launch_bounds__(DSGX_DECODE_THREADS) k_up(DecodeArgs a, int shared_wgs) {
   extern __shared__ uint4 lds[];
   __shared__ Step<M> S;
-  build_union(S, a);
-  fill_slots<FMT, SHFMT, M>(S, a);
   up_phase<FMT, SHFMT, M>(a, lds, S, shared_wgs);
 }
 template <int FMT, int SHFMT, int M>
 __global__ void __launch_bounds__(256) k_down(DecodeArgs a, int spc) {
   extern __shared__ uint4 lds[];
   __shared__ Step<M> S;
-  build_union(S, a);
-  fill_slots<FMT, SHFMT, M>(S, a);
-  const int H = a.L.H, gw = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  {
+    constexpr int NR = resolver_waves<M>();
+    const int wave = uni((int)(threadIdx.x >> 6)), nw = blockDim.x >> 6;
+    ResolveRegs rr;
+    if (wave >= nw - NR) resolve_fetch(S, a, wave - (nw - NR), NR, rr);
+    prep<FMT, SHFMT, M>(S, a);
+    __syncthreads();
+    if (wave >= nw - NR) resolve<FMT, SHFMT, M>(S, a, wave - (nw - NR), NR, rr);
+    __syncthreads();
+  }
+  const int H = a.L.H, gw = uni((int)(blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)));
   const int n_lo = min(H, gw * 2), n_hi = min(H, n_lo + 2);
   down_phase<FMT, SHFMT, M, 4>(a, lds, S, spc, n_lo, n_hi, [] {});
 }
@@ -503,11 +645,9 @@ int launch_decode(const DecodeArgs& a, int parts, hipStream_t st) {
   const int segk = FmtT<FMT>::SEGK;
   size_t lds_up = (size_t)M * ((H + segk - 1) / segk * segk) * 2;
   if (kMixed) lds_up = std::max(lds_up, (size_t)M * ((H + 511) / 512 * 512) * 2);
-  // h of a chunk of slots in LDS for the down phase: all of them when they fit in 64 KiB
+  // h of a chunk of slots in LDS for the down phase: all of them when they fit (96 KiB with one workgroup a CU, 40 with two; the kernels' own tables take up to 36 KiB)
   const size_t slot_bytes = (size_t)M * I * 2;
-  int spc = std::max(1, (int)((64 * 1024) / slot_bytes));
-  spc = std::min(spc, nsl_max);
-  const size_t lds_down = (size_t)spc * slot_bytes;
+  auto slots_per_chunk = [&](size_t lds_bytes) { return std::min(std::max(1, (int)(lds_bytes / slot_bytes)), nsl_max); };
   auto shared_split = [&](int grid) {
     if (!kMixed) return 0;
     // the workgroups split between the BF16 shared expert and the routed experts by their bytes
@@ -517,15 +657,16 @@ int launch_decode(const DecodeArgs& a, int parts, hipStream_t st) {
   (void)SF;
   if (parts == 3) {
     auto kern = k_decode<FMT, SHFMT, M>;
-    const size_t lds = std::max(lds_up, lds_down);
+    const int spc = slots_per_chunk(DSGX_WGS == 1 ? 96 * 1024 : 40 * 1024);
+    const size_t lds = std::max(lds_up, (size_t)spc * slot_bytes);
     if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds)) return rc;
     // every workgroup must be resident: the grid comes from the occupancy of this kernel with this much LDS
     int per_cu = 0;
-    DSGX_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kern, 256, lds));
+    DSGX_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kern, DSGX_DECODE_THREADS, lds));
     if (per_cu >= 1) {
-      per_cu = std::min(per_cu, 2);
+      per_cu = std::min(per_cu, DSGX_WGS);
       const int grid = cus * per_cu;
-      hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, st, a, shared_split(grid), spc);
+      hipLaunchKernelGGL(kern, dim3(grid), dim3(DSGX_DECODE_THREADS), lds, st, a, shared_split(grid), spc);
       DSGX_HIP(hipGetLastError());
       return DSGX_OK;
     }
@@ -534,12 +675,14 @@ int launch_decode(const DecodeArgs& a, int parts, hipStream_t st) {
   if (parts & 1) {
     auto kern = k_up<FMT, SHFMT, M>;
     if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds_up)) return rc;
-    const int grid = cus * (lds_up <= 56 * 1024 ? 2 : 1);
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds_up, st, a, shared_split(grid));
+    const int grid = cus * DSGX_WGS;
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(DSGX_DECODE_THREADS), lds_up, st, a, shared_split(grid));
     DSGX_HIP(hipGetLastError());
   }
   if (parts & 2) {
     auto kern = k_down<FMT, SHFMT, M>;
+    const int spc = slots_per_chunk(40 * 1024);
+    const size_t lds_down = (size_t)spc * slot_bytes;
     if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds_down)) return rc;
     const int waves = (H + 1) / 2, grid = (waves + 3) / 4;
     hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds_down, st, a, spc);

@@ -13,7 +13,10 @@ __global__ void __launch_bounds__(256) k_route(const float* __restrict__ logits,
   if (row >= M) return;
   int id;
   float w;
-  route_row(logits + (size_t)row * E, bias, E, topk, scale, score_fn, lane, id, w);
+  float lg[kRouteRJ], bs[kRouteRJ];
+  route_fetch(logits + (size_t)row * E, E, lane, lg);
+  route_fetch(bias, E, lane, bs);
+  route_row(lg, bs, E, topk, scale, score_fn, lane, id, w);
   if (lane < topk) idx[row * topk + lane] = id, wout[row * topk + lane] = w;
 }
 

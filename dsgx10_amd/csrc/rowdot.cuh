@@ -67,6 +67,44 @@ __device__ __forceinline__ void load_raw(Raw& r, const MatDev& m, int n, int seg
   }
 }
 
+// The same loads with the wave-uniform part of the addresses kept apart: a RowSrc is one weight row's bases, set up
+// once a row on the scalar unit; load_row() then issues the step's loads as scalar base + lane offset.
+struct RowSrc {
+  const uint8_t* w;  // the row's first byte
+  const uint8_t* a;  // FP8: the row's scale row; INT4: the row's scales
+  const uint8_t* z;  // INT4: the zero-point words of the row's group of 8 rows
+  uint32_t zsh;      // INT4: the row's nibble in those words
+};
+// m, n, K wave-uniform
+template <int FMT>
+__device__ __forceinline__ RowSrc row_src(const MatDev& m, int n, int K) {
+  using F = FmtT<FMT>;
+  RowSrc r;
+  r.w = m.w + (size_t)n * F::row_bytes(K);
+  r.a = r.z = nullptr, r.zsh = 0;
+  if constexpr (FMT == DSGX_FMT_FP8_B128) {
+    r.a = m.s + (size_t)(n >> m.lrs) * m.srow * 4;
+  } else if constexpr (FMT == DSGX_FMT_INT4_G32) {
+    const int G = K >> 5;
+    r.a = m.s + (size_t)n * G * 2;
+    r.z = m.zp + (size_t)(n >> 3) * G * 4;
+    r.zsh = 4 * (n & 7);
+  }
+  return r;
+}
+// seg wave-uniform; lks: log2 of the FP8 scale block along k (wave-uniform). No tail handling: K is whole segments.
+template <int FMT>
+__device__ __forceinline__ void load_row(Raw& r, const RowSrc& s, int seg, uint32_t lane, int lks, float pin) {
+  r.v = ldg_stream(s.w + seg * 1024, pin_after(lane * 16u, pin));
+  if constexpr (FMT == DSGX_FMT_FP8_B128) {
+    r.aux = ldg_u32(s.a + (size_t)(seg * FmtT<FMT>::SEGK >> lks) * 4, ((lane * 16u) >> lks) * 4u);
+  } else if constexpr (FMT == DSGX_FMT_INT4_G32) {
+    r.aux = ldg_u16(s.a + seg * 128, lane * 2u) | (((ldg_u32(s.z + seg * 256, lane * 4u) >> s.zsh) & 15u) << 16);
+  } else {
+    r.aux = 0;
+  }
+}
+
 // RB rows of one segment against M activation rows. xs: the workgroup's staged activations, row m at xs + m * nq
 // (nq chunks a row); acc[r][m] are the lanes' running sums.
 template <int FMT, int M, int RB, bool TAIL = false>
