@@ -580,9 +580,12 @@ static void fp8_row_qdot(const Mat& m, const uint8_t* xq, const float* xs, std::
 // One row of the chunk: picks idx[topk], w[topk] of token row x bf16 [H]. hq_out (optional) h bf16 [topk sorted by
 // expert id][I]; yr f32 [H] (sum in expert-id order, acc = fmaf(w_e, d_e, acc)), yr64 / yrmag from the same quantised
 // operands in f64. With a fused FP8 shared expert ys f32 [H] likewise (null allowed).
+// h_in (optional, [topk sorted by expert id (+ 1: the shared expert's last)][I]): the down projections start from
+// these h instead of the ones computed here, which checks the second GEMM alone (a one-step difference in one h
+// is an e4m3 step of its quantised value, or of its whole block when it is the block's maximum).
 ORC void orc_moe_prefill_fp8_row(const dsgx_layer_w* L, const dsgx_mat_desc* desc, const uint16_t* x, const int* idx,
                                  const float* w, uint16_t* h_out, float* yr, double* yr64, double* yrmag, float* ys,
-                                 double* ys64, double* ysmag) {
+                                 double* ys64, double* ysmag, const uint16_t* h_in) {
   const int H = L->H, I = L->I, topk = L->topk;
   std::vector<uint8_t> xq(H), hq(I);
   std::vector<float> xs(H / 128), hs(I / 128);
@@ -603,7 +606,8 @@ ORC void orc_moe_prefill_fp8_row(const dsgx_layer_w* L, const dsgx_mat_desc* des
     fp8_row_qdot(G, xq.data(), xs.data(), g, nullptr, nullptr);
     fp8_row_qdot(Uw, xq.data(), xs.data(), u, nullptr, nullptr);
     for (int c = 0; c < I; ++c) hb[c] = f2bf(silu_mul(bfr(g[c] * G.s2), bfr(u[c] * Uw.s2)));
-    if (h_out && !sh) memcpy(h_out + (size_t)s * I, hb.data(), (size_t)I * 2);
+    if (h_out) memcpy(h_out + (size_t)s * I, hb.data(), (size_t)I * 2);
+    if (h_in) memcpy(hb.data(), h_in + (size_t)s * I, (size_t)I * 2);
     orc_act_quant(hb.data(), 1, I, hq.data(), hs.data());
     fp8_row_qdot(Dn, hq.data(), hs.data(), d, &d64, &dm);
     if (sh) {

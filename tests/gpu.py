@@ -17,6 +17,13 @@ def empty(nbytes, fill=None):
     return t
 
 
+def view(base, ptr, nbytes):
+    """the bytes [ptr, ptr + nbytes) of the device buffer `base` (a pointer the library returned into it)"""
+    o = int(ptr) - base.data_ptr()
+    assert 0 <= o and o + nbytes <= base.numel()
+    return base[o:o + nbytes]
+
+
 def host(t, dtype, shape):
     torch.cuda.synchronize()
     return t.cpu().numpy().view(dtype).reshape(shape).copy()

@@ -212,17 +212,19 @@ def moe_down(hl, h, idx, w, uni, ysum=False, ys_in=None):
     return out
 
 
-def moe_prefill_fp8_row(hl, xrow, idx, w):
+def moe_prefill_fp8_row(hl, xrow, idx, w, h_in=None):
+    """h_in: bf16 [topk in expert-id order (+ 1, the shared expert's)][I] to start the down projections from"""
     xrow = np.ascontiguousarray(xrow, np.uint16)
     idx = np.ascontiguousarray(idx, np.int32)
     w = np.ascontiguousarray(w, np.float32)
     H, I, topk = hl.H, hl.I, hl.topk
-    h = np.empty((topk, I), np.uint16)
+    h = np.empty((topk + 1, I), np.uint16)
+    hin = None if h_in is None else np.ascontiguousarray(h_in, np.uint16)
     out = dict(h=h, yr=np.empty(H, np.float32), yr64=np.empty(H, np.float64), yrmag=np.empty(H, np.float64),
                ys=np.zeros(H, np.float32), ys64=np.zeros(H, np.float64), ysmag=np.zeros(H, np.float64))
     Lw, desc = hl.host_layer_w()
     lib().orc_moe_prefill_fp8_row(C.byref(Lw), _p(desc), _p(xrow), _p(idx), _p(w), _p(h), _p(out["yr"]), _p(out["yr64"]),
-                                  _p(out["yrmag"]), _p(out["ys"]), _p(out["ys64"]), _p(out["ysmag"]))
+                                  _p(out["yrmag"]), _p(out["ys"]), _p(out["ys64"]), _p(out["ysmag"]), _p(hin))
     return out
 
 
