@@ -329,3 +329,42 @@ def gemv_bench(reps=64):
             b = per + M * K * 2 + M * N * 2
             out.append(dict(workload=name, M=M, us_per_call=us, bytes=b, hbm_frac=b / (us * 1e-6) / HBM_PEAK))
     return out
+
+
+class PrefillBench:
+    """One prefill chunk of T rows over a generated FP8 layer: each row picks top-k distinct experts drawn from a
+    Zipf(s) popularity over a seeded permutation of the experts, uniform weights 1/top-k (the reference's
+    bench_prefill input shape, engine/experts/tests/bench_prefill.inc)."""
+
+    def __init__(self, gen, T, zipf_s=1.1, seed=4321):
+        self.gen, self.T = gen, T
+        g = torch.Generator(device="cuda")
+        g.manual_seed(seed)
+        self.x = torch.randn(T, gen.H, generator=g, device="cuda").to(torch.bfloat16)
+        rank = torch.randperm(gen.E, generator=g, device="cuda").to(torch.float32) + 1.0
+        p = rank.pow(-zipf_s)
+        self.idx = torch.multinomial(p.expand(T, gen.E), gen.topk, replacement=False, generator=g).to(torch.int32).contiguous()
+        self.w = torch.full((T, gen.topk), 1.0 / gen.topk, dtype=torch.float32, device="cuda")
+        self.layer = gen.layer_w(0)
+        self.ws = torch.zeros(lib.prefill_ws_bytes(self.layer, T), dtype=torch.uint8, device="cuda")
+        self.yr = torch.zeros(T, gen.H, dtype=torch.float32, device="cuda")
+        self.ys = torch.zeros(T, gen.H, dtype=torch.float32, device="cuda")
+        # useful multiply-adds only: routed picks (and, apart, the shared expert on every row)
+        self.flops_routed = 2.0 * T * gen.topk * 3 * gen.I * gen.H
+        self.flops_shared = 2.0 * T * 3 * gen.I * gen.H
+
+    def run(self, phases=31, shared=True):
+        lib.moe_prefill(self.layer, self.x, self.idx, self.w, self.T, self.ws, self.yr, self.ys, shared=shared, phases=phases)
+
+    def time(self, phases=31, shared=True, reps=5):
+        self.run(phases, shared)
+        torch.cuda.synchronize()
+        ts = []
+        for _ in range(reps):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            self.run(phases, shared)
+            e1.record()
+            torch.cuda.synchronize()
+            ts.append(e0.elapsed_time(e1) * 1e-3)
+        return float(np.median(ts))

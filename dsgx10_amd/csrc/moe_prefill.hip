@@ -29,6 +29,27 @@ __device__ __forceinline__ v16f_t mfma_fp8(v8i_t a, v8i_t b, v16f_t c) {
   return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, c, 0, 0, 0, 0, 0, 0);  // (both scales 0: the unscaled form)
 }
 
+typedef float v4f_t __attribute__((ext_vector_type(4)));
+// D (16 x 16, f32) += A (16 x 128, e4m3) B^T (16 x 128, e4m3): v_mfma_f32_16x16x128_f8f6f4. A lane holds 32 k of one row
+// of A and of one row of B (row lane % 16, k-part lane / 16: which 32 k of the 128 a part holds does not matter as long
+// as A and B agree). The result's register r of lane l is D[4 (l / 16) + r][l % 16].
+__device__ __forceinline__ v4f_t mfma_fp8_k128(v8i_t a, v8i_t b, v4f_t c) {
+  return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, c, 0, 0, 0, 0, 0, 0);
+}
+// the probe of the 16 x 16 x 128 form: a lane's 32 bytes are the 16 bytes at part * 16 and those at 64 + part * 16 of
+// its row (the k order the prefill kernels use, so that four lanes read 64 contiguous bytes of a row an instruction)
+__global__ void __launch_bounds__(64) k_probe_mfma_fp8_k128(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, float* __restrict__ raw) {
+  const int l = threadIdx.x, row = l % 16, part = l / 16;
+  auto frag = [&](const uint8_t* M) {
+    const uint4 lo = *reinterpret_cast<const uint4*>(M + row * 128 + part * 16), hi = *reinterpret_cast<const uint4*>(M + row * 128 + 64 + part * 16);
+    return v8i_t{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
+  };
+  v4f_t c = {};
+  c = mfma_fp8_k128(frag(A), frag(B), c);
+#pragma unroll
+  for (int r = 0; r < 4; ++r) raw[l * 16 + r] = c[r];
+}
+
 __global__ void __launch_bounds__(64) k_probe_mfma_fp8(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, float* __restrict__ raw) {
   const int l = threadIdx.x;
   const v8i_t a = *reinterpret_cast<const v8i_t*>(A + (l % 32) * 64 + (l / 32) * 32);
@@ -126,12 +147,23 @@ __global__ void __launch_bounds__(256) k_pf_rowsort(const int* __restrict__ idx,
 }
 
 // ---- the grouped GEMM ---------------------------------------------------------------------------------------------------
-// A workgroup (4 waves, 2 x 2) computes 128 weight rows x 128 positions of one tile; UP: the weight rows are 64 gate and
-// 64 up channels (a wave: 32 + 32 of the same channels, so g and u of a channel meet in one lane). K in blocks of 128:
-// the block's A and B panels go through LDS (rows padded to 144 bytes: the 32-byte fragment reads of 32 consecutive
-// rows then fall on distinct banks), double buffered, the next block's global loads in flight during the MFMAs.
+// Most experts of a chunk hold fewer rows than a tile, so the step mostly streams weights: it is built like the decode
+// kernels. A workgroup (8 waves) computes one tile of 128 positions against 256 weight rows; a WAVE owns 32 of those
+// rows as two 16-row MFMA tiles (UP: 16 gate rows and the 16 up rows of the same channels, so g and u of a channel meet
+// in one lane) and streams them from memory straight into registers, a ring of kRing 128-k blocks ahead: a lane loads
+// 2 x 16 bytes a tile and block, the four lanes of a row 64 contiguous bytes an instruction. The activations of the
+// tile (shared by the eight waves) go through LDS, kStages blocks ahead, rows padded to 144 bytes (the fragment reads of
+// 16 consecutive rows then fall on distinct banks).
+// v_mfma_f32_16x16x128_f8f6f4 covers one whole 128-k scale block: partial = A B^T from zero, then
+// acc = fma(x_scale * w_scale, partial, acc) on the vector unit (the accumulators therefore stay in ordinary registers).
+// With the weights as the A operand a lane's four accumulators of a tile belong to ONE position, so the combined scale is
+// one value a lane.
 constexpr int kLdsRow = 144;
-constexpr int kPanel = kTile * kLdsRow;  // bytes of one 128-row panel
+constexpr int kPanel = kTile * kLdsRow;          // bytes of one activation panel (128 rows x 128 k)
+constexpr int kStages = 4, kRing = 4;
+constexpr int kStageBytes = kPanel + kTile * 4;  // + the rows' scales of the block
+constexpr int kWgRows = 256;                     // weight rows a workgroup (UP: 128 channels)
+constexpr int kGemmThreads = 512;
 
 struct GemmArgs {
   const uint8_t* aq;   // activations, e4m3 [rows][K]
@@ -148,10 +180,10 @@ struct GemmArgs {
 };
 
 template <bool UP>
-__global__ void __launch_bounds__(256, 2) k_pf_gemm(GemmArgs g) {
+__global__ void __launch_bounds__(kGemmThreads) k_pf_gemm(GemmArgs g) {
   extern __shared__ uint8_t smem[];
   const int K = UP ? g.L.H : g.L.I, KB = K / 128;
-  const int NS = UP ? g.L.I / 64 : g.L.H / kTile;  // workgroups along the weight rows
+  const int NS = UP ? g.L.I / (kWgRows / 2) : g.L.H / kWgRows;  // workgroups along the weight rows
   const int tile = blockIdx.x / NS, ns = blockIdx.x % NS;
   int e = -1, m0 = tile * kTile, mend = g.nrows;
   if (g.tile_e) {
@@ -163,7 +195,7 @@ __global__ void __launch_bounds__(256, 2) k_pf_gemm(GemmArgs g) {
     return;
   }
   // the tile's matrices
-  const uint8_t *wa, *wb;   // UP: gate, up; DOWN: down (wb unused)
+  const uint8_t *wa, *wb;   // UP: gate, up; DOWN: down twice
   const float *sa, *sb;
   float s2a = 1.f, s2b = 1.f;
   const size_t NK = (size_t)g.L.H * g.L.I;
@@ -180,125 +212,132 @@ __global__ void __launch_bounds__(256, 2) k_pf_gemm(GemmArgs g) {
     sa = reinterpret_cast<const float*>(wa + (NK + 255) / 256 * 256);
     sb = reinterpret_cast<const float*>(wb + (NK + 255) / 256 * 256);
   }
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, wn = wave >> 1, wm = wave & 1;
-  const int n0 = UP ? ns * 64 : ns * kTile;  // first channel (UP) / first weight row (DOWN) of the workgroup
+  const int tid = threadIdx.x, lane = tid & 63, wave = uni(tid >> 6), r16 = lane & 15, part = lane >> 4;
+  // the wave's two 16-row weight tiles: the lane's row of each, and the 16-byte column of the block's halves it loads
+  const int n0 = UP ? ns * (kWgRows / 2) + 16 * wave : ns * kWgRows + 32 * wave;  // UP: first channel; DOWN: first row
+  const uint8_t* pa[2];
+  pa[0] = wa + (size_t)(n0 + r16) * K + part * 16;
+  pa[1] = (UP ? wb + (size_t)(n0 + r16) * K : wa + (size_t)(n0 + 16 + r16) * K) + part * 16;
+  const float* swa = sa + (size_t)(n0 / 128) * KB;  // the tiles' scale rows (a wave's 32 rows lie in one 128-row block)
+  const float* swb = UP ? sb + (size_t)(n0 / 128) * KB : swa;
 
-  // staging: thread t brings chunk t % 8 (16 bytes) of panel rows t / 8 + 32 i, i < 4, of A and of B
+  // activation staging: thread t brings chunk t % 8 (16 bytes) of panel rows t / 8 and t / 8 + 64; t < 128 row t's scale
   const int chunk = tid & 7, srow = tid >> 3;
-  const uint8_t* pa[4];
-  const uint8_t* pb[4];
+  const uint8_t* pb[2];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int a = srow + 32 * i;  // panel row of A: wave-major (wn', nt, row)
-    if (UP) {
-      const int c = n0 + 32 * (a >> 6) + (a & 31);
-      pa[i] = ((a >> 5) & 1 ? wb : wa) + (size_t)c * K + chunk * 16;
-    } else {
-      pa[i] = wa + (size_t)(n0 + a) * K + chunk * 16;
-    }
-    int pos = m0 + srow + 32 * i;
+  for (int i = 0; i < 2; ++i) {
+    int pos = m0 + srow + 64 * i;
     if (pos >= mend) pos = mend - 1;  // a ragged tile re-reads its last row (never stored)
-    const int row = g.gather ? g.gather[pos] : pos;
-    pb[i] = g.aq + (size_t)row * K + chunk * 16;
+    pb[i] = g.aq + (size_t)(g.gather ? g.gather[pos] : pos) * K + chunk * 16;
   }
-  // the lane's two token columns (one a 32-column tile) and their activation rows, for the block scales
-  int mpos[2];
-  const float* xs[2];
-#pragma unroll
-  for (int mt = 0; mt < 2; ++mt) {
-    int pos = m0 + 64 * wm + 32 * mt + (lane & 31);
-    mpos[mt] = pos;
+  const float* pxs;
+  {
+    int pos = m0 + (tid & 127);
     if (pos >= mend) pos = mend - 1;
-    xs[mt] = g.as + (size_t)(g.gather ? g.gather[pos] : pos) * KB;
+    pxs = g.as + (size_t)(g.gather ? g.gather[pos] : pos) * KB;
   }
-  // the wave's weight scale rows (its 64 weight rows lie in one 128-row scale block)
-  const float* swa = sa + (size_t)((UP ? n0 + 32 * wn : n0 + 64 * wn) / 128) * KB;
-  const float* swb = UP ? sb + (size_t)((n0 + 32 * wn) / 128) * KB : swa;
 
-  v16f_t acc[2][2];
+  v4f_t acc[2][8];
 #pragma unroll
-  for (int nt = 0; nt < 2; ++nt)
+  for (int t = 0; t < 2; ++t)
 #pragma unroll
-    for (int mt = 0; mt < 2; ++mt) acc[nt][mt] = v16f_t{};
+    for (int mt = 0; mt < 8; ++mt) acc[t][mt] = v4f_t{};
 
-  uint4 ra[4], rb[4];
-  auto fetch = [&](int kb) {
+  u32x4_t ra[kRing][2][2];  // the weight ring: block slot, tile, the block's half
+  auto load_a = [&](int slot, int kb) {
+    const int kc = kb < KB ? kb : KB - 1;  // past the end: the last block again (never used)
 #pragma unroll
-    for (int i = 0; i < 4; ++i) ra[i] = *reinterpret_cast<const uint4*>(pa[i] + (size_t)kb * 128);
-#pragma unroll
-    for (int i = 0; i < 4; ++i) rb[i] = *reinterpret_cast<const uint4*>(pb[i] + (size_t)kb * 128);
+    for (int t = 0; t < 2; ++t) {
+      const uint8_t* p = pin_after(pa[t] + (size_t)kc * 128, acc[t][0][0]);
+      ra[slot][t][0] = ldg_stream(p);
+      ra[slot][t][1] = ldg_stream(p + 64);
+    }
   };
-  auto stash = [&](int buf) {
-    uint8_t* A = smem + (size_t)buf * 2 * kPanel;
-    uint8_t* B = A + kPanel;
+  u32x4_t rx[2][2];
+  float rxs[2];
+  auto fetch_x = [&](int set, int kb) {
+    const int kc = kb < KB ? kb : KB - 1;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) *reinterpret_cast<uint4*>(A + (srow + 32 * i) * kLdsRow + chunk * 16) = ra[i];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) *reinterpret_cast<uint4*>(B + (srow + 32 * i) * kLdsRow + chunk * 16) = rb[i];
+    for (int i = 0; i < 2; ++i) rx[set][i] = *reinterpret_cast<const u32x4_t*>(pb[i] + (size_t)kc * 128);
+    rxs[set] = pxs[kc];
   };
-  fetch(0);
-  stash(0);
-  __syncthreads();
-  for (int kb = 0; kb < KB; ++kb) {
-    if (kb + 1 < KB) fetch(kb + 1);
-    const float x0 = xs[0][kb], x1 = xs[1][kb], wsa = swa[kb], wsb = swb[kb];
-    const uint8_t* A = smem + (size_t)(kb & 1) * 2 * kPanel + (size_t)(wn * 64 + (lane & 31)) * kLdsRow + (lane >> 5) * 32;
-    const uint8_t* B = smem + (size_t)(kb & 1) * 2 * kPanel + kPanel + (size_t)(wm * 64 + (lane & 31)) * kLdsRow + (lane >> 5) * 32;
-    v16f_t p[2][2];
+  auto stash_x = [&](int set, int stage) {
+    uint8_t* B = smem + (size_t)stage * kStageBytes;
 #pragma unroll
-    for (int kc = 0; kc < 2; ++kc) {
-      v8i_t fa[2], fb[2];
+    for (int i = 0; i < 2; ++i) *reinterpret_cast<u32x4_t*>(B + (srow + 64 * i) * kLdsRow + chunk * 16) = rx[set][i];
+    if (tid < kTile) reinterpret_cast<float*>(B + kPanel)[tid] = rxs[set];
+  };
+  auto compute = [&](int slot, int stage, int kb) {
+    const uint8_t* B = smem + (size_t)stage * kStageBytes;
+    const float* XS = reinterpret_cast<const float*>(B + kPanel);
+    const float wsa = swa[kb], wsb = swb[kb];
+    v8i_t fa[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      const u32x4_t lo = keep_whole(ra[slot][t][0]), hi = keep_whole(ra[slot][t][1]);
+      fa[t] = v8i_t{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
+    }
+#pragma unroll
+    for (int mt = 0; mt < 8; ++mt) {
+      const uint8_t* bp = B + (size_t)(16 * mt + r16) * kLdsRow + part * 16;
+      const u32x4_t lo = *reinterpret_cast<const u32x4_t*>(bp), hi = *reinterpret_cast<const u32x4_t*>(bp + 64);
+      const v8i_t fb = v8i_t{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
+      const float x = XS[16 * mt + r16];
 #pragma unroll
       for (int t = 0; t < 2; ++t) {
-        fa[t] = *reinterpret_cast<const v8i_t*>(A + t * 32 * kLdsRow + kc * 64);
-        fb[t] = *reinterpret_cast<const v8i_t*>(B + t * 32 * kLdsRow + kc * 64);
+        const v4f_t p = mfma_fp8_k128(fa[t], fb, v4f_t{});
+        const float sc = __fmul_rn(x, t ? wsb : wsa);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) acc[t][mt][q] = fmaf(sc, p[q], acc[t][mt][q]);
       }
-#pragma unroll
-      for (int nt = 0; nt < 2; ++nt)
-#pragma unroll
-        for (int mt = 0; mt < 2; ++mt) p[nt][mt] = mfma_fp8(fa[nt], fb[mt], kc == 0 ? v16f_t{} : p[nt][mt]);
     }
+  };
+  // prologue: the weight ring, the first activation panels
 #pragma unroll
-    for (int nt = 0; nt < 2; ++nt)
+  for (int d = 0; d < kRing; ++d) load_a(d, d);
 #pragma unroll
-      for (int mt = 0; mt < 2; ++mt) {
-        const float sc = __fmul_rn(mt ? x1 : x0, nt ? wsb : wsa);
+  for (int s = 0; s < kStages - 1; ++s) {
+    fetch_x(0, s);
+    stash_x(0, s);
+  }
+  fetch_x(1, kStages - 1);  // (block 3: written at the end of the first turn)
+  __syncthreads();
+  // turn kb: issue the activation loads of block kb + 4, compute block kb, issue the weight loads of block kb + 4 in
+  // its place, put the activations of block kb + 3 (loaded a turn ago) into their stage
+  for (int kb0 = 0; kb0 < KB; kb0 += 4) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) acc[nt][mt][r] = fmaf(sc, p[nt][mt][r], acc[nt][mt][r]);
-      }
-    if (kb + 1 < KB) stash((kb + 1) & 1);
-    __syncthreads();
+    for (int u = 0; u < 4; ++u) {
+      const int kb = kb0 + u;
+      fetch_x(u & 1, kb + 4);
+      if (kb < KB) compute(u, u, kb);
+      load_a(u, kb + kRing);
+      stash_x((u + 1) & 1, (u + 3) & 3);
+      __syncthreads();
+    }
   }
 
-  // epilogue: register r of lane l is weight row 8 (r / 4) + 4 (l / 32) + r % 4 of the 32-row tile, column l % 32
+  // epilogue: register q of lane l is weight row 4 (l / 16) + q of the 16-row tile, position l % 16 of the 16 positions
   if (UP) {
     const int I = g.L.I;
 #pragma unroll
-    for (int mt = 0; mt < 2; ++mt) {
-      if (mpos[mt] >= mend) continue;
-      uint16_t* hr = g.h + (size_t)mpos[mt] * I + n0 + 32 * wn + 4 * (lane >> 5);
+    for (int mt = 0; mt < 8; ++mt) {
+      const int pos = m0 + 16 * mt + r16;
+      if (pos >= mend) continue;
+      uint32_t hb[4];
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        uint32_t hb[4];
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-          hb[j] = swiglu_bits(bf16_round(__fmul_rn(acc[0][mt][4 * q + j], s2a)), bf16_round(__fmul_rn(acc[1][mt][4 * q + j], s2b)));
-        *reinterpret_cast<uint2*>(hr + 8 * q) = make_uint2(hb[0] | (hb[1] << 16), hb[2] | (hb[3] << 16));
-      }
+      for (int q = 0; q < 4; ++q)
+        hb[q] = swiglu_bits(bf16_round(__fmul_rn(acc[0][mt][q], s2a)), bf16_round(__fmul_rn(acc[1][mt][q], s2b)));
+      *reinterpret_cast<uint2*>(g.h + (size_t)pos * I + n0 + 4 * part) = make_uint2(hb[0] | (hb[1] << 16), hb[2] | (hb[3] << 16));
     }
   } else {
     const int H = g.L.H;
 #pragma unroll
-    for (int mt = 0; mt < 2; ++mt) {
-      if (mpos[mt] >= mend) continue;
+    for (int mt = 0; mt < 8; ++mt) {
+      const int pos = m0 + 16 * mt + r16;
+      if (pos >= mend) continue;
 #pragma unroll
-      for (int nt = 0; nt < 2; ++nt) {
-        float* dr = g.d + (size_t)mpos[mt] * H + n0 + 64 * wn + 32 * nt + 4 * (lane >> 5);
-#pragma unroll
-        for (int q = 0; q < 4; ++q)
-          *reinterpret_cast<float4*>(dr + 8 * q) =
-              make_float4(acc[nt][mt][4 * q], acc[nt][mt][4 * q + 1], acc[nt][mt][4 * q + 2], acc[nt][mt][4 * q + 3]);
-      }
+      for (int t = 0; t < 2; ++t)
+        *reinterpret_cast<float4*>(g.d + (size_t)pos * H + n0 + 16 * t + 4 * part) = make_float4(acc[t][mt][0], acc[t][mt][1], acc[t][mt][2], acc[t][mt][3]);
     }
   }
 }
@@ -328,11 +367,13 @@ using namespace dsgx;
 
 extern "C" {
 
-// raw[lane][r]: the accumulator registers of one v_mfma_f32_32x32x64_f8f6f4 of A [32][64] and B [32][64] (e4m3 codes,
-// k contiguous), so that a test can pin the operand and result layouts the prefill kernels assume.
-int dsgx_probe_mfma_fp8(const void* A, const void* B, float* raw, void* stream) {
-  if (!A || !B || !raw) return fail(DSGX_EINVAL, "probe_mfma_fp8: null argument");
-  hipLaunchKernelGGL(k_probe_mfma_fp8, dim3(1), dim3(64), 0, (hipStream_t)stream, (const uint8_t*)A, (const uint8_t*)B, raw);
+// raw[lane][r]: the accumulator registers of one e4m3 MFMA, so that a test can pin the operand and result layouts the
+// prefill kernels assume. form 0: v_mfma_f32_32x32x64 over A [32][64], B [32][64]; form 1: v_mfma_f32_16x16x128 over
+// A [16][128], B [16][128] (codes, k contiguous; 16 floats a lane, form 1 fills the first four).
+int dsgx_probe_mfma_fp8(const void* A, const void* B, float* raw, int form, void* stream) {
+  if (!A || !B || !raw || form < 0 || form > 1) return fail(DSGX_EINVAL, "probe_mfma_fp8: null argument or form %d", form);
+  if (form == 0) hipLaunchKernelGGL(k_probe_mfma_fp8, dim3(1), dim3(64), 0, (hipStream_t)stream, (const uint8_t*)A, (const uint8_t*)B, raw);
+  else hipLaunchKernelGGL(k_probe_mfma_fp8_k128, dim3(1), dim3(64), 0, (hipStream_t)stream, (const uint8_t*)A, (const uint8_t*)B, raw);
   DSGX_HIP(hipGetLastError());
   return DSGX_OK;
 }
@@ -348,7 +389,8 @@ static int prefill_check(const dsgx_layer_w* L, int T, const char* who) {
   if (!L) return fail(DSGX_EINVAL, "%s: null layer", who);
   if (L->fmt != DSGX_FMT_FP8_B128) return fail(DSGX_EUNSUPPORTED, "%s: only FP8_B128 layers are built (format %u)", who, L->fmt);
   if (T < 1 || T > DSGX_MAX_CHUNK) return fail(DSGX_EINVAL, "%s: T %d (1..%d)", who, T, DSGX_MAX_CHUNK);
-  if (L->H < 128 || L->H % 128 || L->I < 128 || L->I % 128) return fail(DSGX_EINVAL, "%s: H %d, I %d (multiples of 128)", who, L->H, L->I);
+  if (L->H < 256 || L->H % 256 || L->I < 128 || L->I % 128)
+    return fail(DSGX_EINVAL, "%s: H %d (a multiple of 256), I %d (a multiple of 128)", who, L->H, L->I);
   if (L->E < 1 || L->E > DSGX_MAX_EXPERTS || L->topk < 1 || L->topk > DSGX_MAX_TOPK || L->topk > L->E)
     return fail(DSGX_EINVAL, "%s: E %d, top-k %d", who, L->E, L->topk);
   return DSGX_OK;
@@ -377,7 +419,7 @@ int dsgx_moe_prefill(const dsgx_layer_w* L, const uint16_t* x, const int* idx, c
   auto I32 = [&](size_t off) { return reinterpret_cast<int*>(W + off); };
   auto F32 = [&](size_t off) { return reinterpret_cast<float*>(W + off); };
   const int H = L->H, I = L->I, E = L->E, topk = L->topk, P = o.P;
-  const size_t lds = 2 * 2 * (size_t)kPanel;
+  const size_t lds = (size_t)kStages * kStageBytes;
   if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(k_pf_gemm<true>), lds)) return rc;
   if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(k_pf_gemm<false>), lds)) return rc;
 
@@ -398,7 +440,7 @@ int dsgx_moe_prefill(const dsgx_layer_w* L, const uint16_t* x, const int* idx, c
     g.aq = W + o.xq, g.as = F32(o.xs), g.gather = I32(o.perm);
     g.tile_e = I32(o.tile_e), g.tile_m0 = I32(o.tile_m0), g.ntiles = I32(o.ntiles), g.off = I32(o.off), g.nrows = P;
     g.h = reinterpret_cast<uint16_t*>(W + o.h), g.d = nullptr;
-    hipLaunchKernelGGL(k_pf_gemm<true>, dim3((unsigned)o.max_tiles * (I / 64)), dim3(256), lds, st, g);
+    hipLaunchKernelGGL(k_pf_gemm<true>, dim3((unsigned)o.max_tiles * (I / (kWgRows / 2))), dim3(kGemmThreads), lds, st, g);
     DSGX_HIP(hipGetLastError());
   }
   if (cfg.phases & 4) {
@@ -406,7 +448,7 @@ int dsgx_moe_prefill(const dsgx_layer_w* L, const uint16_t* x, const int* idx, c
     g.aq = W + o.hq, g.as = F32(o.hs), g.gather = nullptr;
     g.tile_e = I32(o.tile_e), g.tile_m0 = I32(o.tile_m0), g.ntiles = I32(o.ntiles), g.off = I32(o.off), g.nrows = P;
     g.h = nullptr, g.d = F32(o.d);
-    hipLaunchKernelGGL(k_pf_gemm<false>, dim3((unsigned)o.max_tiles * (H / kTile)), dim3(256), lds, st, g);
+    hipLaunchKernelGGL(k_pf_gemm<false>, dim3((unsigned)o.max_tiles * (H / kWgRows)), dim3(kGemmThreads), lds, st, g);
     DSGX_HIP(hipGetLastError());
   }
   if (cfg.phases & 8) {
@@ -419,10 +461,10 @@ int dsgx_moe_prefill(const dsgx_layer_w* L, const uint16_t* x, const int* idx, c
     g.aq = W + o.xq, g.as = F32(o.xs), g.gather = nullptr;
     g.tile_e = g.tile_m0 = g.ntiles = g.off = nullptr, g.nrows = T;
     g.h = reinterpret_cast<uint16_t*>(W + o.hsh), g.d = nullptr;
-    hipLaunchKernelGGL(k_pf_gemm<true>, dim3((unsigned)tiles * (I / 64)), dim3(256), lds, st, g);
+    hipLaunchKernelGGL(k_pf_gemm<true>, dim3((unsigned)tiles * (I / (kWgRows / 2))), dim3(kGemmThreads), lds, st, g);
     if (int rc = dsgx_act_quant(reinterpret_cast<const uint16_t*>(W + o.hsh), T, I, W + o.hshq, F32(o.hshs), stream)) return rc;
     g.aq = W + o.hshq, g.as = F32(o.hshs), g.h = nullptr, g.d = ys;
-    hipLaunchKernelGGL(k_pf_gemm<false>, dim3((unsigned)tiles * (H / kTile)), dim3(256), lds, st, g);
+    hipLaunchKernelGGL(k_pf_gemm<false>, dim3((unsigned)tiles * (H / kWgRows)), dim3(kGemmThreads), lds, st, g);
     DSGX_HIP(hipGetLastError());
   }
   return DSGX_OK;

@@ -49,7 +49,7 @@ def lib():
         L.dsgx_stream_read.argtypes = [C.c_void_p, C.c_size_t, C.c_void_p, C.c_void_p]
         L.dsgx_stream_read_cfg.argtypes = [C.c_void_p, C.c_size_t, C.c_void_p, C.c_int, C.c_int, C.c_void_p]
         L.dsgx_stream_copy.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]
-        L.dsgx_probe_mfma_fp8.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]
+        L.dsgx_probe_mfma_fp8.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p]
         if hasattr(L, "dsgx_moe_prefill"):
             L.dsgx_prefill_ws_bytes.restype = C.c_size_t
             L.dsgx_prefill_ws_bytes.argtypes = [C.POINTER(abi.LayerW), C.c_int]
@@ -156,6 +156,7 @@ def stream_copy(src, dst, nbytes, stream=None):
     _check(lib().dsgx_stream_copy(_ptr(src), _ptr(dst), nbytes, _stream(stream)))
 
 
-def probe_mfma_fp8(A, B, raw, stream=None):
-    """raw f32 [64][16]: the accumulator registers of one 32x32x64 fp8 MFMA over A [32][64], B [32][64] e4m3 codes"""
-    _check(lib().dsgx_probe_mfma_fp8(_ptr(A), _ptr(B), _ptr(raw), _stream(stream)))
+def probe_mfma_fp8(A, B, raw, form=0, stream=None):
+    """raw f32 [64][16]: the accumulator registers of one e4m3 MFMA; form 0: 32x32x64 over A [32][64], B [32][64];
+    form 1: 16x16x128 over A [16][128], B [16][128]"""
+    _check(lib().dsgx_probe_mfma_fp8(_ptr(A), _ptr(B), _ptr(raw), form, _stream(stream)))

@@ -182,9 +182,10 @@ DSGX_API int dsgx_widen_fp8(const void* codes, int N, int K, uint16_t* out, size
    (ds41f-4xgx10-switchless/ref/torchref/kernel.py:56-77) */
 DSGX_API int dsgx_act_quant(const uint16_t* x, int T, int K, uint8_t* q, float* s, void* stream);
 
-/* Probe: raw[lane][r], the 64 x 16 accumulator registers of one v_mfma_f32_32x32x64_f8f6f4 over A [32][64] and
-   B [32][64] e4m3 codes (k contiguous), loaded the way the prefill kernels load them (pins the layouts in a test). */
-DSGX_API int dsgx_probe_mfma_fp8(const void* A, const void* B, float* raw, void* stream);
+/* Probe: raw[lane][16], the accumulator registers of one e4m3 MFMA with operands loaded the way the prefill kernels
+   load them (pins the layouts in a test). form 0: v_mfma_f32_32x32x64_f8f6f4 over A [32][64], B [32][64];
+   form 1: v_mfma_f32_16x16x128_f8f6f4 over A [16][128], B [16][128] (four registers a lane). */
+DSGX_API int dsgx_probe_mfma_fp8(const void* A, const void* B, float* raw, int form, void* stream);
 
 /* ---- misc ---------------------------------------------------------------------------------------------------- */
 DSGX_API const char* dsgx_last_error(void);

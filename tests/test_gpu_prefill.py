@@ -27,6 +27,22 @@ def test_mfma_fp8_layout():
     assert np.array_equal(got, D)
 
 
+def test_mfma_fp8_k128_layout():
+    """one 16x16x128 e4m3 MFMA with the prefill kernels' k order, against an exact integer product"""
+    rng = np.random.default_rng(6)
+    vals = np.array([0.0, 1.0, -1.0, 2.0, -2.0, 3.0, 0.5, -4.0], dtype=np.float32)
+    A = vals[rng.integers(0, len(vals), (16, 128))]
+    B = vals[rng.integers(0, len(vals), (16, 128))]
+    raw = gpu.empty(64 * 16 * 4, 0xFF)
+    lib.probe_mfma_fp8(gpu.dev(orc.f32_to_e4m3(A)), gpu.dev(orc.f32_to_e4m3(B)), raw, form=1)
+    raw = gpu.host(raw, np.float32, (64, 16))
+    got = np.empty((16, 16), dtype=np.float64)
+    for l in range(64):
+        for r in range(4):
+            got[4 * (l // 16) + r, l % 16] = raw[l, r]
+    assert np.array_equal(got, A.astype(np.float64) @ B.astype(np.float64).T)
+
+
 def test_mfma_fp8_accuracy():
     """What the e4m3 MFMA's own sums are worth: against exact sums of 64 products, the error stays under 1e-4 of
     sum|terms| on data shaped like quantised activations and weights (the GEMV tolerance of the reference,
