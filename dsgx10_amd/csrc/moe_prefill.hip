@@ -158,10 +158,14 @@ __global__ void __launch_bounds__(256) k_pf_rowsort(const int* __restrict__ idx,
 // acc = fma(x_scale * w_scale, partial, acc) on the vector unit (the accumulators therefore stay in ordinary registers).
 // With the weights as the A operand a lane's four accumulators of a tile belong to ONE position, so the combined scale is
 // one value a lane.
-constexpr int kLdsRow = 144;
-constexpr int kPanel = kTile * kLdsRow;          // bytes of one activation panel (128 rows x 128 k)
-constexpr int kStages = 4, kRing = 4;
-constexpr int kStageBytes = kPanel + kTile * 4;  // + the rows' scales of the block
+#ifndef DSGX_PF_BU
+#define DSGX_PF_BU 1
+#endif
+constexpr int kBU = DSGX_PF_BU;                        // 128-k blocks a unit (the bytes of a row that are loaded together)
+constexpr int kLdsRow = kBU * 128 + 16;
+constexpr int kPanel = kTile * kLdsRow;                // bytes of one activation panel (128 rows x a unit)
+constexpr int kStages = 4, kRing = 4 / kBU;
+constexpr int kStageBytes = kPanel + kBU * kTile * 4;  // + the rows' scales of the unit's blocks
 constexpr int kWgRows = 256;                     // weight rows a workgroup (UP: 128 channels)
 constexpr int kGemmThreads = 512;
 
@@ -221,14 +225,20 @@ __global__ void __launch_bounds__(kGemmThreads) k_pf_gemm(GemmArgs g) {
   const float* swa = sa + (size_t)(n0 / 128) * KB;  // the tiles' scale rows (a wave's 32 rows lie in one 128-row block)
   const float* swb = UP ? sb + (size_t)(n0 / 128) * KB : swa;
 
-  // activation staging: thread t brings chunk t % 8 (16 bytes) of panel rows t / 8 and t / 8 + 64; t < 128 row t's scale
-  const int chunk = tid & 7, srow = tid >> 3;
-  const uint8_t* pb[2];
+  // K is walked in units of kBU blocks (kBU * 128 contiguous bytes of every weight and activation row at a time: memory
+  // rows stay open across a unit's lines). NU units; blocks past KB in the last unit are loaded again and not computed.
+  const int NU = (KB + kBU - 1) / kBU;
+  auto blk = [&](int u, int j) { const int kb = u * kBU + j; return kb < KB ? kb : KB - 1; };
+  // activation staging: a unit's panel is 128 rows x kBU * 128 bytes; thread t brings 16-byte chunk t % (8 kBU) of rows
+  // t / (8 kBU) + (64 / kBU) i, i < 2 kBU; thread t < 128 kBU the scale of row t % 128, block t / 128 of the unit
+  constexpr int kCpr = 8 * kBU, kRowsPerPass = kGemmThreads / kCpr, kPass = kTile / kRowsPerPass;
+  const int chunk = tid % kCpr, srow = tid / kCpr;
+  const uint8_t* pb[kPass];
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
-    int pos = m0 + srow + 64 * i;
+  for (int i = 0; i < kPass; ++i) {
+    int pos = m0 + srow + kRowsPerPass * i;
     if (pos >= mend) pos = mend - 1;  // a ragged tile re-reads its last row (never stored)
-    pb[i] = g.aq + (size_t)(g.gather ? g.gather[pos] : pos) * K + chunk * 16;
+    pb[i] = g.aq + (size_t)(g.gather ? g.gather[pos] : pos) * K;
   }
   const float* pxs;
   {
@@ -243,52 +253,80 @@ __global__ void __launch_bounds__(kGemmThreads) k_pf_gemm(GemmArgs g) {
 #pragma unroll
     for (int mt = 0; mt < 8; ++mt) acc[t][mt] = v4f_t{};
 
-  u32x4_t ra[kRing][2][2];  // the weight ring: block slot, tile, the block's half
-  auto load_a = [&](int slot, int kb) {
-    const int kc = kb < KB ? kb : KB - 1;  // past the end: the last block again (never used)
+  u32x4_t ra[kRing][2][kBU][2];  // the weight ring: unit slot, tile, block of the unit, the block's half
+  auto load_a = [&](int slot, int u) {
+    const int uc = u < NU ? u : NU - 1;  // past the end: the last unit again (never used)
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
-      const uint8_t* p = pin_after(pa[t] + (size_t)kc * 128, acc[t][0][0]);
-      ra[slot][t][0] = ldg_stream(p);
-      ra[slot][t][1] = ldg_stream(p + 64);
+      const uint8_t* p = pin_after(pa[t], acc[t][0][0]);
+#pragma unroll
+      for (int j = 0; j < kBU; ++j) {
+        ra[slot][t][j][0] = ldg_stream(p + (size_t)blk(uc, j) * 128);
+        ra[slot][t][j][1] = ldg_stream(p + (size_t)blk(uc, j) * 128 + 64);
+      }
     }
   };
-  u32x4_t rx[2][2];
-  float rxs[2];
-  auto fetch_x = [&](int set, int kb) {
-    const int kc = kb < KB ? kb : KB - 1;
+  u32x4_t rx[kPass];
+  float rxs;
+  auto fetch_x = [&](int u) {
+    const int uc = u < NU ? u : NU - 1;
+    const int kb = blk(uc, chunk >> 3);
 #pragma unroll
-    for (int i = 0; i < 2; ++i) rx[set][i] = *reinterpret_cast<const u32x4_t*>(pb[i] + (size_t)kc * 128);
-    rxs[set] = pxs[kc];
+    for (int i = 0; i < kPass; ++i) rx[i] = *reinterpret_cast<const u32x4_t*>(pb[i] + (size_t)kb * 128 + (chunk & 7) * 16);
+    rxs = tid < kTile * kBU ? pxs[blk(uc, tid >> 7)] : 0.f;
   };
-  auto stash_x = [&](int set, int stage) {
+  auto stash_x = [&](int stage) {
     uint8_t* B = smem + (size_t)stage * kStageBytes;
 #pragma unroll
-    for (int i = 0; i < 2; ++i) *reinterpret_cast<u32x4_t*>(B + (srow + 64 * i) * kLdsRow + chunk * 16) = rx[set][i];
-    if (tid < kTile) reinterpret_cast<float*>(B + kPanel)[tid] = rxs[set];
+    for (int i = 0; i < kPass; ++i) *reinterpret_cast<u32x4_t*>(B + (srow + kRowsPerPass * i) * kLdsRow + chunk * 16) = rx[i];
+    if (tid < kTile * kBU) reinterpret_cast<float*>(B + kPanel)[tid] = rxs;
   };
-  auto compute = [&](int slot, int stage, int kb) {
+  auto compute = [&](int slot, int stage, int u) {
     const uint8_t* B = smem + (size_t)stage * kStageBytes;
     const float* XS = reinterpret_cast<const float*>(B + kPanel);
-    const float wsa = swa[kb], wsb = swb[kb];
-    v8i_t fa[2];
 #pragma unroll
-    for (int t = 0; t < 2; ++t) {
-      const u32x4_t lo = keep_whole(ra[slot][t][0]), hi = keep_whole(ra[slot][t][1]);
-      fa[t] = v8i_t{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
-    }
-#pragma unroll
-    for (int mt = 0; mt < 8; ++mt) {
-      const uint8_t* bp = B + (size_t)(16 * mt + r16) * kLdsRow + part * 16;
-      const u32x4_t lo = *reinterpret_cast<const u32x4_t*>(bp), hi = *reinterpret_cast<const u32x4_t*>(bp + 64);
-      const v8i_t fb = v8i_t{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
-      const float x = XS[16 * mt + r16];
+    for (int j = 0; j < kBU; ++j) {
+      const int kb = u * kBU + j;
+      if (kb >= KB) break;
+      const float wsa = swa[kb], wsb = swb[kb];
+      v8i_t fa[2];
 #pragma unroll
       for (int t = 0; t < 2; ++t) {
-        const v4f_t p = mfma_fp8_k128(fa[t], fb, v4f_t{});
-        const float sc = __fmul_rn(x, t ? wsb : wsa);
+        const u32x4_t lo = keep_whole(ra[slot][t][j][0]), hi = keep_whole(ra[slot][t][j][1]);
+        fa[t] = v8i_t{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
+      }
+      // the eight 16-position tiles in two halves: four activation fragments in registers, eight independent MFMAs
+      // issued back to back, the next half's fragments read while they run, then the scaled adds
+      v8i_t fb[4];
+      float xv[4];
+      auto read_b = [&](int half) {
 #pragma unroll
-        for (int q = 0; q < 4; ++q) acc[t][mt][q] = fmaf(sc, p[q], acc[t][mt][q]);
+        for (int i = 0; i < 4; ++i) {
+          const uint8_t* bp = B + (size_t)(16 * (4 * half + i) + r16) * kLdsRow + j * 128 + part * 16;
+          const u32x4_t lo = *reinterpret_cast<const u32x4_t*>(bp), hi = *reinterpret_cast<const u32x4_t*>(bp + 64);
+          fb[i] = v8i_t{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
+          xv[i] = XS[j * kTile + 16 * (4 * half + i) + r16];
+        }
+      };
+      read_b(0);
+#pragma unroll
+      for (int half = 0; half < 2; ++half) {
+        v4f_t p[2][4];
+        float sc[2][4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+          for (int t = 0; t < 2; ++t) {
+            p[t][i] = mfma_fp8_k128(fa[t], fb[i], v4f_t{});
+            sc[t][i] = __fmul_rn(xv[i], t ? wsb : wsa);
+          }
+        if (half == 0) read_b(1);
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+          for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) acc[t][4 * half + i][q] = fmaf(sc[t][i], p[t][i][q], acc[t][4 * half + i][q]);
       }
     }
   };
@@ -297,21 +335,20 @@ __global__ void __launch_bounds__(kGemmThreads) k_pf_gemm(GemmArgs g) {
   for (int d = 0; d < kRing; ++d) load_a(d, d);
 #pragma unroll
   for (int s = 0; s < kStages - 1; ++s) {
-    fetch_x(0, s);
-    stash_x(0, s);
+    fetch_x(s);
+    stash_x(s);
   }
-  fetch_x(1, kStages - 1);  // (block 3: written at the end of the first turn)
   __syncthreads();
-  // turn kb: issue the activation loads of block kb + 4, compute block kb, issue the weight loads of block kb + 4 in
-  // its place, put the activations of block kb + 3 (loaded a turn ago) into their stage
-  for (int kb0 = 0; kb0 < KB; kb0 += 4) {
+  // turn u: issue the activation loads of unit u + 3, compute unit u, issue the weight loads of unit u + kRing in its
+  // place, put the activations of unit u + 3 into their stage (last read a turn ago)
+  for (int u0 = 0; u0 < NU; u0 += 4) {
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      const int kb = kb0 + u;
-      fetch_x(u & 1, kb + 4);
-      if (kb < KB) compute(u, u, kb);
-      load_a(u, kb + kRing);
-      stash_x((u + 1) & 1, (u + 3) & 3);
+    for (int v = 0; v < 4; ++v) {
+      const int u = u0 + v;
+      fetch_x(u + 3);
+      if (u < NU) compute(v % kRing, v, u);
+      load_a(v % kRing, u + kRing);
+      stash_x((v + 3) & 3);
       __syncthreads();
     }
   }
