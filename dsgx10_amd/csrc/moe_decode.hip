@@ -8,6 +8,7 @@ using namespace dsgx;
 #ifdef DSGX_TRACE
 static unsigned long long* g_trace_buf = nullptr;  // device memory, [workgroups][16]
 extern "C" __attribute__((visibility("default"))) void dsgx_trace_set(void* dev) { g_trace_buf = static_cast<unsigned long long*>(dev); }
+extern "C" unsigned long long* dsgx_trace_buf() { return g_trace_buf; }
 #endif
 
 extern "C" {

@@ -16,6 +16,9 @@
 #include "abi_internal.h"
 #include "common.cuh"
 
+#ifdef DSGX_TRACE
+extern "C" unsigned long long* dsgx_trace_buf();
+#endif
 namespace dsgx {
 namespace {
 
@@ -152,20 +155,15 @@ __global__ void __launch_bounds__(256) k_pf_rowsort(const int* __restrict__ idx,
 // rows as two 16-row MFMA tiles (UP: 16 gate rows and the 16 up rows of the same channels, so g and u of a channel meet
 // in one lane) and streams them from memory straight into registers, a ring of kRing 128-k blocks ahead: a lane loads
 // 2 x 16 bytes a tile and block, the four lanes of a row 64 contiguous bytes an instruction. The activations of the
-// tile (shared by the eight waves) go through LDS, kStages blocks ahead, rows padded to 144 bytes (the fragment reads of
-// 16 consecutive rows then fall on distinct banks).
+// tile (shared by the eight waves) go through LDS, kStages blocks ahead, stored in the order of the MFMA fragments (the
+// operand reads are then linear in the lane: no bank conflicts).
 // v_mfma_f32_16x16x128_f8f6f4 covers one whole 128-k scale block: partial = A B^T from zero, then
 // acc = fma(x_scale * w_scale, partial, acc) on the vector unit (the accumulators therefore stay in ordinary registers).
 // With the weights as the A operand a lane's four accumulators of a tile belong to ONE position, so the combined scale is
 // one value a lane.
-#ifndef DSGX_PF_BU
-#define DSGX_PF_BU 1
-#endif
-constexpr int kBU = DSGX_PF_BU;                        // 128-k blocks a unit (the bytes of a row that are loaded together)
-constexpr int kLdsRow = kBU * 128 + 16;
-constexpr int kPanel = kTile * kLdsRow;                // bytes of one activation panel (128 rows x a unit)
-constexpr int kStages = 4, kRing = 4 / kBU;
-constexpr int kStageBytes = kPanel + kBU * kTile * 4;  // + the rows' scales of the unit's blocks
+constexpr int kPanel = kTile * 128;              // bytes of one activation panel (128 positions x 128 k)
+constexpr int kStages = 4, kRing = 4;
+constexpr int kStageBytes = kPanel + kTile * 4;  // + the positions' scales of the block
 constexpr int kWgRows = 256;                     // weight rows a workgroup (UP: 128 channels)
 constexpr int kGemmThreads = 512;
 
@@ -181,11 +179,23 @@ struct GemmArgs {
   dsgx_layer_w L;
   uint16_t* h;         // UP: h bf16 [position][I]
   float* d;            // DOWN: f32 [position][H]
+#ifdef DSGX_TRACE
+  unsigned long long* trace;  // diagnostic build: [workgroup][16] time stamps
+#endif
 };
+#ifdef DSGX_TRACE
+#define PF_MARK(k)                                                                                       \
+  do {                                                                                                    \
+    if (g.trace && threadIdx.x == 0 && blockIdx.x < 1024) g.trace[blockIdx.x * 16 + (k)] = wall_clock64(); \
+  } while (0)
+#else
+#define PF_MARK(k) do { } while (0)
+#endif
 
 template <bool UP>
 __global__ void __launch_bounds__(kGemmThreads) k_pf_gemm(GemmArgs g) {
   extern __shared__ uint8_t smem[];
+  PF_MARK(0);
   const int K = UP ? g.L.H : g.L.I, KB = K / 128;
   const int NS = UP ? g.L.I / (kWgRows / 2) : g.L.H / kWgRows;  // workgroups along the weight rows
   const int tile = blockIdx.x / NS, ns = blockIdx.x % NS;
@@ -225,20 +235,15 @@ __global__ void __launch_bounds__(kGemmThreads) k_pf_gemm(GemmArgs g) {
   const float* swa = sa + (size_t)(n0 / 128) * KB;  // the tiles' scale rows (a wave's 32 rows lie in one 128-row block)
   const float* swb = UP ? sb + (size_t)(n0 / 128) * KB : swa;
 
-  // K is walked in units of kBU blocks (kBU * 128 contiguous bytes of every weight and activation row at a time: memory
-  // rows stay open across a unit's lines). NU units; blocks past KB in the last unit are loaded again and not computed.
-  const int NU = (KB + kBU - 1) / kBU;
-  auto blk = [&](int u, int j) { const int kb = u * kBU + j; return kb < KB ? kb : KB - 1; };
-  // activation staging: a unit's panel is 128 rows x kBU * 128 bytes; thread t brings 16-byte chunk t % (8 kBU) of rows
-  // t / (8 kBU) + (64 / kBU) i, i < 2 kBU; thread t < 128 kBU the scale of row t % 128, block t / 128 of the unit
-  constexpr int kCpr = 8 * kBU, kRowsPerPass = kGemmThreads / kCpr, kPass = kTile / kRowsPerPass;
-  const int chunk = tid % kCpr, srow = tid / kCpr;
-  const uint8_t* pb[kPass];
-#pragma unroll
-  for (int i = 0; i < kPass; ++i) {
-    int pos = m0 + srow + kRowsPerPass * i;
+  // activation staging: wave w brings the 16 positions 16 w ... of the panel, the lane its MFMA fragment's two 16-byte
+  // pieces (row lane % 16, bytes 16 (lane / 16) of each 64-byte half); in LDS a panel is stored in fragment order,
+  // piece (tile mt, half h, lane) at 16 ((2 mt + h) 64 + lane): the MFMA operand reads are linear in the lane (no
+  // bank conflicts), and so are these writes. Thread t < 128 also brings the scale of position t.
+  const uint8_t* pb;
+  {
+    int pos = m0 + 16 * wave + r16;
     if (pos >= mend) pos = mend - 1;  // a ragged tile re-reads its last row (never stored)
-    pb[i] = g.aq + (size_t)(g.gather ? g.gather[pos] : pos) * K;
+    pb = g.aq + (size_t)(g.gather ? g.gather[pos] : pos) * K + part * 16;
   }
   const float* pxs;
   {
@@ -247,111 +252,110 @@ __global__ void __launch_bounds__(kGemmThreads) k_pf_gemm(GemmArgs g) {
     pxs = g.as + (size_t)(g.gather ? g.gather[pos] : pos) * KB;
   }
 
+  auto blk = [&](int kb) { return kb < KB ? kb : KB - 1; };  // (past the end: the last block again, never used)
   v4f_t acc[2][8];
 #pragma unroll
   for (int t = 0; t < 2; ++t)
 #pragma unroll
     for (int mt = 0; mt < 8; ++mt) acc[t][mt] = v4f_t{};
 
-  u32x4_t ra[kRing][2][kBU][2];  // the weight ring: unit slot, tile, block of the unit, the block's half
-  auto load_a = [&](int slot, int u) {
-    const int uc = u < NU ? u : NU - 1;  // past the end: the last unit again (never used)
+  u32x4_t ra[kRing][2][2];  // the weight ring: block slot, tile, the block's half
+  auto load_a = [&](int slot, int kb) {
+    const int kc = blk(kb);
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
-      const uint8_t* p = pin_after(pa[t], acc[t][0][0]);
-#pragma unroll
-      for (int j = 0; j < kBU; ++j) {
-        ra[slot][t][j][0] = ldg_stream(p + (size_t)blk(uc, j) * 128);
-        ra[slot][t][j][1] = ldg_stream(p + (size_t)blk(uc, j) * 128 + 64);
-      }
+      const uint8_t* p = pin_after(pa[t] + (size_t)kc * 128, acc[t][0][0]);
+      // (ordinary loads, not streaming ones: the other tiles of the same expert read the same lines from L2)
+      ra[slot][t][0] = *reinterpret_cast<const DSGX_GLOBAL u32x4_t*>((uintptr_t)p);
+      ra[slot][t][1] = *reinterpret_cast<const DSGX_GLOBAL u32x4_t*>((uintptr_t)(p + 64));
     }
   };
-  u32x4_t rx[kPass];
-  float rxs;
-  auto fetch_x = [&](int u) {
-    const int uc = u < NU ? u : NU - 1;
-    const int kb = blk(uc, chunk >> 3);
-#pragma unroll
-    for (int i = 0; i < kPass; ++i) rx[i] = *reinterpret_cast<const u32x4_t*>(pb[i] + (size_t)kb * 128 + (chunk & 7) * 16);
-    rxs = tid < kTile * kBU ? pxs[blk(uc, tid >> 7)] : 0.f;
+  struct XRegs {
+    u32x4_t v[2];
+    float s;
   };
-  auto stash_x = [&](int stage) {
+  auto fetch_x = [&](XRegs& r, int kb) {
+    const int kc = blk(kb);
+    r.v[0] = *reinterpret_cast<const u32x4_t*>(pb + (size_t)kc * 128);
+    r.v[1] = *reinterpret_cast<const u32x4_t*>(pb + (size_t)kc * 128 + 64);
+    r.s = pxs[kc];
+  };
+  auto stash_x = [&](const XRegs& r, int stage) {
     uint8_t* B = smem + (size_t)stage * kStageBytes;
-#pragma unroll
-    for (int i = 0; i < kPass; ++i) *reinterpret_cast<u32x4_t*>(B + (srow + kRowsPerPass * i) * kLdsRow + chunk * 16) = rx[i];
-    if (tid < kTile * kBU) reinterpret_cast<float*>(B + kPanel)[tid] = rxs;
+    *reinterpret_cast<u32x4_t*>(B + ((2 * wave + 0) * 64 + lane) * 16) = r.v[0];
+    *reinterpret_cast<u32x4_t*>(B + ((2 * wave + 1) * 64 + lane) * 16) = r.v[1];
+    if (tid < kTile) reinterpret_cast<float*>(B + kPanel)[tid] = r.s;
   };
-  auto compute = [&](int slot, int stage, int u) {
+  auto compute = [&](int slot, int stage, int kb) {
     const uint8_t* B = smem + (size_t)stage * kStageBytes;
     const float* XS = reinterpret_cast<const float*>(B + kPanel);
+    const float wsa = swa[kb], wsb = swb[kb];
+    v8i_t fa[2];
 #pragma unroll
-    for (int j = 0; j < kBU; ++j) {
-      const int kb = u * kBU + j;
-      if (kb >= KB) break;
-      const float wsa = swa[kb], wsb = swb[kb];
-      v8i_t fa[2];
+    for (int t = 0; t < 2; ++t) {
+      const u32x4_t lo = keep_whole(ra[slot][t][0]), hi = keep_whole(ra[slot][t][1]);
+      fa[t] = v8i_t{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
+    }
+    // the eight 16-position tiles in two halves: four activation fragments in registers, eight independent MFMAs
+    // issued back to back, the next half's fragments read while they run, then the scaled adds
+    v8i_t fb[4];
+    float xv[4];
+    auto read_b = [&](int half) {
 #pragma unroll
-      for (int t = 0; t < 2; ++t) {
-        const u32x4_t lo = keep_whole(ra[slot][t][j][0]), hi = keep_whole(ra[slot][t][j][1]);
-        fa[t] = v8i_t{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
+      for (int i = 0; i < 4; ++i) {
+        const int mt = 4 * half + i;
+        const u32x4_t lo = *reinterpret_cast<const u32x4_t*>(B + ((2 * mt + 0) * 64 + lane) * 16);
+        const u32x4_t hi = *reinterpret_cast<const u32x4_t*>(B + ((2 * mt + 1) * 64 + lane) * 16);
+        fb[i] = v8i_t{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
+        xv[i] = XS[16 * mt + r16];
       }
-      // the eight 16-position tiles in two halves: four activation fragments in registers, eight independent MFMAs
-      // issued back to back, the next half's fragments read while they run, then the scaled adds
-      v8i_t fb[4];
-      float xv[4];
-      auto read_b = [&](int half) {
+    };
+    read_b(0);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const uint8_t* bp = B + (size_t)(16 * (4 * half + i) + r16) * kLdsRow + j * 128 + part * 16;
-          const u32x4_t lo = *reinterpret_cast<const u32x4_t*>(bp), hi = *reinterpret_cast<const u32x4_t*>(bp + 64);
-          fb[i] = v8i_t{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
-          xv[i] = XS[j * kTile + 16 * (4 * half + i) + r16];
+    for (int half = 0; half < 2; ++half) {
+      v4f_t p[2][4];
+      float sc[2][4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+          p[t][i] = mfma_fp8_k128(fa[t], fb[i], v4f_t{});
+          sc[t][i] = __fmul_rn(xv[i], t ? wsb : wsa);
         }
-      };
-      read_b(0);
+      if (half == 0) read_b(1);
 #pragma unroll
-      for (int half = 0; half < 2; ++half) {
-        v4f_t p[2][4];
-        float sc[2][4];
+      for (int i = 0; i < 4; ++i)
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
+        for (int t = 0; t < 2; ++t)
 #pragma unroll
-          for (int t = 0; t < 2; ++t) {
-            p[t][i] = mfma_fp8_k128(fa[t], fb[i], v4f_t{});
-            sc[t][i] = __fmul_rn(xv[i], t ? wsb : wsa);
-          }
-        if (half == 0) read_b(1);
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-#pragma unroll
-          for (int t = 0; t < 2; ++t)
-#pragma unroll
-            for (int q = 0; q < 4; ++q) acc[t][4 * half + i][q] = fmaf(sc[t][i], p[t][i][q], acc[t][4 * half + i][q]);
-      }
+          for (int q = 0; q < 4; ++q) acc[t][4 * half + i][q] = fmaf(sc[t][i], p[t][i][q], acc[t][4 * half + i][q]);
     }
   };
+  PF_MARK(1);
   // prologue: the weight ring, the first activation panels
 #pragma unroll
   for (int d = 0; d < kRing; ++d) load_a(d, d);
-#pragma unroll
-  for (int s = 0; s < kStages - 1; ++s) {
-    fetch_x(s);
-    stash_x(s);
-  }
+  XRegs rx, rx1, rx2;
+  fetch_x(rx, 0), fetch_x(rx1, 1), fetch_x(rx2, 2);
+  stash_x(rx, 0), stash_x(rx1, 1), stash_x(rx2, 2);
   __syncthreads();
-  // turn u: issue the activation loads of unit u + 3, compute unit u, issue the weight loads of unit u + kRing in its
-  // place, put the activations of unit u + 3 into their stage (last read a turn ago)
-  for (int u0 = 0; u0 < NU; u0 += 4) {
+  PF_MARK(2);
+  // turn kb: issue the activation loads of block kb + 3, compute block kb, issue the weight loads of block kb + kRing
+  // in its place, put the activations of block kb + 3 into their stage (last read a turn ago)
+  for (int kb0 = 0; kb0 < KB; kb0 += 4) {
 #pragma unroll
     for (int v = 0; v < 4; ++v) {
-      const int u = u0 + v;
-      fetch_x(u + 3);
-      if (u < NU) compute(v % kRing, v, u);
-      load_a(v % kRing, u + kRing);
-      stash_x((v + 3) & 3);
+      const int kb = kb0 + v;
+      fetch_x(rx, kb + 3);
+      if (kb < KB) compute(v, v, kb);
+      load_a(v, kb + kRing);
+      stash_x(rx, (v + 3) & 3);
       __syncthreads();
     }
+    if (kb0 == 0) PF_MARK(3);
+    if (kb0 == 12) PF_MARK(4);
   }
+  PF_MARK(5);
 
   // epilogue: register q of lane l is weight row 4 (l / 16) + q of the 16-row tile, position l % 16 of the 16 positions
   if (UP) {
@@ -377,6 +381,7 @@ __global__ void __launch_bounds__(kGemmThreads) k_pf_gemm(GemmArgs g) {
         *reinterpret_cast<float4*>(g.d + (size_t)pos * H + n0 + 16 * t + 4 * part) = make_float4(acc[t][mt][0], acc[t][mt][1], acc[t][mt][2], acc[t][mt][3]);
     }
   }
+  PF_MARK(6);
 }
 
 // yr[t][n] over the row's picks in expert-id order: acc = fma(s2 * w, d, acc); four columns a thread
@@ -470,6 +475,9 @@ int dsgx_moe_prefill(const dsgx_layer_w* L, const uint16_t* x, const int* idx, c
   }
   GemmArgs g{};
   g.L = *L;
+#ifdef DSGX_TRACE
+  g.trace = dsgx_trace_buf();
+#endif
   if (cfg.phases & (2 | 16)) {
     if (int rc = dsgx_act_quant(x, T, H, W + o.xq, F32(o.xs), stream)) return rc;
   }
