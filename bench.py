@@ -32,6 +32,23 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
+def prefill_extra(gen, T=8192):
+    """the prefill chunk of the benchmark: T rows, top-8 of 256 experts drawn from a Zipf(1.1) popularity, FP8 weights and
+    activations; TFLOP/s over the useful multiply-adds of the routed experts (T * 8 * 3 * I * H * 2)"""
+    from dsgx10_amd.benchdata import PrefillBench
+    pb = PrefillBench(gen, T)
+    t_routed, t_all = pb.time(15, False), pb.time(31, True)
+    d = dict(workload="fp8_moe_prefill", T=T, zipf_s=1.1, ms_routed=t_routed * 1e3, ms_with_shared=t_all * 1e3,
+             tflops_routed=pb.flops_routed / t_routed / 1e12, tflops_with_shared=(pb.flops_routed + pb.flops_shared) / t_all / 1e12,
+             mfma_frac_of_5PFs=pb.flops_routed / t_routed / 5.0e15,
+             phases_ms={n: pb.time(ph, sh) * 1e3 for n, ph, sh in (("bucket", 1, False), ("up", 2, False), ("down", 4, False),
+                                                                      ("combine", 8, False), ("shared", 16, True))})
+    log("  fp8_moe_prefill T=%d: routed %.3f ms (%.0f TFLOP/s, %.1f%% of 5 PFLOP/s), with shared %.3f ms" %
+        (T, d["ms_routed"], d["tflops_routed"], 100 * d["mfma_frac_of_5PFs"], d["ms_with_shared"]))
+    del pb
+    return d
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -109,6 +126,8 @@ def main():
             extra.append(dict(workload=gen.name, M=M, us_per_layer=e["us_per_layer"], bytes=e["bytes_per_layer"],
                               hbm_frac=e["layer_hbm_frac"], up_kernel_us=e["up_us"], up_hbm_frac=e["up_frac"]))
         del b
+        if head_fp8:
+            extra.append(prefill_extra(gen))
         other = Int4LayerGen(seed=0) if head_fp8 else Fp8LayerGen(seed=0)
         for M in (1, 8):
             ob, e = run_decode(other, M, ks if M > 1 else K, min(W, 16))
@@ -133,9 +152,9 @@ def main():
         "higher_is_better": False,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "f32 accumulate over e4m3 weights x bf16 activations" if head_fp8 else "f32 accumulate over int4-g32 weights x bf16 activations",
+        "dtype": "f32",
         "data": "synthetic (torch-seeded N(0,0.02) weights quantised on the GPU, N(0,1) bf16 rows and f32 logits)",
-        "config": {"workload": gen.describe(1), "rows_M": 1, "steps_route_different_experts": True,
+        "config": {"workload": gen.describe(1), "arithmetic": "f32 sums of bf16 x bf16 products (weights decoded to bf16 in registers)", "rows_M": 1, "steps_route_different_experts": True,
                    "bytes_per_layer": r["bytes_per_layer"], "layer_hbm_frac_of_8TBs": r["layer_hbm_frac"],
                    "kernels_per_step": ["k_decode (routing + gate/up + SwiGLU + down + weighted sum, one persistent launch)"], "timed_as": "one HIP graph of all steps, one replay"},
         "roofline": {"bound": "hbm", "kernel": "k_up (gate/up + SwiGLU)", "achieved": r["up_gbs"], "peak": HBM_PEAK_GBS,

@@ -45,12 +45,23 @@ __device__ __forceinline__ void fp8x8_to_bf16(uint32_t w0, uint32_t w1, uint32_t
 // nzs = -(u_z * s). W = bf16_rne((u - u_z) * s): u * s and u_z * s are exact in f32 (4 x 8 significant bits), so
 // fma(u, s, nzs) is the exact product (u - u_z) * s, and the packed conversion rounds it once to nearest even.
 // (Exact while u_z * s stays finite, i.e. |s| < 2^124; dequant_int4's own kernel uses the subtract-first form.)
+// byte k of a word as a float, in one instruction (written as shifts and masks the compiler turns the masked nibbles
+// back into a bit-field extract followed by a conversion: two instructions a value)
+template <int K>
+__device__ __forceinline__ float ubyte_to_f32(uint32_t w) {
+  float f;
+  if (K == 0) asm("v_cvt_f32_ubyte0 %0, %1" : "=v"(f) : "v"(w));
+  else if (K == 1) asm("v_cvt_f32_ubyte1 %0, %1" : "=v"(f) : "v"(w));
+  else if (K == 2) asm("v_cvt_f32_ubyte2 %0, %1" : "=v"(f) : "v"(w));
+  else asm("v_cvt_f32_ubyte3 %0, %1" : "=v"(f) : "v"(w));
+  return f;
+}
 __device__ __forceinline__ void i4x8_to_bf16(uint32_t w, float s, float nzs, uint32_t (&o)[4]) {
   const uint32_t lo = w & 0x0F0F0F0Fu, hi = (w >> 4) & 0x0F0F0F0Fu;  // lo: values 0,2,4,6; hi: 1,3,5,7
-  o[0] = pack_bf16(fmaf((float)(lo & 0xFFu), s, nzs), fmaf((float)(hi & 0xFFu), s, nzs));
-  o[1] = pack_bf16(fmaf((float)((lo >> 8) & 0xFFu), s, nzs), fmaf((float)((hi >> 8) & 0xFFu), s, nzs));
-  o[2] = pack_bf16(fmaf((float)((lo >> 16) & 0xFFu), s, nzs), fmaf((float)((hi >> 16) & 0xFFu), s, nzs));
-  o[3] = pack_bf16(fmaf((float)(lo >> 24), s, nzs), fmaf((float)(hi >> 24), s, nzs));
+  o[0] = pack_bf16(fmaf(ubyte_to_f32<0>(lo), s, nzs), fmaf(ubyte_to_f32<0>(hi), s, nzs));
+  o[1] = pack_bf16(fmaf(ubyte_to_f32<1>(lo), s, nzs), fmaf(ubyte_to_f32<1>(hi), s, nzs));
+  o[2] = pack_bf16(fmaf(ubyte_to_f32<2>(lo), s, nzs), fmaf(ubyte_to_f32<2>(hi), s, nzs));
+  o[3] = pack_bf16(fmaf(ubyte_to_f32<3>(lo), s, nzs), fmaf(ubyte_to_f32<3>(hi), s, nzs));
 }
 // the contract in its subtract-first form, exact for every finite scale: bf16_rne(float(u - u_z) * s)
 __device__ __forceinline__ uint32_t i4_value_bits(int u, int uz, uint32_t sbits) {

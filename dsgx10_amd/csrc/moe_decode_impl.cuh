@@ -392,11 +392,11 @@ __device__ __forceinline__ void up_phase(const DecodeArgs& a, uint4* xs, Step<M>
 }
 
 // ---- down ------------------------------------------------------------------------------------------------------------------
-// The wave's rows [n_lo, n_hi) in sub-batches of RB; per sub-batch every slot in order. hs: LDS for `spc` slots' h.
+// The wave's rows [n_lo, n_hi) in sub-batches of RB (2, or 3 where the rows divide so: the launch picks); per sub-batch
+// every slot in order. hs: LDS for `spc` slots' h.
 // `between` runs after the first loads are issued and before any h is read (the fused kernel's grid barrier).
-template <int FMT, int SHFMT, int M, int D, class Between>
+template <int FMT, int SHFMT, int M, int D, int RB, class Between>
 __device__ __forceinline__ void down_phase(const DecodeArgs& a, uint4* hs, Step<M>& S, int spc, int n_lo, int n_hi, Between&& between) {
-  constexpr int RB = 2;
   constexpr bool kMixed = SHFMT != 0 && SHFMT != FMT;
   constexpr int SF = SHFMT == 0 ? FMT : SHFMT;  // the shared slot's format
   const int H = a.L.H, I = a.L.I;
@@ -595,7 +595,7 @@ __device__ __forceinline__ void grid_barrier(int* bar, int my_gen, int spin_limi
 }
 
 // ---- kernels ----------------------------------------------------------------------------------------------------------------
-template <int FMT, int SHFMT, int M>
+template <int FMT, int SHFMT, int M, int RBD>
 __global__ void __launch_bounds__(DSGX_DECODE_THREADS) k_decode(DecodeArgs a, int shared_wgs, int spc) {
   extern __shared__ uint4 lds[];
   __shared__ Step<M> S;
@@ -606,7 +606,7 @@ __global__ void __launch_bounds__(DSGX_DECODE_THREADS) k_decode(DecodeArgs a, in
   const int H = a.L.H, GW = gridDim.x * (blockDim.x >> 6), gw = uni((int)(blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)));
   const int rpw = uni((H + GW - 1) / GW);
   const int n_lo = min(H, gw * rpw), n_hi = min(H, n_lo + rpw);
-  down_phase<FMT, SHFMT, M, DSGX_DOWND>(a, lds, S, spc, n_lo, n_hi, [&] { DSGX_MARK(5); grid_barrier(a.bar, S.gen, a.spin_limit); DSGX_MARK(6); });
+  down_phase<FMT, SHFMT, M, DSGX_DOWND, RBD>(a, lds, S, spc, n_lo, n_hi, [&] { DSGX_MARK(5); grid_barrier(a.bar, S.gen, a.spin_limit); DSGX_MARK(6); });
   DSGX_MARK(8);
 }
 template <int FMT, int SHFMT, int M>
@@ -631,7 +631,7 @@ __global__ void __launch_bounds__(256) k_down(DecodeArgs a, int spc) {
   }
   const int H = a.L.H, gw = uni((int)(blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)));
   const int n_lo = min(H, gw * 2), n_hi = min(H, n_lo + 2);
-  down_phase<FMT, SHFMT, M, 4>(a, lds, S, spc, n_lo, n_hi, [] {});
+  down_phase<FMT, SHFMT, M, 4, 2>(a, lds, S, spc, n_lo, n_hi, [] {});
 }
 
 // ---- launches ---------------------------------------------------------------------------------------------------------------
@@ -650,13 +650,18 @@ int launch_decode(const DecodeArgs& a, int parts, hipStream_t st) {
   auto slots_per_chunk = [&](size_t lds_bytes) { return std::min(std::max(1, (int)(lds_bytes / slot_bytes)), nsl_max); };
   auto shared_split = [&](int grid) {
     if (!kMixed) return 0;
-    // the workgroups split between the BF16 shared expert and the routed experts by their bytes
-    const double bsh = 2.0 * I * H * 2, bro = (double)std::min(a.M * a.L.topk, a.L.E) * 2.0 * (double)dsgx_mat_bytes(FMT, I, H);
+    // the workgroups split between the BF16 shared expert and the routed experts by their bytes, an INT4 byte counted
+    // as 2.2 BF16 bytes (it holds four times the values, and the gate/up phase is bound by their decoding)
+    const double bsh = 2.0 * I * H * 2, bro = 2.2 * (double)std::min(a.M * a.L.topk, a.L.E) * 2.0 * (double)dsgx_mat_bytes(FMT, I, H);
     return std::max(1, std::min(grid - 1, (int)(grid * bsh / (bsh + bro) + 0.5)));
   };
   (void)SF;
   if (parts == 3) {
-    auto kern = k_decode<FMT, SHFMT, M>;
+    // rows a wave in the down phase: sub-batches of three where that divides them evenly (built for the INT4 layers,
+    // whose hidden size 6144 gives three rows a wave on 256 CUs), else of two
+    const int rpw = (H + cus * (DSGX_DECODE_THREADS / 64) - 1) / (cus * (DSGX_DECODE_THREADS / 64));
+    const bool rb3 = FMT == DSGX_FMT_INT4_G32 && rpw % 3 == 0;
+    auto kern = rb3 ? k_decode<FMT, SHFMT, M, (FMT == DSGX_FMT_INT4_G32 ? 3 : 2)> : k_decode<FMT, SHFMT, M, 2>;
     const int spc = slots_per_chunk(DSGX_WGS == 1 ? 96 * 1024 : 40 * 1024);
     const size_t lds = std::max(lds_up, (size_t)spc * slot_bytes);
     if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds)) return rc;
