@@ -32,6 +32,12 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
+# HBM bytes a launch of the FP8 M=1 gate/up kernel, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs of this script,
+# each scaled by what the counter reads for a kernel of known size in the same run (profiles/): 152,215,347 read +
+# 6,553,600 written (algorithmic bytes: 151,031,808)
+UP_TRAFFIC_FP8_M1 = 158768947
+
+
 def prefill_extra(gen, T=8192):
     """the prefill chunk of the benchmark: T rows, top-8 of 256 experts drawn from a Zipf(1.1) popularity, FP8 weights and
     activations; TFLOP/s over the useful multiply-adds of the routed experts (T * 8 * 3 * I * H * 2)"""
@@ -158,7 +164,7 @@ def main():
                    "bytes_per_layer": r["bytes_per_layer"], "layer_hbm_frac_of_8TBs": r["layer_hbm_frac"],
                    "kernels_per_step": ["k_decode (routing + gate/up + SwiGLU + down + weighted sum, one persistent launch)"], "timed_as": "one HIP graph of all steps, one replay"},
         "roofline": {"bound": "hbm", "kernel": "k_up (gate/up + SwiGLU)", "achieved": r["up_gbs"], "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": r["up_frac"], "traffic": None, "bytes_per_launch": r["up_bytes"],
+                     "unit": "GB/s", "frac": r["up_frac"], "traffic": UP_TRAFFIC_FP8_M1 if head_fp8 else None, "bytes_per_launch": r["up_bytes"],
                      "avg_launch_us": r["up_us"], "measured_stream_read_gbs": stream_gbs},
         "cpu_baseline": cpu,
         "extra": extra,

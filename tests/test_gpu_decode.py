@@ -59,7 +59,7 @@ CASES = [
     (abi.FMT_INT4, 4096, 2048, 168, 8, 3, None, 2.5),
     (abi.FMT_BF16, 1024, 512, 16, 4, 4, None, 2.5),
     # the benchmark's hidden size: three output rows a wave on a 256-CU device, the down phase's sub-batches of three
-    (abi.FMT_INT4, 6144, 256, 16, 4, 3, "bf16", 2.5),
+    (abi.FMT_INT4, 6144, 2048, 16, 4, 2, "bf16", 2.5),
 ]
 
 
