@@ -384,6 +384,210 @@ __global__ void __launch_bounds__(kGemmThreads) k_pf_gemm(GemmArgs g) {
   PF_MARK(6);
 }
 
+// ---- the grouped GEMM with bf16 activations (INT4 layers, and their BF16 shared expert) -----------------------------
+// The same streaming structure for the altar-1 contract (engine/experts/prefill.cu:337-352, 772-831): activations stay
+// bf16, a weight is the bf16 value W = bf16((u - u_z) s) (INT4; decoded in registers by the decode kernels' routine) or
+// the stored bf16 (the shared expert), products are summed in f32 by v_mfma_f32_16x16x32_bf16, whose accumulators the
+// MFMA itself carries across K (no per-block scale here: the scales are inside W).
+// A 128-k block is four MFMAs (j = 0..3) a 16-row tile. INT4: a lane's 16 bytes are the 32 values of ONE scale group:
+// lane (row, part) holds k = 32 part + 8 j + [0, 8) for MFMA j (four lanes a row: 64 contiguous bytes an instruction),
+// one scale and one zero-point word a lane and block. BF16: k = 32 j + 8 part + [0, 8), one 16-byte load an MFMA.
+// The activation panel in LDS is in fragment order for the same k map: piece (tile mt, j, lane) at 16 ((4 mt + j) 64 + lane).
+typedef __bf16 v8bf_t __attribute__((ext_vector_type(8)));
+constexpr int kPanel16 = kTile * 256;  // bytes of one bf16 activation panel (128 positions x 128 k)
+constexpr int kStages16 = 3;
+
+struct Gemm16Args {
+  const uint16_t* x;   // activations bf16 [rows][K]
+  const int* gather;   // position -> activation row (null: the position itself)
+  const int* tile_e;   // (null: the shared expert on rows [0, nrows))
+  const int* tile_m0;
+  const int* ntiles;
+  const int* off;
+  int nrows;
+  dsgx_layer_w L;
+  uint16_t* h;         // UP: h bf16 [position][I]
+  float* d;            // DOWN: f32 [position][H]
+};
+
+// WF: the weights' format (DSGX_FMT_INT4_G32: the routed experts; DSGX_FMT_BF16: the shared expert, gate/up interleaved)
+template <bool UP, int WF>
+__global__ void __launch_bounds__(kGemmThreads) k_pf_gemm16(Gemm16Args g) {
+  extern __shared__ uint8_t smem[];
+  constexpr bool I4 = WF == DSGX_FMT_INT4_G32;
+  const int K = UP ? g.L.H : g.L.I, N = UP ? g.L.I : g.L.H, KB = K / 128;
+  const int NS = UP ? g.L.I / (kWgRows / 2) : g.L.H / kWgRows;
+  const int tile = blockIdx.x / NS, ns = blockIdx.x % NS;
+  int e = -1, m0 = tile * kTile, mend = g.nrows;
+  if (g.tile_e) {
+    if (tile >= *g.ntiles) return;
+    e = g.tile_e[tile];
+    const int o = g.off[e];
+    m0 = o + g.tile_m0[tile], mend = g.off[e + 1];
+  } else if (m0 >= mend) {
+    return;
+  }
+  const int tid = threadIdx.x, lane = tid & 63, wave = uni(tid >> 6), r16 = lane & 15, part = lane >> 4;
+  const int n0 = UP ? ns * (kWgRows / 2) + 16 * wave : ns * kWgRows + 32 * wave;  // UP: first channel; DOWN: first row
+  // the lane's weight row of each of the wave's two tiles
+  const uint8_t* pw[2];
+  const uint8_t* ps[2] = {nullptr, nullptr};
+  const uint8_t* pz[2] = {nullptr, nullptr};
+  uint32_t zsh[2] = {0, 0};
+  float s2a = 1.f, s2b = 1.f;
+  if (I4) {
+    const dsgx_mat_desc* d = g.L.desc + (size_t)e * 3;
+    const int G = K / 32;
+    const size_t soff = ((size_t)N * K / 2 + 255) / 256 * 256, zoff = soff + ((size_t)N * G * 2 + 255) / 256 * 256;
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      const uint8_t* base = g.L.pool + d[UP ? t : 2].off;
+      const int n = UP ? n0 + r16 : n0 + 16 * t + r16;
+      pw[t] = base + (size_t)n * (K / 2) + part * 16;
+      ps[t] = base + soff + ((size_t)n * G + part) * 2;
+      pz[t] = base + zoff + ((size_t)(n >> 3) * G + part) * 4;
+      zsh[t] = 4 * (n & 7);
+    }
+    if (UP) s2a = d[0].s2, s2b = d[1].s2;
+  } else {
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      // shared expert: gate row c is row 2 c of bgu, up row c is row 2 c + 1; down rows plain
+      const size_t row = UP ? 2 * (size_t)(n0 + r16) + t : (size_t)(n0 + 16 * t + r16);
+      pw[t] = reinterpret_cast<const uint8_t*>(UP ? g.L.sh.bgu : g.L.sh.bd) + row * K * 2 + part * 16;
+    }
+  }
+  // activation staging: wave w brings the 16 positions 16 w ..., the lane the four 16-byte pieces of its fragments
+  const uint8_t* px;
+  {
+    int pos = m0 + 16 * wave + r16;
+    if (pos >= mend) pos = mend - 1;
+    px = reinterpret_cast<const uint8_t*>(g.x) + (size_t)(g.gather ? g.gather[pos] : pos) * K * 2;
+  }
+  // byte offset in a 128-k block of the 8 values of MFMA j in lane part p (bf16 activations; and BF16 weights)
+  auto koff = [&](int j) { return I4 ? (32 * part + 8 * j) * 2 : (32 * j + 8 * part) * 2; };
+
+  v4f_t acc[2][8];
+#pragma unroll
+  for (int t = 0; t < 2; ++t)
+#pragma unroll
+    for (int mt = 0; mt < 8; ++mt) acc[t][mt] = v4f_t{};
+
+  constexpr int kRing16 = I4 ? 3 : 2;
+  struct WRegs {
+    u32x4_t v[I4 ? 1 : 4];
+    uint32_t s, z;
+  };
+  WRegs ra[kRing16][2];
+  auto load_a = [&](int slot, int kb) {
+    const int kc = kb < KB ? kb : KB - 1;
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      if (I4) {
+        const uint8_t* p = pin_after(pw[t] + (size_t)kc * 64, acc[t][0][0]);
+        ra[slot][t].v[0] = ldg_stream(p);
+        ra[slot][t].s = ldg_u16(ps[t] + (size_t)kc * 8);
+        ra[slot][t].z = ldg_u32(pz[t] + (size_t)kc * 16);
+      } else {
+        const uint8_t* p = pin_after(pw[t] + (size_t)kc * 256, acc[t][0][0]);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) ra[slot][t].v[j] = ldg_stream(p + 64 * j);
+      }
+    }
+  };
+  u32x4_t rx[4];
+  auto fetch_x = [&](int kb) {
+    const int kc = kb < KB ? kb : KB - 1;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) rx[j] = *reinterpret_cast<const u32x4_t*>(px + (size_t)kc * 256 + koff(j));
+  };
+  auto stash_x = [&](int stage) {
+    uint8_t* B = smem + (size_t)stage * kPanel16;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) *reinterpret_cast<u32x4_t*>(B + ((4 * wave + j) * 64 + lane) * 16) = rx[j];
+  };
+  auto compute = [&](int slot, int stage) {
+    const uint8_t* B = smem + (size_t)stage * kPanel16;
+    // the wave's two A tiles of the block as bf16 fragments
+    u32x4_t fa[2][4];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      if (I4) {
+        const float sc = bf16_bits_to_f32(ra[slot][t].s);
+        const float nzs = -((float)((ra[slot][t].z >> zsh[t]) & 15u) * sc);
+        const u32x4_t w = keep_whole(ra[slot][t].v[0]);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          uint32_t o[4];
+          i4x8_to_bf16(j == 0 ? w.x : j == 1 ? w.y : j == 2 ? w.z : w.w, sc, nzs, o);
+          fa[t][j] = u32x4_t{o[0], o[1], o[2], o[3]};
+        }
+      } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) fa[t][j] = keep_whole(ra[slot][t].v[j]);
+      }
+    }
+#pragma unroll
+    for (int mt = 0; mt < 8; ++mt) {
+      u32x4_t fb[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) fb[j] = *reinterpret_cast<const u32x4_t*>(B + ((4 * mt + j) * 64 + lane) * 16);
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+          acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf_t, fa[t][j]), __builtin_bit_cast(v8bf_t, fb[j]),
+                                                               acc[t][mt], 0, 0, 0);
+    }
+  };
+  // prologue
+#pragma unroll
+  for (int d = 0; d < kRing16; ++d) load_a(d, d);
+  fetch_x(0);
+  stash_x(0);
+  fetch_x(1);
+  stash_x(1);
+  __syncthreads();
+  // turn kb: issue the activation loads of block kb + 2, compute block kb, issue the weight loads of block kb + ring in
+  // its place, put the activations of block kb + 2 into their stage (last read a turn ago)
+  constexpr int kUnroll = kRing16 * kStages16 / (kRing16 == kStages16 ? kRing16 : 1);  // a common multiple of both
+  for (int kb0 = 0; kb0 < KB; kb0 += kUnroll) {
+#pragma unroll
+    for (int v = 0; v < kUnroll; ++v) {
+      const int kb = kb0 + v;
+      fetch_x(kb + 2);
+      if (kb < KB) compute(v % kRing16, v % kStages16);
+      load_a(v % kRing16, kb + kRing16);
+      stash_x((v + 2) % kStages16);
+      __syncthreads();
+    }
+  }
+  // epilogue: register q of lane l is weight row 4 (l / 16) + q of the 16-row tile, position l % 16 of the 16 positions
+  if (UP) {
+    const int I = g.L.I;
+#pragma unroll
+    for (int mt = 0; mt < 8; ++mt) {
+      const int pos = m0 + 16 * mt + r16;
+      if (pos >= mend) continue;
+      uint32_t hb[4];
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+        hb[q] = swiglu_bits(bf16_round(__fmul_rn(acc[0][mt][q], s2a)), bf16_round(__fmul_rn(acc[1][mt][q], s2b)));
+      *reinterpret_cast<uint2*>(g.h + (size_t)pos * I + n0 + 4 * part) = make_uint2(hb[0] | (hb[1] << 16), hb[2] | (hb[3] << 16));
+    }
+  } else {
+    const int H = g.L.H;
+#pragma unroll
+    for (int mt = 0; mt < 8; ++mt) {
+      const int pos = m0 + 16 * mt + r16;
+      if (pos >= mend) continue;
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+        *reinterpret_cast<float4*>(g.d + (size_t)pos * H + n0 + 16 * t + 4 * part) = make_float4(acc[t][mt][0], acc[t][mt][1], acc[t][mt][2], acc[t][mt][3]);
+    }
+  }
+}
+
 // yr[t][n] over the row's picks in expert-id order: acc = fma(s2 * w, d, acc); four columns a thread
 __global__ void __launch_bounds__(256) k_pf_combine(const float* __restrict__ d, const int* __restrict__ rpos, const float* __restrict__ rk,
                                                     int T, int H, int topk, float* __restrict__ yr) {
@@ -429,7 +633,8 @@ void dsgx_prefill_cfg_default(dsgx_prefill_cfg* c) {
 
 static int prefill_check(const dsgx_layer_w* L, int T, const char* who) {
   if (!L) return fail(DSGX_EINVAL, "%s: null layer", who);
-  if (L->fmt != DSGX_FMT_FP8_B128) return fail(DSGX_EUNSUPPORTED, "%s: only FP8_B128 layers are built (format %u)", who, L->fmt);
+  if (L->fmt != DSGX_FMT_FP8_B128 && L->fmt != DSGX_FMT_INT4_G32)
+    return fail(DSGX_EUNSUPPORTED, "%s: FP8_B128 and INT4_G32 layers are built (format %u)", who, L->fmt);
   if (T < 1 || T > DSGX_MAX_CHUNK) return fail(DSGX_EINVAL, "%s: T %d (1..%d)", who, T, DSGX_MAX_CHUNK);
   if (L->H < 256 || L->H % 256 || L->I < 128 || L->I % 128)
     return fail(DSGX_EINVAL, "%s: H %d (a multiple of 256), I %d (a multiple of 128)", who, L->H, L->I);
@@ -451,9 +656,11 @@ int dsgx_moe_prefill(const dsgx_layer_w* L, const uint16_t* x, const int* idx, c
   if (cfg_in) cfg = *cfg_in;
   if (!x || !idx || !w || !ws || !yr) return fail(DSGX_EINVAL, "moe_prefill: null x, idx, w, ws or yr");
   if (!L->pool || !L->desc) return fail(DSGX_EINVAL, "moe_prefill: layer without pool or descriptors");
-  if (!cfg.act_fp8) return fail(DSGX_EUNSUPPORTED, "moe_prefill: bf16 activations (act_fp8 = 0) are not built yet");
-  const bool shared = cfg.shared && layer_has_fp8_shared(L);
-  if (cfg.shared && L->sh.bgu) return fail(DSGX_EUNSUPPORTED, "moe_prefill: BF16 shared expert is not built yet");
+  const bool i4 = L->fmt == DSGX_FMT_INT4_G32;
+  if (!i4 && !cfg.act_fp8) return fail(DSGX_EUNSUPPORTED, "moe_prefill: FP8 layers with bf16 activations (act_fp8 = 0) are not built yet");
+  if (cfg.shared && !i4 && L->sh.bgu) return fail(DSGX_EUNSUPPORTED, "moe_prefill: a BF16 shared expert in an FP8 layer is not built yet");
+  if (cfg.shared && i4 && L->sh.g) return fail(DSGX_EUNSUPPORTED, "moe_prefill: an FP8 shared expert in an INT4 layer is not built yet");
+  const bool shared = cfg.shared && (i4 ? (L->sh.bgu && L->sh.bd) : layer_has_fp8_shared(L));
   if (shared && !ys) return fail(DSGX_EINVAL, "moe_prefill: the layer has a fused shared expert and ys is null");
   hipStream_t st = static_cast<hipStream_t>(stream);
   const PfLayout o = pf_layout(L, T);
@@ -472,6 +679,41 @@ int dsgx_moe_prefill(const dsgx_layer_w* L, const uint16_t* x, const int* idx, c
     hipLaunchKernelGGL(k_pf_rowsort, dim3((T + 255) / 256), dim3(256), 0, st, idx, w, I32(o.pickpos), L->desc, T, topk, I32(o.rpos),
                        I32(o.re), F32(o.rk));
     DSGX_HIP(hipGetLastError());
+  }
+  if (i4) {
+    // bf16 activations throughout: x -> h (bf16) -> d (f32 a pick) -> combine; the BF16 shared expert likewise -> ys
+    const size_t lds16 = (size_t)kStages16 * kPanel16;
+    auto k_up = k_pf_gemm16<true, DSGX_FMT_INT4_G32>;
+    auto k_dn = k_pf_gemm16<false, DSGX_FMT_INT4_G32>;
+    auto k_sup = k_pf_gemm16<true, DSGX_FMT_BF16>;
+    auto k_sdn = k_pf_gemm16<false, DSGX_FMT_BF16>;
+    for (const void* k : {(const void*)k_up, (const void*)k_dn, (const void*)k_sup, (const void*)k_sdn})
+      if (int rc = allow_dynamic_lds(k, lds16)) return rc;
+    Gemm16Args q{};
+    q.L = *L;
+    q.tile_e = I32(o.tile_e), q.tile_m0 = I32(o.tile_m0), q.ntiles = I32(o.ntiles), q.off = I32(o.off), q.nrows = P;
+    if (cfg.phases & 2) {
+      q.x = x, q.gather = I32(o.perm), q.h = reinterpret_cast<uint16_t*>(W + o.h), q.d = nullptr;
+      hipLaunchKernelGGL(k_up, dim3((unsigned)o.max_tiles * (I / (kWgRows / 2))), dim3(kGemmThreads), lds16, st, q);
+    }
+    if (cfg.phases & 4) {
+      q.x = reinterpret_cast<const uint16_t*>(W + o.h), q.gather = nullptr, q.h = nullptr, q.d = F32(o.d);
+      hipLaunchKernelGGL(k_dn, dim3((unsigned)o.max_tiles * (H / kWgRows)), dim3(kGemmThreads), lds16, st, q);
+    }
+    if (cfg.phases & 8) {
+      const size_t n = (size_t)T * (H / 4);
+      hipLaunchKernelGGL(k_pf_combine, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, F32(o.d), I32(o.rpos), F32(o.rk), T, H, topk, yr);
+    }
+    if ((cfg.phases & 16) && shared) {
+      const int tiles = (T + kTile - 1) / kTile;
+      q.tile_e = q.tile_m0 = q.ntiles = q.off = nullptr, q.nrows = T;
+      q.x = x, q.gather = nullptr, q.h = reinterpret_cast<uint16_t*>(W + o.hsh), q.d = nullptr;
+      hipLaunchKernelGGL(k_sup, dim3((unsigned)tiles * (I / (kWgRows / 2))), dim3(kGemmThreads), lds16, st, q);
+      q.x = reinterpret_cast<const uint16_t*>(W + o.hsh), q.h = nullptr, q.d = ys;
+      hipLaunchKernelGGL(k_sdn, dim3((unsigned)tiles * (H / kWgRows)), dim3(kGemmThreads), lds16, st, q);
+    }
+    DSGX_HIP(hipGetLastError());
+    return DSGX_OK;
   }
   GemmArgs g{};
   g.L = *L;

@@ -141,8 +141,43 @@ def test_prefill_rows_do_not_depend_on_the_chunk():
 
 
 def test_prefill_argument_errors():
-    hl = helpers.make_layer(abi.FMT_INT4, 512, 256, 8, 2, 4, seed=1)
+    hl = helpers.make_layer(abi.FMT_BF16, 512, 256, 8, 2, 4, seed=1)
     dl = hl.upload()
     assert lib.prefill_ws_bytes(dl.w, 16) == 0
     with pytest.raises(lib.DsgxError):
         lib.moe_prefill(dl.w, gpu.empty(16), gpu.empty(16), gpu.empty(16), 16, gpu.empty(16), gpu.empty(16), gpu.empty(16))
+
+
+# ---- INT4 layers: bf16 activations, the decode contract row by row ------------------------------------------------
+@pytest.mark.parametrize("H,I,E,topk,T,shared", [(512, 256, 8, 2, 150, "bf16"), (256, 128, 16, 4, 37, None)])
+def test_prefill_int4_against_oracle(H, I, E, topk, T, shared):
+    """a chunk row is a decode row (engine/experts/tests/test_prefill.inc:307-373): h and the outputs against the decode oracle"""
+    hl = helpers.make_layer(abi.FMT_INT4, H, I, E, topk, min(E, 5), seed=6, shared=shared)
+    x, _, idx, w = helpers.rows_and_routing(13, T, H, E, topk, 2.5)
+    yr, ys, ws, dl = _prefill(hl, x, idx, w, T)
+    v = lib.prefill_view(dl.w, ws, T)
+    P = T * topk
+    rpos = gpu.host(gpu.view(ws, v.rpos, P * 4), np.int32, (T, topk))
+    re = gpu.host(gpu.view(ws, v.re, P * 4), np.int32, (T, topk))
+    hg = gpu.host(gpu.view(ws, v.h, P * I * 2), np.uint16, (P, I))
+    hsh = gpu.host(gpu.view(ws, v.hsh, T * I * 2), np.uint16, (T, I)) if shared else None
+    assert np.array_equal(re, np.sort(idx, axis=1))
+    exact = total = 0
+    for t in range(T):
+        uni = orc.union(idx[t:t + 1], E)
+        up = orc.moe_up(hl, x[t:t + 1], uni)
+        mine = np.stack([hg[rpos[t, r]] for r in range(topk)] + ([hsh[t]] if shared else []))[:, None, :]
+        hv = orc.bf16_to_f32(mine)
+        assert np.all((hv >= up["lo"]) & (hv <= up["hi"])), "h outside the range of f32 sums"
+        exact += int(((mine == up["h64"]) | ((hv == 0) & (orc.bf16_to_f32(up["h64"]) == 0))).sum())
+        total += mine.size
+        dn = orc.moe_down(hl, mine, idx[t:t + 1], w[t:t + 1], uni)
+        worst, bad = helpers.check_sums(yr[t:t + 1], dn["yr64"], dn["yrmag"], 1e-4)
+        assert bad == 0, worst
+        full = orc.moe_down(hl, up["h32"], idx[t:t + 1], w[t:t + 1], uni)
+        helpers.check_outputs(yr[t:t + 1], full["yr32"])
+        if shared:
+            worst, bad = helpers.check_sums(ys[t:t + 1], dn["ys64"], dn["ysmag"], 1e-4)
+            assert bad == 0, worst
+            helpers.check_outputs(ys[t:t + 1], full["ys32"])
+    assert exact >= 0.995 * total, (exact, total)
