@@ -38,19 +38,20 @@ def log(*a):
 UP_TRAFFIC_FP8_M1 = 158768947
 
 
-def prefill_extra(gen, T=8192):
-    """the prefill chunk of the benchmark: T rows, top-8 of 256 experts drawn from a Zipf(1.1) popularity, FP8 weights and
-    activations; TFLOP/s over the useful multiply-adds of the routed experts (T * 8 * 3 * I * H * 2)"""
+def prefill_extra(gen, T, name, peak):
+    """a prefill chunk of the benchmark: T rows, top-8 experts drawn from a Zipf(1.1) popularity, uniform weights; FP8
+    weights and activations on the e4m3 MFMA (peak 5 PFLOP/s), or INT4 weights decoded to bf16 on the bf16 MFMA
+    (2.5 PFLOP/s); TFLOP/s over the useful multiply-adds of the routed experts (T * 8 * 3 * I * H * 2)"""
     from dsgx10_amd.benchdata import PrefillBench
     pb = PrefillBench(gen, T)
     t_routed, t_all = pb.time(15, False), pb.time(31, True)
-    d = dict(workload="fp8_moe_prefill", T=T, zipf_s=1.1, ms_routed=t_routed * 1e3, ms_with_shared=t_all * 1e3,
+    d = dict(workload=name, T=T, zipf_s=1.1, ms_routed=t_routed * 1e3, ms_with_shared=t_all * 1e3,
              tflops_routed=pb.flops_routed / t_routed / 1e12, tflops_with_shared=(pb.flops_routed + pb.flops_shared) / t_all / 1e12,
-             mfma_frac_of_5PFs=pb.flops_routed / t_routed / 5.0e15,
+             mfma_peak_tflops=peak / 1e12, mfma_frac=pb.flops_routed / t_routed / peak,
              phases_ms={n: pb.time(ph, sh) * 1e3 for n, ph, sh in (("bucket", 1, False), ("up", 2, False), ("down", 4, False),
                                                                       ("combine", 8, False), ("shared", 16, True))})
-    log("  fp8_moe_prefill T=%d: routed %.3f ms (%.0f TFLOP/s, %.1f%% of 5 PFLOP/s), with shared %.3f ms" %
-        (T, d["ms_routed"], d["tflops_routed"], 100 * d["mfma_frac_of_5PFs"], d["ms_with_shared"]))
+    log("  %s T=%d: routed %.3f ms (%.0f TFLOP/s, %.1f%% of %.1f PFLOP/s), with shared %.3f ms" %
+        (name, T, d["ms_routed"], d["tflops_routed"], 100 * d["mfma_frac"], peak / 1e15, d["ms_with_shared"]))
     del pb
     return d
 
@@ -132,8 +133,7 @@ def main():
             extra.append(dict(workload=gen.name, M=M, us_per_layer=e["us_per_layer"], bytes=e["bytes_per_layer"],
                               hbm_frac=e["layer_hbm_frac"], up_kernel_us=e["up_us"], up_hbm_frac=e["up_frac"]))
         del b
-        if head_fp8:
-            extra.append(prefill_extra(gen))
+        extra.append(prefill_extra(gen, 8192, "fp8_moe_prefill", 5.0e15) if head_fp8 else prefill_extra(gen, 2048, "int4_moe_prefill", 2.5e15))
         other = Int4LayerGen(seed=0) if head_fp8 else Fp8LayerGen(seed=0)
         for M in (1, 8):
             ob, e = run_decode(other, M, ks if M > 1 else K, min(W, 16))
@@ -143,6 +143,7 @@ def main():
                 d["cpu_baseline"] = cpu_baseline(ob, 5.0)
             extra.append(d)
             del ob
+        extra.append(prefill_extra(other, 2048, "int4_moe_prefill", 2.5e15) if head_fp8 else prefill_extra(other, 8192, "fp8_moe_prefill", 5.0e15))
         del other
         from dsgx10_amd.benchdata import gemv_bench
         extra += gemv_bench()

@@ -156,7 +156,8 @@ __global__ void __launch_bounds__(256) k_pf_rowsort(const int* __restrict__ idx,
 // in one lane) and streams them from memory straight into registers, a ring of kRing 128-k blocks ahead: a lane loads
 // 2 x 16 bytes a tile and block, the four lanes of a row 64 contiguous bytes an instruction. The activations of the
 // tile (shared by the eight waves) go through LDS, kStages blocks ahead, stored in the order of the MFMA fragments (the
-// operand reads are then linear in the lane: no bank conflicts).
+// operand reads are then linear in the lane: no bank conflicts). All global loads are issued with four consecutive
+// lanes on 64 contiguous bytes of a row; the weights are brought into the MFMA's lane order by a cross-lane permute.
 // v_mfma_f32_16x16x128_f8f6f4 covers one whole 128-k scale block: partial = A B^T from zero, then
 // acc = fma(x_scale * w_scale, partial, acc) on the vector unit (the accumulators therefore stay in ordinary registers).
 // With the weights as the A operand a lane's four accumulators of a tile belong to ONE position, so the combined scale is
@@ -227,11 +228,17 @@ __global__ void __launch_bounds__(kGemmThreads) k_pf_gemm(GemmArgs g) {
     sb = reinterpret_cast<const float*>(wb + (NK + 255) / 256 * 256);
   }
   const int tid = threadIdx.x, lane = tid & 63, wave = uni(tid >> 6), r16 = lane & 15, part = lane >> 4;
-  // the wave's two 16-row weight tiles: the lane's row of each, and the 16-byte column of the block's halves it loads
+  // Loads are issued with lane l on row l / 4, 16-byte piece l % 4 of a 64-byte half row (four consecutive lanes read 64
+  // contiguous bytes: the texture unit looks up one line for them, not one a lane), and the weights are then moved to the
+  // MFMA's lane order (row l % 16, piece l / 16) with one cross-lane permute a dword. The activations need no permute:
+  // they go to LDS, where each lane writes its piece to the slot of the fragment order.
+  const int lrow = lane >> 2, lq = lane & 3;
+  const int perm_addr = 4 * (4 * r16 + part);  // ds_bpermute: lane (r16, part) takes the dword of lane 4 r16 + part
+  // the wave's two 16-row weight tiles
   const int n0 = UP ? ns * (kWgRows / 2) + 16 * wave : ns * kWgRows + 32 * wave;  // UP: first channel; DOWN: first row
   const uint8_t* pa[2];
-  pa[0] = wa + (size_t)(n0 + r16) * K + part * 16;
-  pa[1] = (UP ? wb + (size_t)(n0 + r16) * K : wa + (size_t)(n0 + 16 + r16) * K) + part * 16;
+  pa[0] = wa + (size_t)(n0 + lrow) * K + lq * 16;
+  pa[1] = (UP ? wb + (size_t)(n0 + lrow) * K : wa + (size_t)(n0 + 16 + lrow) * K) + lq * 16;
   const float* swa = sa + (size_t)(n0 / 128) * KB;  // the tiles' scale rows (a wave's 32 rows lie in one 128-row block)
   const float* swb = UP ? sb + (size_t)(n0 / 128) * KB : swa;
 
@@ -241,9 +248,9 @@ __global__ void __launch_bounds__(kGemmThreads) k_pf_gemm(GemmArgs g) {
   // bank conflicts), and so are these writes. Thread t < 128 also brings the scale of position t.
   const uint8_t* pb;
   {
-    int pos = m0 + 16 * wave + r16;
+    int pos = m0 + 16 * wave + lrow;
     if (pos >= mend) pos = mend - 1;  // a ragged tile re-reads its last row (never stored)
-    pb = g.aq + (size_t)(g.gather ? g.gather[pos] : pos) * K + part * 16;
+    pb = g.aq + (size_t)(g.gather ? g.gather[pos] : pos) * K + lq * 16;
   }
   const float* pxs;
   {
@@ -282,8 +289,8 @@ __global__ void __launch_bounds__(kGemmThreads) k_pf_gemm(GemmArgs g) {
   };
   auto stash_x = [&](const XRegs& r, int stage) {
     uint8_t* B = smem + (size_t)stage * kStageBytes;
-    *reinterpret_cast<u32x4_t*>(B + ((2 * wave + 0) * 64 + lane) * 16) = r.v[0];
-    *reinterpret_cast<u32x4_t*>(B + ((2 * wave + 1) * 64 + lane) * 16) = r.v[1];
+    *reinterpret_cast<u32x4_t*>(B + ((2 * wave + 0) * 64 + lq * 16 + lrow) * 16) = r.v[0];
+    *reinterpret_cast<u32x4_t*>(B + ((2 * wave + 1) * 64 + lq * 16 + lrow) * 16) = r.v[1];
     if (tid < kTile) reinterpret_cast<float*>(B + kPanel)[tid] = r.s;
   };
   auto compute = [&](int slot, int stage, int kb) {
@@ -294,7 +301,8 @@ __global__ void __launch_bounds__(kGemmThreads) k_pf_gemm(GemmArgs g) {
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
       const u32x4_t lo = keep_whole(ra[slot][t][0]), hi = keep_whole(ra[slot][t][1]);
-      fa[t] = v8i_t{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
+      auto mv = [&](uint32_t v) { return __builtin_amdgcn_ds_bpermute(perm_addr, (int)v); };
+      fa[t] = v8i_t{mv(lo.x), mv(lo.y), mv(lo.z), mv(lo.w), mv(hi.x), mv(hi.y), mv(hi.z), mv(hi.w)};
     }
     // the eight 16-position tiles in two halves: four activation fragments in registers, eight independent MFMAs
     // issued back to back, the next half's fragments read while they run, then the scaled adds
