@@ -436,6 +436,10 @@ __global__ void __launch_bounds__(kGemmThreads) k_pf_gemm16(Gemm16Args g) {
     return;
   }
   const int tid = threadIdx.x, lane = tid & 63, wave = uni(tid >> 6), r16 = lane & 15, part = lane >> 4;
+  // loads are issued with lane l on row l / 4, piece l % 4 (four consecutive lanes read 64 contiguous bytes), weights are
+  // then moved to the MFMA's lane order (row l % 16, part l / 16) by a cross-lane permute, activations by their LDS slot
+  const int lrow = lane >> 2, lq = lane & 3;
+  const int perm_addr = 4 * (4 * r16 + part);
   const int n0 = UP ? ns * (kWgRows / 2) + 16 * wave : ns * kWgRows + 32 * wave;  // UP: first channel; DOWN: first row
   // the lane's weight row of each of the wave's two tiles
   const uint8_t* pw[2];
@@ -450,8 +454,9 @@ __global__ void __launch_bounds__(kGemmThreads) k_pf_gemm16(Gemm16Args g) {
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
       const uint8_t* base = g.L.pool + d[UP ? t : 2].off;
-      const int n = UP ? n0 + r16 : n0 + 16 * t + r16;
-      pw[t] = base + (size_t)n * (K / 2) + part * 16;
+      const int ln = UP ? n0 + lrow : n0 + 16 * t + lrow;  // the row this lane loads codes of
+      const int n = UP ? n0 + r16 : n0 + 16 * t + r16;       // the row it holds after the permute (scales: loaded as held)
+      pw[t] = base + (size_t)ln * (K / 2) + lq * 16;
       ps[t] = base + soff + ((size_t)n * G + part) * 2;
       pz[t] = base + zoff + ((size_t)(n >> 3) * G + part) * 4;
       zsh[t] = 4 * (n & 7);
@@ -461,19 +466,23 @@ __global__ void __launch_bounds__(kGemmThreads) k_pf_gemm16(Gemm16Args g) {
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
       // shared expert: gate row c is row 2 c of bgu, up row c is row 2 c + 1; down rows plain
-      const size_t row = UP ? 2 * (size_t)(n0 + r16) + t : (size_t)(n0 + 16 * t + r16);
-      pw[t] = reinterpret_cast<const uint8_t*>(UP ? g.L.sh.bgu : g.L.sh.bd) + row * K * 2 + part * 16;
+      const size_t row = UP ? 2 * (size_t)(n0 + lrow) + t : (size_t)(n0 + 16 * t + lrow);
+      pw[t] = reinterpret_cast<const uint8_t*>(UP ? g.L.sh.bgu : g.L.sh.bd) + row * K * 2 + lq * 16;
     }
   }
   // activation staging: wave w brings the 16 positions 16 w ..., the lane the four 16-byte pieces of its fragments
   const uint8_t* px;
   {
-    int pos = m0 + 16 * wave + r16;
+    int pos = m0 + 16 * wave + lrow;
     if (pos >= mend) pos = mend - 1;
-    px = reinterpret_cast<const uint8_t*>(g.x) + (size_t)(g.gather ? g.gather[pos] : pos) * K * 2;
+    px = reinterpret_cast<const uint8_t*>(g.x) + (size_t)(g.gather ? g.gather[pos] : pos) * K * 2 + lq * 16;
   }
-  // byte offset in a 128-k block of the 8 values of MFMA j in lane part p (bf16 activations; and BF16 weights)
-  auto koff = [&](int j) { return I4 ? (32 * part + 8 * j) * 2 : (32 * j + 8 * part) * 2; };
+  // Activation load i of a lane is the 16-byte piece c = 4 i + lq of its row's block (k = 8 c ...): the piece of MFMA j,
+  // part p with c = 4 p + j (INT4 map: k = 32 p + 8 j) or c = 4 j + p (BF16 map: k = 32 j + 8 p).
+  auto slot_of = [&](int i) {
+    const int c = 4 * i + lq, j = I4 ? c & 3 : c >> 2, p = I4 ? c >> 2 : c & 3;
+    return ((4 * wave + j) * 64 + p * 16 + lrow) * 16;
+  };
 
   v4f_t acc[2][8];
 #pragma unroll
@@ -507,12 +516,12 @@ __global__ void __launch_bounds__(kGemmThreads) k_pf_gemm16(Gemm16Args g) {
   auto fetch_x = [&](int kb) {
     const int kc = kb < KB ? kb : KB - 1;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) rx[j] = *reinterpret_cast<const u32x4_t*>(px + (size_t)kc * 256 + koff(j));
+    for (int j = 0; j < 4; ++j) rx[j] = *reinterpret_cast<const u32x4_t*>(px + (size_t)kc * 256 + 64 * j);
   };
   auto stash_x = [&](int stage) {
     uint8_t* B = smem + (size_t)stage * kPanel16;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) *reinterpret_cast<u32x4_t*>(B + ((4 * wave + j) * 64 + lane) * 16) = rx[j];
+    for (int j = 0; j < 4; ++j) *reinterpret_cast<u32x4_t*>(B + slot_of(j)) = rx[j];
   };
   auto compute = [&](int slot, int stage) {
     const uint8_t* B = smem + (size_t)stage * kPanel16;
@@ -523,7 +532,9 @@ __global__ void __launch_bounds__(kGemmThreads) k_pf_gemm16(Gemm16Args g) {
       if (I4) {
         const float sc = bf16_bits_to_f32(ra[slot][t].s);
         const float nzs = -((float)((ra[slot][t].z >> zsh[t]) & 15u) * sc);
-        const u32x4_t w = keep_whole(ra[slot][t].v[0]);
+        auto mv = [&](uint32_t v) { return (uint32_t)__builtin_amdgcn_ds_bpermute(perm_addr, (int)v); };
+        const u32x4_t wl = keep_whole(ra[slot][t].v[0]);
+        const u32x4_t w = u32x4_t{mv(wl.x), mv(wl.y), mv(wl.z), mv(wl.w)};
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           uint32_t o[4];
@@ -532,7 +543,11 @@ __global__ void __launch_bounds__(kGemmThreads) k_pf_gemm16(Gemm16Args g) {
         }
       } else {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) fa[t][j] = keep_whole(ra[slot][t].v[j]);
+        for (int j = 0; j < 4; ++j) {
+          auto mv = [&](uint32_t v) { return (uint32_t)__builtin_amdgcn_ds_bpermute(perm_addr, (int)v); };
+          const u32x4_t wl = keep_whole(ra[slot][t].v[j]);
+          fa[t][j] = u32x4_t{mv(wl.x), mv(wl.y), mv(wl.z), mv(wl.w)};
+        }
       }
     }
 #pragma unroll
