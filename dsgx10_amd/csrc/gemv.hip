@@ -28,8 +28,6 @@ struct GemvArgs {
 template <int FMT, int M, int RB, int D>
 __global__ void __launch_bounds__(256) k_gemv(GemvArgs a) {
   extern __shared__ uint4 xs[];
-  stage_x<FmtT<FMT>::KL>(xs, a.x, a.ldx, M, a.K, a.nq * 8);
-  __syncthreads();
   const int lane = threadIdx.x & 63;
   const int gw = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6), GW = gridDim.x * (blockDim.x >> 6);
   const int nbatch = a.total_rows / RB;
@@ -92,9 +90,12 @@ __global__ void __launch_bounds__(256) k_gemv(GemvArgs a) {
       static_cast<uint16_t*>(sg.y)[(size_t)m * sg.ldy + n / 2] = (uint16_t)swiglu_bits(bf16_round(mine), bf16_round(mine2));
     }
   };
-  if (nsteps == 0) return;
+  // the first weight loads are issued before the activations are staged: one memory round trip, not two, before the
+  // first product (these calls are a few microseconds long: latency is most of them)
 #pragma unroll
   for (int d = 0; d < D; ++d) load(w[d]);
+  stage_x<FmtT<FMT>::KL>(xs, a.x, a.ldx, M, a.K, a.nq * 8);
+  __syncthreads();
   for (int t = 0; t < nsteps; t += D) {
 #pragma unroll
     for (int d = 0; d < D; ++d) {
