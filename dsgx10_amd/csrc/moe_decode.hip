@@ -67,6 +67,18 @@ int dsgx_moe_decode(const dsgx_layer_w* L, const uint16_t* x, const int* idx, co
   if ((fp8sh || b16sh || c.ysum) && (c.parts & 2) && !ys) return fail(DSGX_EINVAL, "moe_decode: ys (the shared expert's output) is needed");
   if (((uintptr_t)x | (uintptr_t)ws | (uintptr_t)L->pool) & 15) return fail(DSGX_EINVAL, "moe_decode: x, ws and pool must be 16-byte aligned");
 
+  if (M > 8) {
+    // 9-16 rows (the reference's limit, experts.h:104): two passes of the kernels built for up to eight rows, rows 0-7
+    // then the rest; every row's result is what it is alone or in any batch, so the split is invisible in the output.
+    // The second pass reads the weights of its experts again; the workspace is reused in stream order.
+    const int M1 = 8, topk = L->topk, E = L->E;
+    dsgx_decode_cfg c1 = c, c2 = c;
+    c1.parts = c2.parts = c.parts & 3;
+    if (c.logits) c2.logits = c.logits + (size_t)M1 * E;
+    if (int rc = dsgx_moe_decode(L, x, idx, w, M1, ws, yr, ys, stream, &c1)) return rc;
+    return dsgx_moe_decode(L, x + (size_t)M1 * H, idx ? idx + (size_t)M1 * topk : nullptr, w ? w + (size_t)M1 * topk : nullptr, M - M1, ws,
+                           yr ? yr + (size_t)M1 * H : nullptr, ys ? ys + (size_t)M1 * H : nullptr, stream, &c2);
+  }
   DecodeArgs a{};
   a.x = x, a.M = M, a.idx = idx, a.w = w, a.logits = c.logits, a.bias = c.bias, a.route_scale = c.route_scale, a.score_fn = c.score_fn;
   a.L = *L, a.h = static_cast<uint16_t*>(ws), a.yr = yr, a.ys = ys, a.ysum = c.ysum;

@@ -163,3 +163,18 @@ def test_decode_parts_and_duplicate_experts_across_rows():
     assert np.all(gpu.host(yr1, np.uint32, (-1,)) == 0xFFFFFFFF)
     lib.moe_decode(dl.w, gpu.dev(x), gpu.dev(idx), gpu.dev(w), 4, ws, yr1, None, parts=2)   # down only, from ws's h
     assert np.array_equal(gpu.host(yr1, np.float32, (4, H_)).view(np.uint32), yr.view(np.uint32))
+
+
+def test_decode_nine_to_sixteen_rows():
+    """up to 16 rows a call (experts.h:104 of the reference): every row is what it is alone, with idx/w and with logits"""
+    fmt, H, I, E, topk, NS, shared, scale = CASES[0]
+    hl, dl = _layer(fmt, H, I, E, topk, NS, shared)
+    x, logits, idx, w = rows_and_routing(41, 16, H, E, topk, scale)
+    for M in (9, 16):
+        yr, ys, _ = gpu.decode_layer(dl, x[:M], idx[:M], w[:M], M)
+        yl, sl, _ = gpu.decode_layer(dl, x[:M], None, None, M, logits=gpu.dev(logits[:M]), route_scale=scale)
+        assert np.array_equal(yr.view(np.uint32), yl.view(np.uint32)) and np.array_equal(ys.view(np.uint32), sl.view(np.uint32))
+        for m in (0, 7, 8, M - 1):
+            y1, s1, _ = gpu.decode_layer(dl, x[m:m + 1], idx[m:m + 1], w[m:m + 1], 1)
+            assert np.array_equal(y1[0].view(np.uint32), yr[m].view(np.uint32)), (M, m)
+            assert np.array_equal(s1[0].view(np.uint32), ys[m].view(np.uint32)), (M, m)
