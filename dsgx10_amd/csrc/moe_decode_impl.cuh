@@ -122,16 +122,16 @@ template <int FMT, int SHFMT, int M>
 __device__ __forceinline__ void prep(Step<M>& S, const DecodeArgs& a) {
   const int tid = threadIdx.x;
   // every expert's descriptors into S.dtab (their first 16 of 64 bytes), three loads in flight a thread
-  const uint4* d = reinterpret_cast<const uint4*>(a.L.desc);
+  // (loads past the end re-read the last descriptor: unconditional loads into named registers stay in flight together)
+  const DSGX_GLOBAL u32x4_t* d = (const DSGX_GLOBAL u32x4_t*)(uintptr_t)a.L.desc;
+  u32x4_t* tab = reinterpret_cast<u32x4_t*>(S.dtab);
   const int nd = a.L.E * 3, bd = blockDim.x;
   for (int i0 = tid; i0 < nd; i0 += 3 * bd) {
-    uint4 v[3];
-#pragma unroll
-    for (int u = 0; u < 3; ++u)
-      if (i0 + u * bd < nd) v[u] = d[(size_t)(i0 + u * bd) * 4];
-#pragma unroll
-    for (int u = 0; u < 3; ++u)
-      if (i0 + u * bd < nd) S.dtab[i0 + u * bd] = v[u];
+    const int i1 = i0 + bd, i2 = i1 + bd;
+    const u32x4_t v0 = d[(size_t)i0 * 4], v1 = d[(size_t)min(i1, nd - 1) * 4], v2 = d[(size_t)min(i2, nd - 1) * 4];
+    tab[i0] = v0;
+    if (i1 < nd) tab[i1] = v1;
+    if (i2 < nd) tab[i2] = v2;
   }
   if (tid < DSGX_MAX_EXPERTS / 32) S.mask[tid] = 0;
   for (int i = tid; i < M * DSGX_MAX_TOPK * M; i += blockDim.x) (&S.wslot[0][0])[i] = 0.f;
