@@ -356,15 +356,18 @@ class PrefillBench:
     def run(self, phases=31, shared=True):
         lib.moe_prefill(self.layer, self.x, self.idx, self.w, self.T, self.ws, self.yr, self.ys, shared=shared, phases=phases)
 
-    def time(self, phases=31, shared=True, reps=5):
+    def time(self, phases=31, shared=True, reps=8, samples=3):
+        """Seconds per call: `reps` calls back to back between two events (a model's layers follow each other the same
+        way; a lone launch after an idle gap runs at a lower clock), the median of `samples` such runs."""
         self.run(phases, shared)
         torch.cuda.synchronize()
         ts = []
-        for _ in range(reps):
+        for _ in range(samples):
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             e0.record()
-            self.run(phases, shared)
+            for _ in range(reps):
+                self.run(phases, shared)
             e1.record()
             torch.cuda.synchronize()
-            ts.append(e0.elapsed_time(e1) * 1e-3)
+            ts.append(e0.elapsed_time(e1) * 1e-3 / reps)
         return float(np.median(ts))

@@ -163,10 +163,30 @@ __global__ void __launch_bounds__(256) k_pf_rowsort(const int* __restrict__ idx,
 // With the weights as the A operand a lane's four accumulators of a tile belong to ONE position, so the combined scale is
 // one value a lane.
 constexpr int kPanel = kTile * 128;              // bytes of one activation panel (128 positions x 128 k)
-constexpr int kStages = 4, kRing = 4;
+constexpr int kStages = 4, kRing = 3, kHold = 3;  // LDS stages; turns a weight / an activation load is issued ahead of its use
 constexpr int kStageBytes = kPanel + kTile * 4;  // + the positions' scales of the block
 constexpr int kWgRows = 256;                     // weight rows a workgroup (UP: 128 channels)
 constexpr int kGemmThreads = 512;
+
+// Workgroup -> (position tile, group of weight rows). Workgroups go to the eight XCDs round robin by their number, and
+// each XCD has an L2 of its own: what two workgroups share is read from memory once only if they run on the same XCD at
+// about the same time. So the tasks are cut into blocks of kMapTiles consecutive tiles (mostly one expert's: tiles are in
+// expert order) x kMapNs row groups, and a block's 32 tasks get 32 consecutive workgroup numbers OF ONE XCD (numbers
+// x, x + 8, x + 16, ...): they start together and walk K together, a weight line is then fetched by one of the
+// kMapTiles workgroups that use it and an activation line by one of kMapNs, the others hit L2 (measured: 115 GB/s a CU
+// from L2, 28 from beyond).
+constexpr int kMapTiles = 4, kMapNs = 8, kXcds = 8;
+__host__ __device__ inline unsigned pf_grid(int tiles, int NS) {
+  const int blocks = ((tiles + kMapTiles - 1) / kMapTiles) * ((NS + kMapNs - 1) / kMapNs);
+  return (unsigned)((blocks + kXcds - 1) / kXcds) * kXcds * (kMapTiles * kMapNs);
+}
+__device__ __forceinline__ void pf_task(int NS, int& tile, int& ns) {
+  const int x = blockIdx.x % kXcds, j = blockIdx.x / kXcds;
+  const int b = (j / (kMapTiles * kMapNs)) * kXcds + x, i = j % (kMapTiles * kMapNs);
+  const int NG = (NS + kMapNs - 1) / kMapNs;
+  tile = (b / NG) * kMapTiles + i / kMapNs;
+  ns = (b % NG) * kMapNs + i % kMapNs;
+}
 
 struct GemmArgs {
   const uint8_t* aq;   // activations, e4m3 [rows][K]
@@ -187,7 +207,10 @@ struct GemmArgs {
 #ifdef DSGX_TRACE
 #define PF_MARK(k)                                                                                       \
   do {                                                                                                    \
-    if (g.trace && threadIdx.x == 0 && blockIdx.x < 1024) g.trace[blockIdx.x * 16 + (k)] = wall_clock64(); \
+    if (g.trace && threadIdx.x == 0 && blockIdx.x < 1024) {                                                \
+      g.trace[blockIdx.x * 16 + (k)] = wall_clock64();                                                    \
+      g.trace[blockIdx.x * 16 + 8 + (k)] = clock64(); /* (marks 0..7 only) */                            \
+    }                                                                                                     \
   } while (0)
 #else
 #define PF_MARK(k) do { } while (0)
@@ -199,7 +222,9 @@ __global__ void __launch_bounds__(kGemmThreads) k_pf_gemm(GemmArgs g) {
   PF_MARK(0);
   const int K = UP ? g.L.H : g.L.I, KB = K / 128;
   const int NS = UP ? g.L.I / (kWgRows / 2) : g.L.H / kWgRows;  // workgroups along the weight rows
-  const int tile = blockIdx.x / NS, ns = blockIdx.x % NS;
+  int tile, ns;
+  pf_task(NS, tile, ns);
+  if (ns >= NS) return;
   int e = -1, m0 = tile * kTile, mend = g.nrows;
   if (g.tile_e) {
     if (tile >= *g.ntiles) return;
@@ -233,7 +258,6 @@ __global__ void __launch_bounds__(kGemmThreads) k_pf_gemm(GemmArgs g) {
   // MFMA's lane order (row l % 16, piece l / 16) with one cross-lane permute a dword. The activations need no permute:
   // they go to LDS, where each lane writes its piece to the slot of the fragment order.
   const int lrow = lane >> 2, lq = lane & 3;
-  const int perm_addr = 4 * (4 * r16 + part);  // ds_bpermute: lane (r16, part) takes the dword of lane 4 r16 + part
   // the wave's two 16-row weight tiles
   const int n0 = UP ? ns * (kWgRows / 2) + 16 * wave : ns * kWgRows + 32 * wave;  // UP: first channel; DOWN: first row
   const uint8_t* pa[2];
@@ -259,6 +283,11 @@ __global__ void __launch_bounds__(kGemmThreads) k_pf_gemm(GemmArgs g) {
     pxs = g.as + (size_t)(g.gather ? g.gather[pos] : pos) * KB;
   }
 
+  // a fragment's 64 pieces in LDS: piece (row r, part p) at slot 16 p + (r ^ 2 p), 16 bytes a slot. The exclusive-or keeps
+  // both sides free of bank conflicts: the writes (eight consecutive lanes hold two rows x four parts) and the MFMA-order
+  // reads (eight consecutive lanes hold eight rows of one part) each touch eight different slots modulo 8.
+  const int nmt = uni(min(8, (mend - m0 + 15) / 16));  // the tile's 16-position tiles that hold rows
+  const int wr_slot = (lq * 16 + (lrow ^ (2 * lq))) * 16, rd_slot = (part * 16 + (r16 ^ (2 * part))) * 16;
   auto blk = [&](int kb) { return kb < KB ? kb : KB - 1; };  // (past the end: the last block again, never used)
   v4f_t acc[2][8];
 #pragma unroll
@@ -289,79 +318,124 @@ __global__ void __launch_bounds__(kGemmThreads) k_pf_gemm(GemmArgs g) {
   };
   auto stash_x = [&](const XRegs& r, int stage) {
     uint8_t* B = smem + (size_t)stage * kStageBytes;
-    *reinterpret_cast<u32x4_t*>(B + ((2 * wave + 0) * 64 + lq * 16 + lrow) * 16) = r.v[0];
-    *reinterpret_cast<u32x4_t*>(B + ((2 * wave + 1) * 64 + lq * 16 + lrow) * 16) = r.v[1];
+    *reinterpret_cast<u32x4_t*>(B + (2 * wave + 0) * 1024 + wr_slot) = r.v[0];
+    *reinterpret_cast<u32x4_t*>(B + (2 * wave + 1) * 1024 + wr_slot) = r.v[1];
     if (tid < kTile) reinterpret_cast<float*>(B + kPanel)[tid] = r.s;
   };
-  auto compute = [&](int slot, int stage, int kb) {
-    const uint8_t* B = smem + (size_t)stage * kStageBytes;
-    const float* XS = reinterpret_cast<const float*>(B + kPanel);
-    const float wsa = swa[kb], wsb = swb[kb];
-    v8i_t fa[2];
+  // the wave's weight scales: lane l holds those of block kb0 + l for the 64 blocks from kb0 (a multiple of 64)
+  float wsa_l, wsb_l;
+  auto load_ws = [&](int kb0) {
+    const int kc = blk(kb0 + lane);
+    wsa_l = swa[kc], wsb_l = swb[kc];
+  };
+  load_ws(0);
+  // The wave's weights of a block reach the MFMA's lane order through its own LDS (two copies of 4 KiB, written as
+  // loaded, read as fragments, in the activations' slot order: no bank conflicts; the LDS unit serves a wave's
+  // operations in order, so no barrier lies between): a quarter of the LDS time of a cross-lane permute a dword.
+  auto w_to_lds = [&](int slot, int par) {
+    uint8_t* W = smem + (size_t)kStages * kStageBytes + (2 * wave + par) * 4096;
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int h = 0; h < 2; ++h) *reinterpret_cast<u32x4_t*>(W + (2 * t + h) * 1024 + wr_slot) = keep_whole(ra[slot][t][h]);
+  };
+  v8i_t fa[2], fb[3];
+  float xv[3];
+  auto read_fa = [&](int par) {
+    const uint8_t* W = smem + (size_t)kStages * kStageBytes + (2 * wave + par) * 4096;
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
-      const u32x4_t lo = keep_whole(ra[slot][t][0]), hi = keep_whole(ra[slot][t][1]);
-      auto mv = [&](uint32_t v) { return __builtin_amdgcn_ds_bpermute(perm_addr, (int)v); };
-      fa[t] = v8i_t{mv(lo.x), mv(lo.y), mv(lo.z), mv(lo.w), mv(hi.x), mv(hi.y), mv(hi.z), mv(hi.w)};
-    }
-    // the eight 16-position tiles in two halves: four activation fragments in registers, eight independent MFMAs
-    // issued back to back, the next half's fragments read while they run, then the scaled adds
-    v8i_t fb[4];
-    float xv[4];
-    auto read_b = [&](int half) {
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int mt = 4 * half + i;
-        const u32x4_t lo = *reinterpret_cast<const u32x4_t*>(B + ((2 * mt + 0) * 64 + lane) * 16);
-        const u32x4_t hi = *reinterpret_cast<const u32x4_t*>(B + ((2 * mt + 1) * 64 + lane) * 16);
-        fb[i] = v8i_t{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
-        xv[i] = XS[16 * mt + r16];
-      }
-    };
-    read_b(0);
-#pragma unroll
-    for (int half = 0; half < 2; ++half) {
-      v4f_t p[2][4];
-      float sc[2][4];
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int t = 0; t < 2; ++t) {
-          p[t][i] = mfma_fp8_k128(fa[t], fb[i], v4f_t{});
-          sc[t][i] = __fmul_rn(xv[i], t ? wsb : wsa);
-        }
-      if (half == 0) read_b(1);
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int t = 0; t < 2; ++t)
-#pragma unroll
-          for (int q = 0; q < 4; ++q) acc[t][4 * half + i][q] = fmaf(sc[t][i], p[t][i][q], acc[t][4 * half + i][q]);
+      const u32x4_t lo = *reinterpret_cast<const u32x4_t*>(W + (2 * t + 0) * 1024 + rd_slot);
+      const u32x4_t hi = *reinterpret_cast<const u32x4_t*>(W + (2 * t + 1) * 1024 + rd_slot);
+      fa[t] = v8i_t{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
     }
   };
+  auto read_b = [&](int buf, int stage, int mt) {
+    const uint8_t* B = smem + (size_t)stage * kStageBytes;
+    const u32x4_t lo = *reinterpret_cast<const u32x4_t*>(B + (2 * mt + 0) * 1024 + rd_slot);
+    const u32x4_t hi = *reinterpret_cast<const u32x4_t*>(B + (2 * mt + 1) * 1024 + rd_slot);
+    fb[buf] = v8i_t{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
+    xv[buf] = reinterpret_cast<const float*>(B + kPanel)[16 * mt + r16];
+  };
+  // The activations of a block wait in registers for kHold turns between their loads and their LDS writes (the memory
+  // latency is several turns long, and a wait for one load is a wait for every load issued before it): set v holds, at
+  // the start of turn kb = v (mod kHold), block kb + 3.
+  XRegs rx[kHold];
   PF_MARK(1);
-  // prologue: the weight ring, the first activation panels
+  // prologue: the weight ring, the first activation panels, block 0's weights to LDS
 #pragma unroll
   for (int d = 0; d < kRing; ++d) load_a(d, d);
-  XRegs rx, rx1, rx2;
-  fetch_x(rx, 0), fetch_x(rx1, 1), fetch_x(rx2, 2);
-  stash_x(rx, 0), stash_x(rx1, 1), stash_x(rx2, 2);
-  __syncthreads();
-  PF_MARK(2);
-  // turn kb: issue the activation loads of block kb + 3, compute block kb, issue the weight loads of block kb + kRing
-  // in its place, put the activations of block kb + 3 into their stage (last read a turn ago)
-  for (int kb0 = 0; kb0 < KB; kb0 += 4) {
+  {
+    XRegs t0, t1, t2;
+    fetch_x(t0, 0), fetch_x(t1, 1), fetch_x(t2, 2);
 #pragma unroll
-    for (int v = 0; v < 4; ++v) {
+    for (int v = 0; v < kHold; ++v) fetch_x(rx[v], 3 + v);
+    stash_x(t0, 0), stash_x(t1, 1), stash_x(t2, 2);
+  }
+  w_to_lds(0, 0);
+  load_a(0, kRing);
+  __syncthreads();
+  read_fa(0);
+  read_b(0, 0, 0);
+  if (nmt > 1) read_b(1, 0, 1);
+  PF_MARK(2);
+  // Turn kb. On entry the registers hold (or have in flight) block kb's weight fragments and the activation fragments of
+  // its position tiles 0 and 1. The eight tiles run as a pipeline: the fragment of tile mt + 2 is read while tile mt's
+  // two MFMAs (from zero) are issued and tile mt - 1's scaled adds run. In between, work for later turns: the
+  // activations of block kb + 3 (loaded kHold turns ago) go to their stage (last read a turn ago) and the loads of
+  // block kb + 3 + kHold are issued in their place; the ring's block kb + 1 goes to the wave's LDS copy and the loads
+  // of block kb + 1 + kRing are issued in its place; after the last MFMA is issued, the next turn's fragments are
+  // read. Then the barrier: nothing but those reads' latency stands between it and the next turn's first MFMA.
+  // (Unrolled over a common multiple of the rotations.)
+  constexpr int kTurns = 12;
+  static_assert(kTurns % kRing == 0 && kTurns % kHold == 0 && kTurns % kStages == 0 && kTurns % 2 == 0, "unroll");
+  for (int kb0 = 0; kb0 < KB; kb0 += kTurns) {
+#pragma unroll
+    for (int v = 0; v < kTurns; ++v) {
       const int kb = kb0 + v;
-      fetch_x(rx, kb + 3);
-      if (kb < KB) compute(v, v, kb);
-      load_a(v, kb + kRing);
-      stash_x(rx, (v + 3) & 3);
+      if (kb >= KB) break;
+      // the block's weight scales from the lanes that hold them (a load here would be waited for in this same turn, and
+      // a wait for one load is a wait for every load before it: the whole ring)
+      if ((kb & 63) == 0 && kb > 0) load_ws(kb);
+      const float wsa = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, wsa_l), kb & 63));
+      const float wsb = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, wsb_l), kb & 63));
+      v4f_t pp[2] = {v4f_t{}, v4f_t{}};
+      float scp[2] = {0.f, 0.f};
+#pragma unroll
+      for (int mt = 0; mt <= 8; ++mt) {
+        // (a ragged tile's 16-position tiles past its end are skipped: most experts of a chunk hold fewer than 128 rows)
+        if (mt + 2 < 8 && mt + 2 < nmt) read_b((mt + 2) % 3, v % kStages, mt + 2);
+        v4f_t pc[2] = {v4f_t{}, v4f_t{}};
+        float scn[2] = {0.f, 0.f};
+        if (mt < 8 && mt < nmt) {
+#pragma unroll
+          for (int t = 0; t < 2; ++t) pc[t] = mfma_fp8_k128(fa[t], fb[mt % 3], v4f_t{});
+          scn[0] = __fmul_rn(xv[mt % 3], wsa), scn[1] = __fmul_rn(xv[mt % 3], wsb);
+        }
+        if (mt == 7) {  // the last MFMAs are issued: the next turn's fragments
+          read_fa((v + 1) & 1);
+          read_b(0, (v + 1) % kStages, 0);
+          if (nmt > 1) read_b(1, (v + 1) % kStages, 1);
+        }
+        if (mt > 0 && mt - 1 < nmt) {
+#pragma unroll
+          for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) acc[t][mt - 1][q] = fmaf(scp[t], pp[t][q], acc[t][mt - 1][q]);
+        }
+        if (mt < 8) pp[0] = pc[0], pp[1] = pc[1], scp[0] = scn[0], scp[1] = scn[1];
+        if (mt == 2) {
+          stash_x(rx[v % kHold], (v + 3) % kStages);
+          fetch_x(rx[v % kHold], kb + 3 + kHold);
+        }
+        if (mt == 4) {
+          w_to_lds((v + 1) % kRing, (v + 1) & 1);
+          load_a((v + 1) % kRing, kb + 1 + kRing);
+        }
+      }
       __syncthreads();
     }
     if (kb0 == 0) PF_MARK(3);
-    if (kb0 == 12) PF_MARK(4);
   }
   PF_MARK(5);
 
@@ -425,7 +499,9 @@ __global__ void __launch_bounds__(kGemmThreads) k_pf_gemm16(Gemm16Args g) {
   constexpr bool I4 = WF == DSGX_FMT_INT4_G32;
   const int K = UP ? g.L.H : g.L.I, N = UP ? g.L.I : g.L.H, KB = K / 128;
   const int NS = UP ? g.L.I / (kWgRows / 2) : g.L.H / kWgRows;
-  const int tile = blockIdx.x / NS, ns = blockIdx.x % NS;
+  int tile, ns;
+  pf_task(NS, tile, ns);
+  if (ns >= NS) return;
   int e = -1, m0 = tile * kTile, mend = g.nrows;
   if (g.tile_e) {
     if (tile >= *g.ntiles) return;
@@ -691,7 +767,7 @@ int dsgx_moe_prefill(const dsgx_layer_w* L, const uint16_t* x, const int* idx, c
   auto I32 = [&](size_t off) { return reinterpret_cast<int*>(W + off); };
   auto F32 = [&](size_t off) { return reinterpret_cast<float*>(W + off); };
   const int H = L->H, I = L->I, E = L->E, topk = L->topk, P = o.P;
-  const size_t lds = (size_t)kStages * kStageBytes;
+  const size_t lds = (size_t)kStages * kStageBytes + (kGemmThreads / 64) * 2 * 4096;  // activation stages + two weight blocks a wave
   if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(k_pf_gemm<true>), lds)) return rc;
   if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(k_pf_gemm<false>), lds)) return rc;
 
@@ -717,11 +793,11 @@ int dsgx_moe_prefill(const dsgx_layer_w* L, const uint16_t* x, const int* idx, c
     q.tile_e = I32(o.tile_e), q.tile_m0 = I32(o.tile_m0), q.ntiles = I32(o.ntiles), q.off = I32(o.off), q.nrows = P;
     if (cfg.phases & 2) {
       q.x = x, q.gather = I32(o.perm), q.h = reinterpret_cast<uint16_t*>(W + o.h), q.d = nullptr;
-      hipLaunchKernelGGL(k_up, dim3((unsigned)o.max_tiles * (I / (kWgRows / 2))), dim3(kGemmThreads), lds16, st, q);
+      hipLaunchKernelGGL(k_up, dim3(pf_grid(o.max_tiles, I / (kWgRows / 2))), dim3(kGemmThreads), lds16, st, q);
     }
     if (cfg.phases & 4) {
       q.x = reinterpret_cast<const uint16_t*>(W + o.h), q.gather = nullptr, q.h = nullptr, q.d = F32(o.d);
-      hipLaunchKernelGGL(k_dn, dim3((unsigned)o.max_tiles * (H / kWgRows)), dim3(kGemmThreads), lds16, st, q);
+      hipLaunchKernelGGL(k_dn, dim3(pf_grid(o.max_tiles, H / kWgRows)), dim3(kGemmThreads), lds16, st, q);
     }
     if (cfg.phases & 8) {
       const size_t n = (size_t)T * (H / 4);
@@ -731,9 +807,9 @@ int dsgx_moe_prefill(const dsgx_layer_w* L, const uint16_t* x, const int* idx, c
       const int tiles = (T + kTile - 1) / kTile;
       q.tile_e = q.tile_m0 = q.ntiles = q.off = nullptr, q.nrows = T;
       q.x = x, q.gather = nullptr, q.h = reinterpret_cast<uint16_t*>(W + o.hsh), q.d = nullptr;
-      hipLaunchKernelGGL(k_sup, dim3((unsigned)tiles * (I / (kWgRows / 2))), dim3(kGemmThreads), lds16, st, q);
+      hipLaunchKernelGGL(k_sup, dim3(pf_grid(tiles, I / (kWgRows / 2))), dim3(kGemmThreads), lds16, st, q);
       q.x = reinterpret_cast<const uint16_t*>(W + o.hsh), q.h = nullptr, q.d = ys;
-      hipLaunchKernelGGL(k_sdn, dim3((unsigned)tiles * (H / kWgRows)), dim3(kGemmThreads), lds16, st, q);
+      hipLaunchKernelGGL(k_sdn, dim3(pf_grid(tiles, H / kWgRows)), dim3(kGemmThreads), lds16, st, q);
     }
     DSGX_HIP(hipGetLastError());
     return DSGX_OK;
@@ -750,7 +826,7 @@ int dsgx_moe_prefill(const dsgx_layer_w* L, const uint16_t* x, const int* idx, c
     g.aq = W + o.xq, g.as = F32(o.xs), g.gather = I32(o.perm);
     g.tile_e = I32(o.tile_e), g.tile_m0 = I32(o.tile_m0), g.ntiles = I32(o.ntiles), g.off = I32(o.off), g.nrows = P;
     g.h = reinterpret_cast<uint16_t*>(W + o.h), g.d = nullptr;
-    hipLaunchKernelGGL(k_pf_gemm<true>, dim3((unsigned)o.max_tiles * (I / (kWgRows / 2))), dim3(kGemmThreads), lds, st, g);
+    hipLaunchKernelGGL(k_pf_gemm<true>, dim3(pf_grid(o.max_tiles, I / (kWgRows / 2))), dim3(kGemmThreads), lds, st, g);
     DSGX_HIP(hipGetLastError());
   }
   if (cfg.phases & 4) {
@@ -758,7 +834,7 @@ int dsgx_moe_prefill(const dsgx_layer_w* L, const uint16_t* x, const int* idx, c
     g.aq = W + o.hq, g.as = F32(o.hs), g.gather = nullptr;
     g.tile_e = I32(o.tile_e), g.tile_m0 = I32(o.tile_m0), g.ntiles = I32(o.ntiles), g.off = I32(o.off), g.nrows = P;
     g.h = nullptr, g.d = F32(o.d);
-    hipLaunchKernelGGL(k_pf_gemm<false>, dim3((unsigned)o.max_tiles * (H / kWgRows)), dim3(kGemmThreads), lds, st, g);
+    hipLaunchKernelGGL(k_pf_gemm<false>, dim3(pf_grid(o.max_tiles, H / kWgRows)), dim3(kGemmThreads), lds, st, g);
     DSGX_HIP(hipGetLastError());
   }
   if (cfg.phases & 8) {
@@ -771,10 +847,10 @@ int dsgx_moe_prefill(const dsgx_layer_w* L, const uint16_t* x, const int* idx, c
     g.aq = W + o.xq, g.as = F32(o.xs), g.gather = nullptr;
     g.tile_e = g.tile_m0 = g.ntiles = g.off = nullptr, g.nrows = T;
     g.h = reinterpret_cast<uint16_t*>(W + o.hsh), g.d = nullptr;
-    hipLaunchKernelGGL(k_pf_gemm<true>, dim3((unsigned)tiles * (I / (kWgRows / 2))), dim3(kGemmThreads), lds, st, g);
+    hipLaunchKernelGGL(k_pf_gemm<true>, dim3(pf_grid(tiles, I / (kWgRows / 2))), dim3(kGemmThreads), lds, st, g);
     if (int rc = dsgx_act_quant(reinterpret_cast<const uint16_t*>(W + o.hsh), T, I, W + o.hshq, F32(o.hshs), stream)) return rc;
     g.aq = W + o.hshq, g.as = F32(o.hshs), g.h = nullptr, g.d = ys;
-    hipLaunchKernelGGL(k_pf_gemm<false>, dim3((unsigned)tiles * (H / kWgRows)), dim3(kGemmThreads), lds, st, g);
+    hipLaunchKernelGGL(k_pf_gemm<false>, dim3(pf_grid(tiles, H / kWgRows)), dim3(kGemmThreads), lds, st, g);
     DSGX_HIP(hipGetLastError());
   }
   return DSGX_OK;
