@@ -139,6 +139,53 @@ __device__ __forceinline__ float wave_sum(float v) {
   r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
   return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
+// The sums over the wave of N values a lane (N a power of two up to 16) for little more than the price of one: the two
+// widest butterfly steps (lane distance 32, then 16) are done as FOLDS, a lane-half swap of two values' registers
+// leaving one register with the first value's pair sums in one half of the lanes and the second's in the other, so
+// N registers become N / 4 before the four narrow steps (8, 4, 2, 1 within a row of 16 lanes). Every value is summed
+// by the same tree whatever N is, so a result does not depend on how many others were reduced with it.
+// On return v[j] holds, in lane l with l % 16 == j, the sum of value fold_var<N>(l); the other lanes of the row hold the
+// same sum. fold_owner<N>(l): lane l is the one lane that keeps its value (l % 16 < registers left).
+template <int N>
+__device__ __forceinline__ int fold_var(uint32_t lane) {
+  if (N == 1) return 0;
+  if (N == 2) return lane >> 5;
+  return 4 * (lane & 15) + 2 * ((lane >> 4) & 1) + (lane >> 5);
+}
+template <int N>
+__device__ __forceinline__ bool fold_owner(uint32_t lane) {
+  if (N == 1) return lane == 0;
+  if (N == 2) return (lane & 31) == 0;
+  return (lane & 15) < N / 4;
+}
+template <int N>
+__device__ __forceinline__ float fold_sum(float (&v)[N], uint32_t lane) {
+  static_assert(N == 1 || N == 2 || N == 4 || N == 8 || N == 16, "fold_sum: 1, 2, 4, 8 or 16 values");
+  auto add32 = [](float a, float b) {
+    auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(a), __float_as_uint(b), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+  };
+  auto add16 = [](float a, float b) {
+    auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(a), __float_as_uint(b), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+  };
+  constexpr int N1 = N >= 2 ? N / 2 : 1, N2 = N >= 4 ? N / 4 : 1;
+#pragma unroll
+  for (int j = 0; j < N1; ++j) v[j] = N >= 2 ? add32(v[2 * j], v[2 * j + 1]) : add32(v[0], v[0]);
+#pragma unroll
+  for (int j = 0; j < N2; ++j) v[j] = N >= 4 ? add16(v[2 * j], v[2 * j + 1]) : add16(v[0], v[0]);
+#pragma unroll
+  for (int j = 0; j < N2; ++j) {
+    v[j] = dpp_add<0x140>(v[j]);  // row_mirror (distance 8: both lanes' rows of eight hold different eights)
+    v[j] = dpp_add<0x141>(v[j]);  // row_half_mirror
+    v[j] = dpp_add<0x4E>(v[j]);   // quad_perm [2,3,0,1]
+    v[j] = dpp_add<0xB1>(v[j]);   // quad_perm [1,0,3,2]
+  }
+  float r = v[0];
+#pragma unroll
+  for (int j = 1; j < N2; ++j) r = (lane & 15) == (uint32_t)j ? v[j] : r;
+  return r;
+}
 __device__ __forceinline__ uint64_t wave_max_u64(uint64_t v) {
   auto step = [](uint64_t x, uint32_t olo, uint32_t ohi) {
     const uint64_t o = ((uint64_t)ohi << 32) | olo;

@@ -25,9 +25,13 @@ void dsgx_decode_cfg_default(dsgx_decode_cfg* c) {
 }
 
 static size_t ws_h_bytes(const dsgx_layer_w* L) { return (size_t)(DSGX_MAX_UNION + 1) * DSGX_MAX_ROWS * L->I * 2; }
+// after h and the barrier words: the slot-partitioned down phase's slot table (kFacBytes) and its f32 results
+// [slot][8 rows][H]
+static constexpr size_t kFacBytes = (size_t)(8 + (DSGX_MAX_UNION + 1) * 8) * 4 + 192;  // (a multiple of 256)
+static size_t ws_part_bytes(const dsgx_layer_w* L) { return kFacBytes + (size_t)(DSGX_MAX_UNION + 1) * 8 * L->H * 4; }
 size_t dsgx_decode_ws_bytes(const dsgx_layer_w* L) {
-  if (!L || L->I <= 0) return 0;
-  return ws_h_bytes(L) + kBarBytes;
+  if (!L || L->I <= 0 || L->H <= 0) return 0;
+  return ws_h_bytes(L) + kBarBytes + ws_part_bytes(L);
 }
 size_t dsgx_decode_ws_flag_offset(const dsgx_layer_w* L) {
   if (!L || L->I <= 0) return 0;
@@ -83,6 +87,8 @@ int dsgx_moe_decode(const dsgx_layer_w* L, const uint16_t* x, const int* idx, co
   a.x = x, a.M = M, a.idx = idx, a.w = w, a.logits = c.logits, a.bias = c.bias, a.route_scale = c.route_scale, a.score_fn = c.score_fn;
   a.L = *L, a.h = static_cast<uint16_t*>(ws), a.yr = yr, a.ys = ys, a.ysum = c.ysum;
   a.bar = reinterpret_cast<int*>(static_cast<uint8_t*>(ws) + ws_h_bytes(L));
+  a.fac = reinterpret_cast<float*>(static_cast<uint8_t*>(ws) + ws_h_bytes(L) + kBarBytes);
+  a.dpart = reinterpret_cast<float*>(static_cast<uint8_t*>(ws) + ws_h_bytes(L) + kBarBytes + kFacBytes);
   a.spin_limit = 1 << 22;
 #ifdef DSGX_TRACE
   a.trace = g_trace_buf;

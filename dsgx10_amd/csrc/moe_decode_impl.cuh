@@ -71,6 +71,8 @@ struct DecodeArgs {
   float* ys;
   int ysum;
   int* bar;     // the grid barrier's words in the workspace (grid_barrier)
+  float* dpart; // the slot-partitioned down phase's results, f32 [slot][M][H] (k_down_part -> k_down_combine)
+  float* fac;   // its slot table: fac[0] = slots (as int bits), fac[8 + slot * 8 + m] = s2_down * w of row m
 #ifdef DSGX_TRACE
   unsigned long long* trace;
 #endif
@@ -391,6 +393,41 @@ __device__ __forceinline__ void up_phase(const DecodeArgs& a, uint4* xs, Step<M>
   }
 }
 
+// ---- a sub-batch's dot products, reduced over the lanes ----------------------------------------------------------------
+// The RB x M sums of a sub-batch (output q = i * M + m) in groups of up to 16 through fold_sum: own_var<NV>(g, lane) is
+// the output of group g that `lane` keeps after reduce_own (-1: none), red[g] its sum.
+template <int NV> struct Pow2Ceil { static constexpr int v = NV <= 1 ? 1 : NV <= 2 ? 2 : NV <= 4 ? 4 : NV <= 8 ? 8 : 16; };
+template <int NV>
+__device__ __forceinline__ int own_var(int g, uint32_t lane) {
+  const int n = NV - 16 * g < 16 ? NV - 16 * g : 16;
+  int q = -1;
+  // (the group's size is a compile-time value in each branch)
+  if (n <= 1) q = fold_owner<1>(lane) ? fold_var<1>(lane) : -1;
+  else if (n <= 2) q = fold_owner<2>(lane) ? fold_var<2>(lane) : -1;
+  else if (n <= 4) q = fold_owner<4>(lane) ? fold_var<4>(lane) : -1;
+  else if (n <= 8) q = fold_owner<8>(lane) ? fold_var<8>(lane) : -1;
+  else q = fold_owner<16>(lane) ? fold_var<16>(lane) : -1;
+  return q >= 0 && q < n ? 16 * g + q : -1;
+}
+template <int RB, int M, int G>
+__device__ __forceinline__ float reduce_group(float (&acc)[RB][M], uint32_t lane) {
+  constexpr int NV = RB * M, n = NV - 16 * G < 16 ? NV - 16 * G : 16, NP = Pow2Ceil<n>::v;
+  float t[NP];
+#pragma unroll
+  for (int q = 0; q < NP; ++q) {
+    const int idx = 16 * G + q;
+    t[q] = 0.f;
+    if (idx < NV) t[q] = acc[idx / M][idx % M], acc[idx / M][idx % M] = 0.f;
+  }
+  return fold_sum<NP>(t, lane);
+}
+template <int RB, int M>
+__device__ __forceinline__ void reduce_own(float (&acc)[RB][M], uint32_t lane, float (&red)[(RB * M + 15) / 16]) {
+  red[0] = reduce_group<RB, M, 0>(acc, lane);
+  if constexpr (RB * M > 16) red[1] = reduce_group<RB, M, 1>(acc, lane);
+  static_assert(RB * M <= 32, "reduce_own: two groups at most");
+}
+
 // ---- down ------------------------------------------------------------------------------------------------------------------
 // The wave's rows [n_lo, n_hi) in sub-batches of RB (2, or 3 where the rows divide so: the launch picks); per sub-batch
 // every slot in order. hs: LDS for `spc` slots' h.
@@ -413,11 +450,19 @@ __device__ __forceinline__ void down_phase(const DecodeArgs& a, uint4* hs, Step<
   if (lane == 0) atomicMax(&s_maxsub, nsub);
 
   Raw w[D][RB];
-  float yacc[RB][M], sacc[RB][M], acc[RB][M];
+  float acc[RB][M];
 #pragma unroll
   for (int r = 0; r < RB; ++r)
 #pragma unroll
-    for (int m = 0; m < M; ++m) yacc[r][m] = sacc[r][m] = acc[r][m] = 0.f;
+    for (int m = 0; m < M; ++m) acc[r][m] = 0.f;
+  // A slot's dot products are reduced over the lanes when the slot completes (reduce_own: lane l then holds the sum of
+  // ITS output, number own_q of the sub-batch's RB x M), and the lane chains its output's slots in order:
+  // y = fma(s2 w, dot, y) with complete dots, as the reference states it (decode.cu:526-566).
+  constexpr int NG = (RB * M + 15) / 16;
+  float yown[NG], sown[NG];
+  int own_q[NG];
+#pragma unroll
+  for (int g = 0; g < NG; ++g) yown[g] = sown[g] = 0.f, own_q[g] = own_var<RB * M>(g, lane);
   int lsub = 0, ls = 0, lseg = 0;  // the load cursor (scalar): sub-batch, slot, segment
   bool lsh = kMixed && nsh > 0;    // the slot under the load cursor is the shared one in another format
   RowSrc src[RB];
@@ -486,46 +531,37 @@ __device__ __forceinline__ void down_phase(const DecodeArgs& a, uint4* hs, Step<
     }
     if (++cseg < (sh ? segs_s : segs_r)) return;
     cseg = 0;
-    // the slot is complete: into the rows' running sums, in slot (= expert id) order
+    // the slot is complete: into the outputs' running sums, in slot (= expert id) order
     const float s2 = S.slots[cs].d.s2;
+    float red[NG];
+    reduce_own<RB, M>(acc, lane, red);
 #pragma unroll
-    for (int i = 0; i < RB; ++i)
-#pragma unroll
-      for (int m = 0; m < M; ++m) {
-        if (sh) sacc[i][m] = acc[i][m];
-        else yacc[i][m] = fmaf(__fmul_rn(s2, S.wslot[cs - nsh][m]), acc[i][m], yacc[i][m]);
-        acc[i][m] = 0.f;
-      }
+    for (int g = 0; g < NG; ++g) {
+      if (sh) sown[g] = red[g];
+      else yown[g] = fmaf(__fmul_rn(s2, S.wslot[cs - nsh][own_q[g] >= 0 ? own_q[g] % M : 0]), red[g], yown[g]);
+    }
     if (++cs < nsl) {
       if (cs == c0 + spc) c0 += spc;
       return;
     }
     cs = 0, c0 = 0;
-    // the sub-batch is complete: add the lanes; lane i * M + m keeps output (row n0 + i, activation row m)
+    // the sub-batch is complete: the owning lanes store output (row n0 + q / M, activation row q % M)
     const int n0 = n_lo + csub * RB;
     ++csub;
-    float yv = 0.f, sv = 0.f;
 #pragma unroll
-    for (int i = 0; i < RB; ++i)
-#pragma unroll
-      for (int m = 0; m < M; ++m) {
-        const float v = wave_sum(yacc[i][m]);
-        if (lane == i * M + m) yv = v;
-        if (SHFMT != 0) {
-          const float s = wave_sum(sacc[i][m]);
-          if (lane == i * M + m) sv = s;
+    for (int g = 0; g < NG; ++g) {
+      if (live && own_q[g] >= 0) {
+        const int i = own_q[g] / M, m = own_q[g] % M;
+        if (n0 + i < n_hi) {
+          const size_t o = (size_t)m * H + n0 + i;
+          float yv = yown[g], sv = sown[g];
+          if (SHFMT != 0) a.ys[o] = sv;
+          else if (a.ysum) sv = a.ys[o];
+          if (a.ysum) yv = __fadd_rn(yv, sv);
+          a.yr[o] = yv;
         }
-        yacc[i][m] = sacc[i][m] = 0.f;
       }
-    if (live && lane < RB * M) {
-      const int i = lane / M, m = lane % M;
-      if (n0 + i < n_hi) {
-        const size_t o = (size_t)m * H + n0 + i;
-        if (SHFMT != 0) a.ys[o] = sv;
-        else if (a.ysum) sv = a.ys[o];
-        if (a.ysum) yv = __fadd_rn(yv, sv);
-        a.yr[o] = yv;
-      }
+      yown[g] = sown[g] = 0.f;
     }
   };
   if (one_chunk) {
@@ -546,6 +582,131 @@ __device__ __forceinline__ void down_phase(const DecodeArgs& a, uint4* hs, Step<
       }
     }
   }
+}
+
+// ---- down, partitioned by slot ---------------------------------------------------------------------------------------------
+// For steps whose h does not fit LDS (several rows with a large union): the rows-of-all-slots order above would bring
+// every slot's h into every workgroup, as many bytes again as the weights. Here the (slot, row) pairs are cut into equal
+// contiguous ranges, one a workgroup: a range spans two or three slots, whose h is staged once each; the complete dot
+// products go to memory as f32 [slot][M][H] and k_down_combine chains them in slot order: the same sums, by the same
+// tree and in the same order, as down_phase (a row's result is the same bits either way).
+template <int F, int M, int D>
+__device__ __forceinline__ void down_part_body(const DecodeArgs& a, uint4* hs, const Step<M>& S, int s0, int ns, int g, int G) {
+  constexpr int RB = 2;
+  const int H = a.L.H, I = a.L.I, nq = I / 8, segs = num_segs<F>(I);
+  const uint32_t lane = threadIdx.x & 63;
+  const int wave = uni((int)(threadIdx.x >> 6)), nw = blockDim.x >> 6;
+  const int sps = (H + RB - 1) / RB;  // sub-batches a slot
+  const long total = (long)ns * sps;
+  const int t_lo = (int)(total * g / G), t_hi = (int)(total * (g + 1) / G);
+  constexpr int NG = (RB * M + 15) / 16;
+  int own_q[NG];
+#pragma unroll
+  for (int q = 0; q < NG; ++q) own_q[q] = own_var<RB * M>(q, lane);
+  for (int sl = t_lo / sps; sl * sps < t_hi; ++sl) {  // (the same for every wave of the workgroup)
+    const int ta = max(t_lo, sl * sps) - sl * sps, tb = min(t_hi, (sl + 1) * sps) - sl * sps;  // its sub-batches of this slot
+    const Slot& T = S.slots[s0 + sl];
+    __syncthreads();
+    stage_slots<FmtT<F>::KL, false>(hs, 1, M, I, [&](int) { return a.h + (size_t)T.hslot * M * I; });
+    __syncthreads();
+    MatRef dr{};
+    dr.w = uni(T.d.w), dr.s = uni(T.d.s);
+    const MatDev dm = mat_dev<F>(dr, H, I);
+    float* out = a.dpart + (size_t)(s0 + sl) * M * H;
+    const int nsub = uni(tb - ta > wave ? (tb - ta - wave + nw - 1) / nw : 0);  // the wave's: ta + wave, + nw, ...
+    if (nsub == 0) continue;
+    const int steps = nsub * segs;
+    Raw w[D][RB];
+    float acc[RB][M];
+#pragma unroll
+    for (int r = 0; r < RB; ++r)
+#pragma unroll
+      for (int m = 0; m < M; ++m) acc[r][m] = 0.f;
+    int lsub = 0, lseg = 0, csub = 0, cseg = 0;
+    RowSrc src[RB];
+    auto open = [&](int sub) {
+      const int n0 = (ta + wave + min(sub, nsub - 1) * nw) * RB;  // (past the end: the last sub-batch again, unused)
+#pragma unroll
+      for (int i = 0; i < RB; ++i) src[i] = row_src<F>(dm, min(n0 + i, H - 1), I);
+    };
+    open(0);
+    auto load = [&](Raw (&r)[RB]) {
+#pragma unroll
+      for (int i = 0; i < RB; ++i) load_row<F>(r[i], src[i], lseg, lane, 7, acc[i][0]);
+      if (++lseg == segs) lseg = 0, open(++lsub);
+    };
+    auto compute = [&](const Raw (&r)[RB]) {
+      step_dot<F, M, RB>(r, hs, nq, cseg, lane, acc);
+      if (++cseg < segs) return;
+      cseg = 0;
+      float red[NG];
+      reduce_own<RB, M>(acc, lane, red);
+      const int n0 = (ta + wave + csub * nw) * RB;
+      ++csub;
+#pragma unroll
+      for (int q = 0; q < NG; ++q)
+        if (own_q[q] >= 0) {
+          const int i = own_q[q] / M, m = own_q[q] % M;
+          if (n0 + i < H) out[(size_t)m * H + n0 + i] = red[q];
+        }
+    };
+#pragma unroll
+    for (int d = 0; d < D; ++d) load(w[d]);
+    for (int t = 0; t < steps; t += D) {
+#pragma unroll
+      for (int d = 0; d < D; ++d) {
+        if (t + d < steps) compute(w[d]);
+        load(w[d]);
+      }
+    }
+  }
+}
+
+template <int FMT, int SHFMT, int M>
+__global__ void __launch_bounds__(DSGX_DECODE_THREADS) k_down_part(DecodeArgs a, int shared_wgs) {
+  extern __shared__ uint4 lds[];
+  __shared__ Step<M> S;
+  constexpr bool kMixed = SHFMT != 0 && SHFMT != FMT;
+  constexpr int nsh = SHFMT != 0 ? 1 : 0;
+  {
+    constexpr int NR = resolver_waves<M>();
+    const int wave = uni((int)(threadIdx.x >> 6)), nw = blockDim.x >> 6;
+    ResolveRegs rr;
+    if (wave >= nw - NR) resolve_fetch(S, a, wave - (nw - NR), NR, rr);
+    prep<FMT, SHFMT, M>(S, a);
+    __syncthreads();
+    if (wave >= nw - NR) resolve<FMT, SHFMT, M>(S, a, wave - (nw - NR), NR, rr);
+    __syncthreads();
+  }
+  const int nrouted = uni(S.n);
+  if (blockIdx.x == 0) {  // the slot table for k_down_combine
+    if (threadIdx.x == 0) reinterpret_cast<int*>(a.fac)[0] = nrouted;
+    for (int i = threadIdx.x; i < nrouted * M; i += blockDim.x)
+      a.fac[8 + (i / M) * 8 + i % M] = __fmul_rn(S.slots[nsh + i / M].d.s2, S.wslot[i / M][i % M]);
+  }
+  if (kMixed) {
+    if ((int)blockIdx.x < shared_wgs) down_part_body<SHFMT == 0 ? FMT : SHFMT, M, 4>(a, lds, S, 0, 1, blockIdx.x, shared_wgs);
+    else down_part_body<FMT, M, 4>(a, lds, S, 1, nrouted, (int)blockIdx.x - shared_wgs, (int)gridDim.x - shared_wgs);
+  } else {
+    down_part_body<FMT, M, 4>(a, lds, S, 0, nsh + nrouted, blockIdx.x, gridDim.x);
+  }
+}
+
+// yr[m][n] = the slots' dots chained in slot (expert id) order, acc = fma(s2 w, dot, acc); ys = the shared slot's dot
+template <int M, bool SH>
+__global__ void __launch_bounds__(256) k_down_combine(DecodeArgs a) {
+  const int H = a.L.H, nrouted = reinterpret_cast<const int*>(a.fac)[0];
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= M * H) return;
+  const int m = i / H;
+  const float* d = a.dpart + (size_t)(SH ? 1 : 0) * M * H + i;
+  float acc = 0.f;
+  for (int s = 0; s < nrouted; ++s) acc = fmaf(a.fac[8 + s * 8 + m], d[(size_t)s * M * H], acc);
+  float sv = 0.f;
+  if (SH) a.ys[i] = sv = a.dpart[i];
+  else if (a.ysum) sv = a.ys[i];
+  if (a.ysum) acc = __fadd_rn(acc, sv);
+  a.yr[i] = acc;
 }
 
 // ---- the grid barrier ---------------------------------------------------------------------------------------------------------
@@ -656,6 +817,27 @@ int launch_decode(const DecodeArgs& a, int parts, hipStream_t st) {
     return std::max(1, std::min(grid - 1, (int)(grid * bsh / (bsh + bro) + 0.5)));
   };
   (void)SF;
+  // h of all the slots does not fit a workgroup's LDS: gate/up as its own launch, then the down phase partitioned by
+  // slot and its combine (three launches; every row's bits are those of the other paths)
+  const bool part_ok = slot_bytes <= 64 * 1024;
+  if ((parts & 2) && part_ok && nsl_max > slots_per_chunk(parts == 3 && DSGX_WGS == 1 ? 96 * 1024 : 40 * 1024)) {
+    if (parts & 1) {
+      auto kern = k_up<FMT, SHFMT, M>;
+      if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds_up)) return rc;
+      const int grid = cus * DSGX_WGS;
+      hipLaunchKernelGGL(kern, dim3(grid), dim3(DSGX_DECODE_THREADS), lds_up, st, a, shared_split(grid));
+      DSGX_HIP(hipGetLastError());
+    }
+    auto kern = k_down_part<FMT, SHFMT, M>;
+    if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), slot_bytes)) return rc;
+    const int grid = cus * DSGX_WGS;
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(DSGX_DECODE_THREADS), slot_bytes, st, a, shared_split(grid));
+    DSGX_HIP(hipGetLastError());
+    if (SHFMT != 0) hipLaunchKernelGGL((k_down_combine<M, true>), dim3((M * H + 255) / 256), dim3(256), 0, st, a);
+    else hipLaunchKernelGGL((k_down_combine<M, false>), dim3((M * H + 255) / 256), dim3(256), 0, st, a);
+    DSGX_HIP(hipGetLastError());
+    return DSGX_OK;
+  }
   if (parts == 3) {
     // rows a wave in the down phase: sub-batches of three where that divides them evenly (built for the INT4 layers,
     // whose hidden size 6144 gives three rows a wave on 256 CUs), else of two
