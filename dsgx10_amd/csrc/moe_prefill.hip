@@ -516,6 +516,7 @@ __global__ void __launch_bounds__(kGemmThreads) k_pf_gemm16(Gemm16Args g) {
   // then moved to the MFMA's lane order (row l % 16, part l / 16) by a cross-lane permute, activations by their LDS slot
   const int lrow = lane >> 2, lq = lane & 3;
   const int perm_addr = 4 * (4 * r16 + part);
+  const int nmt = uni(min(8, (mend - m0 + 15) / 16));  // the tile's 16-position tiles that hold rows
   const int n0 = UP ? ns * (kWgRows / 2) + 16 * wave : ns * kWgRows + 32 * wave;  // UP: first channel; DOWN: first row
   // the lane's weight row of each of the wave's two tiles
   const uint8_t* pw[2];
@@ -628,6 +629,7 @@ __global__ void __launch_bounds__(kGemmThreads) k_pf_gemm16(Gemm16Args g) {
     }
 #pragma unroll
     for (int mt = 0; mt < 8; ++mt) {
+      if (mt >= nmt) break;  // (a ragged tile's 16-position tiles past its end: most experts hold fewer than 128 rows)
       u32x4_t fb[4];
 #pragma unroll
       for (int j = 0; j < 4; ++j) fb[j] = *reinterpret_cast<const u32x4_t*>(B + ((4 * mt + j) * 64 + lane) * 16);
