@@ -119,24 +119,37 @@ __global__ void __launch_bounds__(256) k_widen_fp8(const uint8_t* __restrict__ c
   *reinterpret_cast<uint4*>(out + (size_t)n * ld + 8 * q) = make_uint4(o[0], o[1], o[2], o[3]);
 }
 
-// act_quant(x, 128): one wavefront a (row, 128-k block), two values a lane
+// act_quant(x, 128): sixteen lanes a (row, 128-k block), eight values (one 16-byte load) a lane; the block's largest
+// magnitude by four DPP steps within the row of 16 lanes
 // (ds41f-4xgx10-switchless/ref/torchref/kernel.py:56-77 of the reference, scale_fmt None)
 __global__ void __launch_bounds__(256) k_act_quant(const uint16_t* __restrict__ x, int T, int K, uint8_t* __restrict__ q, float* __restrict__ s) {
-  const int KB = K / 128, lane = threadIdx.x & 63;
-  const size_t blk = (size_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
-  if (blk >= (size_t)T * KB) return;
-  const size_t t = blk / KB, b = blk % KB;
-  const uint32_t xv = *reinterpret_cast<const uint32_t*>(x + t * K + 128 * b + 2 * lane);
-  const float a = bf16_bits_to_f32(xv & 0xFFFFu), c = bf16_bits_to_f32(xv >> 16);
-  float amax = fmaxf(fabsf(a), fabsf(c));
+  const int KB = K / 128, l16 = threadIdx.x & 15;
+  const size_t blk = (size_t)blockIdx.x * (blockDim.x >> 4) + (threadIdx.x >> 4);
+  if (blk >= (size_t)T * KB) return;  // (whole rows of 16 lanes leave together)
+  const size_t t = blk / KB, b = blk % KB, at = t * K + 128 * b + 8 * l16;
+  const u32x4_t xv = *reinterpret_cast<const DSGX_GLOBAL u32x4_t*>((uintptr_t)(x + at));
+  float v[8];
 #pragma unroll
-  for (int o = 32; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o));
+  for (int i = 0; i < 4; ++i) v[2 * i] = bf16_bits_to_f32(xv[i] & 0xFFFFu), v[2 * i + 1] = bf16_bits_to_f32(xv[i] >> 16);
+  float amax = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(v[i]));
+  amax = dpp_max<0xB1>(amax);
+  amax = dpp_max<0x4E>(amax);
+  amax = dpp_max<0x141>(amax);
+  amax = dpp_max<0x140>(amax);
   amax = fmaxf(amax, 1e-4f);
   const float sc = __fmul_rn(amax, 1.0f / 448.0f);
-  if (lane == 0) s[t * KB + b] = sc;
-  const float qa = fminf(448.f, fmaxf(-448.f, __fdiv_rn(a, sc))), qc = fminf(448.f, fmaxf(-448.f, __fdiv_rn(c, sc)));
-  const uint32_t pk = __builtin_amdgcn_cvt_pk_fp8_f32(qa, qc, 0, false);
-  *reinterpret_cast<uint16_t*>(q + t * K + 128 * b + 2 * lane) = (uint16_t)(pk & 0xFFFFu);
+  if (l16 == 0) s[t * KB + b] = sc;
+  float qv[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) qv[i] = fminf(448.f, fmaxf(-448.f, __fdiv_rn(v[i], sc)));
+  uint32_t o[2];
+  o[0] = __builtin_amdgcn_cvt_pk_fp8_f32(qv[0], qv[1], 0, false);
+  o[0] = __builtin_amdgcn_cvt_pk_fp8_f32(qv[2], qv[3], o[0], true);
+  o[1] = __builtin_amdgcn_cvt_pk_fp8_f32(qv[4], qv[5], 0, false);
+  o[1] = __builtin_amdgcn_cvt_pk_fp8_f32(qv[6], qv[7], o[1], true);
+  *reinterpret_cast<uint2*>(q + at) = make_uint2(o[0], o[1]);
 }
 
 }  // namespace
@@ -227,7 +240,7 @@ int dsgx_widen_fp8(const void* codes, int N, int K, uint16_t* out, size_t ld, vo
 int dsgx_act_quant(const uint16_t* x, int T, int K, uint8_t* q, float* s, void* stream) {
   if (!x || !q || !s || T < 1 || K < 128 || K % 128) return fail(DSGX_EINVAL, "act_quant: [%d][%d] (K a multiple of 128)", T, K);
   const size_t nb = (size_t)T * (K / 128);
-  hipLaunchKernelGGL(k_act_quant, dim3((unsigned)((nb + 3) / 4)), dim3(256), 0, static_cast<hipStream_t>(stream), x, T, K, q, s);
+  hipLaunchKernelGGL(k_act_quant, dim3((unsigned)((nb + 15) / 16)), dim3(256), 0, static_cast<hipStream_t>(stream), x, T, K, q, s);
   DSGX_HIP(hipGetLastError());
   return DSGX_OK;
 }

@@ -812,8 +812,8 @@ int launch_decode(const DecodeArgs& a, int parts, hipStream_t st) {
   auto shared_split = [&](int grid) {
     if (!kMixed) return 0;
     // the workgroups split between the BF16 shared expert and the routed experts by their bytes, an INT4 byte counted
-    // as 2.2 BF16 bytes (it holds four times the values, and the gate/up phase is bound by their decoding)
-    const double bsh = 2.0 * I * H * 2, bro = 2.2 * (double)std::min(a.M * a.L.topk, a.L.E) * 2.0 * (double)dsgx_mat_bytes(FMT, I, H);
+    // as 2.45 BF16 bytes (it holds four times the values, and the gate/up phase is bound by their decoding)
+    const double bsh = 2.0 * I * H * 2, bro = 2.45 * (double)std::min(a.M * a.L.topk, a.L.E) * 2.0 * (double)dsgx_mat_bytes(FMT, I, H);
     return std::max(1, std::min(grid - 1, (int)(grid * bsh / (bsh + bro) + 0.5)));
   };
   (void)SF;
@@ -842,7 +842,11 @@ int launch_decode(const DecodeArgs& a, int parts, hipStream_t st) {
     // rows a wave in the down phase: sub-batches of three where that divides them evenly (built for the INT4 layers,
     // whose hidden size 6144 gives three rows a wave on 256 CUs), else of two
     const int rpw = (H + cus * (DSGX_DECODE_THREADS / 64) - 1) / (cus * (DSGX_DECODE_THREADS / 64));
+#ifdef DSGX_NO_RB3
+    const bool rb3 = false;
+#else
     const bool rb3 = FMT == DSGX_FMT_INT4_G32 && rpw % 3 == 0;
+#endif
     auto kern = rb3 ? k_decode<FMT, SHFMT, M, (FMT == DSGX_FMT_INT4_G32 ? 3 : 2)> : k_decode<FMT, SHFMT, M, 2>;
     const int spc = slots_per_chunk(DSGX_WGS == 1 ? 96 * 1024 : 40 * 1024);
     const size_t lds = std::max(lds_up, (size_t)spc * slot_bytes);

@@ -65,8 +65,9 @@ __global__ void __launch_bounds__(64) k_probe_mfma_fp8(const uint8_t* __restrict
 
 // ---- the workspace -------------------------------------------------------------------------------------------------------
 constexpr int kTile = 128;  // rows of a tile (token positions) and weight rows a workgroup
+constexpr int kRowBlock = 128;  // token rows a workgroup of the bucketing kernels
 struct PfLayout {
-  size_t cnt, off, ntiles, tile_e, tile_m0, perm, pickpos, rpos, re, rk, xq, xs, h, hq, hs, hsh, hshq, hshs, d, total;
+  size_t cnt, off, ntiles, tile_e, tile_m0, perm, pickpos, rpos, re, rk, xq, xs, h, hq, hs, hsh, hshq, hshs, d, bcnt, boff, bmask, total;
   int P, max_tiles;
 };
 PfLayout pf_layout(const dsgx_layer_w* L, int T) {
@@ -83,69 +84,93 @@ PfLayout pf_layout(const dsgx_layer_w* L, int T) {
   o.h = take(P * I * 2), o.hq = take(P * I), o.hs = take(P * (I / 128) * 4);
   o.hsh = take((size_t)T * I * 2), o.hshq = take((size_t)T * I), o.hshs = take((size_t)T * (I / 128) * 4);
   o.d = take(P * H * 4);
+  const size_t NB = ((size_t)T + kRowBlock - 1) / kRowBlock;  // the bucketing's row blocks
+  o.bcnt = take(NB * E * 4), o.boff = take(NB * E * 4), o.bmask = take(NB * E * 16);
   o.total = at;
   return o;
 }
 
 // ---- bucketing -----------------------------------------------------------------------------------------------------------
-// picks of expert e (one workgroup an expert)
-__global__ void __launch_bounds__(256) k_pf_count(const int* __restrict__ idx, int P, int* __restrict__ cnt) {
-  const int e = blockIdx.x;
-  int c = 0;
-  for (int p = threadIdx.x; p < P; p += blockDim.x) c += idx[p] == e;
-  __shared__ int part[4];
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) c += __shfl_xor(c, o);
-  if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = c;
+// Positions inside an expert's bucket follow the picks' order (row-major over [T][topk]); a row picks an expert at most
+// once, so that is the order of the rows. Three launches:
+//   k_pf_mask   a workgroup a block of 128 rows: for every expert the 128-bit mask of the block's rows that picked it
+//               (LDS atomics), stored with its population count;
+//   k_pf_scan   one workgroup, a thread an expert: the blocks' counts summed in block order (each block's offset inside
+//               the bucket), the buckets' offsets and the list of 128-row tiles in expert order by two scans;
+//   k_pf_place  a workgroup a block, a thread a pick: position = bucket offset + block offset + rows of the block below
+//               this one in the expert's mask; and, per row, its picks in expert-id order (ids are distinct in a row):
+//               expert, bucket position, the combine's factor s2 * w.
+__global__ void __launch_bounds__(256) k_pf_mask(const int* __restrict__ idx, int T, int topk, int E, int* __restrict__ bcnt,
+                                                 uint32_t* __restrict__ bmask) {
+  __shared__ uint32_t mask[DSGX_MAX_EXPERTS * 4];
+  const int b = blockIdx.x, t0 = b * kRowBlock, rows = min(kRowBlock, T - t0);
+  for (int i = threadIdx.x; i < E * 4; i += blockDim.x) mask[i] = 0;
   __syncthreads();
-  if (threadIdx.x == 0) cnt[e] = part[0] + part[1] + part[2] + part[3];
-}
-// bucket offsets and the list of 128-row tiles in expert order (one thread: E <= 512)
-__global__ void k_pf_scan(const int* __restrict__ cnt, int E, int* __restrict__ off, int* __restrict__ ntiles, int* __restrict__ tile_e,
-                          int* __restrict__ tile_m0) {
-  if (threadIdx.x != 0 || blockIdx.x != 0) return;
-  int at = 0, nt = 0;
-  for (int e = 0; e < E; ++e) {
-    off[e] = at;
-    for (int m0 = 0; m0 < cnt[e]; m0 += kTile) tile_e[nt] = e, tile_m0[nt] = m0, ++nt;
-    at += cnt[e];
+  for (int i = threadIdx.x; i < rows * topk; i += blockDim.x) {
+    const int r = i / topk, e = idx[(size_t)t0 * topk + i];
+    atomicOr(&mask[e * 4 + (r >> 5)], 1u << (r & 31));
   }
-  off[E] = at;
-  *ntiles = nt;
-}
-// the picks of expert e in pick order (row-major over [T][topk]) to positions off[e] ...: perm[position] = row,
-// pickpos[pick] = position
-__global__ void __launch_bounds__(256) k_pf_scatter(const int* __restrict__ idx, int P, int topk, const int* __restrict__ off,
-                                                    int* __restrict__ perm, int* __restrict__ pickpos) {
-  const int e = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  __shared__ int wcnt[4];
-  int base = off[e];
-  for (int p0 = 0; p0 < P; p0 += 256) {
-    const int p = p0 + threadIdx.x;
-    const bool hit = p < P && idx[p] == e;
-    const uint64_t m = __ballot(hit);
-    if (lane == 0) wcnt[wave] = __popcll(m);
-    __syncthreads();
-    int before = __popcll(m & ((1ull << lane) - 1));
-    for (int w = 0; w < wave; ++w) before += wcnt[w];
-    if (hit) perm[base + before] = p / topk, pickpos[p] = base + before;
-    base += wcnt[0] + wcnt[1] + wcnt[2] + wcnt[3];
-    __syncthreads();
+  __syncthreads();
+  for (int e = threadIdx.x; e < E; e += blockDim.x) {
+    const uint4 m = *reinterpret_cast<const uint4*>(&mask[e * 4]);
+    bcnt[(size_t)b * E + e] = __popc(m.x) + __popc(m.y) + __popc(m.z) + __popc(m.w);
+    *reinterpret_cast<uint4*>(&bmask[((size_t)b * E + e) * 4]) = m;
   }
 }
-// per row: its picks in expert-id order (ids are distinct in a row): expert, bucket position, combine factor s2 * w
-__global__ void __launch_bounds__(256) k_pf_rowsort(const int* __restrict__ idx, const float* __restrict__ w, const int* __restrict__ pickpos,
-                                                    const dsgx_mat_desc* __restrict__ desc, int T, int topk, int* __restrict__ rpos,
-                                                    int* __restrict__ re, float* __restrict__ rk) {
-  const int t = blockIdx.x * blockDim.x + threadIdx.x;
-  if (t >= T) return;
-  for (int k = 0; k < topk; ++k) {
-    const int e = idx[t * topk + k];
-    int r = 0;
-    for (int j = 0; j < topk; ++j) r += idx[t * topk + j] < e;
-    re[t * topk + r] = e;
-    rpos[t * topk + r] = pickpos[t * topk + k];
-    rk[t * topk + r] = __fmul_rn(desc[(size_t)e * 3 + 2].s2, w[t * topk + k]);
+__global__ void __launch_bounds__(DSGX_MAX_EXPERTS) k_pf_scan(const int* __restrict__ bcnt, int NB, int E, int* __restrict__ boff,
+                                                              int* __restrict__ cnt, int* __restrict__ off, int* __restrict__ ntiles,
+                                                              int* __restrict__ tile_e, int* __restrict__ tile_m0) {
+  __shared__ int sa[DSGX_MAX_EXPERTS], sb[DSGX_MAX_EXPERTS];
+  const int e = threadIdx.x;
+  int c = 0;
+  if (e < E)
+    for (int b = 0; b < NB; ++b) {
+      const int v = bcnt[(size_t)b * E + e];
+      boff[(size_t)b * E + e] = c;
+      c += v;
+    }
+  const int nt = (c + kTile - 1) / kTile;
+  sa[e] = e < E ? c : 0, sb[e] = e < E ? nt : 0;
+  __syncthreads();
+  for (int d = 1; d < DSGX_MAX_EXPERTS; d <<= 1) {  // inclusive scans of the counts and of the tile counts
+    const int va = e >= d ? sa[e - d] : 0, vb = e >= d ? sb[e - d] : 0;
+    __syncthreads();
+    sa[e] += va, sb[e] += vb;
+    __syncthreads();
+  }
+  if (e < E) {
+    cnt[e] = c;
+    off[e] = sa[e] - c;
+    if (e == E - 1) off[E] = sa[e], *ntiles = sb[e];
+    const int t0 = sb[e] - nt;
+    for (int i = 0; i < nt; ++i) tile_e[t0 + i] = e, tile_m0[t0 + i] = i * kTile;
+  }
+}
+__global__ void __launch_bounds__(256) k_pf_place(const int* __restrict__ idx, const float* __restrict__ w, int T, int topk, int E,
+                                                  const int* __restrict__ off, const int* __restrict__ boff,
+                                                  const uint32_t* __restrict__ bmask, const dsgx_mat_desc* __restrict__ desc,
+                                                  int* __restrict__ perm, int* __restrict__ pickpos, int* __restrict__ rpos,
+                                                  int* __restrict__ re, float* __restrict__ rk) {
+  __shared__ uint32_t mask[DSGX_MAX_EXPERTS * 4];
+  __shared__ int base[DSGX_MAX_EXPERTS];
+  const int b = blockIdx.x, t0 = b * kRowBlock, rows = min(kRowBlock, T - t0);
+  for (int i = threadIdx.x; i < E * 4; i += blockDim.x) mask[i] = bmask[(size_t)b * E * 4 + i];
+  for (int e = threadIdx.x; e < E; e += blockDim.x) base[e] = off[e] + boff[(size_t)b * E + e];
+  __syncthreads();
+  for (int i = threadIdx.x; i < rows * topk; i += blockDim.x) {
+    const int r = i / topk, k = i % topk, t = t0 + r, e = idx[(size_t)t * topk + k];
+    int below = 0;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const uint32_t m = mask[e * 4 + q];
+      below += q < (r >> 5) ? __popc(m) : q == (r >> 5) ? __popc(m & ((1u << (r & 31)) - 1)) : 0;
+    }
+    const int pos = base[e] + below;
+    perm[pos] = t, pickpos[(size_t)t * topk + k] = pos;
+    int rank = 0;
+    for (int j = 0; j < topk; ++j) rank += idx[(size_t)t * topk + j] < e;
+    const size_t o = (size_t)t * topk + rank;
+    re[o] = e, rpos[o] = pos, rk[o] = __fmul_rn(desc[(size_t)e * 3 + 2].s2, w[(size_t)t * topk + k]);
   }
 }
 
@@ -774,11 +799,13 @@ int dsgx_moe_prefill(const dsgx_layer_w* L, const uint16_t* x, const int* idx, c
   if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(k_pf_gemm<false>), lds)) return rc;
 
   if (cfg.phases & 1) {
-    hipLaunchKernelGGL(k_pf_count, dim3(E), dim3(256), 0, st, idx, P, I32(o.cnt));
-    hipLaunchKernelGGL(k_pf_scan, dim3(1), dim3(64), 0, st, I32(o.cnt), E, I32(o.off), I32(o.ntiles), I32(o.tile_e), I32(o.tile_m0));
-    hipLaunchKernelGGL(k_pf_scatter, dim3(E), dim3(256), 0, st, idx, P, topk, I32(o.off), I32(o.perm), I32(o.pickpos));
-    hipLaunchKernelGGL(k_pf_rowsort, dim3((T + 255) / 256), dim3(256), 0, st, idx, w, I32(o.pickpos), L->desc, T, topk, I32(o.rpos),
-                       I32(o.re), F32(o.rk));
+    const int NB = (T + kRowBlock - 1) / kRowBlock;
+    uint32_t* bmask = reinterpret_cast<uint32_t*>(W + o.bmask);
+    hipLaunchKernelGGL(k_pf_mask, dim3(NB), dim3(256), 0, st, idx, T, topk, E, I32(o.bcnt), bmask);
+    hipLaunchKernelGGL(k_pf_scan, dim3(1), dim3(DSGX_MAX_EXPERTS), 0, st, I32(o.bcnt), NB, E, I32(o.boff), I32(o.cnt), I32(o.off), I32(o.ntiles),
+                       I32(o.tile_e), I32(o.tile_m0));
+    hipLaunchKernelGGL(k_pf_place, dim3(NB), dim3(256), 0, st, idx, w, T, topk, E, I32(o.off), I32(o.boff), bmask, L->desc, I32(o.perm),
+                       I32(o.pickpos), I32(o.rpos), I32(o.re), F32(o.rk));
     DSGX_HIP(hipGetLastError());
   }
   if (i4) {
