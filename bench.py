@@ -33,9 +33,9 @@ def log(*a):
 
 
 # HBM bytes a launch of the FP8 M=1 gate/up kernel, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs of this script,
-# each scaled by what the counter reads for a kernel of known size in the same run (profiles/): 152,215,347 read +
-# 6,553,600 written (algorithmic bytes: 151,031,808)
-UP_TRAFFIC_FP8_M1 = 158768947
+# each scaled by what the counter reads for a kernel of known size in the same run (profiles/): 152,222,720 read +
+# 2,359,296 written (algorithmic bytes: 151,031,808)
+UP_TRAFFIC_FP8_M1 = 154582016
 
 
 def prefill_extra(gen, T, name, peak):
