@@ -517,11 +517,13 @@ struct Gemm16Args {
   float* d;            // DOWN: f32 [position][H]
 };
 
-// WF: the weights' format (DSGX_FMT_INT4_G32: the routed experts; DSGX_FMT_BF16: the shared expert, gate/up interleaved)
+// WF: the weights' format (DSGX_FMT_INT4_G32: the routed experts; DSGX_FMT_BF16: the shared expert, gate/up interleaved;
+// DSGX_FMT_FP8_B128: e4m3 experts or shared expert with bf16 activations, the reference engine's own prefill contract
+// for FP8 weights, prefill.cu:337-352: per 128-k block the bf16 x bf16 products summed from zero, acc = fma(S, sum, acc))
 template <bool UP, int WF>
 __global__ void __launch_bounds__(kGemmThreads) k_pf_gemm16(Gemm16Args g) {
   extern __shared__ uint8_t smem[];
-  constexpr bool I4 = WF == DSGX_FMT_INT4_G32;
+  constexpr bool I4 = WF == DSGX_FMT_INT4_G32, F8 = WF == DSGX_FMT_FP8_B128;
   const int K = UP ? g.L.H : g.L.I, N = UP ? g.L.I : g.L.H, KB = K / 128;
   const int NS = UP ? g.L.I / (kWgRows / 2) : g.L.H / kWgRows;
   int tile, ns;
@@ -564,6 +566,24 @@ __global__ void __launch_bounds__(kGemmThreads) k_pf_gemm16(Gemm16Args g) {
       zsh[t] = 4 * (n & 7);
     }
     if (UP) s2a = d[0].s2, s2b = d[1].s2;
+  } else if (F8) {
+    const uint8_t *wa, *wb;
+    const float *sa, *sb;
+    if (e < 0) {
+      if (UP) wa = g.L.sh.g, sa = g.L.sh.gs, wb = g.L.sh.u, sb = g.L.sh.us;
+      else wa = wb = g.L.sh.d, sa = sb = g.L.sh.ds;
+    } else {
+      const dsgx_mat_desc* d = g.L.desc + (size_t)e * 3;
+      if (UP) wa = g.L.pool + d[0].off, wb = g.L.pool + d[1].off, s2a = d[0].s2, s2b = d[1].s2;
+      else wa = wb = g.L.pool + d[2].off;
+      const size_t NK = (size_t)g.L.H * g.L.I;
+      sa = reinterpret_cast<const float*>(wa + (NK + 255) / 256 * 256);
+      sb = reinterpret_cast<const float*>(wb + (NK + 255) / 256 * 256);
+    }
+    pw[0] = wa + (size_t)(n0 + lrow) * K + lq * 16;
+    pw[1] = (UP ? wb + (size_t)(n0 + lrow) * K : wa + (size_t)(n0 + 16 + lrow) * K) + lq * 16;
+    ps[0] = reinterpret_cast<const uint8_t*>(sa + (size_t)(n0 / 128) * KB);  // the tiles' scale rows (32 rows: one 128-row block)
+    ps[1] = UP ? reinterpret_cast<const uint8_t*>(sb + (size_t)(n0 / 128) * KB) : ps[0];
   } else {
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
@@ -581,8 +601,10 @@ __global__ void __launch_bounds__(kGemmThreads) k_pf_gemm16(Gemm16Args g) {
   }
   // Activation load i of a lane is the 16-byte piece c = 4 i + lq of its row's block (k = 8 c ...): the piece of MFMA j,
   // part p with c = 4 p + j (INT4 map: k = 32 p + 8 j) or c = 4 j + p (BF16 map: k = 32 j + 8 p).
+  // FP8 map: a lane's 32 codes are the 16 at 16 p and the 16 at 64 + 16 p of the block: k = 64 (j / 2) + 16 p + 8 (j % 2), c = k / 8.
   auto slot_of = [&](int i) {
-    const int c = 4 * i + lq, j = I4 ? c & 3 : c >> 2, p = I4 ? c >> 2 : c & 3;
+    const int c = 4 * i + lq;
+    const int j = I4 ? c & 3 : F8 ? 2 * (c >> 3) + (c & 1) : c >> 2, p = I4 ? c >> 2 : F8 ? (c >> 1) & 3 : c & 3;
     return ((4 * wave + j) * 64 + p * 16 + lrow) * 16;
   };
 
@@ -592,11 +614,21 @@ __global__ void __launch_bounds__(kGemmThreads) k_pf_gemm16(Gemm16Args g) {
 #pragma unroll
     for (int mt = 0; mt < 8; ++mt) acc[t][mt] = v4f_t{};
 
-  constexpr int kRing16 = I4 ? 3 : 2;
+  constexpr int kRing16 = I4 || F8 ? 3 : 2;
   struct WRegs {
-    u32x4_t v[I4 ? 1 : 4];
+    u32x4_t v[I4 ? 1 : F8 ? 2 : 4];
     uint32_t s, z;
   };
+  // FP8: the wave's weight scales, lane l holding those of block kb0 + l for the 64 blocks from kb0 (a load inside the
+  // turn would be a wait for every load before it)
+  float ws_l[2] = {1.f, 1.f};
+  auto load_ws = [&](int kb0) {
+    if (F8) {
+      const int kc = min(kb0 + lane, KB - 1);
+      ws_l[0] = reinterpret_cast<const float*>(ps[0])[kc], ws_l[1] = reinterpret_cast<const float*>(ps[1])[kc];
+    }
+  };
+  load_ws(0);
   WRegs ra[kRing16][2];
   auto load_a = [&](int slot, int kb) {
     const int kc = kb < KB ? kb : KB - 1;
@@ -607,10 +639,14 @@ __global__ void __launch_bounds__(kGemmThreads) k_pf_gemm16(Gemm16Args g) {
         ra[slot][t].v[0] = ldg_stream(p);
         ra[slot][t].s = ldg_u16(ps[t] + (size_t)kc * 8);
         ra[slot][t].z = ldg_u32(pz[t] + (size_t)kc * 16);
+      } else if (F8) {
+        const uint8_t* p = pin_after(pw[t] + (size_t)kc * 128, acc[t][0][0]);
+        ra[slot][t].v[0] = *reinterpret_cast<const DSGX_GLOBAL u32x4_t*>((uintptr_t)p);
+        ra[slot][t].v[F8 ? 1 : 0] = *reinterpret_cast<const DSGX_GLOBAL u32x4_t*>((uintptr_t)(p + 64));
       } else {
         const uint8_t* p = pin_after(pw[t] + (size_t)kc * 256, acc[t][0][0]);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) ra[slot][t].v[j] = ldg_stream(p + 64 * j);
+        for (int j = 0; j < 4; ++j) ra[slot][t].v[I4 || F8 ? 0 : j] = ldg_stream(p + 64 * j);
       }
     }
   };
@@ -625,8 +661,14 @@ __global__ void __launch_bounds__(kGemmThreads) k_pf_gemm16(Gemm16Args g) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) *reinterpret_cast<u32x4_t*>(B + slot_of(j)) = rx[j];
   };
-  auto compute = [&](int slot, int stage) {
+  auto compute = [&](int slot, int stage, int kb) {
     const uint8_t* B = smem + (size_t)stage * kPanel16;
+    float wsc[2] = {1.f, 1.f};
+    if (F8) {
+      if ((kb & 63) == 0 && kb > 0) load_ws(kb);
+#pragma unroll
+      for (int t = 0; t < 2; ++t) wsc[t] = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, ws_l[t]), kb & 63));
+    }
     // the wave's two A tiles of the block as bf16 fragments
     u32x4_t fa[2][4];
 #pragma unroll
@@ -643,11 +685,23 @@ __global__ void __launch_bounds__(kGemmThreads) k_pf_gemm16(Gemm16Args g) {
           i4x8_to_bf16(j == 0 ? w.x : j == 1 ? w.y : j == 2 ? w.z : w.w, sc, nzs, o);
           fa[t][j] = u32x4_t{o[0], o[1], o[2], o[3]};
         }
+      } else if (F8) {
+        auto mv = [&](uint32_t v) { return (uint32_t)__builtin_amdgcn_ds_bpermute(perm_addr, (int)v); };
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          const u32x4_t wl = keep_whole(ra[slot][t].v[F8 ? h : 0]);
+          const u32x4_t w = u32x4_t{mv(wl.x), mv(wl.y), mv(wl.z), mv(wl.w)};
+          uint32_t o[4];
+          fp8x8_to_bf16(w.x, w.y, o);
+          fa[t][2 * h] = u32x4_t{o[0], o[1], o[2], o[3]};
+          fp8x8_to_bf16(w.z, w.w, o);
+          fa[t][2 * h + 1] = u32x4_t{o[0], o[1], o[2], o[3]};
+        }
       } else {
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           auto mv = [&](uint32_t v) { return (uint32_t)__builtin_amdgcn_ds_bpermute(perm_addr, (int)v); };
-          const u32x4_t wl = keep_whole(ra[slot][t].v[j]);
+          const u32x4_t wl = keep_whole(ra[slot][t].v[I4 || F8 ? 0 : j]);
           fa[t][j] = u32x4_t{mv(wl.x), mv(wl.y), mv(wl.z), mv(wl.w)};
         }
       }
@@ -658,12 +712,25 @@ __global__ void __launch_bounds__(kGemmThreads) k_pf_gemm16(Gemm16Args g) {
       u32x4_t fb[4];
 #pragma unroll
       for (int j = 0; j < 4; ++j) fb[j] = *reinterpret_cast<const u32x4_t*>(B + ((4 * mt + j) * 64 + lane) * 16);
+      if (F8) {  // the block's sum from zero, then the scaled add
+        v4f_t p[2] = {v4f_t{}, v4f_t{}};
 #pragma unroll
-      for (int j = 0; j < 4; ++j)
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+          for (int t = 0; t < 2; ++t)
+            p[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf_t, fa[t][j]), __builtin_bit_cast(v8bf_t, fb[j]), p[t], 0, 0, 0);
 #pragma unroll
         for (int t = 0; t < 2; ++t)
-          acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf_t, fa[t][j]), __builtin_bit_cast(v8bf_t, fb[j]),
-                                                               acc[t][mt], 0, 0, 0);
+#pragma unroll
+          for (int q = 0; q < 4; ++q) acc[t][mt][q] = fmaf(wsc[t], p[t][q], acc[t][mt][q]);
+      } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+          for (int t = 0; t < 2; ++t)
+            acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf_t, fa[t][j]), __builtin_bit_cast(v8bf_t, fb[j]),
+                                                                 acc[t][mt], 0, 0, 0);
+      }
     }
   };
   // prologue
@@ -682,7 +749,7 @@ __global__ void __launch_bounds__(kGemmThreads) k_pf_gemm16(Gemm16Args g) {
     for (int v = 0; v < kUnroll; ++v) {
       const int kb = kb0 + v;
       fetch_x(kb + 2);
-      if (kb < KB) compute(v % kRing16, v % kStages16);
+      if (kb < KB) compute(v % kRing16, v % kStages16, kb);
       load_a(v % kRing16, kb + kRing16);
       stash_x((v + 2) % kStages16);
       __syncthreads();
@@ -783,7 +850,6 @@ int dsgx_moe_prefill(const dsgx_layer_w* L, const uint16_t* x, const int* idx, c
   if (!x || !idx || !w || !ws || !yr) return fail(DSGX_EINVAL, "moe_prefill: null x, idx, w, ws or yr");
   if (!L->pool || !L->desc) return fail(DSGX_EINVAL, "moe_prefill: layer without pool or descriptors");
   const bool i4 = L->fmt == DSGX_FMT_INT4_G32;
-  if (!i4 && !cfg.act_fp8) return fail(DSGX_EUNSUPPORTED, "moe_prefill: FP8 layers with bf16 activations (act_fp8 = 0) are not built yet");
   if (cfg.shared && !i4 && L->sh.bgu) return fail(DSGX_EUNSUPPORTED, "moe_prefill: a BF16 shared expert in an FP8 layer is not built yet");
   if (cfg.shared && i4 && L->sh.g) return fail(DSGX_EUNSUPPORTED, "moe_prefill: an FP8 shared expert in an INT4 layer is not built yet");
   const bool shared = cfg.shared && (i4 ? (L->sh.bgu && L->sh.bd) : layer_has_fp8_shared(L));
@@ -808,13 +874,14 @@ int dsgx_moe_prefill(const dsgx_layer_w* L, const uint16_t* x, const int* idx, c
                        I32(o.pickpos), I32(o.rpos), I32(o.re), F32(o.rk));
     DSGX_HIP(hipGetLastError());
   }
-  if (i4) {
-    // bf16 activations throughout: x -> h (bf16) -> d (f32 a pick) -> combine; the BF16 shared expert likewise -> ys
+  if (i4 || !cfg.act_fp8) {
+    // bf16 activations throughout: x -> h (bf16) -> d (f32 a pick) -> combine; the shared expert likewise -> ys.
+    // INT4 layers (BF16 shared expert), or FP8 layers under the engine's own contract (act_fp8 = 0; FP8 shared expert)
     const size_t lds16 = (size_t)kStages16 * kPanel16;
-    auto k_up = k_pf_gemm16<true, DSGX_FMT_INT4_G32>;
-    auto k_dn = k_pf_gemm16<false, DSGX_FMT_INT4_G32>;
-    auto k_sup = k_pf_gemm16<true, DSGX_FMT_BF16>;
-    auto k_sdn = k_pf_gemm16<false, DSGX_FMT_BF16>;
+    auto k_up = i4 ? k_pf_gemm16<true, DSGX_FMT_INT4_G32> : k_pf_gemm16<true, DSGX_FMT_FP8_B128>;
+    auto k_dn = i4 ? k_pf_gemm16<false, DSGX_FMT_INT4_G32> : k_pf_gemm16<false, DSGX_FMT_FP8_B128>;
+    auto k_sup = i4 ? k_pf_gemm16<true, DSGX_FMT_BF16> : k_pf_gemm16<true, DSGX_FMT_FP8_B128>;
+    auto k_sdn = i4 ? k_pf_gemm16<false, DSGX_FMT_BF16> : k_pf_gemm16<false, DSGX_FMT_FP8_B128>;
     for (const void* k : {(const void*)k_up, (const void*)k_dn, (const void*)k_sup, (const void*)k_sdn})
       if (int rc = allow_dynamic_lds(k, lds16)) return rc;
     Gemm16Args q{};
