@@ -261,6 +261,41 @@ __device__ __forceinline__ int wait_slots(Step<M>& S) {
 // The routing is resolved late: the workgroup's batches of slot 0 (nsl0 = 1: a fused shared expert; 0: none) need no
 // routing; a wave whose next batch lies beyond them calls wait_nsl(), which waits for the resolvers (wait_slots())
 // and returns the number of slots. Every wave calls it before it leaves (its last claim lies beyond any count).
+// ---- a sub-batch's dot products, reduced over the lanes ----------------------------------------------------------------
+// The RB x M sums of a sub-batch (output q = i * M + m) in groups of up to 16 through fold_sum: own_var<NV>(g, lane) is
+// the output of group g that `lane` keeps after reduce_own (-1: none), red[g] its sum.
+template <int NV> struct Pow2Ceil { static constexpr int v = NV <= 1 ? 1 : NV <= 2 ? 2 : NV <= 4 ? 4 : NV <= 8 ? 8 : 16; };
+template <int NV>
+__device__ __forceinline__ int own_var(int g, uint32_t lane) {
+  const int n = NV - 16 * g < 16 ? NV - 16 * g : 16;
+  int q = -1;
+  // (the group's size is a compile-time value in each branch)
+  if (n <= 1) q = fold_owner<1>(lane) ? fold_var<1>(lane) : -1;
+  else if (n <= 2) q = fold_owner<2>(lane) ? fold_var<2>(lane) : -1;
+  else if (n <= 4) q = fold_owner<4>(lane) ? fold_var<4>(lane) : -1;
+  else if (n <= 8) q = fold_owner<8>(lane) ? fold_var<8>(lane) : -1;
+  else q = fold_owner<16>(lane) ? fold_var<16>(lane) : -1;
+  return q >= 0 && q < n ? 16 * g + q : -1;
+}
+template <int RB, int M, int G>
+__device__ __forceinline__ float reduce_group(float (&acc)[RB][M], uint32_t lane) {
+  constexpr int NV = RB * M, n = NV - 16 * G < 16 ? NV - 16 * G : 16, NP = Pow2Ceil<n>::v;
+  float t[NP];
+#pragma unroll
+  for (int q = 0; q < NP; ++q) {
+    const int idx = 16 * G + q;
+    t[q] = 0.f;
+    if (idx < NV) t[q] = acc[idx / M][idx % M], acc[idx / M][idx % M] = 0.f;
+  }
+  return fold_sum<NP>(t, lane);
+}
+template <int RB, int M>
+__device__ __forceinline__ void reduce_own(float (&acc)[RB][M], uint32_t lane, float (&red)[(RB * M + 15) / 16]) {
+  red[0] = reduce_group<RB, M, 0>(acc, lane);
+  if constexpr (RB * M > 16) red[1] = reduce_group<RB, M, 1>(acc, lane);
+  static_assert(RB * M <= 32, "reduce_own: two groups at most");
+}
+
 template <int FMT, int M, bool INTER, int CH, int D, class WaitNsl>
 __device__ __forceinline__ void up_body(const DecodeArgs& a, const uint4* xs, const Slot* slots, int nsl0, int* counter, int g, int G,
                                         WaitNsl&& wait_nsl) {
@@ -317,34 +352,32 @@ __device__ __forceinline__ void up_body(const DecodeArgs& a, const uint4* xs, co
   auto compute = [&](const Raw (&r)[RB], int csl, int cp, int cseg) {
     step_dot<FMT, M, RB>(r, xs, nq, cseg, lane, acc);
     if (cseg + 1 < nsegk) return;
-    // lane m < M finishes the batch's channel(s) of activation row m and stores them as one 16- or 32-bit word. The
-    // store is coherent at device scope (it bypasses the XCD-local L2): the down phase of the same kernel reads h on
-    // other XCDs right after the grid barrier.
-    float gv[CH], uv[CH];
+    // The batch's CH x M gate sums and up sums are reduced over the lanes by two fold_sums (the same tree whatever their
+    // number), after which output q = c * M + m (channel c, activation row m) is owned by one lane, which finishes it and
+    // stores its 16 bits. The store is coherent at device scope (it bypasses the XCD-local L2): the down phase of the
+    // same kernel reads h on other XCDs right after the grid barrier.
+    constexpr int NP = Pow2Ceil<CH * M>::v;
+    float tg[NP], tu[NP];
 #pragma unroll
-    for (int c = 0; c < CH; ++c) gv[c] = uv[c] = 0.f;
+    for (int q = 0; q < NP; ++q) tg[q] = tu[q] = 0.f;
 #pragma unroll
     for (int i = 0; i < RB; ++i)
 #pragma unroll
       for (int m = 0; m < M; ++m) {
-        const float v = wave_sum(acc[i][m]);
-        acc[i][m] = 0.f;
         const int ch = INTER ? i >> 1 : i % CH;
         const bool up = INTER ? (i & 1) : (i >= CH);
-        if (lane == m) {
-          if (up) uv[ch] = v;
-          else gv[ch] = v;
-        }
+        if (up) tu[ch * M + m] = acc[i][m];
+        else tg[ch * M + m] = acc[i][m];
+        acc[i][m] = 0.f;
       }
-    if (lane < M) {
+    const float gsum = fold_sum<NP>(tg, lane), usum = fold_sum<NP>(tu, lane);
+    const int q = fold_var<NP>(lane);
+    if (fold_owner<NP>(lane) && q < CH * M) {
       const Slot& S = slots[csl];
-      const float sg = S.g.s2, su = S.u.s2;
-      uint32_t hb = 0;
-#pragma unroll
-      for (int c = 0; c < CH; ++c) hb |= swiglu_bits(bf16_round(__fmul_rn(gv[c], sg)), bf16_round(__fmul_rn(uv[c], su))) << (16 * c);
-      uint16_t* dst = a.h + ((size_t)S.hslot * M + lane) * I + CH * cp;
-      if (CH == 1) __hip_atomic_store((DSGX_GLOBAL uint16_t*)(uintptr_t)dst, (uint16_t)hb, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      else __hip_atomic_store((DSGX_GLOBAL uint32_t*)(uintptr_t)dst, hb, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const int c = q / M, m = q % M;
+      const uint32_t hb = swiglu_bits(bf16_round(__fmul_rn(gsum, S.g.s2)), bf16_round(__fmul_rn(usum, S.u.s2)));
+      uint16_t* dst = a.h + ((size_t)S.hslot * M + m) * I + CH * cp + c;
+      __hip_atomic_store((DSGX_GLOBAL uint16_t*)(uintptr_t)dst, (uint16_t)hb, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
   };
   // software pipeline: a ring of D steps in flight; every turn computes the oldest step and issues a load in its place
@@ -391,41 +424,6 @@ __device__ __forceinline__ void up_phase(const DecodeArgs& a, uint4* xs, Step<M>
   } else {
     up_body<FMT, M, false, kUpCH, kUpD>(a, xs, S.slots, nsh, &S.next_up, blockIdx.x, gridDim.x, [&] { return nsh + wait_slots(S); });
   }
-}
-
-// ---- a sub-batch's dot products, reduced over the lanes ----------------------------------------------------------------
-// The RB x M sums of a sub-batch (output q = i * M + m) in groups of up to 16 through fold_sum: own_var<NV>(g, lane) is
-// the output of group g that `lane` keeps after reduce_own (-1: none), red[g] its sum.
-template <int NV> struct Pow2Ceil { static constexpr int v = NV <= 1 ? 1 : NV <= 2 ? 2 : NV <= 4 ? 4 : NV <= 8 ? 8 : 16; };
-template <int NV>
-__device__ __forceinline__ int own_var(int g, uint32_t lane) {
-  const int n = NV - 16 * g < 16 ? NV - 16 * g : 16;
-  int q = -1;
-  // (the group's size is a compile-time value in each branch)
-  if (n <= 1) q = fold_owner<1>(lane) ? fold_var<1>(lane) : -1;
-  else if (n <= 2) q = fold_owner<2>(lane) ? fold_var<2>(lane) : -1;
-  else if (n <= 4) q = fold_owner<4>(lane) ? fold_var<4>(lane) : -1;
-  else if (n <= 8) q = fold_owner<8>(lane) ? fold_var<8>(lane) : -1;
-  else q = fold_owner<16>(lane) ? fold_var<16>(lane) : -1;
-  return q >= 0 && q < n ? 16 * g + q : -1;
-}
-template <int RB, int M, int G>
-__device__ __forceinline__ float reduce_group(float (&acc)[RB][M], uint32_t lane) {
-  constexpr int NV = RB * M, n = NV - 16 * G < 16 ? NV - 16 * G : 16, NP = Pow2Ceil<n>::v;
-  float t[NP];
-#pragma unroll
-  for (int q = 0; q < NP; ++q) {
-    const int idx = 16 * G + q;
-    t[q] = 0.f;
-    if (idx < NV) t[q] = acc[idx / M][idx % M], acc[idx / M][idx % M] = 0.f;
-  }
-  return fold_sum<NP>(t, lane);
-}
-template <int RB, int M>
-__device__ __forceinline__ void reduce_own(float (&acc)[RB][M], uint32_t lane, float (&red)[(RB * M + 15) / 16]) {
-  red[0] = reduce_group<RB, M, 0>(acc, lane);
-  if constexpr (RB * M > 16) red[1] = reduce_group<RB, M, 1>(acc, lane);
-  static_assert(RB * M <= 32, "reduce_own: two groups at most");
 }
 
 // ---- down ------------------------------------------------------------------------------------------------------------------
