@@ -11,8 +11,9 @@
 //   4  down     h quantised; grouped GEMM, each pick's f32 result row kept (d)
 //   8  combine  yr[t] = sum over the row's picks in expert-id order of fma(s2 * w, d, acc) (decode.cu:526-566's order)
 //   16 shared   the fused FP8 shared expert on all T rows with the same two GEMMs -> ys
-// The GEMMs run on v_mfma_f32_32x32x64_f8f6f4: weights are the A operand (rows n), activations the B operand, so a
-// lane's 16 accumulators of a 32 x 32 tile belong to ONE token row and the block's combined scale is one value a lane.
+// The FP8-activation GEMMs run on v_mfma_f32_16x16x128_f8f6f4 (one instruction a 128-k scale block), the bf16-activation
+// ones on v_mfma_f32_16x16x32_bf16: weights are the A operand (rows n), activations the B operand, so a lane's four
+// accumulators of a 16 x 16 tile belong to ONE token row and the block's combined scale is one value a lane.
 #include "abi_internal.h"
 #include "common.cuh"
 
@@ -180,9 +181,10 @@ __global__ void __launch_bounds__(256) k_pf_place(const int* __restrict__ idx, c
 // rows as two 16-row MFMA tiles (UP: 16 gate rows and the 16 up rows of the same channels, so g and u of a channel meet
 // in one lane) and streams them from memory straight into registers, a ring of kRing 128-k blocks ahead: a lane loads
 // 2 x 16 bytes a tile and block, the four lanes of a row 64 contiguous bytes an instruction. The activations of the
-// tile (shared by the eight waves) go through LDS, kStages blocks ahead, stored in the order of the MFMA fragments (the
-// operand reads are then linear in the lane: no bank conflicts). All global loads are issued with four consecutive
-// lanes on 64 contiguous bytes of a row; the weights are brought into the MFMA's lane order by a cross-lane permute.
+// tile (shared by the eight waves) wait kHold turns in registers and go through kStages LDS stages, stored by MFMA
+// fragment with an exclusive-or in the slot number that keeps writes and reads free of bank conflicts. All global loads
+// are issued with four consecutive lanes on 64 contiguous bytes of a row; the weights are brought into the MFMA's lane
+// order through the wave's own piece of LDS (w_to_lds / read_fa).
 // v_mfma_f32_16x16x128_f8f6f4 covers one whole 128-k scale block: partial = A B^T from zero, then
 // acc = fma(x_scale * w_scale, partial, acc) on the vector unit (the accumulators therefore stay in ordinary registers).
 // With the weights as the A operand a lane's four accumulators of a tile belong to ONE position, so the combined scale is
@@ -280,8 +282,8 @@ __global__ void __launch_bounds__(kGemmThreads) k_pf_gemm(GemmArgs g) {
   const int tid = threadIdx.x, lane = tid & 63, wave = uni(tid >> 6), r16 = lane & 15, part = lane >> 4;
   // Loads are issued with lane l on row l / 4, 16-byte piece l % 4 of a 64-byte half row (four consecutive lanes read 64
   // contiguous bytes: the texture unit looks up one line for them, not one a lane), and the weights are then moved to the
-  // MFMA's lane order (row l % 16, piece l / 16) with one cross-lane permute a dword. The activations need no permute:
-  // they go to LDS, where each lane writes its piece to the slot of the fragment order.
+  // MFMA's lane order (row l % 16, piece l / 16) through LDS, as the activations are: each lane writes its piece to the
+  // slot of the fragment order.
   const int lrow = lane >> 2, lq = lane & 3;
   // the wave's two 16-row weight tiles
   const int n0 = UP ? ns * (kWgRows / 2) + 16 * wave : ns * kWgRows + 32 * wave;  // UP: first channel; DOWN: first row
