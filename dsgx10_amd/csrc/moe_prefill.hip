@@ -652,16 +652,21 @@ __global__ void __launch_bounds__(kGemmThreads) k_pf_gemm16(Gemm16Args g) {
       }
     }
   };
-  u32x4_t rx[4];
-  auto fetch_x = [&](int kb) {
+  // The activations of a block wait kHold16 turns in registers between their loads and their LDS writes (the memory
+  // latency is several turns long, and a wait for one load is a wait for every load issued before it).
+  constexpr int kHold16 = F8 ? 2 : 3;
+  struct XRegs16 {
+    u32x4_t v[4];
+  };
+  auto fetch_x = [&](XRegs16& r, int kb) {
     const int kc = kb < KB ? kb : KB - 1;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) rx[j] = *reinterpret_cast<const u32x4_t*>(px + (size_t)kc * 256 + 64 * j);
+    for (int j = 0; j < 4; ++j) r.v[j] = *reinterpret_cast<const u32x4_t*>(px + (size_t)kc * 256 + 64 * j);
   };
-  auto stash_x = [&](int stage) {
+  auto stash_x = [&](const XRegs16& r, int stage) {
     uint8_t* B = smem + (size_t)stage * kPanel16;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) *reinterpret_cast<u32x4_t*>(B + slot_of(j)) = rx[j];
+    for (int j = 0; j < 4; ++j) *reinterpret_cast<u32x4_t*>(B + slot_of(j)) = r.v[j];
   };
   auto compute = [&](int slot, int stage, int kb) {
     const uint8_t* B = smem + (size_t)stage * kPanel16;
@@ -738,22 +743,29 @@ __global__ void __launch_bounds__(kGemmThreads) k_pf_gemm16(Gemm16Args g) {
   // prologue
 #pragma unroll
   for (int d = 0; d < kRing16; ++d) load_a(d, d);
-  fetch_x(0);
-  stash_x(0);
-  fetch_x(1);
-  stash_x(1);
+  XRegs16 rx[kHold16];
+  {
+    XRegs16 t0, t1;
+    fetch_x(t0, 0), fetch_x(t1, 1);
+#pragma unroll
+    for (int v = 0; v < kHold16; ++v) fetch_x(rx[v], 2 + v);
+    stash_x(t0, 0), stash_x(t1, 1);
+  }
   __syncthreads();
-  // turn kb: issue the activation loads of block kb + 2, compute block kb, issue the weight loads of block kb + ring in
-  // its place, put the activations of block kb + 2 into their stage (last read a turn ago)
-  constexpr int kUnroll = kRing16 * kStages16 / (kRing16 == kStages16 ? kRing16 : 1);  // a common multiple of both
+  // turn kb: the activations of block kb + 2 (loaded kHold16 turns ago; set kb % kHold16) go to their stage (last read a
+  // turn ago) and the loads of block kb + 2 + kHold16 are issued in their place; compute block kb; the weight loads of
+  // block kb + ring issued in its place. (Unrolled over a common multiple of the rotations.)
+  constexpr int kUnroll = 6;
+  static_assert(kUnroll % kRing16 == 0 && kUnroll % kStages16 == 0 && kUnroll % kHold16 == 0, "unroll");
   for (int kb0 = 0; kb0 < KB; kb0 += kUnroll) {
 #pragma unroll
     for (int v = 0; v < kUnroll; ++v) {
       const int kb = kb0 + v;
-      fetch_x(kb + 2);
-      if (kb < KB) compute(v % kRing16, v % kStages16, kb);
+      if (kb >= KB) break;
+      stash_x(rx[v % kHold16], (v + 2) % kStages16);
+      fetch_x(rx[v % kHold16], kb + 2 + kHold16);
+      compute(v % kRing16, v % kStages16, kb);
       load_a(v % kRing16, kb + kRing16);
-      stash_x((v + 2) % kStages16);
       __syncthreads();
     }
   }
