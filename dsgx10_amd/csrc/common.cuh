@@ -186,29 +186,6 @@ __device__ __forceinline__ float fold_sum(float (&v)[N], uint32_t lane) {
   for (int j = 1; j < N2; ++j) r = (lane & 15) == (uint32_t)j ? v[j] : r;
   return r;
 }
-__device__ __forceinline__ uint64_t wave_max_u64(uint64_t v) {
-  auto step = [](uint64_t x, uint32_t olo, uint32_t ohi) {
-    const uint64_t o = ((uint64_t)ohi << 32) | olo;
-    return o > x ? o : x;
-  };
-  v = step(v, dpp_mov<0xB1>((uint32_t)v), dpp_mov<0xB1>((uint32_t)(v >> 32)));
-  v = step(v, dpp_mov<0x4E>((uint32_t)v), dpp_mov<0x4E>((uint32_t)(v >> 32)));
-  v = step(v, dpp_mov<0x141>((uint32_t)v), dpp_mov<0x141>((uint32_t)(v >> 32)));
-  v = step(v, dpp_mov<0x140>((uint32_t)v), dpp_mov<0x140>((uint32_t)(v >> 32)));
-  {
-    auto lo = __builtin_amdgcn_permlane16_swap((uint32_t)v, (uint32_t)v, false, false);
-    auto hi = __builtin_amdgcn_permlane16_swap((uint32_t)(v >> 32), (uint32_t)(v >> 32), false, false);
-    const uint64_t a = ((uint64_t)hi[0] << 32) | lo[0], b = ((uint64_t)hi[1] << 32) | lo[1];
-    v = a > b ? a : b;
-  }
-  {
-    auto lo = __builtin_amdgcn_permlane32_swap((uint32_t)v, (uint32_t)v, false, false);
-    auto hi = __builtin_amdgcn_permlane32_swap((uint32_t)(v >> 32), (uint32_t)(v >> 32), false, false);
-    const uint64_t a = ((uint64_t)hi[0] << 32) | lo[0], b = ((uint64_t)hi[1] << 32) | lo[1];
-    v = a > b ? a : b;
-  }
-  return v;
-}
 
 // ---- the activation layout in LDS ---------------------------------------------------------------------------------------------
 // A lane of a wavefront that streams a row holds KL consecutive k per segment of 64 * KL k (KL = 16 for FP8: one
