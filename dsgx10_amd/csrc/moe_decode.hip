@@ -49,7 +49,8 @@ int dsgx_moe_decode(const dsgx_layer_w* L, const uint16_t* x, const int* idx, co
   if (!c.logits && (!idx || !w)) return fail(DSGX_EINVAL, "moe_decode: idx and w, or logits");
   if (c.post) return fail(DSGX_EUNSUPPORTED, "moe_decode: posted outputs need the reference's ring; one GPU has none");
   if (c.parts < 1 || c.parts > 3) return fail(DSGX_EINVAL, "moe_decode: parts %d", c.parts);
-  if (c.up != 0 || c.down < 0 || c.down > 1) return fail(DSGX_EINVAL, "moe_decode: up variant %d / down variant %d", c.up, c.down);
+  if (c.up < 0 || c.up > 1 || c.down < 0 || c.down > 1) return fail(DSGX_EINVAL, "moe_decode: up variant %d / down variant %d", c.up, c.down);
+  if (c.up == 1 && L->fmt != DSGX_FMT_FP8_B128) return fail(DSGX_EUNSUPPORTED, "moe_decode: variant 1 (MFMA) is built for FP8_B128 layers");
   if (c.down == 1 && c.parts == 3) c.parts = 3 | 4;  // variant 1: the two phases as two launches
   if (L->fmt == DSGX_FMT_REF_NVFP4 || L->fmt == DSGX_FMT_REF_INT4 || L->fmt == DSGX_FMT_REF_BF16)
     return fail(DSGX_EFORMAT, "moe_decode: layer expert format %u names a GB10 block tiling; repack to FP8_B128 (16), INT4_G32 (18) or BF16 (19)", L->fmt);
@@ -97,6 +98,7 @@ int dsgx_moe_decode(const dsgx_layer_w* L, const uint16_t* x, const int* idx, co
   const uint32_t f = L->fmt;
   if (f == DSGX_FMT_FP8_B128) {
     if (b16sh) return fail(DSGX_EUNSUPPORTED, "moe_decode: FP8 experts with a BF16 shared expert are not built");
+    if (c.up == 1) return launch_decode_fp8_mfma(a, c.parts & 3, fp8sh, st);
     return launch_decode_fp8(a, c.parts, fp8sh, st);
   }
   if (f == DSGX_FMT_INT4_G32) {

@@ -23,9 +23,9 @@ def _layer(fmt, H, I, E, topk, NS, shared, random_codes=False, seed=1):
     return _cache[key]
 
 
-def _check_step(hl, dl, x, idx, w, M, scale_note=""):
+def _check_step(hl, dl, x, idx, w, M, scale_note="", **kw):
     E = hl.E
-    yr, ys, ws = gpu.decode_layer(dl, x[:M], idx[:M], w[:M], M)
+    yr, ys, ws = gpu.decode_layer(dl, x[:M], idx[:M], w[:M], M, **kw)
     uni = orc.union(idx[:M], E)
     U = len(uni)
     hg = gpu.h_of(ws, dl, M, U)
@@ -178,3 +178,23 @@ def test_decode_nine_to_sixteen_rows():
             y1, s1, _ = gpu.decode_layer(dl, x[m:m + 1], idx[m:m + 1], w[m:m + 1], 1)
             assert np.array_equal(y1[0].view(np.uint32), yr[m].view(np.uint32)), (M, m)
             assert np.array_equal(s1[0].view(np.uint32), ys[m].view(np.uint32)), (M, m)
+
+
+@pytest.mark.parametrize("case", CASES[:2], ids=lambda c: "fmt%d-H%d-I%d-E%d-%s" % (c[0], c[1], c[2], c[3], c[6]))
+def test_decode_mfma_variant(case):
+    """variant 1 (cfg.up = 1): the expert matmuls on the bf16 MFMA, FP8 layers; the same checks as the default's, and a
+    row's bits do not depend on the rows beside it (within the variant)"""
+    fmt, H, I, E, topk, NS, shared, scale = case
+    hl, dl = _layer(fmt, H, I, E, topk, NS, shared)
+    x, logits, idx, w = rows_and_routing(21, 8, H, E, topk, scale)
+    runs = {}
+    for M in (1, 3, 5, 8):
+        runs[M] = _check_step(hl, dl, x, idx, w, M, up=1)
+    for m in range(8):
+        yr1, ys1, _ = gpu.decode_layer(dl, x[m:m + 1], idx[m:m + 1], w[m:m + 1], 1, up=1)
+        assert np.array_equal(yr1[0].view(np.uint32), runs[8][0][m].view(np.uint32)), m
+        if hl.has_shared:
+            assert np.array_equal(ys1[0].view(np.uint32), runs[8][1][m].view(np.uint32)), m
+    # fused routing, and 9-16 rows as two passes
+    yr_l, ys_l, _ = gpu.decode_layer(dl, x, None, None, 8, logits=gpu.dev(logits), route_scale=scale, up=1)
+    assert np.array_equal(yr_l.view(np.uint32), runs[8][0].view(np.uint32))
