@@ -50,7 +50,8 @@ int dsgx_moe_decode(const dsgx_layer_w* L, const uint16_t* x, const int* idx, co
   if (c.post) return fail(DSGX_EUNSUPPORTED, "moe_decode: posted outputs need the reference's ring; one GPU has none");
   if (c.parts < 1 || c.parts > 3) return fail(DSGX_EINVAL, "moe_decode: parts %d", c.parts);
   if (c.up < 0 || c.up > 1 || c.down < 0 || c.down > 1) return fail(DSGX_EINVAL, "moe_decode: up variant %d / down variant %d", c.up, c.down);
-  if (c.up == 1 && L->fmt != DSGX_FMT_FP8_B128) return fail(DSGX_EUNSUPPORTED, "moe_decode: variant 1 (MFMA) is built for FP8_B128 layers");
+  if (c.up == 1 && L->fmt != DSGX_FMT_FP8_B128 && L->fmt != DSGX_FMT_INT4_G32)
+    return fail(DSGX_EUNSUPPORTED, "moe_decode: variant 1 (MFMA) is built for FP8_B128 and INT4_G32 layers");
   if (c.down == 1 && c.parts == 3) c.parts = 3 | 4;  // variant 1: the two phases as two launches
   if (L->fmt == DSGX_FMT_REF_NVFP4 || L->fmt == DSGX_FMT_REF_INT4 || L->fmt == DSGX_FMT_REF_BF16)
     return fail(DSGX_EFORMAT, "moe_decode: layer expert format %u names a GB10 block tiling; repack to FP8_B128 (16), INT4_G32 (18) or BF16 (19)", L->fmt);
@@ -103,6 +104,7 @@ int dsgx_moe_decode(const dsgx_layer_w* L, const uint16_t* x, const int* idx, co
   }
   if (f == DSGX_FMT_INT4_G32) {
     if (fp8sh) return fail(DSGX_EUNSUPPORTED, "moe_decode: INT4 experts with an FP8 shared expert are not built");
+    if (c.up == 1) return launch_decode_int4_mfma(a, c.parts & 3, b16sh, st);
     return launch_decode_int4(a, c.parts, b16sh, st);
   }
   if (fp8sh || b16sh) return fail(DSGX_EUNSUPPORTED, "moe_decode: BF16 experts with a fused shared expert are not built");

@@ -6,6 +6,6 @@ int launch_decode_fp8(const DecodeArgs& a, int parts, bool shared, hipStream_t s
   return shared ? launch_decode_m<DSGX_FMT_FP8_B128, DSGX_FMT_FP8_B128>(a, parts, st) : launch_decode_m<DSGX_FMT_FP8_B128, 0>(a, parts, st);
 }
 int launch_decode_fp8_mfma(const DecodeArgs& a, int parts, bool shared, hipStream_t st) {
-  return shared ? launch_decode_mfma_m<true>(a, parts, st) : launch_decode_mfma_m<false>(a, parts, st);
+  return shared ? launch_decode_mfma_m<DSGX_FMT_FP8_B128, DSGX_FMT_FP8_B128>(a, parts, st) : launch_decode_mfma_m<DSGX_FMT_FP8_B128, 0>(a, parts, st);
 }
 }  // namespace dsgx

@@ -1,13 +1,18 @@
-// Decode variant 1 (dsgx_decode_cfg::up = 1) for FP8-128x128 layers: the expert matmuls on v_mfma_f32_16x16x32_bf16.
+// Decode variant 1 (dsgx_decode_cfg::up = 1) for FP8-128x128 layers (with or without the fused FP8 shared expert) and
+// INT4-g32 layers (with or without the fused BF16 shared expert): the expert matmuls on v_mfma_f32_16x16x32_bf16.
 // The reference's decode kernels are tensor-core kernels too (engine/experts/decode.cu:307-343, 526-587: one MMA tile
 // holds up to 16 activation rows); here a tile is 16 WEIGHT rows as the MFMA's A operand and the step's rows (up to 16,
 // zero beyond M) as its B operand, so a row count costs nothing extra and no sum crosses lanes.
-//   * a unit = 16 weight rows x all of K; the eight waves of a workgroup split K in eight slices and walk the slice in
-//     steps of 64 k (1 KiB: lane l loads 16 bytes of row l / 4, four lanes 64 contiguous bytes of a row), a register ring
-//     kD steps ahead; the bytes reach the MFMA's lane order (row l % 16, k part l / 16) through 1 KiB of the wave's LDS;
-//   * e4m3 -> bf16 exactly in registers; per 128-k scale block the four MFMAs sum from zero, then
+//   * a unit = 16 weight rows x all of K; K is cut into `ns` slices (mf_slices) and the workgroup's eight waves form
+//     8 / ns groups: the waves of a group walk one unit, a slice each, in steps of 128 bytes a row (2 KiB a step: two
+//     loads, each eight rows x 128 contiguous bytes; 128 k of FP8, 256 k of INT4, 64 k of BF16), a register ring kMfD
+//     steps ahead; the bytes reach the MFMA's lane order (row l % 16, k part l / 16) through 2 KiB of the wave's LDS;
+//   * FP8: e4m3 -> bf16 exactly in registers; per 128-k scale block the four MFMAs sum from zero, then
 //     acc = fma(S, sum, acc) (the contract of the FP8 paths: decode.cu:269-306);
-//   * the waves' slice sums are added in wave order through LDS (one workgroup barrier a unit), then the epilogue.
+//   * INT4: a lane reads 16 bytes = the 32 values of one scale group of its row and feeds them to four MFMAs, eight
+//     values each (the activation fragment of MFMA j takes the same k: a sum does not mind the order of k inside a
+//     step); W = bf16((u - u_z) s) in registers, the decode kernels' routine and bits; the MFMAs accumulate over K;
+//   * the slices' sums are added in slice order through LDS (one workgroup barrier a round of units), then the epilogue.
 // gate/up: unit = 8 channels, rows interleaved (g0, u0, g1, u1, ...), so that g and u of a channel meet in one lane.
 // down: units are (slot, 16 output rows), cut into equal contiguous ranges a workgroup; the complete dots go to memory
 // as f32 [slot][M][H] and k_down_combine chains them in slot order (as after k_down_part).
@@ -19,15 +24,29 @@ namespace dsgx {
 
 typedef __bf16 v8bf_t __attribute__((ext_vector_type(8)));
 typedef float v4f_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
 constexpr int kMfD = 4;           // ring depth in steps
 constexpr int kMfPad = 64;        // bytes between activation rows in LDS beyond their length (bank spread)
 constexpr int kMfThreads = 512;   // eight waves a workgroup, one workgroup a CU
 constexpr int kMfWaves = kMfThreads / 64;
 
-// K is cut into slices of whole 128-k scale blocks, one a wave (waves beyond the slices idle: small K only)
-__host__ __device__ inline int mf_slices(int K) { return K / 128 < kMfWaves ? K / 128 : kMfWaves; }
+// k a step (128 bytes of a weight row)
+template <int FMT> struct MfFmt;
+template <> struct MfFmt<DSGX_FMT_FP8_B128> { static constexpr int STEPK = 128; };
+template <> struct MfFmt<DSGX_FMT_INT4_G32> { static constexpr int STEPK = 256; };
+template <> struct MfFmt<DSGX_FMT_BF16> { static constexpr int STEPK = 64; };
+
+// The slices of K: a power of two (1 .. 8) that divides the steps of K, four steps or more a slice where K allows
+// (fewer steps between two workgroup barriers cost more than they spread). With ns < 8 slices, 8 / ns groups of waves
+// work on different units at a time.
+__host__ __device__ inline int mf_slices(int K, int stepk) {
+  const int steps = K / stepk;
+  int ns = kMfWaves;
+  while (ns > 1 && (steps % ns || steps / ns < 4)) ns >>= 1;
+  return ns;
+}
 __host__ __device__ inline size_t mf_rows_bytes(int M, int K) { return (size_t)M * ((size_t)K * 2 + kMfPad) + 64; }
-// + two steps' weights a wave + the waves' slice sums of two units (the lanes of positions < M only: 4 M x 16 bytes a wave)
+// + one step's weights a wave + the waves' slice sums of two rounds (the lanes of positions < M only: 4 M x 16 bytes a wave)
 __host__ __device__ inline size_t mf_lds_bytes(int M, int K) { return mf_rows_bytes(M, K) + kMfWaves * 2048 + 2 * kMfWaves * 64 * M; }
 
 // M rows of K bf16 (row m at src + m * ld) to LDS with the padded stride; 64 zero bytes after them
@@ -50,97 +69,157 @@ __device__ __forceinline__ void mf_stage_rows(uint8_t* lds, const uint16_t* src,
   if (threadIdx.x < 4) *reinterpret_cast<uint4*>(lds + (size_t)M * rs + 16 * threadIdx.x) = make_uint4(0, 0, 0, 0);
 }
 
-// What a lane needs to walk units: set per unit by the caller's `open`
+// What a lane needs to walk a unit: set per unit by the caller's `open`. The weight loads are row-major (lane l: rows
+// l / 8 and 8 + l / 8 of the unit, piece l % 8 of the step's 128 bytes); scales and zero points are loaded by the lane
+// that uses them, in the MFMA's order (unit row l % 16, k part l / 16).
 struct MfUnit {
-  const uint8_t* wp;  // the lane's 16 bytes of the unit's first step: row l / 8 (and 8 rows on), piece l % 8, this wave's K slice
+  const uint8_t* wp;  // the lane's 16 bytes of the unit's first step, this wave's K slice
   size_t half;        // bytes from row l / 8 to row 8 + l / 8
-  const float* sp;    // the first step's scale of the unit's even rows (lanes 0, 2, ...) or odd rows (lanes 1, 3, ...)
+  const uint8_t* sp;  // FP8: the first step's f32 scale of the unit's even rows (even lanes) or odd rows (odd lanes);
+                      // INT4: the bf16 scales of groups 2 (l / 16), 2 (l / 16) + 1 of the first step, row l % 16
+  const uint8_t* zp;  // INT4: the zero-point words of the same two groups (the row's group of 8 rows)
+  uint32_t zsh;       // INT4: the row's nibble in those words
 };
 
-// The core: `nu` units of `steps` steps each; a step is one 128-k scale block of the unit's 16 rows (2 KiB: two loads,
-// each eight rows x 128 contiguous bytes, eight lanes a row). open(u) -> MfUnit; done(u, sum) is called by one wave
-// (they take turns) with the unit's complete sums (v4f: rows 4 (l / 16) + q, position l % 16). k0: the first k of this
-// wave's slice; ns: the slices (= the waves that work). Every wave of the workgroup calls this with the same nu.
-template <int M, class Open, class Done>
+// The core: `nu` units of `steps` steps each. Wave w works on slice w % ns of the units of group w / ns: in round i the
+// groups work on units i ng + group; with ns > 1 a workgroup barrier ends the round and one wave of each group (they
+// take turns) adds the slices' sums in slice order. open(u) -> MfUnit (for this wave's slice); done(u, sum) gets the
+// unit's complete sums (v4f: rows 4 (l / 16) + q, position l % 16). k0: the first k of this wave's slice. Every wave
+// of the workgroup calls this with the same nu, ns, steps.
+template <int FMT, int M, class Open, class Done>
 __device__ __forceinline__ void mf_stream(uint8_t* smem, size_t rows_bytes, int K, int k0, int ns, int nu, int steps, Open&& open, Done&& done) {
+  constexpr int STEPK = MfFmt<FMT>::STEPK;
   const uint32_t lane = threadIdx.x & 63;
   const int wave = uni((int)(threadIdx.x >> 6));
+  const int ng = kMfWaves / ns, grp = wave / ns, slice = wave - grp * ns, rounds = (nu + ng - 1) / ng;
   float* red = reinterpret_cast<float*>(smem + rows_bytes + kMfWaves * 2048);
-  auto finish = [&](int u) {  // after the unit's barrier: one wave adds the slices' sums in wave order
-    if (wave == u % ns) {
+  auto finish = [&](int rnd) {  // after the round's barrier: one wave a group adds the slices' sums in slice order
+    const int u = rnd * ng + grp;
+    if (u < nu && slice == rnd % ns) {
       v4f_t sum = {0.f, 0.f, 0.f, 0.f};
       const int pos = lane & 15, part4 = lane >> 4;
       if (pos < M)
-        for (int w = 0; w < ns; ++w) sum += *reinterpret_cast<const v4f_t*>(red + (((size_t)(u & 1) * kMfWaves + w) * 4 * M + part4 * M + pos) * 4);
+        for (int w = 0; w < ns; ++w)
+          sum += *reinterpret_cast<const v4f_t*>(red + (((size_t)(rnd & 1) * kMfWaves + grp * ns + w) * 4 * M + part4 * M + pos) * 4);
       done(u, sum);
     }
   };
-  if (wave >= ns) {  // (no slice: only the barriers)
-    for (int u = 0; u < nu; ++u) __syncthreads();
+  const int mine = (nu - grp + ng - 1) / ng;  // this wave's units: grp, grp + ng, ...
+  if (mine <= 0) {  // (no unit: only the barriers)
+    if (ns > 1)
+      for (int i = 0; i < rounds; ++i) __syncthreads();
     return;
   }
   const int r8 = lane >> 3, q = lane & 7, r16 = lane & 15, part = lane >> 4;
   uint8_t* W = smem + rows_bytes + wave * 2048;  // one step's weights: 16 rows x 128 bytes
   const size_t rs = (size_t)K * 2 + kMfPad;
-  // LDS offsets. A row's eight 16-byte pieces are exchanged by (row / 2) % 8: the MFMA-order reads of 8 bytes (16 lanes:
-  // 16 rows, one k part) then touch every bank once, and the row-major writes stay whole 128-byte rows.
-  int wr_off[2], rd_off[4];
+  // LDS offsets. The row-major writes stay whole 128-byte rows; a row's eight 16-byte pieces are exchanged so that the
+  // MFMA-order reads (16 lanes: 16 rows, one k part) touch every bank once: by (row / 2) % 8 for FP8's reads of 8 bytes,
+  // by row % 8 for the reads of 16 bytes.
+  constexpr int RSH = FMT == DSGX_FMT_FP8_B128 ? 1 : 0;
+  int wr_off[2], rd_off[FMT == DSGX_FMT_FP8_B128 ? 4 : 2];
 #pragma unroll
-  for (int h = 0; h < 2; ++h) wr_off[h] = (8 * h + r8) * 128 + ((q ^ (((8 * h + r8) >> 1) & 7)) * 16);
+  for (int h = 0; h < 2; ++h) wr_off[h] = (8 * h + r8) * 128 + ((q ^ (((8 * h + r8) >> RSH) & 7)) * 16);
+  if constexpr (FMT == DSGX_FMT_FP8_B128) {
 #pragma unroll
-  for (int j = 0; j < 4; ++j) rd_off[j] = r16 * 128 + (((2 * j + (part >> 1)) ^ ((r16 >> 1) & 7)) * 16) + 8 * (part & 1);
+    for (int j = 0; j < 4; ++j) rd_off[j] = r16 * 128 + (((2 * j + (part >> 1)) ^ ((r16 >> 1) & 7)) * 16) + 8 * (part & 1);
+  } else if constexpr (FMT == DSGX_FMT_INT4_G32) {  // pieces 2 part, 2 part + 1: two scale groups
+#pragma unroll
+    for (int j = 0; j < 2; ++j) rd_off[j] = r16 * 128 + (((2 * part + j) ^ (r16 & 7)) * 16);
+  } else {  // pieces part, 4 + part: the lane's 8 k of the step's two MFMAs
+#pragma unroll
+    for (int j = 0; j < 2; ++j) rd_off[j] = r16 * 128 + (((4 * j + part) ^ (r16 & 7)) * 16);
+  }
   const bool live = r16 < M;  // positions beyond the step's rows read the zero bytes
-  const uint32_t xb = live ? (uint32_t)(r16 * rs) + (uint32_t)(k0 + 8 * part) * 2 : (uint32_t)(M * rs);
+  // the lane's activations: row r16 from k0 + (FP8, BF16: 8 part; INT4: 64 part)
+  constexpr int XPART = FMT == DSGX_FMT_INT4_G32 ? 64 : 8;
+  const uint32_t xb = live ? (uint32_t)(r16 * rs) + (uint32_t)(k0 + XPART * part) * 2 : (uint32_t)(M * rs);
   const uint32_t xk = live ? 2u : 0u;
 
   struct Entry {
     u32x4_t a, b;  // rows l / 8 and 8 + l / 8
-    float s;       // the block's scale (even lanes: of the even rows; odd lanes: of the odd rows)
+    uint32_t s;    // FP8: the block's scale (even lanes: of the even rows; odd lanes: of the odd rows); INT4: two scales
+    u32x2_t z;     // INT4: the two groups' zero-point words
   };
   Entry ring[kMfD];
   int lu = 0, lstep = 0, cu = 0, cstep = 0;
-  MfUnit cur = open(0);
+  MfUnit cur = open(grp);
   v4f_t acc = {0.f, 0.f, 0.f, 0.f};
   auto load = [&](Entry& e) {
     const uint8_t* p = pin_after(cur.wp + (size_t)lstep * 128, acc[0]);
     e.a = ldg_stream(p);
     e.b = ldg_stream(p + cur.half);
-    e.s = *(const DSGX_GLOBAL float*)(uintptr_t)(cur.sp + lstep);
+    if constexpr (FMT == DSGX_FMT_FP8_B128) {
+      e.s = ldg_u32(cur.sp + (size_t)lstep * 4);
+    } else if constexpr (FMT == DSGX_FMT_INT4_G32) {
+      e.s = ldg_u32(cur.sp + (size_t)lstep * 16);
+      e.z = *(const DSGX_GLOBAL u32x2_t*)(uintptr_t)(cur.zp + (size_t)lstep * 32);
+    }
     if (++lstep == steps) {
       lstep = 0;
-      if (++lu < nu) cur = open(lu);  // (past the end the ring re-reads the last unit: unused)
+      if (++lu < mine) cur = open(lu * ng + grp);  // (past the end the ring re-reads the last unit: unused)
     }
+  };
+  const uint32_t zsh = cur.zsh;  // (the same for every unit of a stream)
+  auto mfma = [&](const uint32_t (&o)[4], uint32_t koff, v4f_t c) {
+    const u32x4_t av = u32x4_t{o[0], o[1], o[2], o[3]};
+    const u32x4_t bv = *reinterpret_cast<const u32x4_t*>(smem + xb + xk * koff);
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf_t, av), __builtin_bit_cast(v8bf_t, bv), c, 0, 0, 0);
   };
   auto compute = [&](const Entry& e) {
     *reinterpret_cast<u32x4_t*>(W + wr_off[0]) = keep_whole(e.a);
     *reinterpret_cast<u32x4_t*>(W + wr_off[1]) = keep_whole(e.b);
-    v4f_t part_sum = {0.f, 0.f, 0.f, 0.f};
+    if constexpr (FMT == DSGX_FMT_FP8_B128) {
+      v4f_t part_sum = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const uint2 wq = *reinterpret_cast<const uint2*>(W + rd_off[j]);
-      uint32_t o[4];
-      fp8x8_to_bf16(wq.x, wq.y, o);
-      const u32x4_t av = u32x4_t{o[0], o[1], o[2], o[3]};
-      const u32x4_t bv = *reinterpret_cast<const u32x4_t*>(smem + xb + xk * (uint32_t)(cstep * 128 + 32 * j));
-      part_sum = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf_t, av), __builtin_bit_cast(v8bf_t, bv), part_sum, 0, 0, 0);
+      for (int j = 0; j < 4; ++j) {
+        const uint2 wq = *reinterpret_cast<const uint2*>(W + rd_off[j]);
+        uint32_t o[4];
+        fp8x8_to_bf16(wq.x, wq.y, o);
+        part_sum = mfma(o, (uint32_t)(cstep * STEPK + 32 * j), part_sum);
+      }
+      // the 128-k block is complete: the scaled add (even rows of the unit: lane 0's scale, odd rows: lane 1's)
+      const float s0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane((int)e.s, 0));
+      const float s1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane((int)e.s, 1));
+      acc[0] = fmaf(s0, part_sum[0], acc[0]), acc[1] = fmaf(s1, part_sum[1], acc[1]);
+      acc[2] = fmaf(s0, part_sum[2], acc[2]), acc[3] = fmaf(s1, part_sum[3], acc[3]);
+    } else if constexpr (FMT == DSGX_FMT_INT4_G32) {
+#pragma unroll
+      for (int jj = 0; jj < 2; ++jj) {
+        const u32x4_t pc = *reinterpret_cast<const u32x4_t*>(W + rd_off[jj]);
+        const float s = bf16_bits_to_f32(jj ? e.s >> 16 : e.s & 0xFFFFu);
+        const float nzs = -((float)(((jj ? e.z.y : e.z.x) >> zsh) & 15u) * s);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          uint32_t o[4];
+          i4x8_to_bf16(pc[j], s, nzs, o);
+          acc = mfma(o, (uint32_t)(cstep * STEPK + 32 * jj + 8 * j), acc);
+        }
+      }
+    } else {
+#pragma unroll
+      for (int jj = 0; jj < 2; ++jj) {
+        const u32x4_t pc = *reinterpret_cast<const u32x4_t*>(W + rd_off[jj]);
+        const uint32_t o[4] = {pc[0], pc[1], pc[2], pc[3]};
+        acc = mfma(o, (uint32_t)(cstep * STEPK + 32 * jj), acc);
+      }
     }
-    // the 128-k block is complete: the scaled add (even rows of the unit: lane 0's scale, odd rows: lane 1's)
-    const float s0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, e.s), 0));
-    const float s1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, e.s), 1));
-    acc[0] = fmaf(s0, part_sum[0], acc[0]), acc[1] = fmaf(s1, part_sum[1], acc[1]);
-    acc[2] = fmaf(s0, part_sum[2], acc[2]), acc[3] = fmaf(s1, part_sum[3], acc[3]);
     if (++cstep < steps) return;
     cstep = 0;
-    // the unit is complete in this wave's slice: the slices' sums through LDS, added in wave order by one wave
-    if (live) *reinterpret_cast<v4f_t*>(red + (((size_t)(cu & 1) * kMfWaves + wave) * 4 * M + part * M + r16) * 4) = acc;
+    // the unit is complete in this wave's slice
+    if (ns == 1) {
+      done(cu * ng + grp, acc);
+    } else {
+      if (live) *reinterpret_cast<v4f_t*>(red + (((size_t)(cu & 1) * kMfWaves + wave) * 4 * M + part * M + r16) * 4) = acc;
+      __syncthreads();
+      finish(cu);  // (cu: the round)
+    }
     acc = v4f_t{0.f, 0.f, 0.f, 0.f};
-    __syncthreads();
-    finish(cu);
     ++cu;
   };
 #pragma unroll
   for (int d = 0; d < kMfD; ++d) load(ring[d]);
-  const int total = nu * steps;
+  const int total = mine * steps;
   for (int t = 0; t < total; t += kMfD) {
 #pragma unroll
     for (int d = 0; d < kMfD; ++d) {
@@ -148,50 +227,94 @@ __device__ __forceinline__ void mf_stream(uint8_t* smem, size_t rows_bytes, int 
       load(ring[d]);
     }
   }
+  if (ns > 1 && mine < rounds) __syncthreads();  // (the last round has no unit for this group)
 }
 
-template <int M, bool SH>
+template <int FMT, int SHFMT, int M>
 __device__ __forceinline__ void mf_setup(Step<M>& S, const DecodeArgs& a) {
   constexpr int NR = resolver_waves<M>();
   const int wave = uni((int)(threadIdx.x >> 6)), nw = blockDim.x >> 6;
   ResolveRegs rr;
   if (wave >= nw - NR) resolve_fetch(S, a, wave - (nw - NR), NR, rr);
-  prep<DSGX_FMT_FP8_B128, SH ? DSGX_FMT_FP8_B128 : 0, M>(S, a);
+  prep<FMT, SHFMT, M>(S, a);
   __syncthreads();
-  if (wave >= nw - NR) resolve<DSGX_FMT_FP8_B128, SH ? DSGX_FMT_FP8_B128 : 0, M>(S, a, wave - (nw - NR), NR, rr);
+  if (wave >= nw - NR) resolve<FMT, SHFMT, M>(S, a, wave - (nw - NR), NR, rr);
   __syncthreads();
 }
 
-template <int M, bool SH>
+// A unit of a gate/up matrix pair in format F: tile t = channels 8 t .. 8 t + 7, unit rows 2 c and 2 c + 1 gate and up of
+// channel 8 t + c. (BF16: the shared expert's interleaved matrix, whose rows already come in this order.)
+template <int F>
+__device__ __forceinline__ MfUnit mf_open_up(const Slot& T, int t, int H, int I, int k0, uint32_t lane) {
+  const int r8 = lane >> 3, p8 = lane & 7, r16 = lane & 15, part = lane >> 4;
+  const uint8_t* gw = T.g.w;
+  const uint8_t* uw = T.u.w;
+  const uint8_t* gs = T.g.s;
+  const uint8_t* us = T.u.s;
+  MfUnit q{};
+  if constexpr (F == DSGX_FMT_FP8_B128) {
+    q.wp = ((r8 & 1) ? uw : gw) + (size_t)(8 * t + (r8 >> 1)) * H + k0 + p8 * 16;
+    q.half = (size_t)4 * H;  // row 8 + r is gate / up (the same parity) of channel 4 further
+    q.sp = ((lane & 1) ? us : gs) + ((size_t)((8 * t) >> 7) * (H >> 7) + (k0 >> 7)) * 4;
+  } else if constexpr (F == DSGX_FMT_INT4_G32) {
+    const int G = H >> 5;
+    q.wp = ((r8 & 1) ? uw : gw) + (size_t)(8 * t + (r8 >> 1)) * (H >> 1) + (k0 >> 1) + p8 * 16;
+    q.half = (size_t)4 * (H >> 1);
+    const uint8_t* sb = (r16 & 1) ? us : gs;
+    const size_t g0 = (size_t)(k0 >> 5) + 2 * part;
+    q.sp = sb + ((size_t)(8 * t + (r16 >> 1)) * G + g0) * 2;
+    q.zp = sb + al256d((size_t)I * G * 2) + ((size_t)t * G + g0) * 4;
+    q.zsh = 4 * (r16 >> 1);
+  } else {
+    q.wp = gw + ((size_t)(16 * t + r8) * H + k0) * 2 + p8 * 16;
+    q.half = (size_t)16 * H;
+  }
+  return q;
+}
+// A unit of a down matrix: tile t = output rows 16 t .. 16 t + 15
+template <int F>
+__device__ __forceinline__ MfUnit mf_open_down(const Slot& T, int t, int H, int I, int k0, uint32_t lane) {
+  const int r8 = lane >> 3, p8 = lane & 7, r16 = lane & 15, part = lane >> 4;
+  const uint8_t* dw = T.d.w;
+  const uint8_t* ds = T.d.s;
+  MfUnit q{};
+  if constexpr (F == DSGX_FMT_FP8_B128) {
+    q.wp = dw + (size_t)(16 * t + r8) * I + k0 + p8 * 16;
+    q.half = (size_t)8 * I;
+    q.sp = ds + ((size_t)((16 * t) >> 7) * (I >> 7) + (k0 >> 7)) * 4;
+  } else if constexpr (F == DSGX_FMT_INT4_G32) {
+    const int G = I >> 5;
+    q.wp = dw + (size_t)(16 * t + r8) * (I >> 1) + (k0 >> 1) + p8 * 16;
+    q.half = (size_t)8 * (I >> 1);
+    const size_t g0 = (size_t)(k0 >> 5) + 2 * part;
+    q.sp = ds + ((size_t)(16 * t + r16) * G + g0) * 2;
+    q.zp = ds + al256d((size_t)H * G * 2) + ((size_t)(2 * t + (r16 >> 3)) * G + g0) * 4;
+    q.zsh = 4 * (r16 & 7);
+  } else {
+    q.wp = dw + ((size_t)(16 * t + r8) * I + k0) * 2 + p8 * 16;
+    q.half = (size_t)16 * I;
+  }
+  return q;
+}
+
+// SHFMT: 0 (no fused shared expert), FMT (slot 0 streams with the routed slots) or another format (slot 0 first, in a
+// stream of its own)
+template <int FMT, int SHFMT, int M>
 __global__ void __launch_bounds__(kMfThreads) k_up_mfma(DecodeArgs a) {
   extern __shared__ uint8_t mf_smem[];
   __shared__ Step<M> S;
-  mf_setup<M, SH>(S, a);
+  mf_setup<FMT, SHFMT, M>(S, a);
+  constexpr int nsh = SHFMT != 0 ? 1 : 0;
   const int H = a.L.H, I = a.L.I;
   const uint32_t lane = threadIdx.x & 63;
   const int wave = uni((int)(threadIdx.x >> 6));
   mf_stage_rows(mf_smem, a.x, H, M, H);
   __syncthreads();
-  const int nsl = (SH ? 1 : 0) + uni(S.n), tiles = I / 8, g = blockIdx.x, G = gridDim.x;
+  const int tiles = I / 8, g = blockIdx.x, G = gridDim.x;
   const int tpw = uni(g < tiles ? (tiles - g + G - 1) / G : 0);  // this workgroup's tiles a slot
-  const int ns = mf_slices(H), KS = H / ns, k0 = min(wave, ns - 1) * KS;
-  const int r8 = lane >> 3, p8 = lane & 7;
-  auto open = [&](int u) {
-    const int sl = uni(u / tpw), t = g + (u - sl * tpw) * G;
-    const Slot& T = S.slots[sl];
-    const uint8_t* gw = T.g.w;
-    const uint8_t* uw = T.u.w;
-    const uint8_t* gs = T.g.s;
-    const uint8_t* us = T.u.s;
-    // rows of the unit: 2 c and 2 c + 1 are gate and up of channel 8 t + c; this lane loads rows l / 8 and 8 + l / 8
-    MfUnit q;
-    q.wp = ((r8 & 1) ? uw : gw) + (size_t)(8 * t + (r8 >> 1)) * H + k0 + p8 * 16;
-    q.half = (size_t)4 * H;  // row 8 + r is gate / up (the same parity) of channel 4 further
-    q.sp = reinterpret_cast<const float*>((lane & 1) ? us : gs) + (size_t)((8 * t) >> 7) * (H >> 7) + (k0 >> 7);
-    return q;
-  };
-  auto done = [&](int u, v4f_t sum) {
-    const int sl = uni(u / tpw), t = g + (u - sl * tpw) * G, pos = lane & 15, part = lane >> 4;
+  if (tpw == 0) return;
+  auto done = [&](int sl, int t, v4f_t sum) {
+    const int pos = lane & 15, part = lane >> 4;
     if (pos >= M) return;
     const Slot& T = S.slots[sl];
     const float sg = T.g.s2, su = T.u.s2;
@@ -200,92 +323,115 @@ __global__ void __launch_bounds__(kMfThreads) k_up_mfma(DecodeArgs a) {
     uint16_t* dst = a.h + ((size_t)T.hslot * M + pos) * I + 8 * t + 2 * part;
     __hip_atomic_store((DSGX_GLOBAL uint32_t*)(uintptr_t)dst, h0 | (h1 << 16), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   };
-  if (tpw > 0) mf_stream<M>(mf_smem, mf_rows_bytes(M, H), H, k0, ns, nsl * tpw, KS / 128, open, done);
+  auto run = [&](auto fmt_tag, int s0, int nslots) {  // slots s0 .. s0 + nslots - 1 in format F
+    constexpr int F = decltype(fmt_tag)::value;
+    const int ns = mf_slices(H, MfFmt<F>::STEPK), KS = H / ns, k0 = (wave % ns) * KS;
+    auto open = [&](int u) {
+      const int sl = uni(u / tpw);
+      return mf_open_up<F>(S.slots[s0 + sl], g + (u - sl * tpw) * G, H, I, k0, lane);
+    };
+    auto fin = [&](int u, v4f_t sum) {
+      const int sl = uni(u / tpw);
+      done(s0 + sl, g + (u - sl * tpw) * G, sum);
+    };
+    mf_stream<F, M>(mf_smem, mf_rows_bytes(M, H), H, k0, ns, nslots * tpw, KS / MfFmt<F>::STEPK, open, fin);
+  };
+  const int nrouted = uni(S.n);
+  if constexpr (SHFMT != 0 && SHFMT != FMT) {
+    run(std::integral_constant<int, SHFMT>{}, 0, 1);
+    __syncthreads();
+    if (nrouted > 0) run(std::integral_constant<int, FMT>{}, 1, nrouted);
+  } else {
+    if (nsh + nrouted > 0) run(std::integral_constant<int, FMT>{}, 0, nsh + nrouted);
+  }
 }
 
-template <int M, bool SH>
+// The units (slot, tile of 16 output rows) are cut into equal contiguous ranges a workgroup; a shared slot in another
+// format counts WSH units a tile (BF16 beside INT4: four times the bytes).
+template <int FMT, int SHFMT, int M>
 __global__ void __launch_bounds__(kMfThreads) k_down_mfma(DecodeArgs a) {
   extern __shared__ uint8_t mf_smem[];
   __shared__ Step<M> S;
-  mf_setup<M, SH>(S, a);
-  constexpr int nsh = SH ? 1 : 0;
+  mf_setup<FMT, SHFMT, M>(S, a);
+  constexpr int nsh = SHFMT != 0 ? 1 : 0;
+  constexpr bool SH2 = SHFMT != 0 && SHFMT != FMT;
+  constexpr int WSH = 4;
   const int H = a.L.H, I = a.L.I;
   const uint32_t lane = threadIdx.x & 63;
   const int wave = uni((int)(threadIdx.x >> 6));
-  const int nrouted = uni(S.n), nsl = nsh + nrouted;
+  const int nrouted = uni(S.n);
   if (blockIdx.x == 0) {  // the slot table for k_down_combine
     if (threadIdx.x == 0) reinterpret_cast<int*>(a.fac)[0] = nrouted;
     for (int i = threadIdx.x; i < nrouted * M; i += blockDim.x)
       a.fac[8 + (i / M) * 8 + i % M] = __fmul_rn(S.slots[nsh + i / M].d.s2, S.wslot[i / M][i % M]);
   }
   const int tps = H / 16;  // tiles a slot
-  const long total = (long)nsl * tps;
-  const int u_lo = (int)(total * blockIdx.x / gridDim.x), u_hi = (int)(total * (blockIdx.x + 1) / gridDim.x);
-  const int ns = mf_slices(I), KS = I / ns, k0 = min(wave, ns - 1) * KS;
-  const int r8 = lane >> 3, p8 = lane & 7;
-  for (int sl = u_lo / tps; sl * tps < u_hi; ++sl) {  // (the same for every wave of the workgroup)
-    const int ta = max(u_lo, sl * tps) - sl * tps, tb = min(u_hi, (sl + 1) * tps) - sl * tps;
+  const int s0 = SH2 ? 1 : 0, nsl = nsh + nrouted - s0;  // the slots in format FMT
+  const long csh = SH2 ? (long)WSH * tps : 0;
+  const long total = csh + (long)nsl * tps;
+  const long c_lo = total * blockIdx.x / gridDim.x, c_hi = total * (blockIdx.x + 1) / gridDim.x;
+  auto run = [&](auto fmt_tag, int sl, int ta, int tb) {  // tiles ta .. tb - 1 of slot sl in format F
+    constexpr int F = decltype(fmt_tag)::value;
     const Slot& T = S.slots[sl];
     __syncthreads();
     mf_stage_rows(mf_smem, a.h + (size_t)T.hslot * M * I, I, M, I);
     __syncthreads();
-    if (tb <= ta) continue;
-    const uint8_t* dw = T.d.w;
-    const uint8_t* ds = T.d.s;
+    if (tb <= ta) return;
+    const int ns = mf_slices(I, MfFmt<F>::STEPK), KS = I / ns, k0 = (wave % ns) * KS;
     float* out = a.dpart + (size_t)sl * M * H;
-    auto open = [&](int u) {
-      const int t = ta + u;
-      MfUnit q;
-      q.wp = dw + (size_t)(16 * t + r8) * I + k0 + p8 * 16;
-      q.half = (size_t)8 * I;
-      q.sp = reinterpret_cast<const float*>(ds) + (size_t)((16 * t) >> 7) * (I >> 7) + (k0 >> 7);
-      return q;
-    };
-    auto done = [&](int u, v4f_t sum) {
+    auto open = [&](int u) { return mf_open_down<F>(T, ta + u, H, I, k0, lane); };
+    auto fin = [&](int u, v4f_t sum) {
       const int t = ta + u, pos = lane & 15, part = lane >> 4;
       if (pos < M) *reinterpret_cast<v4f_t*>(out + (size_t)pos * H + 16 * t + 4 * part) = sum;
     };
-    mf_stream<M>(mf_smem, mf_rows_bytes(M, I), I, k0, ns, tb - ta, KS / 128, open, done);
+    mf_stream<F, M>(mf_smem, mf_rows_bytes(M, I), I, k0, ns, tb - ta, KS / MfFmt<F>::STEPK, open, fin);
+  };
+  if constexpr (SH2) {  // the shared slot's tiles whose first cost unit lies in this workgroup's range
+    const long lo = c_lo < csh ? c_lo : csh, hi = c_hi < csh ? c_hi : csh;
+    const int ta = (int)((lo + WSH - 1) / WSH), tb = (int)((hi + WSH - 1) / WSH);
+    if (tb > ta) run(std::integral_constant<int, SHFMT>{}, 0, ta, tb);
+  }
+  const int u_lo = (int)((c_lo > csh ? c_lo : csh) - csh), u_hi = (int)((c_hi > csh ? c_hi : csh) - csh);
+  for (int sl = u_lo / tps; sl * tps < u_hi; ++sl) {  // (the same for every wave of the workgroup)
+    const int ta = max(u_lo, sl * tps) - sl * tps, tb = min(u_hi, (sl + 1) * tps) - sl * tps;
+    run(std::integral_constant<int, FMT>{}, s0 + sl, ta, tb);
   }
 }
 
-template <bool SH>
-int launch_decode_mfma_m(const DecodeArgs& a, int parts, hipStream_t st);
-
-template <int M, bool SH>
+template <int FMT, int SHFMT, int M>
 int launch_decode_mfma(const DecodeArgs& a, int parts, hipStream_t st) {
   const int H = a.L.H, I = a.L.I, cus = num_cus_cached();
-  if (H % 128 || I % 128 || H % mf_slices(H) || (H / mf_slices(H)) % 128 || (I / mf_slices(I)) % 128)
-    return fail(DSGX_EINVAL, "moe_decode (variant 1): hidden %d, intermediate %d (slices of whole 128-k blocks)", H, I);
+  if (H % 256 || I % 256)
+    return fail(DSGX_EINVAL, "moe_decode (variant 1): hidden %d, intermediate %d (whole steps of 256 k)", H, I);
   if (parts & 1) {
-    auto kern = k_up_mfma<M, SH>;
+    auto kern = k_up_mfma<FMT, SHFMT, M>;
     const size_t lds = mf_lds_bytes(M, H);
     if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds)) return rc;
     hipLaunchKernelGGL(kern, dim3(cus), dim3(kMfThreads), lds, st, a);
     DSGX_HIP(hipGetLastError());
   }
   if (parts & 2) {
-    auto kern = k_down_mfma<M, SH>;
+    auto kern = k_down_mfma<FMT, SHFMT, M>;
     const size_t lds = mf_lds_bytes(M, I);
     if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds)) return rc;
     hipLaunchKernelGGL(kern, dim3(cus), dim3(kMfThreads), lds, st, a);
-    hipLaunchKernelGGL((k_down_combine<M, SH>), dim3((M * H + 255) / 256), dim3(256), 0, st, a);
+    hipLaunchKernelGGL((k_down_combine<M, SHFMT != 0>), dim3((M * H + 255) / 256), dim3(256), 0, st, a);
     DSGX_HIP(hipGetLastError());
   }
   return DSGX_OK;
 }
 
-template <bool SH>
+template <int FMT, int SHFMT>
 int launch_decode_mfma_m(const DecodeArgs& a, int parts, hipStream_t st) {
   switch (a.M) {
-    case 1: return launch_decode_mfma<1, SH>(a, parts, st);
-    case 2: return launch_decode_mfma<2, SH>(a, parts, st);
-    case 3: return launch_decode_mfma<3, SH>(a, parts, st);
-    case 4: return launch_decode_mfma<4, SH>(a, parts, st);
-    case 5: return launch_decode_mfma<5, SH>(a, parts, st);
-    case 6: return launch_decode_mfma<6, SH>(a, parts, st);
-    case 7: return launch_decode_mfma<7, SH>(a, parts, st);
-    case 8: return launch_decode_mfma<8, SH>(a, parts, st);
+    case 1: return launch_decode_mfma<FMT, SHFMT, 1>(a, parts, st);
+    case 2: return launch_decode_mfma<FMT, SHFMT, 2>(a, parts, st);
+    case 3: return launch_decode_mfma<FMT, SHFMT, 3>(a, parts, st);
+    case 4: return launch_decode_mfma<FMT, SHFMT, 4>(a, parts, st);
+    case 5: return launch_decode_mfma<FMT, SHFMT, 5>(a, parts, st);
+    case 6: return launch_decode_mfma<FMT, SHFMT, 6>(a, parts, st);
+    case 7: return launch_decode_mfma<FMT, SHFMT, 7>(a, parts, st);
+    case 8: return launch_decode_mfma<FMT, SHFMT, 8>(a, parts, st);
   }
   return fail(DSGX_EUNSUPPORTED, "moe_decode (variant 1): %d rows", a.M);
 }

@@ -88,6 +88,7 @@ def test_decode_random_codes_asymmetric_int4_and_fp8():
         hl, dl = _layer(fmt, 2048, 2048, 64, 8, 3, shared, random_codes=True, seed=3)
         x, logits, idx, w = rows_and_routing(5, 4, 2048, 64, 8, 2.5)
         _check_step(hl, dl, x, idx, w, 4)
+        _check_step(hl, dl, x, idx, w, 4, up=1)  # variant 1: the same decode through the MFMA's lane order
 
 
 def test_decode_fused_routing_and_ysum():
@@ -180,10 +181,11 @@ def test_decode_nine_to_sixteen_rows():
             assert np.array_equal(s1[0].view(np.uint32), ys[m].view(np.uint32)), (M, m)
 
 
-@pytest.mark.parametrize("case", CASES[:2], ids=lambda c: "fmt%d-H%d-I%d-E%d-%s" % (c[0], c[1], c[2], c[3], c[6]))
+@pytest.mark.parametrize("case", CASES[:4] + CASES[5:], ids=lambda c: "fmt%d-H%d-I%d-E%d-%s" % (c[0], c[1], c[2], c[3], c[6]))
 def test_decode_mfma_variant(case):
-    """variant 1 (cfg.up = 1): the expert matmuls on the bf16 MFMA, FP8 layers; the same checks as the default's, and a
-    row's bits do not depend on the rows beside it (within the variant)"""
+    """variant 1 (cfg.up = 1): the expert matmuls on the bf16 MFMA, FP8 layers (FP8 shared expert) and INT4 layers (BF16
+    shared expert); the same checks as the default's, and a row's bits do not depend on the rows beside it (within the
+    variant)"""
     fmt, H, I, E, topk, NS, shared, scale = case
     hl, dl = _layer(fmt, H, I, E, topk, NS, shared)
     x, logits, idx, w = rows_and_routing(21, 8, H, E, topk, scale)
