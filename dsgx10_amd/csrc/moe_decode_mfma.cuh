@@ -25,7 +25,10 @@ namespace dsgx {
 typedef __bf16 v8bf_t __attribute__((ext_vector_type(8)));
 typedef float v4f_t __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
-constexpr int kMfD = 4;           // ring depth in steps
+#ifndef DSGX_MFD
+#define DSGX_MFD 4
+#endif
+constexpr int kMfD = DSGX_MFD;    // ring depth in steps
 constexpr int kMfPad = 64;        // bytes between activation rows in LDS beyond their length (bank spread)
 constexpr int kMfThreads = 512;   // eight waves a workgroup, one workgroup a CU
 constexpr int kMfWaves = kMfThreads / 64;
@@ -49,7 +52,9 @@ __host__ __device__ inline size_t mf_rows_bytes(int M, int K) { return (size_t)M
 // + one step's weights a wave + the waves' slice sums of two rounds (the lanes of positions < M only: 4 M x 16 bytes a wave)
 __host__ __device__ inline size_t mf_lds_bytes(int M, int K) { return mf_rows_bytes(M, K) + kMfWaves * 2048 + 2 * kMfWaves * 64 * M; }
 
-// M rows of K bf16 (row m at src + m * ld) to LDS with the padded stride; 64 zero bytes after them
+// M rows of K bf16 (row m at src + m * ld) to LDS with the padded stride.
+// COHERENT: rows written by other workgroups of the same kernel (h after the grid barrier)
+template <bool COHERENT>
 __device__ __forceinline__ void mf_stage_rows(uint8_t* lds, const uint16_t* src, size_t ld, int M, int K) {
   const int nq = K / 8, total = M * nq;
   const size_t rs = (size_t)K * 2 + kMfPad;
@@ -58,7 +63,7 @@ __device__ __forceinline__ void mf_stage_rows(uint8_t* lds, const uint16_t* src,
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
       const int i = min(i0 + u * (int)blockDim.x, total - 1);
-      v[u] = load_chunk<false>(src + (size_t)(i / nq) * ld + 8 * (i % nq));
+      v[u] = load_chunk<COHERENT>(src + (size_t)(i / nq) * ld + 8 * (i % nq));
     }
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
@@ -66,7 +71,10 @@ __device__ __forceinline__ void mf_stage_rows(uint8_t* lds, const uint16_t* src,
       if (i < total) *reinterpret_cast<uint4*>(lds + (size_t)(i / nq) * rs + 16 * (i % nq)) = v[u];
     }
   }
-  if (threadIdx.x < 4) *reinterpret_cast<uint4*>(lds + (size_t)M * rs + 16 * threadIdx.x) = make_uint4(0, 0, 0, 0);
+}
+// the 64 zero bytes that the lanes of positions beyond the step's rows read
+__device__ __forceinline__ void mf_zero_bytes(uint8_t* at) {
+  if (threadIdx.x < 4) *reinterpret_cast<uint4*>(at + 16 * threadIdx.x) = make_uint4(0, 0, 0, 0);
 }
 
 // What a lane needs to walk a unit: set per unit by the caller's `open`. The weight loads are row-major (lane l: rows
@@ -85,9 +93,13 @@ struct MfUnit {
 // groups work on units i ng + group; with ns > 1 a workgroup barrier ends the round and one wave of each group (they
 // take turns) adds the slices' sums in slice order. open(u) -> MfUnit (for this wave's slice); done(u, sum) gets the
 // unit's complete sums (v4f: rows 4 (l / 16) + q, position l % 16). k0: the first k of this wave's slice. Every wave
-// of the workgroup calls this with the same nu, ns, steps.
-template <int FMT, int M, class Open, class Done>
-__device__ __forceinline__ void mf_stream(uint8_t* smem, size_t rows_bytes, int K, int k0, int ns, int nu, int steps, Open&& open, Done&& done) {
+// of the workgroup calls this with the same nu, ns, steps. The activation rows of unit u start xoff_of(u) bytes into
+// the LDS (units of different slots in one stream); zoff: 64 zero bytes. pre() is called once by every wave, after
+// its first kMfD steps' loads are issued and before anything is read from LDS: the caller waits for and stages the
+// activations there (a workgroup barrier at its end), with the first weights already on their way.
+template <int FMT, int M, class Open, class XOff, class Done, class Pre>
+__device__ __forceinline__ void mf_stream(uint8_t* smem, size_t rows_bytes, uint32_t zoff, int K, int k0, int ns, int nu, int steps, Open&& open,
+                                          XOff&& xoff_of, Done&& done, Pre&& pre) {
   constexpr int STEPK = MfFmt<FMT>::STEPK;
   const uint32_t lane = threadIdx.x & 63;
   const int wave = uni((int)(threadIdx.x >> 6));
@@ -106,6 +118,7 @@ __device__ __forceinline__ void mf_stream(uint8_t* smem, size_t rows_bytes, int 
   };
   const int mine = (nu - grp + ng - 1) / ng;  // this wave's units: grp, grp + ng, ...
   if (mine <= 0) {  // (no unit: only the barriers)
+    pre();
     if (ns > 1)
       for (int i = 0; i < rounds; ++i) __syncthreads();
     return;
@@ -133,7 +146,8 @@ __device__ __forceinline__ void mf_stream(uint8_t* smem, size_t rows_bytes, int 
   const bool live = r16 < M;  // positions beyond the step's rows read the zero bytes
   // the lane's activations: row r16 from k0 + (FP8, BF16: 8 part; INT4: 64 part)
   constexpr int XPART = FMT == DSGX_FMT_INT4_G32 ? 64 : 8;
-  const uint32_t xb = live ? (uint32_t)(r16 * rs) + (uint32_t)(k0 + XPART * part) * 2 : (uint32_t)(M * rs);
+  const uint32_t xl = (uint32_t)(r16 * rs) + (uint32_t)(k0 + XPART * part) * 2;
+  uint32_t xb = live ? xl + xoff_of(grp) : zoff;
   const uint32_t xk = live ? 2u : 0u;
 
   struct Entry {
@@ -215,10 +229,11 @@ __device__ __forceinline__ void mf_stream(uint8_t* smem, size_t rows_bytes, int 
       finish(cu);  // (cu: the round)
     }
     acc = v4f_t{0.f, 0.f, 0.f, 0.f};
-    ++cu;
+    if (++cu < mine && live) xb = xl + xoff_of(cu * ng + grp);
   };
 #pragma unroll
   for (int d = 0; d < kMfD; ++d) load(ring[d]);
+  pre();
   const int total = mine * steps;
   for (int t = 0; t < total; t += kMfD) {
 #pragma unroll
@@ -300,19 +315,17 @@ __device__ __forceinline__ MfUnit mf_open_down(const Slot& T, int t, int H, int 
 // SHFMT: 0 (no fused shared expert), FMT (slot 0 streams with the routed slots) or another format (slot 0 first, in a
 // stream of its own)
 template <int FMT, int SHFMT, int M>
-__global__ void __launch_bounds__(kMfThreads) k_up_mfma(DecodeArgs a) {
-  extern __shared__ uint8_t mf_smem[];
-  __shared__ Step<M> S;
-  mf_setup<FMT, SHFMT, M>(S, a);
+__device__ __forceinline__ void mf_up_phase(Step<M>& S, const DecodeArgs& a, uint8_t* mf_smem) {
   constexpr int nsh = SHFMT != 0 ? 1 : 0;
   const int H = a.L.H, I = a.L.I;
   const uint32_t lane = threadIdx.x & 63;
   const int wave = uni((int)(threadIdx.x >> 6));
-  mf_stage_rows(mf_smem, a.x, H, M, H);
+  mf_stage_rows<false>(mf_smem, a.x, H, M, H);
+  mf_zero_bytes(mf_smem + (size_t)M * ((size_t)H * 2 + kMfPad));
   __syncthreads();
   const int tiles = I / 8, g = blockIdx.x, G = gridDim.x;
   const int tpw = uni(g < tiles ? (tiles - g + G - 1) / G : 0);  // this workgroup's tiles a slot
-  if (tpw == 0) return;
+  if (tpw == 0) return;  // (a workgroup beyond the tiles: no barrier of the workgroup follows in this phase)
   auto done = [&](int sl, int t, v4f_t sum) {
     const int pos = lane & 15, part = lane >> 4;
     if (pos >= M) return;
@@ -334,7 +347,8 @@ __global__ void __launch_bounds__(kMfThreads) k_up_mfma(DecodeArgs a) {
       const int sl = uni(u / tpw);
       done(s0 + sl, g + (u - sl * tpw) * G, sum);
     };
-    mf_stream<F, M>(mf_smem, mf_rows_bytes(M, H), H, k0, ns, nslots * tpw, KS / MfFmt<F>::STEPK, open, fin);
+    mf_stream<F, M>(mf_smem, mf_rows_bytes(M, H), (uint32_t)(M * ((size_t)H * 2 + kMfPad)), H, k0, ns, nslots * tpw, KS / MfFmt<F>::STEPK, open,
+                    [](int) { return 0u; }, fin, [] {});
   };
   const int nrouted = uni(S.n);
   if constexpr (SHFMT != 0 && SHFMT != FMT) {
@@ -347,12 +361,12 @@ __global__ void __launch_bounds__(kMfThreads) k_up_mfma(DecodeArgs a) {
 }
 
 // The units (slot, tile of 16 output rows) are cut into equal contiguous ranges a workgroup; a shared slot in another
-// format counts WSH units a tile (BF16 beside INT4: four times the bytes).
-template <int FMT, int SHFMT, int M>
-__global__ void __launch_bounds__(kMfThreads) k_down_mfma(DecodeArgs a) {
-  extern __shared__ uint8_t mf_smem[];
-  __shared__ Step<M> S;
-  mf_setup<FMT, SHFMT, M>(S, a);
+// format counts WSH units a tile (BF16 beside INT4: four times the bytes). A workgroup's range is walked in segments of
+// up to two slots, a stream each (with no more slots than workgroups, the whole range is one segment): the h rows of
+// the segment's slots are staged together and the ring runs on across the slot boundary. FUSED: h was written by this
+// launch; the first segment's weights are requested before the grid barrier is waited for.
+template <int FMT, int SHFMT, int M, bool FUSED>
+__device__ __forceinline__ void mf_down_phase(Step<M>& S, const DecodeArgs& a, uint8_t* mf_smem) {
   constexpr int nsh = SHFMT != 0 ? 1 : 0;
   constexpr bool SH2 = SHFMT != 0 && SHFMT != FMT;
   constexpr int WSH = 4;
@@ -370,21 +384,33 @@ __global__ void __launch_bounds__(kMfThreads) k_down_mfma(DecodeArgs a) {
   const long csh = SH2 ? (long)WSH * tps : 0;
   const long total = csh + (long)nsl * tps;
   const long c_lo = total * blockIdx.x / gridDim.x, c_hi = total * (blockIdx.x + 1) / gridDim.x;
-  auto run = [&](auto fmt_tag, int sl, int ta, int tb) {  // tiles ta .. tb - 1 of slot sl in format F
+  const size_t rs = (size_t)I * 2 + kMfPad;
+  const size_t rows_bytes = mf_rows_bytes(2 * M, I);
+  bool waited = !FUSED;  // the grid barrier is behind this workgroup
+  // units [ua, ub) of the slots from sl0 on (unit = slot * tps + tile, slots counted from sl0), all in format F
+  auto run = [&](auto fmt_tag, int sl0, int ua, int ub) {
     constexpr int F = decltype(fmt_tag)::value;
-    const Slot& T = S.slots[sl];
-    __syncthreads();
-    mf_stage_rows(mf_smem, a.h + (size_t)T.hslot * M * I, I, M, I);
-    __syncthreads();
-    if (tb <= ta) return;
-    const int ns = mf_slices(I, MfFmt<F>::STEPK), KS = I / ns, k0 = (wave % ns) * KS;
-    float* out = a.dpart + (size_t)sl * M * H;
-    auto open = [&](int u) { return mf_open_down<F>(T, ta + u, H, I, k0, lane); };
-    auto fin = [&](int u, v4f_t sum) {
-      const int t = ta + u, pos = lane & 15, part = lane >> 4;
-      if (pos < M) *reinterpret_cast<v4f_t*>(out + (size_t)pos * H + 16 * t + 4 * part) = sum;
+    const int nss = (ub - 1) / tps + 1;  // 1 or 2 slots
+    auto pre = [&] {
+      if (!waited) grid_barrier(a.bar, S.gen, a.spin_limit);
+      else __syncthreads();
+      waited = true;
+      for (int j = 0; j < nss; ++j)
+        mf_stage_rows<FUSED>(mf_smem + (size_t)j * M * rs, a.h + (size_t)S.slots[sl0 + j].hslot * M * I, I, M, I);
+      mf_zero_bytes(mf_smem + (size_t)2 * M * rs);
+      __syncthreads();
     };
-    mf_stream<F, M>(mf_smem, mf_rows_bytes(M, I), I, k0, ns, tb - ta, KS / MfFmt<F>::STEPK, open, fin);
+    const int ns = mf_slices(I, MfFmt<F>::STEPK), KS = I / ns, k0 = (wave % ns) * KS;
+    auto open = [&](int u) {
+      const int j = uni((ua + u) / tps);
+      return mf_open_down<F>(S.slots[sl0 + j], ua + u - j * tps, H, I, k0, lane);
+    };
+    auto xoff = [&](int u) { return (uint32_t)(uni((ua + u) / tps) * M * rs); };
+    auto fin = [&](int u, v4f_t sum) {
+      const int j = uni((ua + u) / tps), t = ua + u - j * tps, pos = lane & 15, part = lane >> 4;
+      if (pos < M) *reinterpret_cast<v4f_t*>(a.dpart + ((size_t)(sl0 + j) * M + pos) * H + 16 * t + 4 * part) = sum;
+    };
+    mf_stream<F, M>(mf_smem, rows_bytes, (uint32_t)(2 * M * rs), I, k0, ns, ub - ua, KS / MfFmt<F>::STEPK, open, xoff, fin, pre);
   };
   if constexpr (SH2) {  // the shared slot's tiles whose first cost unit lies in this workgroup's range
     const long lo = c_lo < csh ? c_lo : csh, hi = c_hi < csh ? c_hi : csh;
@@ -392,10 +418,36 @@ __global__ void __launch_bounds__(kMfThreads) k_down_mfma(DecodeArgs a) {
     if (tb > ta) run(std::integral_constant<int, SHFMT>{}, 0, ta, tb);
   }
   const int u_lo = (int)((c_lo > csh ? c_lo : csh) - csh), u_hi = (int)((c_hi > csh ? c_hi : csh) - csh);
-  for (int sl = u_lo / tps; sl * tps < u_hi; ++sl) {  // (the same for every wave of the workgroup)
-    const int ta = max(u_lo, sl * tps) - sl * tps, tb = min(u_hi, (sl + 1) * tps) - sl * tps;
-    run(std::integral_constant<int, FMT>{}, s0 + sl, ta, tb);
+  for (int sl = u_lo / tps; sl * tps < u_hi; sl += 2) {  // (the same for every wave of the workgroup)
+    const int ua = max(u_lo, sl * tps) - sl * tps, ub = min(u_hi, (sl + 2) * tps) - sl * tps;
+    run(std::integral_constant<int, FMT>{}, s0 + sl, ua, ub);
   }
+  if (!waited) grid_barrier(a.bar, S.gen, a.spin_limit);  // (a workgroup without a unit)
+}
+
+template <int FMT, int SHFMT, int M>
+__global__ void __launch_bounds__(kMfThreads) k_up_mfma(DecodeArgs a) {
+  extern __shared__ uint8_t mf_smem[];
+  __shared__ Step<M> S;
+  mf_setup<FMT, SHFMT, M>(S, a);
+  mf_up_phase<FMT, SHFMT, M>(S, a, mf_smem);
+}
+template <int FMT, int SHFMT, int M>
+__global__ void __launch_bounds__(kMfThreads) k_down_mfma(DecodeArgs a) {
+  extern __shared__ uint8_t mf_smem[];
+  __shared__ Step<M> S;
+  mf_setup<FMT, SHFMT, M>(S, a);
+  mf_down_phase<FMT, SHFMT, M, false>(S, a, mf_smem);
+}
+// Both phases in one launch, a grid barrier between them (every workgroup resident: one a CU); the step's set-up runs once
+template <int FMT, int SHFMT, int M>
+__global__ void __launch_bounds__(kMfThreads) k_decode_mfma(DecodeArgs a) {
+  extern __shared__ uint8_t mf_smem[];
+  __shared__ Step<M> S;
+  if (threadIdx.x == 0) S.gen = grid_barrier_gen(a.bar);
+  mf_setup<FMT, SHFMT, M>(S, a);
+  mf_up_phase<FMT, SHFMT, M>(S, a, mf_smem);
+  mf_down_phase<FMT, SHFMT, M, true>(S, a, mf_smem);
 }
 
 template <int FMT, int SHFMT, int M>
@@ -403,6 +455,19 @@ int launch_decode_mfma(const DecodeArgs& a, int parts, hipStream_t st) {
   const int H = a.L.H, I = a.L.I, cus = num_cus_cached();
   if (H % 256 || I % 256)
     return fail(DSGX_EINVAL, "moe_decode (variant 1): hidden %d, intermediate %d (whole steps of 256 k)", H, I);
+  if (parts == 3) {
+    auto kern = k_decode_mfma<FMT, SHFMT, M>;
+    const size_t lds = std::max(mf_lds_bytes(M, H), mf_lds_bytes(2 * M, I));
+    if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds)) return rc;
+    int per_cu = 0;  // the grid barrier needs every workgroup resident
+    DSGX_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kern, kMfThreads, lds));
+    if (per_cu >= 1) {
+      hipLaunchKernelGGL(kern, dim3(cus), dim3(kMfThreads), lds, st, a);
+      hipLaunchKernelGGL((k_down_combine<M, SHFMT != 0>), dim3((M * H + 255) / 256), dim3(256), 0, st, a);
+      DSGX_HIP(hipGetLastError());
+      return DSGX_OK;
+    }
+  }
   if (parts & 1) {
     auto kern = k_up_mfma<FMT, SHFMT, M>;
     const size_t lds = mf_lds_bytes(M, H);
@@ -412,7 +477,7 @@ int launch_decode_mfma(const DecodeArgs& a, int parts, hipStream_t st) {
   }
   if (parts & 2) {
     auto kern = k_down_mfma<FMT, SHFMT, M>;
-    const size_t lds = mf_lds_bytes(M, I);
+    const size_t lds = mf_lds_bytes(2 * M, I);
     if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds)) return rc;
     hipLaunchKernelGGL(kern, dim3(cus), dim3(kMfThreads), lds, st, a);
     hipLaunchKernelGGL((k_down_combine<M, SHFMT != 0>), dim3((M * H + 255) / 256), dim3(256), 0, st, a);

@@ -197,6 +197,13 @@ def test_decode_mfma_variant(case):
         assert np.array_equal(yr1[0].view(np.uint32), runs[8][0][m].view(np.uint32)), m
         if hl.has_shared:
             assert np.array_equal(ys1[0].view(np.uint32), runs[8][1][m].view(np.uint32)), m
+    # the two phases as two launches (parts 1, then 2): the one-launch form's bits
+    for M in (1, 8):
+        ws = gpu.decode_layer(dl, x[:M], idx[:M], w[:M], M, up=1, parts=1)[2]
+        yr_p, ys_p, _ = gpu.decode_layer(dl, x[:M], idx[:M], w[:M], M, up=1, parts=2, ws=ws)
+        assert np.array_equal(yr_p.view(np.uint32), runs[M][0].view(np.uint32))
+        if hl.has_shared:
+            assert np.array_equal(ys_p.view(np.uint32), runs[M][1].view(np.uint32))
     # fused routing, and 9-16 rows as two passes
     yr_l, ys_l, _ = gpu.decode_layer(dl, x, None, None, 8, logits=gpu.dev(logits), route_scale=scale, up=1)
     assert np.array_equal(yr_l.view(np.uint32), runs[8][0].view(np.uint32))
