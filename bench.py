@@ -11,7 +11,8 @@ expert rotates over copies that together exceed the 256 MB Infinity Cache.
 
 Prints ONE JSON line: metric us_per_moe_layer (lower is better), the roofline of the dominant kernel (the gate/up
 kernel, timed alone with HIP events on its launch stream), the CPU baseline (the C++ oracle on the host cores over
-the same step) and, unless --no-extra, the other benchmark configurations.
+the same step) and, unless --no-extra, the other benchmark configurations, each decode configuration with both kernel
+variants (dsgx_decode_cfg::up: 0 = dot products on the vector unit, the headline; 1 = on the bf16 MFMA).
 """
 import argparse
 import ctypes as C
@@ -82,13 +83,19 @@ def main():
     K, W = args.steps, args.warmup
     t_start = time.time()
 
-    def run_decode(gen, M, steps, warmup):
-        b = DecodeBench(gen, M, steps)
+    VARIANTS = ("vector", "mfma")  # dsgx_decode_cfg::up = 0, 1
+
+    def run_decode(gen, M, steps, warmup, up=0):
+        b = DecodeBench(gen, M, steps, up=up)
         r = b.time_layer(warmup)
         r.update(b.time_up_kernel())
-        log("  %s M=%d: %.2f us/layer (%.1f%% of 8 TB/s), gate/up kernel %.2f us (%.1f%%)" %
-            (gen.name, M, r["us_per_layer"], 100 * r["layer_hbm_frac"], r["up_us"], 100 * r["up_frac"]))
+        log("  %s M=%d (%s kernels): %.2f us/layer (%.1f%% of 8 TB/s), gate/up kernel %.2f us (%.1f%%)" %
+            (gen.name, M, VARIANTS[up], r["us_per_layer"], 100 * r["layer_hbm_frac"], r["up_us"], 100 * r["up_frac"]))
         return b, r
+
+    def decode_entry(gen, M, e, up):
+        return dict(workload=gen.name, M=M, variant=VARIANTS[up], us_per_layer=e["us_per_layer"], bytes=e["bytes_per_layer"],
+                    hbm_frac=e["layer_hbm_frac"], up_kernel_us=e["up_us"], up_hbm_frac=e["up_frac"])
 
     def cpu_baseline(b, budget_s):
         """The C++ oracle on the host cores over step 0 of the same workload (f32 contract sums only), repeated for about
@@ -128,21 +135,23 @@ def main():
     extra = []
     if not args.no_extra:
         ks = min(K, 128)
-        for M in (4, 8):
-            _, e = run_decode(gen, M, ks, min(W, 16))
-            extra.append(dict(workload=gen.name, M=M, us_per_layer=e["us_per_layer"], bytes=e["bytes_per_layer"],
-                              hbm_frac=e["layer_hbm_frac"], up_kernel_us=e["up_us"], up_hbm_frac=e["up_frac"]))
         del b
+        _, e = run_decode(gen, 1, K, W, up=1)
+        extra.append(decode_entry(gen, 1, e, 1))
+        for M in (4, 8):
+            for up in (0, 1):
+                _, e = run_decode(gen, M, ks, min(W, 16), up)
+                extra.append(decode_entry(gen, M, e, up))
         extra.append(prefill_extra(gen, 8192, "fp8_moe_prefill", 5.0e15) if head_fp8 else prefill_extra(gen, 2048, "int4_moe_prefill", 2.5e15))
         other = Int4LayerGen(seed=0) if head_fp8 else Fp8LayerGen(seed=0)
         for M in (1, 8):
-            ob, e = run_decode(other, M, ks if M > 1 else K, min(W, 16))
-            d = dict(workload=other.name, M=M, us_per_layer=e["us_per_layer"], bytes=e["bytes_per_layer"],
-                     hbm_frac=e["layer_hbm_frac"], up_kernel_us=e["up_us"], up_hbm_frac=e["up_frac"])
-            if M == 1 and not args.no_cpu:
-                d["cpu_baseline"] = cpu_baseline(ob, 5.0)
-            extra.append(d)
-            del ob
+            for up in (0, 1):
+                ob, e = run_decode(other, M, ks if M > 1 else K, min(W, 16), up)
+                d = decode_entry(other, M, e, up)
+                if M == 1 and not args.no_cpu:
+                    d["cpu_baseline"] = cpu_baseline(ob, 3.0)
+                extra.append(d)
+                del ob
         extra.append(prefill_extra(other, 2048, "int4_moe_prefill", 2.5e15) if head_fp8 else prefill_extra(other, 8192, "fp8_moe_prefill", 5.0e15))
         del other
         from dsgx10_amd.benchdata import gemv_bench

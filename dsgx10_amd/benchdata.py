@@ -206,8 +206,9 @@ class Int4LayerGen(_LayerGen):
 class DecodeBench:
     """`steps` decode steps of M rows over a generated layer; step s routes logits[s] (seeded N(0,1))."""
 
-    def __init__(self, gen, M, steps, seed=1234):
-        self.gen, self.M, self.steps = gen, M, steps
+    def __init__(self, gen, M, steps, seed=1234, up=0):
+        """up: the decode variant (dsgx_decode_cfg::up): 0 the vector-unit kernels, 1 the MFMA kernels"""
+        self.gen, self.M, self.steps, self.up = gen, M, steps, up
         g = torch.Generator(device="cuda")
         g.manual_seed(seed)
         self.x = torch.randn(M, gen.H, generator=g, device="cuda").to(torch.bfloat16)
@@ -230,11 +231,11 @@ class DecodeBench:
         g = self.gen
         if fused_routing:
             lib.moe_decode(self.layers[s % g.NSH], self.x, None, None, self.M, self.ws, self.yr, self.ys, parts=parts,
-                           logits=self.logits[s], route_scale=g.route_scale)
+                           logits=self.logits[s], route_scale=g.route_scale, up=self.up)
             return
         if route:
             lib.route(self.logits[s], None, self.idx[s], self.w[s], g.route_scale)
-        lib.moe_decode(self.layers[s % g.NSH], self.x, self.idx[s], self.w[s], self.M, self.ws, self.yr, self.ys, parts=parts)
+        lib.moe_decode(self.layers[s % g.NSH], self.x, self.idx[s], self.w[s], self.M, self.ws, self.yr, self.ys, parts=parts, up=self.up)
 
     def _graph(self, fn):
         gr = torch.cuda.CUDAGraph()
