@@ -29,7 +29,10 @@ typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
 #define DSGX_MFD 4
 #endif
 constexpr int kMfD = DSGX_MFD;    // ring depth in steps
-constexpr int kMfPad = 64;        // bytes between activation rows in LDS beyond their length (bank spread)
+// Bytes between activation rows in LDS beyond their length, by the routed experts' format: the lanes of one MFMA
+// operand read (position l % 16, k part l / 16) 16 bytes each, parts 16 bytes apart (FP8, BF16: rows 64 bytes apart
+// mod 256 spread four rows over the banks) or 128 bytes apart (INT4: rows 16 bytes apart spread eight).
+__host__ __device__ constexpr int mf_pad(int fmt) { return fmt == DSGX_FMT_INT4_G32 ? 16 : 64; }
 constexpr int kMfThreads = 512;   // eight waves a workgroup, one workgroup a CU
 constexpr int kMfWaves = kMfThreads / 64;
 
@@ -48,16 +51,16 @@ __host__ __device__ inline int mf_slices(int K, int stepk) {
   while (ns > 1 && (steps % ns || steps / ns < 4)) ns >>= 1;
   return ns;
 }
-__host__ __device__ inline size_t mf_rows_bytes(int M, int K) { return (size_t)M * ((size_t)K * 2 + kMfPad) + 64; }
+__host__ __device__ inline size_t mf_rows_bytes(int M, int K, int pad) { return (size_t)M * ((size_t)K * 2 + pad) + 64; }
 // + one step's weights a wave + the waves' slice sums of two rounds (the lanes of positions < M only: 4 M x 16 bytes a wave)
-__host__ __device__ inline size_t mf_lds_bytes(int M, int K) { return mf_rows_bytes(M, K) + kMfWaves * 2048 + 2 * kMfWaves * 64 * M; }
+__host__ __device__ inline size_t mf_lds_bytes(int M, int K, int pad) { return mf_rows_bytes(M, K, pad) + kMfWaves * 2048 + 2 * kMfWaves * 64 * M; }
 
 // M rows of K bf16 (row m at src + m * ld) to LDS with the padded stride.
 // COHERENT: rows written by other workgroups of the same kernel (h after the grid barrier)
 template <bool COHERENT>
-__device__ __forceinline__ void mf_stage_rows(uint8_t* lds, const uint16_t* src, size_t ld, int M, int K) {
+__device__ __forceinline__ void mf_stage_rows(uint8_t* lds, const uint16_t* src, size_t ld, int M, int K, int pad) {
   const int nq = K / 8, total = M * nq;
-  const size_t rs = (size_t)K * 2 + kMfPad;
+  const size_t rs = (size_t)K * 2 + pad;
   for (int i0 = threadIdx.x; i0 < total; i0 += 4 * blockDim.x) {
     uint4 v[4];
 #pragma unroll
@@ -98,7 +101,7 @@ struct MfUnit {
 // its first kMfD steps' loads are issued and before anything is read from LDS: the caller waits for and stages the
 // activations there (a workgroup barrier at its end), with the first weights already on their way.
 template <int FMT, int M, class Open, class XOff, class Done, class Pre>
-__device__ __forceinline__ void mf_stream(uint8_t* smem, size_t rows_bytes, uint32_t zoff, int K, int k0, int ns, int nu, int steps, Open&& open,
+__device__ __forceinline__ void mf_stream(uint8_t* smem, size_t rows_bytes, uint32_t zoff, int pad, int K, int k0, int ns, int nu, int steps, Open&& open,
                                           XOff&& xoff_of, Done&& done, Pre&& pre) {
   constexpr int STEPK = MfFmt<FMT>::STEPK;
   const uint32_t lane = threadIdx.x & 63;
@@ -125,7 +128,7 @@ __device__ __forceinline__ void mf_stream(uint8_t* smem, size_t rows_bytes, uint
   }
   const int r8 = lane >> 3, q = lane & 7, r16 = lane & 15, part = lane >> 4;
   uint8_t* W = smem + rows_bytes + wave * 2048;  // one step's weights: 16 rows x 128 bytes
-  const size_t rs = (size_t)K * 2 + kMfPad;
+  const size_t rs = (size_t)K * 2 + pad;
   // LDS offsets. The row-major writes stay whole 128-byte rows; a row's eight 16-byte pieces are exchanged so that the
   // MFMA-order reads (16 lanes: 16 rows, one k part) touch every bank once: by (row / 2) % 8 for FP8's reads of 8 bytes,
   // by row % 8 for the reads of 16 bytes.
@@ -320,8 +323,9 @@ __device__ __forceinline__ void mf_up_phase(Step<M>& S, const DecodeArgs& a, uin
   const int H = a.L.H, I = a.L.I;
   const uint32_t lane = threadIdx.x & 63;
   const int wave = uni((int)(threadIdx.x >> 6));
-  mf_stage_rows<false>(mf_smem, a.x, H, M, H);
-  mf_zero_bytes(mf_smem + (size_t)M * ((size_t)H * 2 + kMfPad));
+  constexpr int pad = mf_pad(FMT);
+  mf_stage_rows<false>(mf_smem, a.x, H, M, H, pad);
+  mf_zero_bytes(mf_smem + (size_t)M * ((size_t)H * 2 + pad));
   __syncthreads();
   const int tiles = I / 8, g = blockIdx.x, G = gridDim.x;
   const int tpw = uni(g < tiles ? (tiles - g + G - 1) / G : 0);  // this workgroup's tiles a slot
@@ -347,7 +351,7 @@ __device__ __forceinline__ void mf_up_phase(Step<M>& S, const DecodeArgs& a, uin
       const int sl = uni(u / tpw);
       done(s0 + sl, g + (u - sl * tpw) * G, sum);
     };
-    mf_stream<F, M>(mf_smem, mf_rows_bytes(M, H), (uint32_t)(M * ((size_t)H * 2 + kMfPad)), H, k0, ns, nslots * tpw, KS / MfFmt<F>::STEPK, open,
+    mf_stream<F, M>(mf_smem, mf_rows_bytes(M, H, pad), (uint32_t)(M * ((size_t)H * 2 + pad)), pad, H, k0, ns, nslots * tpw, KS / MfFmt<F>::STEPK, open,
                     [](int) { return 0u; }, fin, [] {});
   };
   const int nrouted = uni(S.n);
@@ -384,8 +388,9 @@ __device__ __forceinline__ void mf_down_phase(Step<M>& S, const DecodeArgs& a, u
   const long csh = SH2 ? (long)WSH * tps : 0;
   const long total = csh + (long)nsl * tps;
   const long c_lo = total * blockIdx.x / gridDim.x, c_hi = total * (blockIdx.x + 1) / gridDim.x;
-  const size_t rs = (size_t)I * 2 + kMfPad;
-  const size_t rows_bytes = mf_rows_bytes(2 * M, I);
+  constexpr int pad = mf_pad(FMT);
+  const size_t rs = (size_t)I * 2 + pad;
+  const size_t rows_bytes = mf_rows_bytes(2 * M, I, pad);
   bool waited = !FUSED;  // the grid barrier is behind this workgroup
   // units [ua, ub) of the slots from sl0 on (unit = slot * tps + tile, slots counted from sl0), all in format F
   auto run = [&](auto fmt_tag, int sl0, int ua, int ub) {
@@ -396,7 +401,7 @@ __device__ __forceinline__ void mf_down_phase(Step<M>& S, const DecodeArgs& a, u
       else __syncthreads();
       waited = true;
       for (int j = 0; j < nss; ++j)
-        mf_stage_rows<FUSED>(mf_smem + (size_t)j * M * rs, a.h + (size_t)S.slots[sl0 + j].hslot * M * I, I, M, I);
+        mf_stage_rows<FUSED>(mf_smem + (size_t)j * M * rs, a.h + (size_t)S.slots[sl0 + j].hslot * M * I, I, M, I, pad);
       mf_zero_bytes(mf_smem + (size_t)2 * M * rs);
       __syncthreads();
     };
@@ -410,7 +415,7 @@ __device__ __forceinline__ void mf_down_phase(Step<M>& S, const DecodeArgs& a, u
       const int j = uni((ua + u) / tps), t = ua + u - j * tps, pos = lane & 15, part = lane >> 4;
       if (pos < M) *reinterpret_cast<v4f_t*>(a.dpart + ((size_t)(sl0 + j) * M + pos) * H + 16 * t + 4 * part) = sum;
     };
-    mf_stream<F, M>(mf_smem, rows_bytes, (uint32_t)(2 * M * rs), I, k0, ns, ub - ua, KS / MfFmt<F>::STEPK, open, xoff, fin, pre);
+    mf_stream<F, M>(mf_smem, rows_bytes, (uint32_t)(2 * M * rs), pad, I, k0, ns, ub - ua, KS / MfFmt<F>::STEPK, open, xoff, fin, pre);
   };
   if constexpr (SH2) {  // the shared slot's tiles whose first cost unit lies in this workgroup's range
     const long lo = c_lo < csh ? c_lo : csh, hi = c_hi < csh ? c_hi : csh;
@@ -457,7 +462,7 @@ int launch_decode_mfma(const DecodeArgs& a, int parts, hipStream_t st) {
     return fail(DSGX_EINVAL, "moe_decode (variant 1): hidden %d, intermediate %d (whole steps of 256 k)", H, I);
   if (parts == 3) {
     auto kern = k_decode_mfma<FMT, SHFMT, M>;
-    const size_t lds = std::max(mf_lds_bytes(M, H), mf_lds_bytes(2 * M, I));
+    const size_t lds = std::max(mf_lds_bytes(M, H, mf_pad(FMT)), mf_lds_bytes(2 * M, I, mf_pad(FMT)));
     if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds)) return rc;
     int per_cu = 0;  // the grid barrier needs every workgroup resident
     DSGX_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kern, kMfThreads, lds));
@@ -470,14 +475,14 @@ int launch_decode_mfma(const DecodeArgs& a, int parts, hipStream_t st) {
   }
   if (parts & 1) {
     auto kern = k_up_mfma<FMT, SHFMT, M>;
-    const size_t lds = mf_lds_bytes(M, H);
+    const size_t lds = mf_lds_bytes(M, H, mf_pad(FMT));
     if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds)) return rc;
     hipLaunchKernelGGL(kern, dim3(cus), dim3(kMfThreads), lds, st, a);
     DSGX_HIP(hipGetLastError());
   }
   if (parts & 2) {
     auto kern = k_down_mfma<FMT, SHFMT, M>;
-    const size_t lds = mf_lds_bytes(2 * M, I);
+    const size_t lds = mf_lds_bytes(2 * M, I, mf_pad(FMT));
     if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds)) return rc;
     hipLaunchKernelGGL(kern, dim3(cus), dim3(kMfThreads), lds, st, a);
     hipLaunchKernelGGL((k_down_combine<M, SHFMT != 0>), dim3((M * H + 255) / 256), dim3(256), 0, st, a);
