@@ -51,7 +51,7 @@ __host__ __device__ inline int mf_slices(int K, int stepk) {
   while (ns > 1 && (steps % ns || steps / ns < 4)) ns >>= 1;
   return ns;
 }
-__host__ __device__ inline size_t mf_rows_bytes(int M, int K, int pad) { return (size_t)M * ((size_t)K * 2 + pad) + 64; }
+__host__ __device__ inline size_t mf_rows_bytes(int M, int K, int pad) { return (size_t)M * ((size_t)K * 2 + pad) + 256; }
 // + one step's weights a wave + the waves' slice sums of two rounds (the lanes of positions < M only: 4 M x 16 bytes a wave)
 __host__ __device__ inline size_t mf_lds_bytes(int M, int K, int pad) { return mf_rows_bytes(M, K, pad) + kMfWaves * 2048 + 2 * kMfWaves * 64 * M; }
 
@@ -75,9 +75,9 @@ __device__ __forceinline__ void mf_stage_rows(uint8_t* lds, const uint16_t* src,
     }
   }
 }
-// the 64 zero bytes that the lanes of positions beyond the step's rows read
+// the 256 zero bytes that the lanes of positions beyond the step's rows read (a step's fragments lie within 208 bytes)
 __device__ __forceinline__ void mf_zero_bytes(uint8_t* at) {
-  if (threadIdx.x < 4) *reinterpret_cast<uint4*>(at + 16 * threadIdx.x) = make_uint4(0, 0, 0, 0);
+  if (threadIdx.x < 16) *reinterpret_cast<uint4*>(at + 16 * threadIdx.x) = make_uint4(0, 0, 0, 0);
 }
 
 // What a lane needs to walk a unit: set per unit by the caller's `open`. The weight loads are row-major (lane l: rows
@@ -97,7 +97,7 @@ struct MfUnit {
 // take turns) adds the slices' sums in slice order. open(u) -> MfUnit (for this wave's slice); done(u, sum) gets the
 // unit's complete sums (v4f: rows 4 (l / 16) + q, position l % 16). k0: the first k of this wave's slice. Every wave
 // of the workgroup calls this with the same nu, ns, steps. The activation rows of unit u start xoff_of(u) bytes into
-// the LDS (units of different slots in one stream); zoff: 64 zero bytes. pre() is called once by every wave, after
+// the LDS (units of different slots in one stream); zoff: 256 zero bytes. pre() is called once by every wave, after
 // its first kMfD steps' loads are issued and before anything is read from LDS: the caller waits for and stages the
 // activations there (a workgroup barrier at its end), with the first weights already on their way.
 template <int FMT, int M, class Open, class XOff, class Done, class Pre>
@@ -150,8 +150,10 @@ __device__ __forceinline__ void mf_stream(uint8_t* smem, size_t rows_bytes, uint
   // the lane's activations: row r16 from k0 + (FP8, BF16: 8 part; INT4: 64 part)
   constexpr int XPART = FMT == DSGX_FMT_INT4_G32 ? 64 : 8;
   const uint32_t xl = (uint32_t)(r16 * rs) + (uint32_t)(k0 + XPART * part) * 2;
-  uint32_t xb = live ? xl + xoff_of(grp) : zoff;
-  const uint32_t xk = live ? 2u : 0u;
+  // xp: the lane's activations of the step at hand (the fragments' offsets within a step are immediates); the lanes of
+  // positions beyond the step's rows stay on the zero bytes
+  uint32_t xp = live ? xl + xoff_of(grp) : zoff;
+  const uint32_t xstep = live ? (uint32_t)STEPK * 2 : 0u;
 
   struct Entry {
     u32x4_t a, b;  // rows l / 8 and 8 + l / 8
@@ -178,9 +180,9 @@ __device__ __forceinline__ void mf_stream(uint8_t* smem, size_t rows_bytes, uint
     }
   };
   const uint32_t zsh = cur.zsh;  // (the same for every unit of a stream)
-  auto mfma = [&](const uint32_t (&o)[4], uint32_t koff, v4f_t c) {
+  auto mfma = [&](const uint32_t (&o)[4], uint32_t koff, v4f_t c) {  // koff: k within the step
     const u32x4_t av = u32x4_t{o[0], o[1], o[2], o[3]};
-    const u32x4_t bv = *reinterpret_cast<const u32x4_t*>(smem + xb + xk * koff);
+    const u32x4_t bv = *reinterpret_cast<const u32x4_t*>(smem + xp + 2 * koff);
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf_t, av), __builtin_bit_cast(v8bf_t, bv), c, 0, 0, 0);
   };
   auto compute = [&](const Entry& e) {
@@ -193,7 +195,7 @@ __device__ __forceinline__ void mf_stream(uint8_t* smem, size_t rows_bytes, uint
         const uint2 wq = *reinterpret_cast<const uint2*>(W + rd_off[j]);
         uint32_t o[4];
         fp8x8_to_bf16(wq.x, wq.y, o);
-        part_sum = mfma(o, (uint32_t)(cstep * STEPK + 32 * j), part_sum);
+        part_sum = mfma(o, 32 * j, part_sum);
       }
       // the 128-k block is complete: the scaled add (even rows of the unit: lane 0's scale, odd rows: lane 1's)
       const float s0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane((int)e.s, 0));
@@ -210,7 +212,7 @@ __device__ __forceinline__ void mf_stream(uint8_t* smem, size_t rows_bytes, uint
         for (int j = 0; j < 4; ++j) {
           uint32_t o[4];
           i4x8_to_bf16(pc[j], s, nzs, o);
-          acc = mfma(o, (uint32_t)(cstep * STEPK + 32 * jj + 8 * j), acc);
+          acc = mfma(o, 32 * jj + 8 * j, acc);
         }
       }
     } else {
@@ -218,9 +220,10 @@ __device__ __forceinline__ void mf_stream(uint8_t* smem, size_t rows_bytes, uint
       for (int jj = 0; jj < 2; ++jj) {
         const u32x4_t pc = *reinterpret_cast<const u32x4_t*>(W + rd_off[jj]);
         const uint32_t o[4] = {pc[0], pc[1], pc[2], pc[3]};
-        acc = mfma(o, (uint32_t)(cstep * STEPK + 32 * jj), acc);
+        acc = mfma(o, 32 * jj, acc);
       }
     }
+    xp += xstep;
     if (++cstep < steps) return;
     cstep = 0;
     // the unit is complete in this wave's slice
@@ -232,7 +235,7 @@ __device__ __forceinline__ void mf_stream(uint8_t* smem, size_t rows_bytes, uint
       finish(cu);  // (cu: the round)
     }
     acc = v4f_t{0.f, 0.f, 0.f, 0.f};
-    if (++cu < mine && live) xb = xl + xoff_of(cu * ng + grp);
+    if (++cu < mine && live) xp = xl + xoff_of(cu * ng + grp);
   };
 #pragma unroll
   for (int d = 0; d < kMfD; ++d) load(ring[d]);
