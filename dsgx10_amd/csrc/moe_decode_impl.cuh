@@ -701,7 +701,19 @@ __global__ void __launch_bounds__(256) k_down_combine(DecodeArgs a) {
   const int m = i / H;
   const float* d = a.dpart + (size_t)(SH ? 1 : 0) * M * H + i;
   float acc = 0.f;
-  for (int s = 0; s < nrouted; ++s) acc = fmaf(a.fac[8 + s * 8 + m], d[(size_t)s * M * H], acc);
+  // sixteen slots' loads in flight together (past the end: the last slot again, unused), then their adds in slot order
+  constexpr int B = 16;
+  for (int s0 = 0; s0 < nrouted; s0 += B) {
+    float v[B], f[B];
+#pragma unroll
+    for (int j = 0; j < B; ++j) {
+      const int s = min(s0 + j, nrouted - 1);
+      v[j] = d[(size_t)s * M * H], f[j] = a.fac[8 + s * 8 + m];
+    }
+#pragma unroll
+    for (int j = 0; j < B; ++j)
+      if (s0 + j < nrouted) acc = fmaf(f[j], v[j], acc);
+  }
   float sv = 0.f;
   if (SH) a.ys[i] = sv = a.dpart[i];
   else if (a.ysum) sv = a.ys[i];
