@@ -65,6 +65,8 @@ def main():
     ap.add_argument("--no-extra", action="store_true", help="only the headline workload")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--workload", default="fp8_m1", help="headline workload: fp8_m1 | int4_m1")
+    ap.add_argument("--variant", default="vector", choices=("vector", "mfma"),
+                    help="the headline's decode kernels (dsgx_decode_cfg::up = 0 | 1); --no-extra then runs nothing else")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs on one GPU (the whole layer is resident; no collectives are built); "
@@ -127,7 +129,8 @@ def main():
     gen = Fp8LayerGen(seed=0) if head_fp8 else Int4LayerGen(seed=0)
     log("  %.1f s, pool %.2f GB" % (time.time() - t_start, gen.pool.numel() / 1e9))
     stream_gbs = gen.stream_read_gbs()
-    b, r = run_decode(gen, 1, K, W)
+    head_up = 1 if args.variant == "mfma" else 0
+    b, r = run_decode(gen, 1, K, W, head_up)
     cpu = None
     if not args.no_cpu:
         cpu = cpu_baseline(b, 10.0)
@@ -136,8 +139,8 @@ def main():
     if not args.no_extra:
         ks = min(K, 128)
         del b
-        _, e = run_decode(gen, 1, K, W, up=1)
-        extra.append(decode_entry(gen, 1, e, 1))
+        _, e = run_decode(gen, 1, K, W, up=1 - head_up)
+        extra.append(decode_entry(gen, 1, e, 1 - head_up))
         for M in (4, 8):
             for up in (0, 1):
                 _, e = run_decode(gen, M, ks, min(W, 16), up)
@@ -172,9 +175,12 @@ def main():
         "data": "synthetic (torch-seeded N(0,0.02) weights quantised on the GPU, N(0,1) bf16 rows and f32 logits)",
         "config": {"workload": gen.describe(1), "arithmetic": "f32 sums of bf16 x bf16 products (weights decoded to bf16 in registers)", "rows_M": 1, "steps_route_different_experts": True,
                    "bytes_per_layer": r["bytes_per_layer"], "layer_hbm_frac_of_8TBs": r["layer_hbm_frac"],
-                   "kernels_per_step": ["k_decode (routing + gate/up + SwiGLU + down + weighted sum, one persistent launch)"], "timed_as": "one HIP graph of all steps, one replay"},
-        "roofline": {"bound": "hbm", "kernel": "k_up (gate/up + SwiGLU)", "achieved": r["up_gbs"], "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": r["up_frac"], "traffic": UP_TRAFFIC_FP8_M1 if head_fp8 else None, "bytes_per_launch": r["up_bytes"],
+                   "variant": args.variant,
+                   "kernels_per_step": ["k_decode (routing + gate/up + SwiGLU + down + weighted sum, one persistent launch)"] if head_up == 0 else
+                                       ["k_decode_mfma (routing + gate/up + SwiGLU + down, one persistent launch)", "k_down_combine (weighted sum in expert order)"],
+                   "timed_as": "one HIP graph of all steps, one replay"},
+        "roofline": {"bound": "hbm", "kernel": "k_up (gate/up + SwiGLU)" if head_up == 0 else "k_up_mfma (gate/up + SwiGLU)", "achieved": r["up_gbs"], "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": r["up_frac"], "traffic": UP_TRAFFIC_FP8_M1 if head_fp8 and head_up == 0 else None, "bytes_per_launch": r["up_bytes"],
                      "avg_launch_us": r["up_us"], "measured_stream_read_gbs": stream_gbs},
         "cpu_baseline": cpu,
         "extra": extra,
