@@ -102,7 +102,10 @@ DSGX_API int dsgx_route(const float* logits, const float* bias, int M, int E, in
 
 /* ---- decode: gx::moe_decode (engine/experts/experts.h:104-147, decode.cu:708-730) ------------------------------- */
 typedef struct dsgx_decode_cfg {
-  int32_t up, down;        /* kernel variants: up 0 only; down 0 = both phases in one persistent kernel, 1 = two launches */
+  int32_t up, down;        /* kernel variants. up 0: dot products on the vector unit; up 1: on the bf16 MFMA (FP8_B128 and
+                              INT4_G32 layers, 1-16 rows; a row's bits are the same in any batch within a variant, but differ
+                              between the variants in the order of the f32 adds). down (with up 0) 0: both phases in one
+                              persistent kernel; 1: two launches */
   int32_t parts;           /* 1 up only, 2 down only, 3 both (bench) */
   int32_t ysum;            /* 1: yr += ys in f32 after the routed experts (experts.h:132-136) */
   const float* logits;     /* fused routing (experts.h:123-127): with logits (+ optional bias) idx, w are not read */

@@ -93,10 +93,10 @@ inline void moe_decode(const LayerW& L, const uint16_t* x, const int* idx, const
   d.route_scale = cfg.route_scale, d.post = cfg.post;
   DSGX_DIE_ON(dsgx_moe_decode(&c, x, idx, w, M, ws, yr, ys, st, &d));
 }
-inline int decode_up_variants() { return 1; }
-inline int decode_down_variants() { return 1; }
-inline const char* decode_up_name(int) { return "rows4 lanes64"; }
-inline const char* decode_down_name(int) { return "rows2 lanes64"; }
+inline int decode_up_variants() { return 2; }
+inline int decode_down_variants() { return 2; }
+inline const char* decode_up_name(int v) { return v == 1 ? "mfma16 kslices" : "rows4 lanes64"; }
+inline const char* decode_down_name(int v) { return v == 1 ? "two launches" : "rows2 lanes64"; }
 inline void finalize(const float* R, const float* S, int M, uint16_t* out, void* st, bool pdl = true, int H = kH) {
   (void)pdl;
   DSGX_DIE_ON(dsgx_finalize(R, S, M * H, out, st));
