@@ -7,7 +7,8 @@
 // Each function names the reference lines it restates (paths relative to the reference tree; A/ =
 // altar1-4xgx10-switchless/, D/ = ds41f-4xgx10-switchless/). The reference's own implementation of this path is CUDA
 // for sm_121a with inline PTX and cannot be compiled here, so there is no oracle/_ref build; the functions below are
-// pinned by closed forms, exhaustive checks, torch-CPU library routines and brute force in tests/test_oracle_*.py.
+// pinned by closed forms, exhaustive checks, torch-CPU library routines and brute force in tests/test_oracle_*.py, and
+// orc_moe_prefill_fp8_row also by vectors from the reference's own torch kernels (tests/golden/prefill_fp8_expert.npz).
 //
 // Pinned: bf16 RNE, e4m3 decode/encode, INT4 dequant, FP8 quantiser and dequant, act_quant, router, union,
 // GEMV and MoE sums (f32 contract order, f64 and sum of |terms|). Parity unpinned: none of the functions here; the
