@@ -38,17 +38,19 @@ constexpr int kMfWaves = kMfThreads / 64;
 
 // k a step (128 bytes of a weight row)
 template <int FMT> struct MfFmt;
-template <> struct MfFmt<DSGX_FMT_FP8_B128> { static constexpr int STEPK = 128; };
-template <> struct MfFmt<DSGX_FMT_INT4_G32> { static constexpr int STEPK = 256; };
-template <> struct MfFmt<DSGX_FMT_BF16> { static constexpr int STEPK = 64; };
+// MINSTEPS: the fewest steps of a K slice (mf_slices), measured: 4 for FP8; 8 for the steps of INT4, which hold four
+// times the arithmetic
+template <> struct MfFmt<DSGX_FMT_FP8_B128> { static constexpr int STEPK = 128, MINSTEPS = 4; };
+template <> struct MfFmt<DSGX_FMT_INT4_G32> { static constexpr int STEPK = 256, MINSTEPS = 8; };
+template <> struct MfFmt<DSGX_FMT_BF16> { static constexpr int STEPK = 64, MINSTEPS = 8; };
 
-// The slices of K: a power of two (1 .. 8) that divides the steps of K, four steps or more a slice where K allows
+// The slices of K: a power of two (1 .. 8) that divides the steps of K, `minsteps` steps or more a slice where K allows
 // (fewer steps between two workgroup barriers cost more than they spread). With ns < 8 slices, 8 / ns groups of waves
 // work on different units at a time.
-__host__ __device__ inline int mf_slices(int K, int stepk) {
+__host__ __device__ inline int mf_slices(int K, int stepk, int minsteps) {
   const int steps = K / stepk;
   int ns = kMfWaves;
-  while (ns > 1 && (steps % ns || steps / ns < 4)) ns >>= 1;
+  while (ns > 1 && (steps % ns || steps / ns < minsteps)) ns >>= 1;
   return ns;
 }
 __host__ __device__ inline size_t mf_rows_bytes(int M, int K, int pad) { return (size_t)M * ((size_t)K * 2 + pad) + 256; }
@@ -345,7 +347,7 @@ __device__ __forceinline__ void mf_up_phase(Step<M>& S, const DecodeArgs& a, uin
   };
   auto run = [&](auto fmt_tag, int s0, int nslots) {  // slots s0 .. s0 + nslots - 1 in format F
     constexpr int F = decltype(fmt_tag)::value;
-    const int ns = mf_slices(H, MfFmt<F>::STEPK), KS = H / ns, k0 = (wave % ns) * KS;
+    const int ns = mf_slices(H, MfFmt<F>::STEPK, MfFmt<F>::MINSTEPS), KS = H / ns, k0 = (wave % ns) * KS;
     auto open = [&](int u) {
       const int sl = uni(u / tpw);
       return mf_open_up<F>(S.slots[s0 + sl], g + (u - sl * tpw) * G, H, I, k0, lane);
@@ -408,7 +410,7 @@ __device__ __forceinline__ void mf_down_phase(Step<M>& S, const DecodeArgs& a, u
       mf_zero_bytes(mf_smem + (size_t)2 * M * rs);
       __syncthreads();
     };
-    const int ns = mf_slices(I, MfFmt<F>::STEPK), KS = I / ns, k0 = (wave % ns) * KS;
+    const int ns = mf_slices(I, MfFmt<F>::STEPK, MfFmt<F>::MINSTEPS), KS = I / ns, k0 = (wave % ns) * KS;
     auto open = [&](int u) {
       const int j = uni((ua + u) / tps);
       return mf_open_down<F>(S.slots[sl0 + j], ua + u - j * tps, H, I, k0, lane);
