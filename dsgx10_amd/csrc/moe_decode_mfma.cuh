@@ -370,7 +370,8 @@ __device__ __forceinline__ void mf_up_phase(Step<M>& S, const DecodeArgs& a, uin
 }
 
 // The units (slot, tile of 16 output rows) are cut into equal contiguous ranges a workgroup; a shared slot in another
-// format counts WSH units a tile (BF16 beside INT4: four times the bytes). A workgroup's range is walked in segments of
+// format counts WSH units a tile (BF16 beside INT4: 3.5 times the bytes, but streamed at the memory's rate where an INT4
+// tile waits for the vector unit: twice the time, measured). A workgroup's range is walked in segments of
 // up to two slots, a stream each (with no more slots than workgroups, the whole range is one segment): the h rows of
 // the segment's slots are staged together and the ring runs on across the slot boundary. FUSED: h was written by this
 // launch; the first segment's weights are requested before the grid barrier is waited for.
@@ -378,7 +379,7 @@ template <int FMT, int SHFMT, int M, bool FUSED>
 __device__ __forceinline__ void mf_down_phase(Step<M>& S, const DecodeArgs& a, uint8_t* mf_smem) {
   constexpr int nsh = SHFMT != 0 ? 1 : 0;
   constexpr bool SH2 = SHFMT != 0 && SHFMT != FMT;
-  constexpr int WSH = 4;
+  constexpr int WSH = 2;
   const int H = a.L.H, I = a.L.I;
   const uint32_t lane = threadIdx.x & 63;
   const int wave = uni((int)(threadIdx.x >> 6));
