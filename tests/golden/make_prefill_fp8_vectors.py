@@ -2,7 +2,7 @@
 """Writes tests/golden/prefill_fp8_expert.npz: input/output vectors of the reference's FP8-activation expert
 (ds41f-4xgx10-switchless/ref/inference/model.py:841-851 over linear() :181-205) computed by the reference's own
 pure-torch kernels (ds41f-4xgx10-switchless/ref/torchref/kernel.py: act_quant :56-77, fp8_gemm :118-125), in the
-128 x 128 / 1 x 128 f32-scale form BASELINE's FP8 prefill configuration names (act_quant(x, 128, None),
+128 x 128 / 1 x 128 f32-scale form of the benchmark's FP8 prefill configuration (act_quant(x, 128, None),
 fp8_gemm(..., block_size=128)).
 
 Run in the build container only (the reference is not on the GPU box):  python tests/golden/make_prefill_fp8_vectors.py
