@@ -9,10 +9,12 @@ experts + 1 shared, intermediate 2048, e4m3 weights with 128 x 128 block scales,
 step routes a different seeded logits row, so its experts come from a 6.4 GB pool and not from the caches; the shared
 expert rotates over copies that together exceed the 256 MB Infinity Cache.
 
-Prints ONE JSON line: metric us_per_moe_layer (lower is better), the roofline of the dominant kernel (the gate/up
-kernel, timed alone with HIP events on its launch stream), the CPU baseline (the C++ oracle on the host cores over
-the same step) and, unless --no-extra, the other benchmark configurations, each decode configuration with both kernel
-variants (dsgx_decode_cfg::up: 0 = dot products on the vector unit, the headline; 1 = on the bf16 MFMA).
+Prints ONE JSON line: metric us_per_moe_layer (lower is better), the roofline of the kernel the timed step launches
+(the layer's algorithmic bytes over its time in the timed graph, HIP events on the launch stream; the gate/up kernel
+launched alone is an extra field), the CPU baseline (the C++ oracle on the host cores over the same step, which also
+checks the GPU's outputs) and, unless --no-extra, the other benchmark configurations, each decode configuration with
+both kernel variants (dsgx_decode_cfg::up: 0 = dot products on the vector unit; 1 = on the bf16 MFMA) and each prefill
+chunk with a few of its rows checked against the oracle.
 """
 import argparse
 import ctypes as C
@@ -33,13 +35,13 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
-# HBM bytes a launch of the FP8 M=1 gate/up kernel, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs of this script,
-# each scaled by what the counter reads for a kernel of known size in the same run (profiles/): 152,222,720 read +
-# 2,359,296 written (algorithmic bytes: 151,031,808)
-UP_TRAFFIC_FP8_M1 = 154582016
+# HBM bytes a launch of the FP8 M=1 decode kernel (k_decode), from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs of this
+# script, each scaled by what the counter reads for a kernel of known size in the same run (profiles/): the algorithmic
+# bytes are 226,547,712
+LAYER_TRAFFIC_FP8_M1 = 231007642
 
 
-def prefill_extra(gen, T, name, peak):
+def prefill_extra(gen, T, name, peak, check=True):
     """a prefill chunk of the benchmark: T rows, top-8 experts drawn from a Zipf(1.1) popularity, uniform weights; FP8
     weights and activations on the e4m3 MFMA (peak 5 PFLOP/s), or INT4 weights decoded to bf16 on the bf16 MFMA
     (2.5 PFLOP/s); TFLOP/s over the useful multiply-adds of the routed experts (T * 8 * 3 * I * H * 2)"""
@@ -53,8 +55,46 @@ def prefill_extra(gen, T, name, peak):
                                                                       ("combine", 8, False), ("shared", 16, True))})
     log("  %s T=%d: routed %.3f ms (%.0f TFLOP/s, %.1f%% of %.1f PFLOP/s), with shared %.3f ms" %
         (name, T, d["ms_routed"], d["tflops_routed"], 100 * d["mfma_frac"], peak / 1e15, d["ms_with_shared"]))
+    if check:
+        d["gpu_vs_oracle"] = prefill_check_rows(pb)
+        log("  %s: rows %s against the oracle: max-abs %.2e, rel-L2 %.2e" %
+            (name, d["gpu_vs_oracle"]["rows"], d["gpu_vs_oracle"]["max_abs_err"], d["gpu_vs_oracle"]["rel_l2"]))
     del pb
     return d
+
+
+def prefill_check_rows(pb, nrows=4):
+    """Part of the CPU leg: a few rows of the chunk just timed against the C++ oracle (FP8 layers: the FP8-activation
+    contract row by row; INT4 layers: a chunk row is a decode row). Returns the worst errors over the rows."""
+    import torch
+    from dsgx10_amd import abi
+    from tests import orc   # the oracle: test infrastructure, used here as the checker only
+    pb.run(31, True)
+    torch.cuda.synchronize()
+    T, gen = pb.T, pb.gen
+    cnt = torch.bincount(pb.idx.reshape(-1).long(), minlength=gen.E).cpu().numpy()
+    idx_h = pb.idx.cpu().numpy()
+    hot, cold = int(np.argmax(cnt)), int(np.argmin(np.where(cnt > 0, cnt, 1 << 30)))
+    rows = [int(np.nonzero((idx_h == hot).any(1))[0][-1]), int(np.nonzero((idx_h == cold).any(1))[0][0]), 0, T - 1][:nrows]
+    worst = dict(rows=rows, max_abs_err=0.0, rel_l2=0.0)
+    for t in rows:
+        experts = sorted(int(e) for e in idx_h[t])
+        hl = gen.host_sublayer(experts, 0)
+        li = np.array([experts.index(int(e)) for e in idx_h[t]], np.int32)
+        x = pb.x[t:t + 1].view(torch.int16).cpu().numpy().view(np.uint16)
+        w = pb.w[t:t + 1].cpu().numpy()
+        if gen.fmt == abi.FMT_FP8:
+            o = orc.moe_prefill_fp8_row(hl, x[0], li, w[0])
+            ref = [o["yr"], o["ys"]]
+        else:
+            uni = np.arange(len(experts), dtype=np.int32)
+            up = orc.moe_up(hl, x, uni, want_range=False)
+            dn = orc.moe_down(hl, up["h32"], li[None, :], w, uni)
+            ref = [dn["yr32"][0], dn["ys32"][0]]
+        for got, r in zip((pb.yr[t].cpu().numpy(), pb.ys[t].cpu().numpy()), ref):
+            worst["max_abs_err"] = max(worst["max_abs_err"], float(np.abs(got - r).max()))
+            worst["rel_l2"] = max(worst["rel_l2"], float(np.sqrt(((got - r).astype(np.float64) ** 2).sum() / max((r.astype(np.float64) ** 2).sum(), 1e-300))))
+    return worst
 
 
 def main():
@@ -145,7 +185,7 @@ def main():
             for up in (0, 1):
                 _, e = run_decode(gen, M, ks, min(W, 16), up)
                 extra.append(decode_entry(gen, M, e, up))
-        extra.append(prefill_extra(gen, 8192, "fp8_moe_prefill", 5.0e15) if head_fp8 else prefill_extra(gen, 2048, "int4_moe_prefill", 2.5e15))
+        extra.append(prefill_extra(gen, 8192, "fp8_moe_prefill", 5.0e15, not args.no_cpu) if head_fp8 else prefill_extra(gen, 2048, "int4_moe_prefill", 2.5e15, not args.no_cpu))
         other = Int4LayerGen(seed=0) if head_fp8 else Fp8LayerGen(seed=0)
         for M in (1, 8):
             for up in (0, 1):
@@ -155,7 +195,7 @@ def main():
                     d["cpu_baseline"] = cpu_baseline(ob, 3.0)
                 extra.append(d)
                 del ob
-        extra.append(prefill_extra(other, 2048, "int4_moe_prefill", 2.5e15) if head_fp8 else prefill_extra(other, 8192, "fp8_moe_prefill", 5.0e15))
+        extra.append(prefill_extra(other, 2048, "int4_moe_prefill", 2.5e15, not args.no_cpu) if head_fp8 else prefill_extra(other, 8192, "fp8_moe_prefill", 5.0e15, not args.no_cpu))
         del other
         from dsgx10_amd.benchdata import gemv_bench
         extra += gemv_bench()
@@ -179,9 +219,18 @@ def main():
                    "kernels_per_step": ["k_decode (routing + gate/up + SwiGLU + down + weighted sum, one persistent launch)"] if head_up == 0 else
                                        ["k_decode_mfma (routing + gate/up + SwiGLU + down, one persistent launch)", "k_down_combine (weighted sum in expert order)"],
                    "timed_as": "one HIP graph of all steps, one replay"},
-        "roofline": {"bound": "hbm", "kernel": "k_up (gate/up + SwiGLU)" if head_up == 0 else "k_up_mfma (gate/up + SwiGLU)", "achieved": r["up_gbs"], "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": r["up_frac"], "traffic": UP_TRAFFIC_FP8_M1 if head_fp8 and head_up == 0 else None, "bytes_per_launch": r["up_bytes"],
-                     "avg_launch_us": r["up_us"], "measured_stream_read_gbs": stream_gbs},
+        # the kernel(s) of the timed step: the algorithmic bytes of a layer (every weight byte of the picked experts and the
+        # shared expert once, scales included) over the step's time in the timed graph (HIP events on the launch stream)
+        "roofline": {"bound": "hbm",
+                     "kernel": "k_decode<FP8_B128, FP8_B128, 1, 2>" if head_fp8 and head_up == 0 else
+                               ("k_decode" if head_up == 0 else "k_decode_mfma + k_down_combine"),
+                     "achieved": r["bytes_per_layer"] / (r["us_per_layer"] * 1e-6) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": r["layer_hbm_frac"], "traffic": LAYER_TRAFFIC_FP8_M1 if head_fp8 and head_up == 0 else None,
+                     "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of an earlier run of this command (profiles/), not measured in this run",
+                     "bytes_per_launch": r["bytes_per_layer"], "avg_launch_us": r["us_per_layer"],
+                     "gate_up_kernel_alone": {"kernel": "k_up" if head_up == 0 else "k_up_mfma", "avg_launch_us": r["up_us"],
+                                              "bytes_per_launch": r["up_bytes"], "achieved": r["up_gbs"], "frac": r["up_frac"]},
+                     "measured_stream_read_gbs": stream_gbs},
         "cpu_baseline": cpu,
         "extra": extra,
         "wall_s": round(time.time() - t_start, 1),

@@ -15,13 +15,23 @@ extern "C" {
 
 void dsgx_decode_cfg_default(dsgx_decode_cfg* c) {
   if (!c) return;
-  c->up = c->down = 0;
+  c->up = -1;  // the faster variant for the layer's format and the row count (decode_variant)
+  c->down = 0;
   c->parts = 3;
   c->ysum = 0;
   c->logits = c->bias = nullptr;
   c->route_scale = 1.f;
   c->score_fn = 0;
   c->post = nullptr;
+}
+
+// dsgx_decode_cfg::up = -1: INT4 layers run on the MFMA kernels at every row count; FP8 layers on the vector-unit
+// kernels at one row (the stream is then bound by memory alone) and on the MFMA kernels from two rows on; BF16 layers
+// have the vector-unit kernels only.
+static int decode_variant(uint32_t fmt, int M) {
+  if (fmt == DSGX_FMT_INT4_G32) return 1;
+  if (fmt == DSGX_FMT_FP8_B128) return M >= 2 ? 1 : 0;
+  return 0;
 }
 
 static size_t ws_h_bytes(const dsgx_layer_w* L) { return (size_t)(DSGX_MAX_UNION + 1) * DSGX_MAX_ROWS * L->I * 2; }
@@ -49,7 +59,8 @@ int dsgx_moe_decode(const dsgx_layer_w* L, const uint16_t* x, const int* idx, co
   if (!c.logits && (!idx || !w)) return fail(DSGX_EINVAL, "moe_decode: idx and w, or logits");
   if (c.post) return fail(DSGX_EUNSUPPORTED, "moe_decode: posted outputs need the reference's ring; one GPU has none");
   if (c.parts < 1 || c.parts > 3) return fail(DSGX_EINVAL, "moe_decode: parts %d", c.parts);
-  if (c.up < 0 || c.up > 1 || c.down < 0 || c.down > 1) return fail(DSGX_EINVAL, "moe_decode: up variant %d / down variant %d", c.up, c.down);
+  if (c.up < -1 || c.up > 1 || c.down < 0 || c.down > 1) return fail(DSGX_EINVAL, "moe_decode: up variant %d / down variant %d", c.up, c.down);
+  if (c.up == -1) c.up = c.down == 1 ? 0 : decode_variant(L->fmt, M);  // (the two-launch form is the vector-unit kernels')
   if (c.up == 1 && L->fmt != DSGX_FMT_FP8_B128 && L->fmt != DSGX_FMT_INT4_G32)
     return fail(DSGX_EUNSUPPORTED, "moe_decode: variant 1 (MFMA) is built for FP8_B128 and INT4_G32 layers");
   if (c.down == 1 && c.parts == 3) c.parts = 3 | 4;  // variant 1: the two phases as two launches
@@ -109,6 +120,24 @@ int dsgx_moe_decode(const dsgx_layer_w* L, const uint16_t* x, const int* idx, co
   }
   if (fp8sh || b16sh) return fail(DSGX_EUNSUPPORTED, "moe_decode: BF16 experts with a fused shared expert are not built");
   return launch_decode_bf16(a, c.parts, st);
+}
+
+// ---- the barrier's error flag ------------------------------------------------------------------------------------------
+int dsgx_decode_status(const dsgx_layer_w* L, void* ws, void* stream) {
+  if (!L || L->I <= 0 || L->H <= 0) return fail(DSGX_EINVAL, "decode_status: null or empty layer");
+  if (!ws) return fail(DSGX_EINVAL, "decode_status: null workspace");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  uint8_t* bar = static_cast<uint8_t*>(ws) + ws_h_bytes(L);
+  int flag = 0;
+  DSGX_HIP(hipMemcpyAsync(&flag, bar + (size_t)(2 * kBarGroups + 1) * kBarLine * 4, 4, hipMemcpyDeviceToHost, st));
+  DSGX_HIP(hipStreamSynchronize(st));
+  if (!flag) return DSGX_OK;
+  // the barrier's counters may be anywhere after a wait that gave up: all of its words back to zero
+  DSGX_HIP(hipMemsetAsync(bar, 0, kBarBytes, st));
+  DSGX_HIP(hipStreamSynchronize(st));
+  return fail(DSGX_ETIMEOUT, "moe_decode: a workgroup gave up waiting at the fused kernel's grid barrier (the grid was not resident: "
+                             "another kernel or process held part of the GPU); the outputs of the steps since the last check are invalid. "
+                             "The workspace is usable again; dsgx_decode_cfg::down = 1 runs the step without a grid barrier");
 }
 
 }  // extern "C"

@@ -426,6 +426,11 @@ __device__ __forceinline__ void up_phase(const DecodeArgs& a, uint4* xs, Step<M>
   } else {
     up_body<FMT, M, false, kUpCH, kUpD>(a, xs, S.slots, nsh, &S.next_up, blockIdx.x, gridDim.x, [&] { return nsh + wait_slots(S); });
   }
+  // Every wave waits here for its own h stores to be acknowledged by the memory system (the stores are device-scope
+  // write-through; the ring's trailing loads, which hit the cache, complete with them). The fused kernel's grid barrier
+  // then needs only the workgroup barrier in front of its arrival: a workgroup-scope release alone does not wait for
+  // the vector memory counter.
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 }
 
 // ---- down ------------------------------------------------------------------------------------------------------------------
@@ -736,8 +741,10 @@ constexpr size_t kBarBytes = (size_t)(2 * kBarGroups + 2) * kBarLine * 4;
 __device__ __forceinline__ int bar_load(int* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 __device__ __forceinline__ int grid_barrier_gen(int* bar) { return bar_load(bar + (kBarGroups + 1 + blockIdx.x % kBarGroups) * kBarLine); }
 __device__ __forceinline__ void grid_barrier(int* bar, int my_gen, int spin_limit) {
-  // h was stored with device-scope coherent stores; __syncthreads() waits for every wave's stores to complete, so no
-  // cache write-back or invalidate is needed around the counters (a device-scope fence would flush the whole L2 here)
+  // h was stored with device-scope write-through stores and every wave has waited for its own to complete (the
+  // s_waitcnt vmcnt(0) that ends the gate/up phase), so after the workgroup barrier all of this workgroup's h is in
+  // memory and no cache write-back or invalidate is needed around the counters (a device-scope fence would flush the
+  // whole L2 here)
   __syncthreads();
   if (threadIdx.x == 0) {
     const int g = blockIdx.x % kBarGroups;

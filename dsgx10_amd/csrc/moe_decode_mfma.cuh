@@ -367,6 +367,8 @@ __device__ __forceinline__ void mf_up_phase(Step<M>& S, const DecodeArgs& a, uin
   } else {
     if (nsh + nrouted > 0) run(std::integral_constant<int, FMT>{}, 0, nsh + nrouted);
   }
+  // the wave's h stores are complete before it goes on to the grid barrier (see up_phase)
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 }
 
 // The units (slot, tile of 16 output rows) are cut into equal contiguous ranges a workgroup; a shared slot in another

@@ -32,7 +32,8 @@ typedef enum dsgx_status {
   DSGX_EINVAL = 1,      /* an argument the reference would die() on */
   DSGX_EFORMAT = 2,     /* unknown / unsupported weight format tag (never guessed) */
   DSGX_EUNSUPPORTED = 3,/* a reference feature that has no meaning on one GPU (ring posting) or is not built */
-  DSGX_EHIP = 4         /* a HIP runtime error (message has hipGetErrorString) */
+  DSGX_EHIP = 4,        /* a HIP runtime error (message has hipGetErrorString) */
+  DSGX_ETIMEOUT = 5     /* dsgx_decode_status: a fused decode step gave up at its grid barrier; its outputs are invalid */
 } dsgx_status;
 
 /* Weight format tags (dsgx_mat_desc::fmt, dsgx_layer_w::fmt, dsgx_gemv_seg::fmt). */
@@ -102,10 +103,13 @@ DSGX_API int dsgx_route(const float* logits, const float* bias, int M, int E, in
 
 /* ---- decode: gx::moe_decode (engine/experts/experts.h:104-147, decode.cu:708-730) ------------------------------- */
 typedef struct dsgx_decode_cfg {
-  int32_t up, down;        /* kernel variants. up 0: dot products on the vector unit; up 1: on the bf16 MFMA (FP8_B128 and
-                              INT4_G32 layers, 1-16 rows; a row's bits are the same in any batch within a variant, but differ
-                              between the variants in the order of the f32 adds). down (with up 0) 0: both phases in one
-                              persistent kernel; 1: two launches */
+  int32_t up, down;        /* kernel variants (the reference's DecodeCfg::up / down choose among its launch shapes too).
+                              up -1 (the default): the faster of the two below for the layer's format and row count
+                              (INT4_G32: 1; FP8_B128: 0 at one row, 1 from two rows on; BF16: 0). up 0: dot products on the
+                              vector unit; up 1: on the bf16 MFMA (FP8_B128 and INT4_G32 layers, 1-16 rows). A row's bits are
+                              the same in any batch within a variant; the two variants differ in the order of the f32 adds
+                              inside a dot product, so a caller that needs a row's bits not to depend on the row count
+                              names the variant. down (with up 0) 0: both phases in one persistent kernel; 1: two launches */
   int32_t parts;           /* 1 up only, 2 down only, 3 both (bench) */
   int32_t ysum;            /* 1: yr += ys in f32 after the routed experts (experts.h:132-136) */
   const float* logits;     /* fused routing (experts.h:123-127): with logits (+ optional bias) idx, w are not read */
@@ -123,6 +127,12 @@ DSGX_API size_t dsgx_decode_ws_bytes(const dsgx_layer_w* L);
    happen when the grid is not resident, e.g. the GPU is shared with another process) sets this flag to 1 and the step's
    outputs are invalid. No counterpart in the reference (its two kernels are ordered by the stream). */
 DSGX_API size_t dsgx_decode_ws_flag_offset(const dsgx_layer_w* L);
+/* Reads that flag: waits for `stream`, returns DSGX_OK when no step since the last check gave up at the barrier, else
+   DSGX_ETIMEOUT after putting the barrier's words back to their initial state (the workspace is usable again; the outputs
+   of the steps since the last check are invalid). Synchronous, so not for
+   use under stream capture: call it where the host waits for results anyway. No counterpart in the reference (its two
+   kernels are ordered by the stream and cannot time out); the C++ mirrors expose it as gx::decode_check(). */
+DSGX_API int dsgx_decode_status(const dsgx_layer_w* L, void* ws, void* stream);
 /* x bf16 [M][H]; idx, w from dsgx_route; yr, ys f32 [M][H]. ys is written when the layer has a fused shared expert,
    otherwise it is an input (only read with ysum). h of the step stays in ws: slot s (the s-th picked expert in
    expert-id order) at ((s * M + m) * I + c), the shared expert's at slot DSGX_SH_SLOT. */

@@ -261,12 +261,14 @@ static inline float route_sum(const float* p, int k) {
 }
 // A/engine/experts/tests/testdata.h:339-355 (route_ref) with E, top-k and the scale as arguments; bias may be null.
 // score_fn 1: sqrt(softplus(l)), softplus as torch's (l > 20 ? l : log1p(exp(l))): D/engine/kernels/common.cuh:261-315.
+static inline float route_score(float v, int score_fn) { return score_fn == 0 ? route_sigmoid(v) : sqrtf(v > 20.f ? v : log1pf(expf(v))); }
+ORC float orc_route_score(float l, int score_fn) { return route_score(l, score_fn); }
 ORC void orc_route(const float* l, const float* bias, int M, int E, int topk, float scale, int score_fn, int* idx, float* w) {
   std::vector<float> s(E), key(E);
   for (int m = 0; m < M; ++m) {
     for (int e = 0; e < E; ++e) {
       const float v = l[(size_t)m * E + e];
-      s[e] = score_fn == 0 ? route_sigmoid(v) : sqrtf(v > 20.f ? v : log1pf(expf(v)));
+      s[e] = route_score(v, score_fn);
       key[e] = s[e] + (bias ? bias[e] : 0.f);
     }
     float p[8];
@@ -630,6 +632,44 @@ ORC void orc_moe_prefill_fp8_row(const dsgx_layer_w* L, const dsgx_mat_desc* des
     if (yr) yr[n] = acc[n];
     if (yr64) yr64[n] = a64[n];
     if (yrmag) yrmag[n] = am[n];
+  }
+}
+
+// The range h of one chunk row can take under the FP8-activation contract when each gate and up sum moves by
+// sum_tol * its sum of |terms| (the rule of orc_moe_up's lo / hi, A/engine/experts/tests/test_experts.cu:395-404, applied
+// to the sums of orc_moe_prefill_fp8_row): lo, hi f32 [topk in expert-id order (+ 1, the shared expert's)][I].
+ORC void orc_moe_prefill_fp8_row_range(const dsgx_layer_w* L, const dsgx_mat_desc* desc, const uint16_t* x, const int* idx,
+                                       double sum_tol, float* lo, float* hi) {
+  const int H = L->H, I = L->I, topk = L->topk;
+  std::vector<uint8_t> xq(H);
+  std::vector<float> xs(H / 128), g, u;
+  std::vector<double> g64, gm, u64, um;
+  orc_act_quant(x, 1, H, xq.data(), xs.data());
+  int ord[8];
+  for (int k = 0; k < topk; ++k) ord[k] = k;
+  std::sort(ord, ord + topk, [&](int a, int b) { return idx[a] < idx[b]; });
+  const int nsl = topk + (sh_fp8(L) ? 1 : 0);
+  for (int s = 0; s < nsl; ++s) {
+    const bool sh = s == topk;
+    const int e = sh ? -1 : idx[ord[s]];
+    const Mat G = sh ? shared_mat(L, 0) : expert_mat(L, desc, e, 0);
+    const Mat Uw = sh ? shared_mat(L, 1) : expert_mat(L, desc, e, 1);
+    fp8_row_qdot(G, xq.data(), xs.data(), g, &g64, &gm);
+    fp8_row_qdot(Uw, xq.data(), xs.data(), u, &u64, &um);
+    for (int c = 0; c < I; ++c) {
+      const double kg = G.s2, ku = Uw.s2;
+      const float hv = silu_mul(bfr((float)(g64[c] * kg)), bfr((float)(u64[c] * ku)));
+      float l = hv, hh = hv;
+      const double g0 = (g64[c] - sum_tol * gm[c]) * kg, g1 = (g64[c] + sum_tol * gm[c]) * kg;
+      const double u0 = (u64[c] - sum_tol * um[c]) * ku, u1 = (u64[c] + sum_tol * um[c]) * ku;
+      const double gs[3] = {g0, g1, std::min(std::max(-1.2785, g0), g1)};  // (silu's minimum lies at -1.2785)
+      for (double gg : gs)
+        for (double uu : {u0, u1}) {
+          const float v = silu_mul(bfr((float)gg), bfr((float)uu));
+          l = std::min(l, v), hh = std::max(hh, v);
+        }
+      lo[(size_t)s * I + c] = l, hi[(size_t)s * I + c] = hh;
+    }
   }
 }
 

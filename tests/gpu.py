@@ -36,11 +36,13 @@ def decode_layer(dl, x, idx, w, M, ws=None, **kw):
         ws = empty(lib.decode_ws_bytes(dl.w), 0)
     dx, di, dw = dev(x), (None if idx is None else dev(idx)), (None if w is None else dev(w))
     yr, ys = empty(M * H * 4, 0xFF), empty(M * H * 4, 0xFF)
+    kw.setdefault("up", 0)  # a named variant: a row's bits are then the same at every row count
     if kw.get("ys_in") is not None:
         ys = dev(kw.pop("ys_in"))
     else:
         kw.pop("ys_in", None)
     lib.moe_decode(dl.w, dx, di, dw, M, ws, yr, ys, **kw)
+    lib.decode_status(dl.w, ws)  # (raises if a fused step gave up at its grid barrier)
     return host(yr, np.float32, (M, H)), host(ys, np.float32, (M, H)), ws
 
 

@@ -61,13 +61,13 @@ def check_sums(got, ref64, mag, tol=1e-4):
     return float(e.max()), int((~(e <= tol)).sum())
 
 
-def check_outputs(got, ref, bf16_rel=True):
+def check_outputs(got, ref, bf16_rel=True, stress=False):
     """The benchmark's bar on outputs against the f32-accumulated oracle: relative L2 <= 1e-3 and max-abs-err <= 2e-2,
     on the f32 outputs and on their bf16 roundings. The absolute bar is stated for outputs of order one (weights
-    ~ N(0, 0.02), activations ~ N(0, 1)): where a value is large enough for one bf16 step to exceed 2e-2 the step is
-    allowed, and for the stress layers made of random codes (outputs of order 1e3) it scales with max|ref| / 8."""
+    ~ N(0, 0.02), activations ~ N(0, 1)); a value large enough for one bf16 step to exceed 2e-2 is allowed that step.
+    stress: the layers made of random codes (outputs of order 1e3), where the absolute bar scales with max|ref| / 8."""
     got, ref = np.asarray(got, np.float32), np.asarray(ref, np.float32)
-    scale = max(1.0, float(np.abs(ref).max()) / 8.0)
+    scale = max(1.0, float(np.abs(ref).max()) / 8.0) if stress else 1.0
     assert rel_l2(got, ref) <= 1e-3, rel_l2(got, ref)
     assert np.abs(got - ref).max() <= 2e-2 * scale, np.abs(got - ref).max()
     g16, r16 = orc.bf16_to_f32(orc.f32_to_bf16(got)), orc.bf16_to_f32(orc.f32_to_bf16(ref))

@@ -40,6 +40,8 @@ def lib():
         L.orc_int4_value_bits.argtypes = [C.c_int, C.c_int, C.c_uint16]
         L.orc_route_sigmoid.restype = C.c_float
         L.orc_route_sigmoid.argtypes = [C.c_float]
+        L.orc_route_score.restype = C.c_float
+        L.orc_route_score.argtypes = [C.c_float, C.c_int]
         L.orc_union.restype = C.c_int
         L.orc_threads.restype = C.c_int
     return _lib
@@ -226,6 +228,18 @@ def moe_prefill_fp8_row(hl, xrow, idx, w, h_in=None):
     lib().orc_moe_prefill_fp8_row(C.byref(Lw), _p(desc), _p(xrow), _p(idx), _p(w), _p(h), _p(out["yr"]), _p(out["yr64"]),
                                   _p(out["yrmag"]), _p(out["ys"]), _p(out["ys64"]), _p(out["ysmag"]), _p(hin))
     return out
+
+
+def moe_prefill_fp8_row_range(hl, xrow, idx, sum_tol):
+    """(lo, hi) f32 [topk in expert-id order (+ 1)][I]: the values h may take when the gate and up sums move by
+    sum_tol * their sums of |terms|"""
+    xrow = np.ascontiguousarray(xrow, np.uint16)
+    idx = np.ascontiguousarray(idx, np.int32)
+    n = hl.topk + (1 if hl.has_shared else 0)
+    lo, hi = np.empty((n, hl.I), np.float32), np.empty((n, hl.I), np.float32)
+    Lw, desc = hl.host_layer_w()
+    lib().orc_moe_prefill_fp8_row_range(C.byref(Lw), _p(desc), _p(xrow), _p(idx), C.c_double(sum_tol), _p(lo), _p(hi))
+    return lo, hi
 
 
 def finalize(R, S):

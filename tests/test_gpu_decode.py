@@ -23,7 +23,8 @@ def _layer(fmt, H, I, E, topk, NS, shared, random_codes=False, seed=1):
     return _cache[key]
 
 
-def _check_step(hl, dl, x, idx, w, M, scale_note="", **kw):
+def _check_step(hl, dl, x, idx, w, M, scale_note="", stress=False, **kw):
+    """stress: a layer of random codes (outputs of order 1e3: the absolute bar scales, helpers.check_outputs)"""
     E = hl.E
     yr, ys, ws = gpu.decode_layer(dl, x[:M], idx[:M], w[:M], M, **kw)
     uni = orc.union(idx[:M], E)
@@ -47,7 +48,7 @@ def _check_step(hl, dl, x, idx, w, M, scale_note="", **kw):
     # end to end against the f32-accumulated oracle: bf16 outputs
     full = orc.moe_down(hl, up["h32"], idx[:M], w[:M], uni)
     for got, ref in ((yr, full["yr32"]),) + (((ys, full["ys32"]),) if hl.has_shared else ()):
-        check_outputs(got, ref)
+        check_outputs(got, ref, stress=stress)
     return yr, ys, hg
 
 
@@ -87,8 +88,8 @@ def test_decode_random_codes_asymmetric_int4_and_fp8():
     for fmt, shared in ((abi.FMT_INT4, None), (abi.FMT_FP8, None)):
         hl, dl = _layer(fmt, 2048, 2048, 64, 8, 3, shared, random_codes=True, seed=3)
         x, logits, idx, w = rows_and_routing(5, 4, 2048, 64, 8, 2.5)
-        _check_step(hl, dl, x, idx, w, 4)
-        _check_step(hl, dl, x, idx, w, 4, up=1)  # variant 1: the same decode through the MFMA's lane order
+        _check_step(hl, dl, x, idx, w, 4, stress=True)
+        _check_step(hl, dl, x, idx, w, 4, up=1, stress=True)  # variant 1: the same decode through the MFMA's lane order
 
 
 def test_decode_fused_routing_and_ysum():
@@ -160,9 +161,9 @@ def test_decode_parts_and_duplicate_experts_across_rows():
     _check_step(hl, dl, x, idx, w, 4)
     H_ = hl.H
     yr1 = gpu.empty(4 * H_ * 4, 0xFF)
-    lib.moe_decode(dl.w, gpu.dev(x), gpu.dev(idx), gpu.dev(w), 4, ws, yr1, None, parts=1)   # up only: yr untouched
+    lib.moe_decode(dl.w, gpu.dev(x), gpu.dev(idx), gpu.dev(w), 4, ws, yr1, None, parts=1, up=0)   # up only: yr untouched
     assert np.all(gpu.host(yr1, np.uint32, (-1,)) == 0xFFFFFFFF)
-    lib.moe_decode(dl.w, gpu.dev(x), gpu.dev(idx), gpu.dev(w), 4, ws, yr1, None, parts=2)   # down only, from ws's h
+    lib.moe_decode(dl.w, gpu.dev(x), gpu.dev(idx), gpu.dev(w), 4, ws, yr1, None, parts=2, up=0)   # down only, from ws's h
     assert np.array_equal(gpu.host(yr1, np.float32, (4, H_)).view(np.uint32), yr.view(np.uint32))
 
 

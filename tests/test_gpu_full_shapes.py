@@ -1,0 +1,202 @@
+"""GPU parity at the benchmark's own shapes (marked gpu): the decode layers of configurations 3 and 4 at their full
+sizes, the FP8 prefill chunk of configuration 5 (T = 8192, hidden 4096, intermediate 2048, 256 experts + FP8 shared,
+Zipf(1.1) top-8) and configuration 4's INT4 prefill chunk (T = 2048, hidden 6144, intermediate 2048, 168 experts + BF16
+shared). The layers alias a handful of stored experts under all expert ids (testdata.h:197 of the reference does the
+same), so the host copies stay small while every index, offset and launch shape is the benchmark's. Shaped after the
+reference's prefill tests (altar1-4xgx10-switchless/engine/experts/tests/test_prefill.inc:36-62, 103-305): bucket
+invariants on all rows, sampled rows against the CPU reference, chunk independence."""
+import numpy as np
+import pytest
+import torch
+
+from dsgx10_amd import abi, lib
+from tests import gpu, helpers, orc
+from tests.test_gpu_decode import _check_step
+
+pytestmark = pytest.mark.gpu
+
+
+def zipf_picks(T, E, topk, s=1.1, seed=4321):
+    """top-k distinct experts a row drawn (without replacement) from a Zipf(s) popularity over a seeded permutation of the
+    experts: the k largest of log p + Gumbel noise; uniform weights 1 / top-k (the bench's prefill input)"""
+    rng = np.random.default_rng(seed)
+    logp = -s * np.log(rng.permutation(E) + 1.0)
+    idx = np.argsort(-(logp[None, :] + rng.gumbel(size=(T, E))), axis=1, kind="stable")[:, :topk]
+    return np.ascontiguousarray(idx, np.int32), np.full((T, topk), 1.0 / topk, np.float32)
+
+
+def _run_prefill(hl, dl, x, idx, w, **kw):
+    T = x.shape[0]
+    ws = gpu.empty(lib.prefill_ws_bytes(dl.w, T), 0)
+    yr, ys = gpu.empty(T * hl.H * 4, 0xFF), gpu.empty(T * hl.H * 4, 0xFF)
+    lib.moe_prefill(dl.w, gpu.dev(x), gpu.dev(idx), gpu.dev(w), T, ws, yr, ys, **kw)
+    return gpu.host(yr, np.float32, (T, hl.H)), gpu.host(ys, np.float32, (T, hl.H)), ws
+
+
+def _buckets(dl, ws, idx, T, E, topk):
+    """the bucketing's outputs checked on ALL rows against numpy; returns (off, perm, rpos, re, view)"""
+    v = lib.prefill_view(dl.w, ws, T)
+    P = T * topk
+    off = gpu.host(gpu.view(ws, v.off, (E + 1) * 4), np.int32, (E + 1,))
+    perm = gpu.host(gpu.view(ws, v.perm, P * 4), np.int32, (P,))
+    re = gpu.host(gpu.view(ws, v.re, P * 4), np.int32, (T, topk))
+    rpos = gpu.host(gpu.view(ws, v.rpos, P * 4), np.int32, (T, topk))
+    cnt = np.bincount(idx.reshape(-1), minlength=E)
+    assert np.array_equal(off, np.concatenate([[0], np.cumsum(cnt)])), "off is not the prefix sum of the experts' counts"
+    e_flat, t_flat = idx.reshape(-1), np.repeat(np.arange(T, dtype=np.int32), topk)
+    assert np.array_equal(perm, t_flat[np.lexsort((t_flat, e_flat))]), "perm: an expert's rows are not in row order"
+    assert np.array_equal(re, np.sort(idx, axis=1)), "re: a row's picks are not in expert-id order"
+    assert np.array_equal(perm[rpos], np.repeat(np.arange(T)[:, None], topk, 1)), "rpos does not lead back to the row"
+    assert np.all((off[re] <= rpos) & (rpos < off[re + 1])), "rpos outside its expert's bucket"
+    return off, perm, rpos, re, v
+
+
+def _sample_rows(off, perm, T, n=64, seed=1):
+    """rows of the hottest experts (first and last row of the bucket, both sides of every 128-row tile boundary, rows of
+    the ragged last tile), rows of the coldest non-empty experts, then random rows up to n"""
+    cnt = np.diff(off)
+    rows = []
+    for e in np.argsort(-cnt)[:3]:
+        o, c = off[e], cnt[e]
+        nt = (c + 127) // 128
+        pos = [0, c - 1] + [128 * i + d for i in range(1, min(nt, 4)) for d in (-1, 0)] + [128 * (nt - 1) + (c - 128 * (nt - 1)) // 2]
+        rows += [int(perm[o + p]) for p in pos if 0 <= p < c]
+    for e in [e for e in np.argsort(cnt) if cnt[e] > 0][:6]:
+        rows += [int(perm[off[e]]), int(perm[off[e + 1] - 1])]
+    rng = np.random.default_rng(seed)
+    rows += [int(t) for t in rng.integers(0, T, 4 * n)]
+    out = []
+    for t in rows:
+        if t not in out:
+            out.append(t)
+    return out[:n], cnt
+
+
+def _h_rows(ws, ptr, nrows, I, rows):
+    """rows of a bf16 [nrows][I] tensor inside the workspace (only the sampled rows cross PCIe)"""
+    t = gpu.view(ws, ptr, nrows * I * 2).view(nrows, I * 2)
+    sel = t[torch.as_tensor(np.asarray(rows, np.int64), device=t.device)]
+    torch.cuda.synchronize()
+    return sel.cpu().numpy().view(np.uint16).reshape(len(rows), I)
+
+
+def test_prefill_fp8_at_the_benchmark_shape():
+    T, H, I, E, topk = 8192, 4096, 2048, 256, 8
+    hl = helpers.make_layer(abi.FMT_FP8, H, I, E, topk, 6, seed=3, shared="fp8")
+    dl = hl.upload()
+    x = orc.normal_bf16(11, 1, (T, H), 1.0)
+    idx, w = zipf_picks(T, E, topk)
+    yr, ys, ws = _run_prefill(hl, dl, x, idx, w)
+    off, perm, rpos, re, v = _buckets(dl, ws, idx, T, E, topk)
+    rows, cnt = _sample_rows(off, perm, T)
+    assert cnt.max() > 4 * 128 and np.median(cnt) < 128, "the draw should give multi-tile hot experts and sub-tile cold ones"
+    nh = nbad = 0
+    worst_sum = 0.0
+    ref_r, ref_s, got_r, got_s = [], [], [], []
+    for t in rows:
+        o = orc.moe_prefill_fp8_row(hl, x[t], idx[t], w[t])
+        mine = np.concatenate([_h_rows(ws, v.h, T * topk, I, rpos[t]), _h_rows(ws, v.hsh, T, I, [t])])
+        # (1) h: most values equal, every one inside the range the contract allows when the gate and up sums move by
+        # 1e-4 of their sums of |terms| (the reference's tolerance on such sums, test_experts.cu:352-361, which is also
+        # what the e4m3 MFMA's own additions are good for: test_mfma_fp8_accuracy)
+        nbad += int((mine != o["h"]).sum())
+        nh += mine.size
+        lo, hi = orc.moe_prefill_fp8_row_range(hl, x[t], idx[t], 1e-4)
+        hv = orc.bf16_to_f32(mine)
+        far = ~((hv >= lo[:mine.shape[0]]) & (hv <= hi[:mine.shape[0]]))
+        assert far.sum() == 0, (t, int(far.sum()), float(np.abs(hv - orc.bf16_to_f32(o["h"])).max()))
+        # (2) down + combine from the GPU's own h: the reference's GEMV tolerance and the benchmark's bar
+        o2 = orc.moe_prefill_fp8_row(hl, x[t], idx[t], w[t], h_in=mine)
+        for got, r64, mag, r32 in ((yr[t], o2["yr64"], o2["yrmag"], o2["yr"]), (ys[t], o2["ys64"], o2["ysmag"], o2["ys"])):
+            worst, bad = helpers.check_sums(got, r64, mag)
+            worst_sum = max(worst_sum, worst)
+            assert bad == 0, (t, worst)
+            helpers.check_outputs(got, r32, bf16_rel=False)
+        ref_r.append(o["yr"]), ref_s.append(o["ys"]), got_r.append(yr[t]), got_s.append(ys[t])
+    assert nbad <= 0.05 * nh, (nbad, nh)
+    # (3) end to end against the oracle's own h on the sampled rows. Two correct evaluations of this contract do not
+    # agree to the benchmark's 1e-3 / 2e-2 here: ~2% of the gate and up sums fall on the other side of a bf16 rounding
+    # (the MFMA's additions against the oracle's f32 ones), one such h in sixteen then moves a whole e4m3 step (6-12% of
+    # its value) when h is quantised for the down projection, and at this shape the outputs are of order 1-3. The bar
+    # is held stage by stage in (2); end to end the sampled rows stay within 3e-3 / 6e-2 (measured: 1.3e-3 routed,
+    # 2.4e-3 shared, max-abs 3.9e-2).
+    e2e_r, e2e_s = helpers.rel_l2(np.stack(got_r), np.stack(ref_r)), helpers.rel_l2(np.stack(got_s), np.stack(ref_s))
+    mx = max(np.abs(np.stack(got_r) - np.stack(ref_r)).max(), np.abs(np.stack(got_s) - np.stack(ref_s)).max())
+    print("fp8 prefill T=8192: %d rows sampled, h equal %.2f%%, staged |err|/sum|terms| %.2e, end-to-end rel-L2 routed %.2e shared %.2e, max-abs %.2e"
+          % (len(rows), 100 - 100.0 * nbad / nh, worst_sum, e2e_r, e2e_s, mx))
+    assert e2e_r <= 3e-3 and e2e_s <= 3e-3 and mx <= 6e-2
+    # (4) a row's bits do not depend on the chunk: a slice of rows as a chunk of its own
+    a, b = 4000, 4100
+    yr2, ys2, _ = _run_prefill(hl, dl, x[a:b], idx[a:b], w[a:b])
+    assert np.array_equal(yr[a:b].view(np.uint32), yr2.view(np.uint32)) and np.array_equal(ys[a:b].view(np.uint32), ys2.view(np.uint32))
+
+
+def test_prefill_int4_chunk_at_the_benchmark_shape():
+    T, H, I, E, topk = 2048, 6144, 2048, 168, 8
+    hl = helpers.make_layer(abi.FMT_INT4, H, I, E, topk, 5, seed=6, shared="bf16")
+    dl = hl.upload()
+    x = orc.normal_bf16(13, 1, (T, H), 1.0)
+    idx, w = zipf_picks(T, E, topk, seed=77)
+    w *= np.float32(2.5)
+    yr, ys, ws = _run_prefill(hl, dl, x, idx, w)
+    off, perm, rpos, re, v = _buckets(dl, ws, idx, T, E, topk)
+    rows, cnt = _sample_rows(off, perm, T)
+    assert cnt.max() > 2 * 128 and np.median(cnt) < 128
+    exact = total = 0
+    worst_row, row_l2 = 0.0, []
+    ref_yr, ref_ys, got_yr, got_ys = [], [], [], []
+    for t in rows:
+        # a chunk row is a decode row (test_prefill.inc:307-373): h and the outputs against the decode oracle
+        uni = orc.union(idx[t:t + 1], E)
+        up = orc.moe_up(hl, x[t:t + 1], uni)
+        mine = np.concatenate([_h_rows(ws, v.h, T * topk, I, rpos[t]), _h_rows(ws, v.hsh, T, I, [t])])[:, None, :]
+        hv = orc.bf16_to_f32(mine)
+        assert np.all((hv >= up["lo"]) & (hv <= up["hi"])), "h outside the range of f32 sums (row %d)" % t
+        exact += int(((mine == up["h64"]) | ((hv == 0) & (orc.bf16_to_f32(up["h64"]) == 0))).sum())
+        total += mine.size
+        dn = orc.moe_down(hl, mine, idx[t:t + 1], w[t:t + 1], uni)
+        for got, k in ((yr, "yr"), (ys, "ys")):
+            worst, bad = helpers.check_sums(got[t:t + 1], dn[k + "64"], dn[k + "mag"], 1e-4)
+            assert bad == 0, (t, k, worst)
+        full = orc.moe_down(hl, up["h32"], idx[t:t + 1], w[t:t + 1], uni)
+        # per row, the reference's own bar between a chunk row and the decode path: 2e-3 of the row's largest output
+        # (test_prefill.inc:220-248)
+        for got, k in ((yr, "yr32"), (ys, "ys32")):
+            err = float(np.abs(got[t] - full[k][0]).max() / np.abs(full[k][0]).max())
+            worst_row = max(worst_row, err)
+            assert err <= 2e-3, (t, k, err)
+            row_l2.append(helpers.rel_l2(got[t], full[k][0]))
+        ref_yr.append(full["yr32"][0]), ref_ys.append(full["ys32"][0]), got_yr.append(yr[t]), got_ys.append(ys[t])
+    print("int4 prefill T=2048: %d rows sampled, h bit-equal %.3f%%, worst row error %.2e of the row's max, per-row rel-L2 median %.2e max %.2e, "
+          "sampled rows together rel-L2 routed %.2e shared %.2e, max-abs %.2e"
+          % (len(rows), 100.0 * exact / total, worst_row, np.median(row_l2), np.max(row_l2), helpers.rel_l2(np.stack(got_yr), np.stack(ref_yr)),
+             helpers.rel_l2(np.stack(got_ys), np.stack(ref_ys)), max(np.abs(np.stack(got_yr) - np.stack(ref_yr)).max(), np.abs(np.stack(got_ys) - np.stack(ref_ys)).max())))
+    # h against the f64 sums: the reference asks 98.5% bit-equal of a prefill chunk (test_prefill.inc:186), 99.5% of decode
+    assert exact >= 0.985 * total, (exact, total)
+    # the benchmark's bar (relative L2 1e-3, max-abs 2e-2) on the sampled rows' f32 outputs taken together. (Their bf16
+    # roundings are held to max-abs only: where got and ref differ by ~3e-4 relative, ~6% of the values round to different
+    # bf16 neighbours, a step of 4-8e-3 each, which is 1.4e-3 in relative L2 although the values agree within the bar.)
+    helpers.check_outputs(np.stack(got_yr), np.stack(ref_yr), bf16_rel=False)
+    helpers.check_outputs(np.stack(got_ys), np.stack(ref_ys), bf16_rel=False)
+    a, b = 1000, 1050
+    yr2, ys2, _ = _run_prefill(hl, dl, x[a:b], idx[a:b], w[a:b])
+    assert np.array_equal(yr[a:b].view(np.uint32), yr2.view(np.uint32)) and np.array_equal(ys[a:b].view(np.uint32), ys2.view(np.uint32))
+
+
+@pytest.mark.parametrize("fmt,H,I,E,shared,scale,NS", [(abi.FMT_FP8, 4096, 2048, 256, "fp8", 1.0, 6), (abi.FMT_INT4, 6144, 2048, 168, "bf16", 2.5, 5)],
+                         ids=["fp8-config3", "int4-config4"])
+def test_decode_layers_at_the_benchmark_shapes(fmt, H, I, E, shared, scale, NS):
+    """configuration 3 (M = 1, 4, 8) and configuration 4 (M = 1, 8) at their full shapes, both kernel variants and the
+    library's own choice of variant, against the oracle; fused routing gives the same bits as routing apart"""
+    topk = 8
+    hl = helpers.make_layer(fmt, H, I, E, topk, NS, seed=9, shared=shared)
+    dl = hl.upload()
+    x, logits, idx, w = helpers.rows_and_routing(29, 8, H, E, topk, scale)
+    for M in (1, 4, 8):
+        outs = {}
+        for up in (0, 1):
+            outs[up] = _check_step(hl, dl, x, idx, w, M, up=up)
+        yr_a, ys_a, _ = gpu.decode_layer(dl, x[:M], None, None, M, logits=gpu.dev(logits[:M]), route_scale=scale, up=-1)
+        pick = 1 if fmt == abi.FMT_INT4 or M >= 2 else 0   # the library's table
+        assert np.array_equal(yr_a.view(np.uint32), outs[pick][0].view(np.uint32)), (M, "auto variant / fused routing")
+        assert np.array_equal(ys_a.view(np.uint32), outs[pick][1].view(np.uint32))

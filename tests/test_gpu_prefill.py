@@ -99,6 +99,7 @@ def test_prefill_fp8_against_oracle(H, I, E, topk, T, shared):
     hg = gpu.host(gpu.view(ws, v.h, P * I * 2), np.uint16, (P, I))
     hsh = gpu.host(gpu.view(ws, v.hsh, T * I * 2), np.uint16, (T, I)) if shared else None
     nh = nbad = 0
+    worst_sum = 0.0
     ref_r, ref_s = np.empty((T, H), np.float32), np.empty((T, H), np.float32)
     for t in range(T):
         # (1) gate/up + SwiGLU. The e4m3 MFMA does not add its products in full f32 precision (test_mfma_fp8_accuracy:
@@ -115,12 +116,19 @@ def test_prefill_fp8_against_oracle(H, I, E, topk, T, shared):
             assert np.all(np.abs(a - b) <= 4 * step + 5e-5), np.abs(a - b).max()  # (5e-5: values that are a difference of large terms)
         # (2) down + combine from the very h the GPU made: the GEMV tolerance of the reference (:352-361) and the bar
         o = orc.moe_prefill_fp8_row(hl, x[t], idx[t], w[t], h_in=np.stack(mine))
-        helpers.check_sums(yr[t], o["yr64"], o["yrmag"])
+        worst, bad = helpers.check_sums(yr[t], o["yr64"], o["yrmag"])
+        assert bad == 0, (t, worst)
+        worst_sum = max(worst_sum, worst)
         helpers.check_outputs(yr[t], o["yr"], bf16_rel=False)  # (the MFMA's ~1e-5 relative error flips bf16 roundings too)
         if shared:
-            helpers.check_sums(ys[t], o["ys64"], o["ysmag"])
+            worst, bad = helpers.check_sums(ys[t], o["ys64"], o["ysmag"])
+            assert bad == 0, (t, worst)
+            worst_sum = max(worst_sum, worst)
             helpers.check_outputs(ys[t], o["ys"], bf16_rel=False)
     assert nbad <= 0.05 * nh, (nbad, nh)
+    print("fp8 prefill H=%d I=%d T=%d: h equal %.2f%%, staged |err|/sum|terms| %.2e, end-to-end rel-L2 routed %.2e%s, max-abs %.2e"
+          % (H, I, T, 100 - 100.0 * nbad / nh, worst_sum, helpers.rel_l2(yr, ref_r),
+             " shared %.2e" % helpers.rel_l2(ys, ref_s) if shared else "", np.abs(yr - ref_r).max()))
     # (3) end to end against the oracle's own h. A bf16 step of one h is, one time in ten or so, an e4m3 step of its
     # quantised value (6-12% of it), or of its whole block of 128 when it is the block's maximum: two correct
     # evaluations of this contract differ by about 1e-3 in relative L2 (measured here: 0.6e-3 to 1.4e-3). The bar of

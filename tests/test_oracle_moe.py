@@ -164,3 +164,21 @@ def test_finalize():
     S = orc.normal_f32(0, 2, (64,), 1.0)
     want = (torch.from_numpy(R).to(torch.bfloat16) + torch.from_numpy(S).to(torch.bfloat16)).view(torch.int16).numpy().view(np.uint16)
     assert np.array_equal(orc.finalize(R, S), want)
+
+
+def test_prefill_fp8_row_range_brackets_h():
+    """the allowed range of a chunk row's h under the FP8-activation contract: it collapses to the f64 sums' h at
+    tolerance 0, widens with the tolerance, and holds the f32 contract's h at the reference's sum tolerance"""
+    from dsgx10_amd import abi
+    from tests import helpers
+    hl = helpers.make_layer(abi.FMT_FP8, 512, 256, 16, 4, 6, seed=3, shared="fp8")
+    x, _, idx, w = helpers.rows_and_routing(11, 3, 512, 16, 4, 2.5)
+    for t in range(3):
+        h = orc.bf16_to_f32(orc.moe_prefill_fp8_row(hl, x[t], idx[t], w[t])["h"])
+        lo0, hi0 = orc.moe_prefill_fp8_row_range(hl, x[t], idx[t], 0.0)
+        assert np.array_equal(lo0, hi0) and (lo0 == h).mean() > 0.99
+        lo1, hi1 = orc.moe_prefill_fp8_row_range(hl, x[t], idx[t], 2e-5)
+        lo2, hi2 = orc.moe_prefill_fp8_row_range(hl, x[t], idx[t], 1e-4)
+        assert np.all(lo2 <= lo1) and np.all(lo1 <= lo0) and np.all(hi0 <= hi1) and np.all(hi1 <= hi2)
+        assert np.all((h >= lo1) & (h <= hi1))
+        assert (hi2 > lo2).any() and np.all(hi2 - lo2 <= 0.05 * np.maximum(np.abs(h), 0.05) + 1e-3)

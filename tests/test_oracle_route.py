@@ -89,3 +89,63 @@ def test_route_top6_sum_order_and_bias_is_selection_only():
 def test_union_sorted_unique():
     idx = np.array([[5, 3, 9], [3, 200, 0]], np.int32)
     assert list(orc.union(idx, 256)) == [0, 3, 5, 9, 200]
+
+
+# ---- DeepSeek's score function: sqrt(softplus(l)) (ds41f-4xgx10-switchless/engine/kernels/common.cuh:266-315) ----------
+def _ulp32(v):
+    v = np.abs(np.asarray(v, np.float64))
+    return 2.0 ** (np.floor(np.log2(np.maximum(v, 2.0 ** -126))) - 23)
+
+
+def test_sqrt_softplus_score_against_f64():
+    """score(l) = sqrt(l > 20 ? l : log1p(exp(l))) within 2 f32 ulp of the f64 value on a grid that covers both branches,
+    the switch at 20 itself, large negative logits (softplus -> exp(l)) and the overflow side of expf"""
+    L = orc.lib()
+    xs = np.concatenate([np.linspace(-30, 30, 6001), np.linspace(19.9, 20.1, 401), [20.0, np.nextafter(np.float32(20), np.float32(21)), 25.0, 60.0, 88.0, 100.0, -80.0, 0.0]]).astype(np.float32)
+    got = np.array([L.orc_route_score(float(v), 1) for v in xs], np.float64)
+    x64 = xs.astype(np.float64)
+    want = np.sqrt(np.where(xs > np.float32(20), x64, np.log1p(np.exp(np.minimum(x64, 50.0)))))
+    assert np.all(np.abs(got - want) <= 2 * _ulp32(want)), float((np.abs(got - want) / _ulp32(want)).max())
+    assert np.all(np.diff(got[:6001]) >= 0)  # monotone over the grid
+    # the branch: exactly l above 20 (the square root of the logit itself, correctly rounded)
+    for v in (20.5, 33.0, 100.0):
+        assert L.orc_route_score(v, 1) == float(np.sqrt(np.float32(v)))
+    # a different function (the sigmoid, or softplus without the root) is far outside the tolerance
+    assert abs(L.orc_route_score(1.0, 1) - L.orc_route_score(1.0, 0)) > 0.1
+    assert abs(L.orc_route_score(1.0, 1) - np.log1p(np.exp(1.0))) > 0.1
+
+
+def test_sqrt_softplus_route_top6_order_and_sum_order():
+    """the whole DeepSeek selection (router_row, common.cuh:266-315): keys = score + bias, top-6 by (key descending, id
+    ascending) found by brute force, weights = score / (((p0+p4)+p2)+((p1+p5)+p3) + 1e-20) * scale with the bias left
+    out of the weights; a sequential sum of the six gives other bits on some rows"""
+    E, M, topk, scale = 384, 64, 6, 1.5
+    l = orc.normal_f32(7, 2, (M, E), 1.0)
+    l[0, :4] = [25.0, 21.0, 30.0, 20.5]      # rows that take the l > 20 branch
+    l[1, 5] = l[1, 300] = l[1, 17] = 3.25      # a three-way tie inside the top six
+    bias = orc.normal_f32(7, 3, (E,), 0.05)
+    bias[5] = bias[300] = bias[17] = 0.0
+    idx, w = orc.route(l, bias, topk, scale, score_fn=1)
+    other_order = 0
+    for m in range(M):
+        s = np.array([orc.lib().orc_route_score(float(v), 1) for v in l[m]], np.float32)
+        key = (s + bias).astype(np.float32)
+        order = sorted(range(E), key=lambda e: (-float(key[e]), e))[:topk]
+        assert list(idx[m]) == order
+        p = s[idx[m]]
+        tot = np.float32(np.float32(np.float32(p[0] + p[4]) + p[2]) + np.float32(np.float32(p[1] + p[5]) + p[3]))
+        want = (p / np.float32(tot + np.float32(1e-20))) * np.float32(scale)
+        assert np.array_equal(w[m].view(np.uint32), want.astype(np.float32).view(np.uint32))
+        seq = np.float32(0)
+        for v in p:
+            seq = np.float32(seq + v)
+        other_order += not np.array_equal((p / np.float32(seq + np.float32(1e-20)) * np.float32(scale)).astype(np.float32), w[m])
+        assert abs(float(w[m].astype(np.float64).sum()) - scale) < 1e-5
+    assert list(idx[1][:3]) == [5, 17, 300] or {5, 17, 300} <= set(idx[1])  # ties go to the lower id, in id order
+    pos = [list(idx[1]).index(e) for e in (5, 17, 300)]
+    assert pos == sorted(pos)
+    assert other_order > 0
+    # no bias (null) is bias 0
+    i2, w2 = orc.route(l, None, topk, scale, score_fn=1)
+    i3, w3 = orc.route(l, np.zeros(E, np.float32), topk, scale, score_fn=1)
+    assert np.array_equal(i2, i3) and np.array_equal(w2.view(np.uint32), w3.view(np.uint32))
