@@ -6,6 +6,7 @@ FMT_FP8, FMT_INT4, FMT_BF16 = 16, 18, 19
 OUT_BF16, OUT_F32, OUT_SWIGLU = 0, 1, 2
 MAX_ROWS, MAX_TOPK, MAX_UNION, SH_SLOT, MAX_EXPERTS, MAX_CHUNK = 16, 8, 128, 128, 512, 8192
 OK, EINVAL, EFORMAT, EUNSUPPORTED, EHIP, ETIMEOUT = 0, 1, 2, 3, 4, 5
+NOALLOC_MAX_H, NOALLOC_MAX_I = 6144, 2048
 
 
 class MatDesc(C.Structure):
@@ -45,7 +46,7 @@ assert C.sizeof(MatDesc) == 64
 # every symbol include/dsgx.h declares
 SYMBOLS = [
     "dsgx_mat_bytes", "dsgx_mat_scale_off", "dsgx_mat_zp_off", "dsgx_route", "dsgx_decode_cfg_default",
-    "dsgx_decode_ws_bytes", "dsgx_decode_ws_flag_offset", "dsgx_decode_status", "dsgx_moe_decode", "dsgx_finalize", "dsgx_prefill_cfg_default", "dsgx_prefill_ws_bytes",
+    "dsgx_decode_ws_bytes", "dsgx_decode_ws_flag_offset", "dsgx_decode_status", "dsgx_moe_decode", "dsgx_moe_decode_noalloc", "dsgx_finalize", "dsgx_prefill_cfg_default", "dsgx_prefill_ws_bytes",
     "dsgx_moe_prefill", "dsgx_prefill_view_get", "dsgx_gemv", "dsgx_dequant_int4", "dsgx_probe_dequant_int4", "dsgx_probe_mfma_fp8",
     "dsgx_widen_fp8", "dsgx_act_quant", "dsgx_last_error", "dsgx_version", "dsgx_stream_read", "dsgx_stream_read_cfg", "dsgx_stream_copy",
 ]

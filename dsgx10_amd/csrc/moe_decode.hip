@@ -1,6 +1,8 @@
 // The C ABI of the decode expert step (dsgx_moe_decode = gx::moe_decode of the reference,
 // altar1-4xgx10-switchless/engine/experts/decode.cu:708-730): argument checks and the dispatch on the layer's format.
 // The kernels are in moe_decode_impl.cuh, instantiated per format in moe_decode_{fp8,int4,bf16}.hip.
+#include <mutex>
+
 #include "moe_decode_impl.cuh"
 
 using namespace dsgx;
@@ -10,6 +12,37 @@ static unsigned long long* g_trace_buf = nullptr;  // device memory, [workgroups
 extern "C" __attribute__((visibility("default"))) void dsgx_trace_set(void* dev) { g_trace_buf = static_cast<unsigned long long*>(dev); }
 extern "C" unsigned long long* dsgx_trace_buf() { return g_trace_buf; }
 #endif
+
+// The workspace of dsgx_moe_decode_noalloc: a device array of the library itself, sized for the largest layer that entry
+// point takes (h of 129 slots x 16 rows x DSGX_NOALLOC_MAX_I, the barrier's words, the slot-partitioned down phase's
+// table and its f32 [129][8][DSGX_NOALLOC_MAX_H] results: 33.8 MB on every GPU the library runs on, zero when the
+// module loads, which is the barrier's initial state). In host code the array's name is not a device address: the
+// address is asked for once a device (static_ws) and only that pointer is used.
+static constexpr size_t kStaticWsBytes = (size_t)(DSGX_MAX_UNION + 1) * DSGX_MAX_ROWS * DSGX_NOALLOC_MAX_I * 2 + dsgx::kBarBytes +
+                                         (size_t)(8 + (DSGX_MAX_UNION + 1) * 8) * 4 + 192 +
+                                         (size_t)(DSGX_MAX_UNION + 1) * 8 * DSGX_NOALLOC_MAX_H * 4;
+static __device__ __align__(256) uint8_t scratch[kStaticWsBytes];
+// (never launched: keeps the array referenced from device code of this file)
+__global__ void k_scratch_probe(uint8_t* out) {
+  if (out) *out = scratch[0];
+}
+static int static_ws(void** out) {
+  constexpr int kMaxDev = 64;
+  static void* ptr[kMaxDev] = {};
+  static std::mutex mu;
+  int dev = 0;
+  DSGX_HIP(hipGetDevice(&dev));
+  if (dev < 0 || dev >= kMaxDev) return fail(DSGX_EINVAL, "moe_decode_noalloc: device %d", dev);
+  std::lock_guard<std::mutex> lk(mu);
+  if (!ptr[dev]) {
+    void* p = nullptr;
+    DSGX_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));  // (the current device's copy of the array)
+    if (!p) return fail(DSGX_EHIP, "moe_decode_noalloc: no address for the built-in workspace");
+    ptr[dev] = p;
+  }
+  *out = ptr[dev];
+  return DSGX_OK;
+}
 
 extern "C" {
 
@@ -125,7 +158,11 @@ int dsgx_moe_decode(const dsgx_layer_w* L, const uint16_t* x, const int* idx, co
 // ---- the barrier's error flag ------------------------------------------------------------------------------------------
 int dsgx_decode_status(const dsgx_layer_w* L, void* ws, void* stream) {
   if (!L || L->I <= 0 || L->H <= 0) return fail(DSGX_EINVAL, "decode_status: null or empty layer");
-  if (!ws) return fail(DSGX_EINVAL, "decode_status: null workspace");
+  if (!ws) {
+    void* p = nullptr;
+    if (int rc = static_ws(&p)) return rc;
+    ws = p;
+  }
   hipStream_t st = static_cast<hipStream_t>(stream);
   uint8_t* bar = static_cast<uint8_t*>(ws) + ws_h_bytes(L);
   int flag = 0;
@@ -138,6 +175,19 @@ int dsgx_decode_status(const dsgx_layer_w* L, void* ws, void* stream) {
   return fail(DSGX_ETIMEOUT, "moe_decode: a workgroup gave up waiting at the fused kernel's grid barrier (the grid was not resident: "
                              "another kernel or process held part of the GPU); the outputs of the steps since the last check are invalid. "
                              "The workspace is usable again; dsgx_decode_cfg::down = 1 runs the step without a grid barrier");
+}
+
+// ---- the decode step on the library's own workspace ----------------------------------------------------------------------
+int dsgx_moe_decode_noalloc(const dsgx_layer_w* L, const uint16_t* x, const int* idx, const float* w, int M, float* yr, float* ys,
+                            void* stream, const dsgx_decode_cfg* cfg) {
+  if (!L) return fail(DSGX_EINVAL, "moe_decode_noalloc: null layer");
+  if (L->I < 1 || L->I > DSGX_NOALLOC_MAX_I || L->H < 1 || L->H > DSGX_NOALLOC_MAX_H)
+    return fail(DSGX_EINVAL, "moe_decode_noalloc: hidden %d, intermediate %d exceed the built-in workspace (hidden <= %d, intermediate <= %d); "
+                             "use dsgx_moe_decode with a workspace of dsgx_decode_ws_bytes()", L->H, L->I, DSGX_NOALLOC_MAX_H, DSGX_NOALLOC_MAX_I);
+  if (dsgx_decode_ws_bytes(L) > kStaticWsBytes) return fail(DSGX_EINVAL, "moe_decode_noalloc: the layer's workspace exceeds the built-in one");
+  void* ws = nullptr;
+  if (int rc = static_ws(&ws)) return rc;
+  return dsgx_moe_decode(L, x, idx, w, M, ws, yr, ys, stream, cfg);
 }
 
 }  // extern "C"

@@ -40,6 +40,8 @@ def lib():
         L.dsgx_route.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_float, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]
         L.dsgx_moe_decode.argtypes = [C.POINTER(abi.LayerW), C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p,
                                       C.c_void_p, C.c_void_p, C.c_void_p, C.POINTER(abi.DecodeCfg)]
+        L.dsgx_moe_decode_noalloc.argtypes = [C.POINTER(abi.LayerW), C.c_void_p, C.c_void_p, C.c_void_p, C.c_int,
+                                              C.c_void_p, C.c_void_p, C.c_void_p, C.POINTER(abi.DecodeCfg)]
         L.dsgx_decode_status.argtypes = [C.POINTER(abi.LayerW), C.c_void_p, C.c_void_p]
         L.dsgx_finalize.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p]
         L.dsgx_gemv.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.POINTER(abi.GemvSeg), C.c_int, C.c_int, C.c_int, C.c_void_p]
@@ -95,15 +97,19 @@ def decode_ws_flag_offset(layer_w):
 
 def moe_decode(layer_w, x, idx, w, M, ws, yr, ys, stream=None, parts=3, ysum=False, logits=None, bias=None,
                route_scale=1.0, score_fn=0, up=-1, down=0, post=None):
-    """up -1: the library's choice of variant."""
+    """ws None: the library's own workspace (dsgx_moe_decode_noalloc). up -1: the library's choice of variant."""
     cfg = abi.DecodeCfg(up, down, parts, int(ysum), _ptr(logits), _ptr(bias), route_scale, score_fn, post)
+    if ws is None:
+        _check(lib().dsgx_moe_decode_noalloc(C.byref(layer_w), _ptr(x), _ptr(idx), _ptr(w), M, _ptr(yr), _ptr(ys),
+                                             _stream(stream), C.byref(cfg)))
+        return
     _check(lib().dsgx_moe_decode(C.byref(layer_w), _ptr(x), _ptr(idx), _ptr(w), M, _ptr(ws), _ptr(yr), _ptr(ys),
                                  _stream(stream), C.byref(cfg)))
 
 
 def decode_status(layer_w, ws, stream=None):
     """waits for the stream; raises DsgxError(ETIMEOUT) if a fused decode step gave up at its grid barrier since the last
-    check"""
+    check (ws None: the library's own workspace)"""
     _check(lib().dsgx_decode_status(C.byref(layer_w), _ptr(ws), _stream(stream)))
 
 

@@ -129,7 +129,7 @@ DSGX_API size_t dsgx_decode_ws_bytes(const dsgx_layer_w* L);
 DSGX_API size_t dsgx_decode_ws_flag_offset(const dsgx_layer_w* L);
 /* Reads that flag: waits for `stream`, returns DSGX_OK when no step since the last check gave up at the barrier, else
    DSGX_ETIMEOUT after putting the barrier's words back to their initial state (the workspace is usable again; the outputs
-   of the steps since the last check are invalid). Synchronous, so not for
+   of the steps since the last check are invalid). ws null: the workspace of dsgx_moe_decode_noalloc. Synchronous, so not for
    use under stream capture: call it where the host waits for results anyway. No counterpart in the reference (its two
    kernels are ordered by the stream and cannot time out); the C++ mirrors expose it as gx::decode_check(). */
 DSGX_API int dsgx_decode_status(const dsgx_layer_w* L, void* ws, void* stream);
@@ -138,6 +138,17 @@ DSGX_API int dsgx_decode_status(const dsgx_layer_w* L, void* ws, void* stream);
    expert-id order) at ((s * M + m) * I + c), the shared expert's at slot DSGX_SH_SLOT. */
 DSGX_API int dsgx_moe_decode(const dsgx_layer_w* L, const uint16_t* x, const int* idx, const float* w, int M, void* ws,
                              float* yr, float* ys, void* stream, const dsgx_decode_cfg* cfg);
+/* dsgx_moe_decode on a workspace inside the library, for callers that cannot allocate device memory (code under HIP graph
+   capture, serving loops and harnesses that forbid hipMalloc): no workspace argument, no allocation of any kind. It has
+   no counterpart in the reference, whose moe_decode always takes the caller's workspace. The workspace is one array of
+   33.8 MB on every GPU the library runs on, held until the process ends; it fits layers with hidden <= DSGX_NOALLOC_MAX_H
+   and intermediate <= DSGX_NOALLOC_MAX_I (larger ones: DSGX_EINVAL). All calls on a GPU share it: calls that overlap on
+   one GPU (two streams) race; stream-ordered calls are fine (h and the barrier's words are rewritten by every step).
+   Same arguments, bits and errors as dsgx_moe_decode otherwise. */
+#define DSGX_NOALLOC_MAX_H 6144
+#define DSGX_NOALLOC_MAX_I 2048
+DSGX_API int dsgx_moe_decode_noalloc(const dsgx_layer_w* L, const uint16_t* x, const int* idx, const float* w, int M, float* yr,
+                                     float* ys, void* stream, const dsgx_decode_cfg* cfg);
 /* out = bf16(bf16(R) + bf16(S)): gx::finalize (engine/experts/experts.h:146-147, decode.cu:591-598) */
 DSGX_API int dsgx_finalize(const float* R, const float* S, int n, uint16_t* out, void* stream);
 
