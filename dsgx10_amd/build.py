@@ -54,7 +54,24 @@ def build(jobs=None, force=False, extra=(), suffix=""):
     if force or _stale(so, objs):
         cmd = ["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", "-o", so] + objs
         subprocess.check_call(cmd)
+    if not suffix:
+        build_mirror_run(force)
     return so
+
+
+def build_mirror_run(force=False):
+    """tests/mirror_run: the test program that drives the C++ mirror headers on the GPU (host code only; it links the
+    library just built and finds it relative to its own place)"""
+    root = os.path.dirname(HERE)
+    src, exe = os.path.join(root, "tests", "mirror_run.cpp"), os.path.join(root, "tests", "mirror_run")
+    if not os.path.exists(src):
+        return None
+    inc = os.path.join(root, "include")
+    hdrs = [os.path.join(dp, f) for dp, _, fs in os.walk(inc) for f in fs]
+    if force or _stale(exe, [src, SO] + hdrs):
+        subprocess.check_call(["hipcc", "-std=c++17", "-O1", "-Wall", "-I", inc, src, "-o", exe, "-L", CSRC, "-ldsgx",
+                               "-Wl,-rpath,$ORIGIN/../dsgx10_amd/csrc"])
+    return exe
 
 
 if __name__ == "__main__":

@@ -61,9 +61,9 @@ void dsgx_decode_cfg_default(dsgx_decode_cfg* c) {
 // dsgx_decode_cfg::up = -1: INT4 layers run on the MFMA kernels at every row count; FP8 layers on the vector-unit
 // kernels at one row (the stream is then bound by memory alone) and on the MFMA kernels from two rows on; BF16 layers
 // have the vector-unit kernels only.
-static int decode_variant(uint32_t fmt, int M) {
+static int decode_variant(uint32_t fmt, int M, int H, int I) {
   if (fmt == DSGX_FMT_INT4_G32) return 1;
-  if (fmt == DSGX_FMT_FP8_B128) return M >= 2 ? 1 : 0;
+  if (fmt == DSGX_FMT_FP8_B128) return M >= 2 || H % 1024 || I % 1024 ? 1 : 0;  // (shapes only the MFMA kernels' steps divide)
   return 0;
 }
 
@@ -93,7 +93,7 @@ int dsgx_moe_decode(const dsgx_layer_w* L, const uint16_t* x, const int* idx, co
   if (c.post) return fail(DSGX_EUNSUPPORTED, "moe_decode: posted outputs need the reference's ring; one GPU has none");
   if (c.parts < 1 || c.parts > 3) return fail(DSGX_EINVAL, "moe_decode: parts %d", c.parts);
   if (c.up < -1 || c.up > 1 || c.down < 0 || c.down > 1) return fail(DSGX_EINVAL, "moe_decode: up variant %d / down variant %d", c.up, c.down);
-  if (c.up == -1) c.up = c.down == 1 ? 0 : decode_variant(L->fmt, M);  // (the two-launch form is the vector-unit kernels')
+  if (c.up == -1) c.up = c.down == 1 ? 0 : decode_variant(L->fmt, M, L->H, L->I);  // (the two-launch form is the vector-unit kernels')
   if (c.up == 1 && L->fmt != DSGX_FMT_FP8_B128 && L->fmt != DSGX_FMT_INT4_G32)
     return fail(DSGX_EUNSUPPORTED, "moe_decode: variant 1 (MFMA) is built for FP8_B128 and INT4_G32 layers");
   if (c.down == 1 && c.parts == 3) c.parts = 3 | 4;  // variant 1: the two phases as two launches
@@ -105,13 +105,15 @@ int dsgx_moe_decode(const dsgx_layer_w* L, const uint16_t* x, const int* idx, co
   const int H = L->H, I = L->I;
   if (L->E < 1 || L->E > DSGX_MAX_EXPERTS || L->topk < 1 || L->topk > DSGX_MAX_TOPK || L->topk > L->E)
     return fail(DSGX_EINVAL, "moe_decode: E %d, top-k %d", L->E, L->topk);
-  const int kmul = L->fmt == DSGX_FMT_INT4_G32 ? 2048 : L->fmt == DSGX_FMT_FP8_B128 ? 1024 : 512;
+  // the vector-unit kernels walk whole 1 KiB segments of a row (2048 INT4, 1024 FP8, 512 BF16 values); the MFMA kernels
+  // steps of 256 k, so they also take the narrow per-rank shapes (the reference's intermediate 512, experts.h:18-22)
+  const int kmul = c.up == 1 ? 256 : L->fmt == DSGX_FMT_INT4_G32 ? 2048 : L->fmt == DSGX_FMT_FP8_B128 ? 1024 : 512;
   if (H < kmul || H % kmul || I < kmul || I % kmul || I % 128 || H % 128)
-    return fail(DSGX_EINVAL, "moe_decode: hidden %d, intermediate %d (multiples of %d for this format)", H, I, kmul);
+    return fail(DSGX_EINVAL, "moe_decode: hidden %d, intermediate %d (multiples of %d for this format and variant)", H, I, kmul);
   const bool fp8sh = L->sh.g != nullptr, b16sh = L->sh.bgu != nullptr;
   if (fp8sh && b16sh) return fail(DSGX_EINVAL, "moe_decode: an FP8 and a BF16 shared expert");
   if (fp8sh && (!L->sh.u || !L->sh.d || !L->sh.gs || !L->sh.us || !L->sh.ds)) return fail(DSGX_EINVAL, "moe_decode: the FP8 shared expert needs g, u, d and their scales");
-  if (fp8sh && (H % 1024 || I % 1024)) return fail(DSGX_EINVAL, "moe_decode: the FP8 shared expert needs hidden and intermediate multiples of 1024");
+  if (fp8sh && c.up != 1 && (H % 1024 || I % 1024)) return fail(DSGX_EINVAL, "moe_decode: the FP8 shared expert needs hidden and intermediate multiples of 1024");
   if (b16sh && !L->sh.bd) return fail(DSGX_EINVAL, "moe_decode: the BF16 shared expert needs its down");
   if ((c.parts & 2) && !yr) return fail(DSGX_EINVAL, "moe_decode: null yr");
   if ((fp8sh || b16sh || c.ysum) && (c.parts & 2) && !ys) return fail(DSGX_EINVAL, "moe_decode: ys (the shared expert's output) is needed");
@@ -147,8 +149,8 @@ int dsgx_moe_decode(const dsgx_layer_w* L, const uint16_t* x, const int* idx, co
     return launch_decode_fp8(a, c.parts, fp8sh, st);
   }
   if (f == DSGX_FMT_INT4_G32) {
-    if (fp8sh) return fail(DSGX_EUNSUPPORTED, "moe_decode: INT4 experts with an FP8 shared expert are not built");
-    if (c.up == 1) return launch_decode_int4_mfma(a, c.parts & 3, b16sh, st);
+    if (c.up == 1) return launch_decode_int4_mfma(a, c.parts & 3, b16sh ? DSGX_FMT_BF16 : fp8sh ? DSGX_FMT_FP8_B128 : 0, st);
+    if (fp8sh) return fail(DSGX_EUNSUPPORTED, "moe_decode: INT4 experts with an FP8 shared expert run on variant 1 only (dsgx_decode_cfg::up = 1 or -1)");
     return launch_decode_int4(a, c.parts, b16sh, st);
   }
   if (fp8sh || b16sh) return fail(DSGX_EUNSUPPORTED, "moe_decode: BF16 experts with a fused shared expert are not built");

@@ -82,7 +82,7 @@ struct DecodeArgs {
 int launch_decode_fp8(const DecodeArgs& a, int parts, bool shared, hipStream_t st);
 int launch_decode_fp8_mfma(const DecodeArgs& a, int parts, bool shared, hipStream_t st);  // variant 1 (moe_decode_mfma.cuh)
 int launch_decode_int4(const DecodeArgs& a, int parts, bool shared_bf16, hipStream_t st);
-int launch_decode_int4_mfma(const DecodeArgs& a, int parts, bool shared_bf16, hipStream_t st);  // variant 1
+int launch_decode_int4_mfma(const DecodeArgs& a, int parts, int shared_fmt, hipStream_t st);  // variant 1 (shared: 0, BF16 or FP8_B128)
 int launch_decode_bf16(const DecodeArgs& a, int parts, hipStream_t st);
 
 // ---- what a workgroup knows about the step -------------------------------------------------------------------------

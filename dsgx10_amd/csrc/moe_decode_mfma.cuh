@@ -332,9 +332,10 @@ __device__ __forceinline__ void mf_up_phase(Step<M>& S, const DecodeArgs& a, uin
   mf_stage_rows<false>(mf_smem, a.x, H, M, H, pad);
   mf_zero_bytes(mf_smem + (size_t)M * ((size_t)H * 2 + pad));
   __syncthreads();
+  // Units are (slot, tile of 8 channels), numbered slot-major; workgroup g of G walks the units g, g + G, g + 2 G, ...
+  // (with as many tiles a slot as workgroups that is one tile of every slot; with fewer, a narrow intermediate size, the
+  // workgroups still share the slots' tiles evenly)
   const int tiles = I / 8, g = blockIdx.x, G = gridDim.x;
-  const int tpw = uni(g < tiles ? (tiles - g + G - 1) / G : 0);  // this workgroup's tiles a slot
-  if (tpw == 0) return;  // (a workgroup beyond the tiles: no barrier of the workgroup follows in this phase)
   auto done = [&](int sl, int t, v4f_t sum) {
     const int pos = lane & 15, part = lane >> 4;
     if (pos >= M) return;
@@ -347,16 +348,19 @@ __device__ __forceinline__ void mf_up_phase(Step<M>& S, const DecodeArgs& a, uin
   };
   auto run = [&](auto fmt_tag, int s0, int nslots) {  // slots s0 .. s0 + nslots - 1 in format F
     constexpr int F = decltype(fmt_tag)::value;
+    const int total = nslots * tiles;
+    const int mine = uni(g < total ? (total - g + G - 1) / G : 0);  // this workgroup's units
+    if (mine == 0) return;  // (the same for every wave of the workgroup)
     const int ns = mf_slices(H, MfFmt<F>::STEPK, MfFmt<F>::MINSTEPS), KS = H / ns, k0 = (wave % ns) * KS;
     auto open = [&](int u) {
-      const int sl = uni(u / tpw);
-      return mf_open_up<F>(S.slots[s0 + sl], g + (u - sl * tpw) * G, H, I, k0, lane);
+      const int q = g + u * G, sl = uni(q / tiles);
+      return mf_open_up<F>(S.slots[s0 + sl], q - sl * tiles, H, I, k0, lane);
     };
     auto fin = [&](int u, v4f_t sum) {
-      const int sl = uni(u / tpw);
-      done(s0 + sl, g + (u - sl * tpw) * G, sum);
+      const int q = g + u * G, sl = uni(q / tiles);
+      done(s0 + sl, q - sl * tiles, sum);
     };
-    mf_stream<F, M>(mf_smem, mf_rows_bytes(M, H, pad), (uint32_t)(M * ((size_t)H * 2 + pad)), pad, H, k0, ns, nslots * tpw, KS / MfFmt<F>::STEPK, open,
+    mf_stream<F, M>(mf_smem, mf_rows_bytes(M, H, pad), (uint32_t)(M * ((size_t)H * 2 + pad)), pad, H, k0, ns, mine, KS / MfFmt<F>::STEPK, open,
                     [](int) { return 0u; }, fin, [] {});
   };
   const int nrouted = uni(S.n);

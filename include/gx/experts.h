@@ -63,43 +63,65 @@ struct LayerW {
 };
 
 // ---- routing (experts.h:99-102) -----------------------------------------------------------------------------------
+// The first seven arguments are the reference's; the rest carry what its compile-time constants fix (168 experts, top-8,
+// sigmoid scores scaled by 2.5). score_fn: 0 sigmoid, 1 sqrt(softplus) (the DeepSeek engine's router).
 inline void route(const float* logits, const float* bias, int M, int* idx, float* w, void* st, bool pdl = true, int E = kE,
-                  int topk = kTopK, float scale = kRouteScale) {
+                  int topk = kTopK, float scale = kRouteScale, int score_fn = 0) {
   (void)pdl;
-  DSGX_DIE_ON(dsgx_route(logits, bias, M, E, topk, scale, 0, idx, w, st));
+  DSGX_DIE_ON(dsgx_route(logits, bias, M, E, topk, scale, score_fn, idx, w, st));
 }
 
 // ---- decode (experts.h:104-147) -----------------------------------------------------------------------------------
+// The reference's variant numbers name its launch shapes (decode.cu:624-698); here up / down are this build's variants
+// (dsgx_decode_cfg). kUpPrefillOrder (experts.h:111-113,138: decode = prefill bit for bit) has no counterpart yet and is
+// refused by name rather than mapped to something else.
+constexpr int kUpPrefillOrder = 6;
 struct DecodeCfg {
-  int up = 0, down = 0;
+  int up = -1, down = 0;   // up -1: the faster variant for the layer's format and the row count
   int up_ctas_per_sm = 0;  // accepted, unused: the grid is sized to the chip
   bool pdl = true;         // accepted, unused
-  bool dyn = true;         // accepted, unused: batches are walked round-robin, no task counter
+  bool dyn = true;         // accepted, unused: batches are claimed from a counter in LDS
   bool xpf = true;         // accepted, unused
   int parts = 3;
   const float* logits = nullptr;
   const float* bias = nullptr;
   float route_scale = kRouteScale;  // fused routing's scale (the reference's is the constant 2.5)
+  int score_fn = 0;                 // fused routing's score: 0 sigmoid, 1 sqrt(softplus)
   const void* post = nullptr;       // must be null
   bool ysum = false;
 };
 inline size_t decode_ws_bytes(const LayerW& L) { const dsgx_layer_w c = L.c(); return dsgx_decode_ws_bytes(&c); }
+// the reference's form (experts.h:139): the workspace of a layer of its compile-time shape (LayerW's defaults)
+inline size_t decode_ws_bytes() { return decode_ws_bytes(LayerW()); }
 inline void moe_decode(const LayerW& L, const uint16_t* x, const int* idx, const float* w, int M, void* ws, float* yr, float* ys,
                        void* st, const DecodeCfg& cfg = DecodeCfg()) {
+  if (cfg.up == kUpPrefillOrder) die("moe_decode: up variant %d (decode in the prefill kernels' order of adds) is not built", cfg.up);
   const dsgx_layer_w c = L.c();
   dsgx_decode_cfg d;
   dsgx_decode_cfg_default(&d);
   d.up = cfg.up, d.down = cfg.down, d.parts = cfg.parts, d.ysum = cfg.ysum, d.logits = cfg.logits, d.bias = cfg.bias;
-  d.route_scale = cfg.route_scale, d.post = cfg.post;
+  d.route_scale = cfg.route_scale, d.score_fn = cfg.score_fn, d.post = cfg.post;
   DSGX_DIE_ON(dsgx_moe_decode(&c, x, idx, w, M, ws, yr, ys, st, &d));
+}
+// Dies if a fused decode step since the last check gave up at its grid barrier (its outputs are invalid). Waits for the
+// stream: call it where the host waits for results anyway. No counterpart in the reference, whose two kernels are
+// ordered by the stream.
+inline void decode_check(const LayerW& L, void* ws, void* st) {
+  const dsgx_layer_w c = L.c();
+  DSGX_DIE_ON(dsgx_decode_status(&c, ws, st));
 }
 inline int decode_up_variants() { return 2; }
 inline int decode_down_variants() { return 2; }
 inline const char* decode_up_name(int v) { return v == 1 ? "mfma16 kslices" : "rows4 lanes64"; }
 inline const char* decode_down_name(int v) { return v == 1 ? "two launches" : "rows2 lanes64"; }
-inline void finalize(const float* R, const float* S, int M, uint16_t* out, void* st, bool pdl = true, int H = kH) {
+// out[m][n] = bf16(bf16(R) + bf16(S)) over M rows (experts.h:146-147, decode.cu:591-598). The reference's form takes M and
+// uses its compile-time hidden size, 6144: for a layer of another width pass the layer.
+inline void finalize(const float* R, const float* S, int M, uint16_t* out, void* st, bool pdl = true) {
   (void)pdl;
-  DSGX_DIE_ON(dsgx_finalize(R, S, M * H, out, st));
+  DSGX_DIE_ON(dsgx_finalize(R, S, M * kH, out, st));
+}
+inline void finalize(const LayerW& L, const float* R, const float* S, int M, uint16_t* out, void* st) {
+  DSGX_DIE_ON(dsgx_finalize(R, S, M * L.H, out, st));
 }
 
 // ---- prefill (experts.h:149-193) ----------------------------------------------------------------------------------
@@ -113,6 +135,7 @@ struct PrefillCfg {
   bool act_fp8 = true;      // FP8 layers: e4m3 activations on the fp8 MFMA (see dsgx_prefill_cfg)
 };
 inline size_t prefill_ws_bytes(const LayerW& L, int T) { const dsgx_layer_w c = L.c(); return dsgx_prefill_ws_bytes(&c, T); }
+inline size_t prefill_ws_bytes(int T) { return prefill_ws_bytes(LayerW(), T); }  // the reference's form (experts.h:180)
 inline void moe_prefill_phases(const LayerW& L, const uint16_t* x, const int* idx, const float* w, int T, void* ws, float* yr,
                                float* ys, void* st, const PrefillCfg& cfg, int phases) {
   if (cfg.diag || cfg.ddiag) die("moe_prefill: bench diagnostics are not built");
@@ -136,5 +159,6 @@ inline PrefillView prefill_view(const LayerW& L, void* ws, int T) {
   DSGX_DIE_ON(dsgx_prefill_view_get(&c, ws, T, &v));
   return PrefillView{v.rpos, v.re, v.h, v.hsh};
 }
+inline PrefillView prefill_view(void* ws, int T) { return prefill_view(LayerW(), ws, T); }  // the reference's form (experts.h:190)
 
 }  // namespace gx

@@ -208,3 +208,25 @@ def test_decode_mfma_variant(case):
     # fused routing, and 9-16 rows as two passes
     yr_l, ys_l, _ = gpu.decode_layer(dl, x, None, None, 8, logits=gpu.dev(logits), route_scale=scale, up=1)
     assert np.array_equal(yr_l.view(np.uint32), runs[8][0].view(np.uint32))
+
+
+@pytest.mark.parametrize("fmt,H,I,E,shared,scale", [(abi.FMT_INT4, 6144, 512, 168, "bf16", 2.5), (abi.FMT_INT4, 2048, 2048, 32, "fp8", 2.5),
+                                                   (abi.FMT_FP8, 1280, 768, 32, "fp8", 1.0)],
+                         ids=["int4-per-rank-I512", "int4-fp8-shared", "fp8-H1280-I768"])
+def test_decode_variant1_narrow_shapes_and_fp8_shared_beside_int4(fmt, H, I, E, shared, scale):
+    """what only the MFMA kernels take: the reference's per-rank intermediate size (512: experts.h:18-22), hidden and
+    intermediate sizes that are multiples of 256 only, and GLM-5.3's combination of INT4 experts with a fused FP8 shared
+    expert (experts.h:66-87); the library's own choice of variant runs them too"""
+    hl, dl = _layer(fmt, H, I, E, 8, 4, shared, seed=7)
+    x, logits, idx, w = rows_and_routing(23, 8, H, E, 8, scale)
+    runs = {}
+    for M in (1, 3, 8):
+        runs[M] = _check_step(hl, dl, x, idx, w, M, up=1)
+        yr, ys, _ = gpu.decode_layer(dl, x[:M], idx[:M], w[:M], M, up=-1)
+        assert np.array_equal(yr.view(np.uint32), runs[M][0].view(np.uint32)) and np.array_equal(ys.view(np.uint32), runs[M][1].view(np.uint32))
+    for m in (0, 5):
+        yr1, ys1, _ = gpu.decode_layer(dl, x[m:m + 1], idx[m:m + 1], w[m:m + 1], 1, up=1)
+        assert np.array_equal(yr1[0].view(np.uint32), runs[8][0][m].view(np.uint32)) and np.array_equal(ys1[0].view(np.uint32), runs[8][1][m].view(np.uint32))
+    if fmt == abi.FMT_INT4 and shared == "fp8":
+        with pytest.raises(lib.DsgxError):
+            gpu.decode_layer(dl, x[:1], idx[:1], w[:1], 1, up=0)

@@ -1,0 +1,68 @@
+"""The C++ mirror headers on the GPU (marked gpu): tests/mirror_run (tests/mirror_run.cpp, compiled by
+dsgx10_amd.build against include/gx/experts.h and include/glm/attn.h) runs route -> moe_decode -> finalize, the fused
+form and a dense GEMV through the gx:: / glm:: forwarders; every output must equal, bit for bit, what the same calls
+give through the ctypes binding of the C ABI."""
+import os
+import subprocess
+import tempfile
+
+import numpy as np
+import pytest
+import torch
+
+from dsgx10_amd import abi, lib
+from tests import gpu, orc
+from tests.helpers import make_layer, rows_and_routing
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+EXE = os.path.join(ROOT, "tests", "mirror_run")
+
+
+@pytest.mark.parametrize("fmt,shared,scale,up", [(abi.FMT_FP8, "fp8", 1.0, -1), (abi.FMT_FP8, "fp8", 1.0, 0), (abi.FMT_INT4, "bf16", 2.5, 1)])
+def test_cpp_mirrors_give_the_c_abi_bits(fmt, shared, scale, up):
+    assert os.path.exists(EXE), "tests/mirror_run is not built (python -m dsgx10_amd.build)"
+    H, I, E, topk, M = 2048, 2048, 32, 8, 3
+    hl = make_layer(fmt, H, I, E, topk, 4, seed=12, shared=shared)
+    dl = hl.upload()
+    x, logits, _, _ = rows_and_routing(51, M, H, E, topk, scale)
+    bias = orc.normal_f32(51, 3, (E,), 0.3)
+    resid = orc.normal_f32(51, 4, (M, H), 1.0)
+    with tempfile.TemporaryDirectory() as d:
+        def put(name, a):
+            np.ascontiguousarray(a).tofile(os.path.join(d, name + ".bin"))
+        put("pool", hl.pool), put("desc", hl.desc), put("x", x), put("logits", logits), put("bias", bias), put("resid", resid)
+        if hl.shared_fp8 is not None:
+            for n, (c, s) in zip("gud", hl.shared_fp8):
+                put("sh_" + n, c), put("sh_" + n + "s", s)
+        if hl.shared_bf16 is not None:
+            put("sh_bgu", hl.shared_bf16[0]), put("sh_bd", hl.shared_bf16[1])
+        r = subprocess.run([EXE, d, str(fmt), str(H), str(I), str(E), str(topk), str(M), repr(scale), str(up)], capture_output=True, text=True, timeout=120)
+        assert r.returncode == 0 and "CHECK mirror_run ok" in r.stdout, r.stdout + r.stderr
+        got = {n: np.fromfile(os.path.join(d, "o_%s.bin" % n), dt) for n, dt in
+               (("idx", np.int32), ("w", np.uint32), ("yr", np.uint32), ("ys", np.uint32), ("out", np.uint16), ("yr2", np.uint32), ("ys2", np.uint32), ("gemv", np.uint32))}
+    # the same calls through ctypes
+    dlog, dbias = gpu.dev(logits), gpu.dev(bias)
+    gi, gw = gpu.empty(M * topk * 4), gpu.empty(M * topk * 4)
+    lib.route(dlog.view(torch.float32).view(M, E), dbias, gi.view(torch.int32).view(M, topk), gw.view(torch.float32).view(M, topk), scale)
+    idx, w = gpu.host(gi, np.int32, (M, topk)), gpu.host(gw, np.float32, (M, topk))
+    assert np.array_equal(got["idx"], idx.reshape(-1)) and np.array_equal(got["w"], w.view(np.uint32).reshape(-1))
+    ridx, rw = orc.route(logits, bias, topk, scale)
+    assert np.array_equal(idx, ridx) and np.array_equal(w.view(np.uint32), rw.view(np.uint32))
+    yr, ys, _ = gpu.decode_layer(dl, x, idx, w, M, up=up)
+    assert np.array_equal(got["yr"], yr.view(np.uint32).reshape(-1)) and np.array_equal(got["ys"], ys.view(np.uint32).reshape(-1))
+    out = gpu.empty(M * H * 2, 0)
+    lib.finalize(gpu.dev(resid), gpu.dev(yr), M * H, out)
+    assert np.array_equal(got["out"], gpu.host(out, np.uint16, (-1,)))
+    yr2, ys2, _ = gpu.decode_layer(dl, x, None, None, M, logits=dlog, bias=dbias, route_scale=scale, ysum=True, up=up)
+    assert np.array_equal(got["yr2"], yr2.view(np.uint32).reshape(-1)) and np.array_equal(got["ys2"], ys2.view(np.uint32).reshape(-1))
+    assert np.array_equal(yr2, yr + ys)
+    # the dense GEMV
+    gn = I if shared == "fp8" else 2 * I
+    y = gpu.empty(M * gn * 4, 0)
+    if shared == "fp8":
+        seg = dict(fmt=abi.FMT_FP8, w=gpu.dev(hl.shared_fp8[0][0]), s=gpu.dev(hl.shared_fp8[0][1]), n=gn, y=y, ldy=gn)
+    else:
+        seg = dict(fmt=abi.FMT_BF16, w=gpu.dev(hl.shared_bf16[0]), n=gn, y=y, ldy=gn)
+    lib.gemv(gpu.dev(x), H, M, H, [seg], abi.OUT_F32)
+    assert np.array_equal(got["gemv"], gpu.host(y, np.uint32, (-1,)))
