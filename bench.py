@@ -104,7 +104,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=64)
     ap.add_argument("--no-extra", action="store_true", help="only the headline workload")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
-    ap.add_argument("--workload", default="fp8_m1", help="headline workload: fp8_m1 | int4_m1")
+    ap.add_argument("--workload", default="fp8_m1", help="headline workload: fp8_m1 | int4_m1; fp8_prefill | int4_prefill time only that prefill chunk")
     ap.add_argument("--variant", default="vector", choices=("vector", "mfma"),
                     help="the headline's decode kernels (dsgx_decode_cfg::up = 0 | 1); --no-extra then runs nothing else")
     args = ap.parse_args()
@@ -164,6 +164,19 @@ def main():
                            "C++ oracle, OpenMP, f32 sums" % (b.M, len(d["experts"]), len(ts) - 1),
                     gpu_vs_oracle=par)
 
+    if args.workload in ("fp8_prefill", "int4_prefill"):
+        # only the prefill chunk (for profiler runs of the grouped-GEMM kernels): its own JSON line, TFLOP/s over useful MACs
+        fp8 = args.workload == "fp8_prefill"
+        gen = Fp8LayerGen(seed=0) if fp8 else Int4LayerGen(seed=0)
+        d = prefill_extra(gen, 8192 if fp8 else 2048, args.workload.replace("_", "_moe_"), 5.0e15 if fp8 else 2.5e15, not args.no_cpu)
+        print(json.dumps({"metric": "prefill_grouped_gemm_tflops", "value": d["tflops_routed"], "unit": "TFLOP/s", "n_gpus": 1, "steps": 8,
+                          "warmup": 1, "ms_per_step": d["ms_routed"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+                          "dtype": "fp8 (e4m3 x e4m3, f32 sums)" if fp8 else "bf16 (INT4 weights decoded to bf16, f32 sums)", "data": "synthetic",
+                          "config": {"workload": d["workload"], "T": d["T"]},
+                          "roofline": {"bound": "mfma", "achieved": d["tflops_routed"], "peak": d["mfma_peak_tflops"], "unit": "TFLOP/s",
+                                       "frac": d["mfma_frac"], "traffic": None},
+                          "cpu_baseline": None, "extra": [d], "wall_s": round(time.time() - t_start, 1)}))
+        return
     head_fp8 = args.workload == "fp8_m1"
     log("generating the %s layer ..." % ("FP8 256-expert" if head_fp8 else "INT4 168-expert"))
     gen = Fp8LayerGen(seed=0) if head_fp8 else Int4LayerGen(seed=0)

@@ -16,6 +16,7 @@
 // accumulators of a 16 x 16 tile belong to ONE token row and the block's combined scale is one value a lane.
 #include "abi_internal.h"
 #include "common.cuh"
+#include "pf_gemm_fp8.cuh"
 
 #ifdef DSGX_TRACE
 extern "C" unsigned long long* dsgx_trace_buf();
@@ -69,7 +70,8 @@ constexpr int kTile = 128;  // rows of a tile (token positions) and weight rows 
 constexpr int kRowBlock = 128;  // token rows a workgroup of the bucketing kernels
 struct PfLayout {
   size_t cnt, off, ntiles, tile_e, tile_m0, perm, pickpos, rpos, re, rk, xq, xs, h, hq, hs, hsh, hshq, hshs, d, bcnt, boff, bmask, total;
-  int P, max_tiles;
+  size_t nbig, big_e, big_m0, nsmall, small_e, small_m0;  // the FP8 kernels' lists: 256-position tiles, and the experts' remainders
+  int P, max_tiles, max_big;
 };
 PfLayout pf_layout(const dsgx_layer_w* L, int T) {
   PfLayout o{};
@@ -80,6 +82,9 @@ PfLayout pf_layout(const dsgx_layer_w* L, int T) {
   auto take = [&](size_t bytes) { const size_t a = at; at += align256(bytes); return a; };
   o.cnt = take(E * 4), o.off = take((E + 1) * 4), o.ntiles = take(4);
   o.tile_e = take((size_t)o.max_tiles * 4), o.tile_m0 = take((size_t)o.max_tiles * 4);
+  o.max_big = (int)(P / 256 + E);
+  o.nbig = take(4), o.big_e = take((size_t)o.max_big * 4), o.big_m0 = take((size_t)o.max_big * 4);
+  o.nsmall = take(4), o.small_e = take(E * 4), o.small_m0 = take(E * 4);
   o.perm = take(P * 4), o.pickpos = take(P * 4), o.rpos = take(P * 4), o.re = take(P * 4), o.rk = take(P * 4);
   o.xq = take((size_t)T * H), o.xs = take((size_t)T * (H / 128) * 4);
   o.h = take(P * I * 2), o.hq = take(P * I), o.hs = take(P * (I / 128) * 4);
@@ -118,10 +123,16 @@ __global__ void __launch_bounds__(256) k_pf_mask(const int* __restrict__ idx, in
     *reinterpret_cast<uint4*>(&bmask[((size_t)b * E + e) * 4]) = m;
   }
 }
+// The FP8 kernels' two lists: an expert of c rows gives c / 256 tiles of 256 positions, one more if over 128 rows are left,
+// else (if any are left) one tile of up to 128 positions.
+struct TileLists {
+  int *ntiles, *tile_e, *tile_m0;     // all rows in 128-position tiles
+  int *nbig, *big_e, *big_m0;         // 256-position tiles
+  int *nsmall, *small_e, *small_m0;   // the remainders of up to 128 positions
+};
 __global__ void __launch_bounds__(DSGX_MAX_EXPERTS) k_pf_scan(const int* __restrict__ bcnt, int NB, int E, int* __restrict__ boff,
-                                                              int* __restrict__ cnt, int* __restrict__ off, int* __restrict__ ntiles,
-                                                              int* __restrict__ tile_e, int* __restrict__ tile_m0) {
-  __shared__ int sa[DSGX_MAX_EXPERTS], sb[DSGX_MAX_EXPERTS];
+                                                              int* __restrict__ cnt, int* __restrict__ off, TileLists tl) {
+  __shared__ int sa[DSGX_MAX_EXPERTS], sb[DSGX_MAX_EXPERTS], sc[DSGX_MAX_EXPERTS], sd[DSGX_MAX_EXPERTS];
   const int e = threadIdx.x;
   int c = 0;
   if (e < E)
@@ -131,20 +142,24 @@ __global__ void __launch_bounds__(DSGX_MAX_EXPERTS) k_pf_scan(const int* __restr
       c += v;
     }
   const int nt = (c + kTile - 1) / kTile;
-  sa[e] = e < E ? c : 0, sb[e] = e < E ? nt : 0;
+  const int rem = c % 256, nbig = c / 256 + (rem > 128 ? 1 : 0), nsmall = rem > 0 && rem <= 128 ? 1 : 0;
+  sa[e] = e < E ? c : 0, sb[e] = e < E ? nt : 0, sc[e] = e < E ? nbig : 0, sd[e] = e < E ? nsmall : 0;
   __syncthreads();
   for (int d = 1; d < DSGX_MAX_EXPERTS; d <<= 1) {  // inclusive scans of the counts and of the tile counts
-    const int va = e >= d ? sa[e - d] : 0, vb = e >= d ? sb[e - d] : 0;
+    const int va = e >= d ? sa[e - d] : 0, vb = e >= d ? sb[e - d] : 0, vc = e >= d ? sc[e - d] : 0, vd = e >= d ? sd[e - d] : 0;
     __syncthreads();
-    sa[e] += va, sb[e] += vb;
+    sa[e] += va, sb[e] += vb, sc[e] += vc, sd[e] += vd;
     __syncthreads();
   }
   if (e < E) {
     cnt[e] = c;
     off[e] = sa[e] - c;
-    if (e == E - 1) off[E] = sa[e], *ntiles = sb[e];
+    if (e == E - 1) off[E] = sa[e], *tl.ntiles = sb[e], *tl.nbig = sc[e], *tl.nsmall = sd[e];
     const int t0 = sb[e] - nt;
-    for (int i = 0; i < nt; ++i) tile_e[t0 + i] = e, tile_m0[t0 + i] = i * kTile;
+    for (int i = 0; i < nt; ++i) tl.tile_e[t0 + i] = e, tl.tile_m0[t0 + i] = i * kTile;
+    const int b0 = sc[e] - nbig;
+    for (int i = 0; i < nbig; ++i) tl.big_e[b0 + i] = e, tl.big_m0[b0 + i] = i * 256;
+    if (nsmall) tl.small_e[sd[e] - 1] = e, tl.small_m0[sd[e] - 1] = (c / 256) * 256;
   }
 }
 __global__ void __launch_bounds__(256) k_pf_place(const int* __restrict__ idx, const float* __restrict__ w, int T, int topk, int E,
@@ -175,23 +190,8 @@ __global__ void __launch_bounds__(256) k_pf_place(const int* __restrict__ idx, c
   }
 }
 
-// ---- the grouped GEMM ---------------------------------------------------------------------------------------------------
-// Most experts of a chunk hold fewer rows than a tile, so the step mostly streams weights: it is built like the decode
-// kernels. A workgroup (8 waves) computes one tile of 128 positions against 256 weight rows; a WAVE owns 32 of those
-// rows as two 16-row MFMA tiles (UP: 16 gate rows and the 16 up rows of the same channels, so g and u of a channel meet
-// in one lane) and streams them from memory straight into registers, a ring of kRing 128-k blocks ahead: a lane loads
-// 2 x 16 bytes a tile and block, the four lanes of a row 64 contiguous bytes an instruction. The activations of the
-// tile (shared by the eight waves) wait kHold turns in registers and go through kStages LDS stages, stored by MFMA
-// fragment with an exclusive-or in the slot number that keeps writes and reads free of bank conflicts. All global loads
-// are issued with four consecutive lanes on 64 contiguous bytes of a row; the weights are brought into the MFMA's lane
-// order through the wave's own piece of LDS (w_to_lds / read_fa).
-// v_mfma_f32_16x16x128_f8f6f4 covers one whole 128-k scale block: partial = A B^T from zero, then
-// acc = fma(x_scale * w_scale, partial, acc) on the vector unit (the accumulators therefore stay in ordinary registers).
-// With the weights as the A operand a lane's four accumulators of a tile belong to ONE position, so the combined scale is
-// one value a lane.
-constexpr int kPanel = kTile * 128;              // bytes of one activation panel (128 positions x 128 k)
-constexpr int kStages = 4, kRing = 3, kHold = 3;  // LDS stages; turns a weight / an activation load is issued ahead of its use
-constexpr int kStageBytes = kPanel + kTile * 4;  // + the positions' scales of the block
+// ---- the grouped GEMMs ---------------------------------------------------------------------------------------------------
+// FP8 activations (e4m3 MFMA): pf_gemm_fp8.cuh. bf16 activations (bf16 MFMA): k_pf_gemm16 below.
 constexpr int kWgRows = 256;                     // weight rows a workgroup (UP: 128 channels)
 constexpr int kGemmThreads = 512;
 
@@ -213,284 +213,6 @@ __device__ __forceinline__ void pf_task(int NS, int& tile, int& ns) {
   const int NG = (NS + kMapNs - 1) / kMapNs;
   tile = (b / NG) * kMapTiles + i / kMapNs;
   ns = (b % NG) * kMapNs + i % kMapNs;
-}
-
-struct GemmArgs {
-  const uint8_t* aq;   // activations, e4m3 [rows][K]
-  const float* as;     // their scales [rows][K / 128]
-  const int* gather;   // position -> activation row (null: the position itself)
-  const int* tile_e;   // (null: one pseudo-expert -1 holding rows [0, nrows): the shared expert)
-  const int* tile_m0;
-  const int* ntiles;
-  const int* off;
-  int nrows;           // shared expert: T
-  dsgx_layer_w L;
-  uint16_t* h;         // UP: h bf16 [position][I]
-  float* d;            // DOWN: f32 [position][H]
-#ifdef DSGX_TRACE
-  unsigned long long* trace;  // diagnostic build: [workgroup][16] time stamps
-#endif
-};
-#ifdef DSGX_TRACE
-#define PF_MARK(k)                                                                                       \
-  do {                                                                                                    \
-    if (g.trace && threadIdx.x == 0 && blockIdx.x < 1024) {                                                \
-      g.trace[blockIdx.x * 16 + (k)] = wall_clock64();                                                    \
-      g.trace[blockIdx.x * 16 + 8 + (k)] = clock64(); /* (marks 0..7 only) */                            \
-    }                                                                                                     \
-  } while (0)
-#else
-#define PF_MARK(k) do { } while (0)
-#endif
-
-template <bool UP>
-__global__ void __launch_bounds__(kGemmThreads) k_pf_gemm(GemmArgs g) {
-  extern __shared__ uint8_t smem[];
-  PF_MARK(0);
-  const int K = UP ? g.L.H : g.L.I, KB = K / 128;
-  const int NS = UP ? g.L.I / (kWgRows / 2) : g.L.H / kWgRows;  // workgroups along the weight rows
-  int tile, ns;
-  pf_task(NS, tile, ns);
-  if (ns >= NS) return;
-  int e = -1, m0 = tile * kTile, mend = g.nrows;
-  if (g.tile_e) {
-    if (tile >= *g.ntiles) return;
-    e = g.tile_e[tile];
-    const int o = g.off[e];
-    m0 = o + g.tile_m0[tile], mend = g.off[e + 1];
-  } else if (m0 >= mend) {
-    return;
-  }
-  // the tile's matrices
-  const uint8_t *wa, *wb;   // UP: gate, up; DOWN: down twice
-  const float *sa, *sb;
-  float s2a = 1.f, s2b = 1.f;
-  const size_t NK = (size_t)g.L.H * g.L.I;
-  if (e < 0) {
-    if (UP) wa = g.L.sh.g, sa = g.L.sh.gs, wb = g.L.sh.u, sb = g.L.sh.us;
-    else wa = wb = g.L.sh.d, sa = sb = g.L.sh.ds;
-  } else {
-    const dsgx_mat_desc* d = g.L.desc + (size_t)e * 3;
-    if (UP) {
-      wa = g.L.pool + d[0].off, wb = g.L.pool + d[1].off, s2a = d[0].s2, s2b = d[1].s2;
-    } else {
-      wa = wb = g.L.pool + d[2].off;
-    }
-    sa = reinterpret_cast<const float*>(wa + (NK + 255) / 256 * 256);
-    sb = reinterpret_cast<const float*>(wb + (NK + 255) / 256 * 256);
-  }
-  const int tid = threadIdx.x, lane = tid & 63, wave = uni(tid >> 6), r16 = lane & 15, part = lane >> 4;
-  // Loads are issued with lane l on row l / 4, 16-byte piece l % 4 of a 64-byte half row (four consecutive lanes read 64
-  // contiguous bytes: the texture unit looks up one line for them, not one a lane), and the weights are then moved to the
-  // MFMA's lane order (row l % 16, piece l / 16) through LDS, as the activations are: each lane writes its piece to the
-  // slot of the fragment order.
-  const int lrow = lane >> 2, lq = lane & 3;
-  // the wave's two 16-row weight tiles
-  const int n0 = UP ? ns * (kWgRows / 2) + 16 * wave : ns * kWgRows + 32 * wave;  // UP: first channel; DOWN: first row
-  const uint8_t* pa[2];
-  pa[0] = wa + (size_t)(n0 + lrow) * K + lq * 16;
-  pa[1] = (UP ? wb + (size_t)(n0 + lrow) * K : wa + (size_t)(n0 + 16 + lrow) * K) + lq * 16;
-  const float* swa = sa + (size_t)(n0 / 128) * KB;  // the tiles' scale rows (a wave's 32 rows lie in one 128-row block)
-  const float* swb = UP ? sb + (size_t)(n0 / 128) * KB : swa;
-
-  // activation staging: wave w brings the 16 positions 16 w ... of the panel, the lane its MFMA fragment's two 16-byte
-  // pieces (row lane % 16, bytes 16 (lane / 16) of each 64-byte half); in LDS a panel is stored in fragment order,
-  // piece (tile mt, half h, lane) at 16 ((2 mt + h) 64 + lane): the MFMA operand reads are linear in the lane (no
-  // bank conflicts), and so are these writes. Thread t < 128 also brings the scale of position t.
-  const uint8_t* pb;
-  {
-    int pos = m0 + 16 * wave + lrow;
-    if (pos >= mend) pos = mend - 1;  // a ragged tile re-reads its last row (never stored)
-    pb = g.aq + (size_t)(g.gather ? g.gather[pos] : pos) * K + lq * 16;
-  }
-  const float* pxs;
-  {
-    int pos = m0 + (tid & 127);
-    if (pos >= mend) pos = mend - 1;
-    pxs = g.as + (size_t)(g.gather ? g.gather[pos] : pos) * KB;
-  }
-
-  // a fragment's 64 pieces in LDS: piece (row r, part p) at slot 16 p + (r ^ 2 p), 16 bytes a slot. The exclusive-or keeps
-  // both sides free of bank conflicts: the writes (eight consecutive lanes hold two rows x four parts) and the MFMA-order
-  // reads (eight consecutive lanes hold eight rows of one part) each touch eight different slots modulo 8.
-  const int nmt = uni(min(8, (mend - m0 + 15) / 16));  // the tile's 16-position tiles that hold rows
-  const int wr_slot = (lq * 16 + (lrow ^ (2 * lq))) * 16, rd_slot = (part * 16 + (r16 ^ (2 * part))) * 16;
-  auto blk = [&](int kb) { return kb < KB ? kb : KB - 1; };  // (past the end: the last block again, never used)
-  v4f_t acc[2][8];
-#pragma unroll
-  for (int t = 0; t < 2; ++t)
-#pragma unroll
-    for (int mt = 0; mt < 8; ++mt) acc[t][mt] = v4f_t{};
-
-  u32x4_t ra[kRing][2][2];  // the weight ring: block slot, tile, the block's half
-  auto load_a = [&](int slot, int kb) {
-    const int kc = blk(kb);
-#pragma unroll
-    for (int t = 0; t < 2; ++t) {
-      const uint8_t* p = pin_after(pa[t] + (size_t)kc * 128, acc[t][0][0]);
-      // (ordinary loads, not streaming ones: the other tiles of the same expert read the same lines from L2)
-      ra[slot][t][0] = *reinterpret_cast<const DSGX_GLOBAL u32x4_t*>((uintptr_t)p);
-      ra[slot][t][1] = *reinterpret_cast<const DSGX_GLOBAL u32x4_t*>((uintptr_t)(p + 64));
-    }
-  };
-  struct XRegs {
-    u32x4_t v[2];
-    float s;
-  };
-  auto fetch_x = [&](XRegs& r, int kb) {
-    const int kc = blk(kb);
-    r.v[0] = *reinterpret_cast<const u32x4_t*>(pb + (size_t)kc * 128);
-    r.v[1] = *reinterpret_cast<const u32x4_t*>(pb + (size_t)kc * 128 + 64);
-    r.s = pxs[kc];
-  };
-  auto stash_x = [&](const XRegs& r, int stage) {
-    uint8_t* B = smem + (size_t)stage * kStageBytes;
-    *reinterpret_cast<u32x4_t*>(B + (2 * wave + 0) * 1024 + wr_slot) = r.v[0];
-    *reinterpret_cast<u32x4_t*>(B + (2 * wave + 1) * 1024 + wr_slot) = r.v[1];
-    if (tid < kTile) reinterpret_cast<float*>(B + kPanel)[tid] = r.s;
-  };
-  // the wave's weight scales: lane l holds those of block kb0 + l for the 64 blocks from kb0 (a multiple of 64)
-  float wsa_l, wsb_l;
-  auto load_ws = [&](int kb0) {
-    const int kc = blk(kb0 + lane);
-    wsa_l = swa[kc], wsb_l = swb[kc];
-  };
-  load_ws(0);
-  // The wave's weights of a block reach the MFMA's lane order through its own LDS (two copies of 4 KiB, written as
-  // loaded, read as fragments, in the activations' slot order: no bank conflicts; the LDS unit serves a wave's
-  // operations in order, so no barrier lies between): a quarter of the LDS time of a cross-lane permute a dword.
-  auto w_to_lds = [&](int slot, int par) {
-    uint8_t* W = smem + (size_t)kStages * kStageBytes + (2 * wave + par) * 4096;
-#pragma unroll
-    for (int t = 0; t < 2; ++t)
-#pragma unroll
-      for (int h = 0; h < 2; ++h) *reinterpret_cast<u32x4_t*>(W + (2 * t + h) * 1024 + wr_slot) = keep_whole(ra[slot][t][h]);
-  };
-  v8i_t fa[2], fb[3];
-  float xv[3];
-  auto read_fa = [&](int par) {
-    const uint8_t* W = smem + (size_t)kStages * kStageBytes + (2 * wave + par) * 4096;
-#pragma unroll
-    for (int t = 0; t < 2; ++t) {
-      const u32x4_t lo = *reinterpret_cast<const u32x4_t*>(W + (2 * t + 0) * 1024 + rd_slot);
-      const u32x4_t hi = *reinterpret_cast<const u32x4_t*>(W + (2 * t + 1) * 1024 + rd_slot);
-      fa[t] = v8i_t{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
-    }
-  };
-  auto read_b = [&](int buf, int stage, int mt) {
-    const uint8_t* B = smem + (size_t)stage * kStageBytes;
-    const u32x4_t lo = *reinterpret_cast<const u32x4_t*>(B + (2 * mt + 0) * 1024 + rd_slot);
-    const u32x4_t hi = *reinterpret_cast<const u32x4_t*>(B + (2 * mt + 1) * 1024 + rd_slot);
-    fb[buf] = v8i_t{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
-    xv[buf] = reinterpret_cast<const float*>(B + kPanel)[16 * mt + r16];
-  };
-  // The activations of a block wait in registers for kHold turns between their loads and their LDS writes (the memory
-  // latency is several turns long, and a wait for one load is a wait for every load issued before it): set v holds, at
-  // the start of turn kb = v (mod kHold), block kb + 3.
-  XRegs rx[kHold];
-  PF_MARK(1);
-  // prologue: the weight ring, the first activation panels, block 0's weights to LDS
-#pragma unroll
-  for (int d = 0; d < kRing; ++d) load_a(d, d);
-  {
-    XRegs t0, t1, t2;
-    fetch_x(t0, 0), fetch_x(t1, 1), fetch_x(t2, 2);
-#pragma unroll
-    for (int v = 0; v < kHold; ++v) fetch_x(rx[v], 3 + v);
-    stash_x(t0, 0), stash_x(t1, 1), stash_x(t2, 2);
-  }
-  w_to_lds(0, 0);
-  load_a(0, kRing);
-  __syncthreads();
-  read_fa(0);
-  read_b(0, 0, 0);
-  if (nmt > 1) read_b(1, 0, 1);
-  PF_MARK(2);
-  // Turn kb. On entry the registers hold (or have in flight) block kb's weight fragments and the activation fragments of
-  // its position tiles 0 and 1. The eight tiles run as a pipeline: the fragment of tile mt + 2 is read while tile mt's
-  // two MFMAs (from zero) are issued and tile mt - 1's scaled adds run. In between, work for later turns: the
-  // activations of block kb + 3 (loaded kHold turns ago) go to their stage (last read a turn ago) and the loads of
-  // block kb + 3 + kHold are issued in their place; the ring's block kb + 1 goes to the wave's LDS copy and the loads
-  // of block kb + 1 + kRing are issued in its place; after the last MFMA is issued, the next turn's fragments are
-  // read. Then the barrier: nothing but those reads' latency stands between it and the next turn's first MFMA.
-  // (Unrolled over a common multiple of the rotations.)
-  constexpr int kTurns = 12;
-  static_assert(kTurns % kRing == 0 && kTurns % kHold == 0 && kTurns % kStages == 0 && kTurns % 2 == 0, "unroll");
-  for (int kb0 = 0; kb0 < KB; kb0 += kTurns) {
-#pragma unroll
-    for (int v = 0; v < kTurns; ++v) {
-      const int kb = kb0 + v;
-      if (kb >= KB) break;
-      // the block's weight scales from the lanes that hold them (a load here would be waited for in this same turn, and
-      // a wait for one load is a wait for every load before it: the whole ring)
-      if ((kb & 63) == 0 && kb > 0) load_ws(kb);
-      const float wsa = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, wsa_l), kb & 63));
-      const float wsb = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, wsb_l), kb & 63));
-      v4f_t pp[2] = {v4f_t{}, v4f_t{}};
-      float scp[2] = {0.f, 0.f};
-#pragma unroll
-      for (int mt = 0; mt <= 8; ++mt) {
-        // (a ragged tile's 16-position tiles past its end are skipped: most experts of a chunk hold fewer than 128 rows)
-        if (mt + 2 < 8 && mt + 2 < nmt) read_b((mt + 2) % 3, v % kStages, mt + 2);
-        v4f_t pc[2] = {v4f_t{}, v4f_t{}};
-        float scn[2] = {0.f, 0.f};
-        if (mt < 8 && mt < nmt) {
-#pragma unroll
-          for (int t = 0; t < 2; ++t) pc[t] = mfma_fp8_k128(fa[t], fb[mt % 3], v4f_t{});
-          scn[0] = __fmul_rn(xv[mt % 3], wsa), scn[1] = __fmul_rn(xv[mt % 3], wsb);
-        }
-        if (mt == 7) {  // the last MFMAs are issued: the next turn's fragments
-          read_fa((v + 1) & 1);
-          read_b(0, (v + 1) % kStages, 0);
-          if (nmt > 1) read_b(1, (v + 1) % kStages, 1);
-        }
-        if (mt > 0 && mt - 1 < nmt) {
-#pragma unroll
-          for (int t = 0; t < 2; ++t)
-#pragma unroll
-            for (int q = 0; q < 4; ++q) acc[t][mt - 1][q] = fmaf(scp[t], pp[t][q], acc[t][mt - 1][q]);
-        }
-        if (mt < 8) pp[0] = pc[0], pp[1] = pc[1], scp[0] = scn[0], scp[1] = scn[1];
-        if (mt == 2) {
-          stash_x(rx[v % kHold], (v + 3) % kStages);
-          fetch_x(rx[v % kHold], kb + 3 + kHold);
-        }
-        if (mt == 4) {
-          w_to_lds((v + 1) % kRing, (v + 1) & 1);
-          load_a((v + 1) % kRing, kb + 1 + kRing);
-        }
-      }
-      __syncthreads();
-    }
-    if (kb0 == 0) PF_MARK(3);
-  }
-  PF_MARK(5);
-
-  // epilogue: register q of lane l is weight row 4 (l / 16) + q of the 16-row tile, position l % 16 of the 16 positions
-  if (UP) {
-    const int I = g.L.I;
-#pragma unroll
-    for (int mt = 0; mt < 8; ++mt) {
-      const int pos = m0 + 16 * mt + r16;
-      if (pos >= mend) continue;
-      uint32_t hb[4];
-#pragma unroll
-      for (int q = 0; q < 4; ++q)
-        hb[q] = swiglu_bits(bf16_round(__fmul_rn(acc[0][mt][q], s2a)), bf16_round(__fmul_rn(acc[1][mt][q], s2b)));
-      *reinterpret_cast<uint2*>(g.h + (size_t)pos * I + n0 + 4 * part) = make_uint2(hb[0] | (hb[1] << 16), hb[2] | (hb[3] << 16));
-    }
-  } else {
-    const int H = g.L.H;
-#pragma unroll
-    for (int mt = 0; mt < 8; ++mt) {
-      const int pos = m0 + 16 * mt + r16;
-      if (pos >= mend) continue;
-#pragma unroll
-      for (int t = 0; t < 2; ++t)
-        *reinterpret_cast<float4*>(g.d + (size_t)pos * H + n0 + 16 * t + 4 * part) = make_float4(acc[t][mt][0], acc[t][mt][1], acc[t][mt][2], acc[t][mt][3]);
-    }
-  }
-  PF_MARK(6);
 }
 
 // ---- the grouped GEMM with bf16 activations (INT4 layers, and their BF16 shared expert) -----------------------------
@@ -874,16 +596,13 @@ int dsgx_moe_prefill(const dsgx_layer_w* L, const uint16_t* x, const int* idx, c
   auto I32 = [&](size_t off) { return reinterpret_cast<int*>(W + off); };
   auto F32 = [&](size_t off) { return reinterpret_cast<float*>(W + off); };
   const int H = L->H, I = L->I, E = L->E, topk = L->topk, P = o.P;
-  const size_t lds = (size_t)kStages * kStageBytes + (kGemmThreads / 64) * 2 * 4096;  // activation stages + two weight blocks a wave
-  if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(k_pf_gemm<true>), lds)) return rc;
-  if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(k_pf_gemm<false>), lds)) return rc;
 
   if (cfg.phases & 1) {
     const int NB = (T + kRowBlock - 1) / kRowBlock;
     uint32_t* bmask = reinterpret_cast<uint32_t*>(W + o.bmask);
     hipLaunchKernelGGL(k_pf_mask, dim3(NB), dim3(256), 0, st, idx, T, topk, E, I32(o.bcnt), bmask);
-    hipLaunchKernelGGL(k_pf_scan, dim3(1), dim3(DSGX_MAX_EXPERTS), 0, st, I32(o.bcnt), NB, E, I32(o.boff), I32(o.cnt), I32(o.off), I32(o.ntiles),
-                       I32(o.tile_e), I32(o.tile_m0));
+    const TileLists tl{I32(o.ntiles), I32(o.tile_e), I32(o.tile_m0), I32(o.nbig), I32(o.big_e), I32(o.big_m0), I32(o.nsmall), I32(o.small_e), I32(o.small_m0)};
+    hipLaunchKernelGGL(k_pf_scan, dim3(1), dim3(DSGX_MAX_EXPERTS), 0, st, I32(o.bcnt), NB, E, I32(o.boff), I32(o.cnt), I32(o.off), tl);
     hipLaunchKernelGGL(k_pf_place, dim3(NB), dim3(256), 0, st, idx, w, T, topk, E, I32(o.off), I32(o.boff), bmask, L->desc, I32(o.perm),
                        I32(o.pickpos), I32(o.rpos), I32(o.re), F32(o.rk));
     DSGX_HIP(hipGetLastError());
@@ -924,27 +643,41 @@ int dsgx_moe_prefill(const dsgx_layer_w* L, const uint16_t* x, const int* idx, c
     DSGX_HIP(hipGetLastError());
     return DSGX_OK;
   }
-  GemmArgs g{};
+  // FP8 activations: x quantised -> gate/up + SwiGLU (h bf16 for the view, and quantised for the down projection in the
+  // same kernel) -> down (f32 a pick) -> ordered combine. Every GEMM runs twice: the 256-position tiles, then the
+  // experts' remainders of up to 128 positions.
+  if (H > 8192 || I > 8192) return fail(DSGX_EUNSUPPORTED, "moe_prefill: FP8 activations: hidden %d, intermediate %d (up to 8192)", H, I);
+  auto k_up1 = pf8::k_gemm<true, 1>, k_up2 = pf8::k_gemm<true, 2>, k_dn1 = pf8::k_gemm<false, 1>, k_dn2 = pf8::k_gemm<false, 2>;
+  for (const void* k : {(const void*)k_up1, (const void*)k_dn1})
+    if (int rc = allow_dynamic_lds(k, pf8::Shape<1>::kLds)) return rc;
+  for (const void* k : {(const void*)k_up2, (const void*)k_dn2})
+    if (int rc = allow_dynamic_lds(k, pf8::Shape<2>::kLds)) return rc;
+  pf8::Args g{};
   g.L = *L;
-#ifdef DSGX_TRACE
-  g.trace = dsgx_trace_buf();
-#endif
+  const int NSU = I / (pf8::kWgRows / 2), NSD = H / pf8::kWgRows;
+  auto routed = [&](bool big) {
+    g.tile_e = I32(big ? o.big_e : o.small_e), g.tile_m0 = I32(big ? o.big_m0 : o.small_m0), g.ntiles = I32(big ? o.nbig : o.nsmall);
+    g.off = I32(o.off), g.nrows = P;
+  };
   if (cfg.phases & (2 | 16)) {
     if (int rc = dsgx_act_quant(x, T, H, W + o.xq, F32(o.xs), stream)) return rc;
   }
   if (cfg.phases & 2) {
     g.aq = W + o.xq, g.as = F32(o.xs), g.gather = I32(o.perm);
-    g.tile_e = I32(o.tile_e), g.tile_m0 = I32(o.tile_m0), g.ntiles = I32(o.ntiles), g.off = I32(o.off), g.nrows = P;
-    g.h = reinterpret_cast<uint16_t*>(W + o.h), g.d = nullptr;
-    hipLaunchKernelGGL(k_pf_gemm<true>, dim3(pf_grid(o.max_tiles, I / (kWgRows / 2))), dim3(kGemmThreads), lds, st, g);
+    g.h = reinterpret_cast<uint16_t*>(W + o.h), g.hq = W + o.hq, g.hs = F32(o.hs), g.d = nullptr;
+    routed(true);
+    hipLaunchKernelGGL(k_up2, dim3(pf8::grid_of(o.max_big, NSU)), dim3(pf8::kThreads), pf8::Shape<2>::kLds, st, g);
+    routed(false);
+    hipLaunchKernelGGL(k_up1, dim3(pf8::grid_of(E, NSU)), dim3(pf8::kThreads), pf8::Shape<1>::kLds, st, g);
     DSGX_HIP(hipGetLastError());
   }
   if (cfg.phases & 4) {
-    if (int rc = dsgx_act_quant(reinterpret_cast<const uint16_t*>(W + o.h), P, I, W + o.hq, F32(o.hs), stream)) return rc;
     g.aq = W + o.hq, g.as = F32(o.hs), g.gather = nullptr;
-    g.tile_e = I32(o.tile_e), g.tile_m0 = I32(o.tile_m0), g.ntiles = I32(o.ntiles), g.off = I32(o.off), g.nrows = P;
-    g.h = nullptr, g.d = F32(o.d);
-    hipLaunchKernelGGL(k_pf_gemm<false>, dim3(pf_grid(o.max_tiles, H / kWgRows)), dim3(kGemmThreads), lds, st, g);
+    g.h = nullptr, g.hq = nullptr, g.hs = nullptr, g.d = F32(o.d);
+    routed(true);
+    hipLaunchKernelGGL(k_dn2, dim3(pf8::grid_of(o.max_big, NSD)), dim3(pf8::kThreads), pf8::Shape<2>::kLds, st, g);
+    routed(false);
+    hipLaunchKernelGGL(k_dn1, dim3(pf8::grid_of(E, NSD)), dim3(pf8::kThreads), pf8::Shape<1>::kLds, st, g);
     DSGX_HIP(hipGetLastError());
   }
   if (cfg.phases & 8) {
@@ -953,14 +686,13 @@ int dsgx_moe_prefill(const dsgx_layer_w* L, const uint16_t* x, const int* idx, c
     DSGX_HIP(hipGetLastError());
   }
   if ((cfg.phases & 16) && shared) {
-    const int tiles = (T + kTile - 1) / kTile;
-    g.aq = W + o.xq, g.as = F32(o.xs), g.gather = nullptr;
+    const int tiles = (T + 255) / 256;
     g.tile_e = g.tile_m0 = g.ntiles = g.off = nullptr, g.nrows = T;
-    g.h = reinterpret_cast<uint16_t*>(W + o.hsh), g.d = nullptr;
-    hipLaunchKernelGGL(k_pf_gemm<true>, dim3(pf_grid(tiles, I / (kWgRows / 2))), dim3(kGemmThreads), lds, st, g);
-    if (int rc = dsgx_act_quant(reinterpret_cast<const uint16_t*>(W + o.hsh), T, I, W + o.hshq, F32(o.hshs), stream)) return rc;
-    g.aq = W + o.hshq, g.as = F32(o.hshs), g.h = nullptr, g.d = ys;
-    hipLaunchKernelGGL(k_pf_gemm<false>, dim3(pf_grid(tiles, H / kWgRows)), dim3(kGemmThreads), lds, st, g);
+    g.aq = W + o.xq, g.as = F32(o.xs), g.gather = nullptr;
+    g.h = reinterpret_cast<uint16_t*>(W + o.hsh), g.hq = W + o.hshq, g.hs = F32(o.hshs), g.d = nullptr;
+    hipLaunchKernelGGL(k_up2, dim3(pf8::grid_of(tiles, NSU)), dim3(pf8::kThreads), pf8::Shape<2>::kLds, st, g);
+    g.aq = W + o.hshq, g.as = F32(o.hshs), g.h = nullptr, g.hq = nullptr, g.hs = nullptr, g.d = ys;
+    hipLaunchKernelGGL(k_dn2, dim3(pf8::grid_of(tiles, NSD)), dim3(pf8::kThreads), pf8::Shape<2>::kLds, st, g);
     DSGX_HIP(hipGetLastError());
   }
   return DSGX_OK;
