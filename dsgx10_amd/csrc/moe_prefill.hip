@@ -14,6 +14,8 @@
 // The FP8-activation GEMMs run on v_mfma_f32_16x16x128_f8f6f4 (one instruction a 128-k scale block), the bf16-activation
 // ones on v_mfma_f32_16x16x32_bf16: weights are the A operand (rows n), activations the B operand, so a lane's four
 // accumulators of a 16 x 16 tile belong to ONE token row and the block's combined scale is one value a lane.
+#include <cstdlib>
+
 #include "abi_internal.h"
 #include "common.cuh"
 #include "pf_gemm_fp8.cuh"
@@ -71,6 +73,7 @@ constexpr int kRowBlock = 128;  // token rows a workgroup of the bucketing kerne
 struct PfLayout {
   size_t cnt, off, ntiles, tile_e, tile_m0, perm, pickpos, rpos, re, rk, xq, xs, h, hq, hs, hsh, hshq, hshs, d, bcnt, boff, bmask, total;
   size_t nbig, big_e, big_m0, nsmall, small_e, small_m0;  // the FP8 kernels' lists: 256-position tiles, and the experts' remainders
+  size_t nmix, mix_e, mix_m0;                             // ... and the two merged into the order the kernels run them in
   int P, max_tiles, max_big;
 };
 PfLayout pf_layout(const dsgx_layer_w* L, int T) {
@@ -85,6 +88,7 @@ PfLayout pf_layout(const dsgx_layer_w* L, int T) {
   o.max_big = (int)(P / 256 + E);
   o.nbig = take(4), o.big_e = take((size_t)o.max_big * 4), o.big_m0 = take((size_t)o.max_big * 4);
   o.nsmall = take(4), o.small_e = take(E * 4), o.small_m0 = take(E * 4);
+  o.nmix = take(4), o.mix_e = take((size_t)(o.max_big + E) * 4), o.mix_m0 = take((size_t)(o.max_big + E) * 4);
   o.perm = take(P * 4), o.pickpos = take(P * 4), o.rpos = take(P * 4), o.re = take(P * 4), o.rk = take(P * 4);
   o.xq = take((size_t)T * H), o.xs = take((size_t)T * (H / 128) * 4);
   o.h = take(P * I * 2), o.hq = take(P * I), o.hs = take(P * (I / 128) * 4);
@@ -129,6 +133,7 @@ struct TileLists {
   int *ntiles, *tile_e, *tile_m0;     // all rows in 128-position tiles
   int *nbig, *big_e, *big_m0;         // 256-position tiles
   int *nsmall, *small_e, *small_m0;   // the remainders of up to 128 positions
+  int *nmix, *mix_e, *mix_m0;         // both, merged evenly (expert | 1 << 30 for a 256-position tile)
 };
 __global__ void __launch_bounds__(DSGX_MAX_EXPERTS) k_pf_scan(const int* __restrict__ bcnt, int NB, int E, int* __restrict__ boff,
                                                               int* __restrict__ cnt, int* __restrict__ off, TileLists tl) {
@@ -161,6 +166,21 @@ __global__ void __launch_bounds__(DSGX_MAX_EXPERTS) k_pf_scan(const int* __restr
     for (int i = 0; i < nbig; ++i) tl.big_e[b0 + i] = e, tl.big_m0[b0 + i] = i * 256;
     if (nsmall) tl.small_e[sd[e] - 1] = e, tl.small_m0[sd[e] - 1] = (c / 256) * 256;
   }
+  __syncthreads();
+  // The merged list: the small tiles (they mostly stream an expert's weights) spread evenly among the big ones (they
+  // mostly multiply), each kind in expert order: entry i of the small list goes in after floor(i nb / ns) big ones.
+  const int nb = sc[DSGX_MAX_EXPERTS - 1], nsm = sd[DSGX_MAX_EXPERTS - 1];
+  __threadfence_block();
+  for (int i = e; i < nb; i += DSGX_MAX_EXPERTS) {
+    // small entries before big entry i: those j with floor(j nb / nsm) <= i, j < nsm
+    const int before = nsm ? min(nsm, (int)(((long)(i + 1) * nsm + nb - 1) / nb)) : 0;
+    tl.mix_e[i + before] = tl.big_e[i] | (1 << 30), tl.mix_m0[i + before] = tl.big_m0[i];
+  }
+  for (int j = e; j < nsm; j += DSGX_MAX_EXPERTS) {
+    const int before = (int)((long)j * nb / nsm);  // big entries before small entry j
+    tl.mix_e[j + before] = tl.small_e[j], tl.mix_m0[j + before] = tl.small_m0[j];
+  }
+  if (e == 0) *tl.nmix = nb + nsm;
 }
 __global__ void __launch_bounds__(256) k_pf_place(const int* __restrict__ idx, const float* __restrict__ w, int T, int topk, int E,
                                                   const int* __restrict__ off, const int* __restrict__ boff,
@@ -601,7 +621,8 @@ int dsgx_moe_prefill(const dsgx_layer_w* L, const uint16_t* x, const int* idx, c
     const int NB = (T + kRowBlock - 1) / kRowBlock;
     uint32_t* bmask = reinterpret_cast<uint32_t*>(W + o.bmask);
     hipLaunchKernelGGL(k_pf_mask, dim3(NB), dim3(256), 0, st, idx, T, topk, E, I32(o.bcnt), bmask);
-    const TileLists tl{I32(o.ntiles), I32(o.tile_e), I32(o.tile_m0), I32(o.nbig), I32(o.big_e), I32(o.big_m0), I32(o.nsmall), I32(o.small_e), I32(o.small_m0)};
+    const TileLists tl{I32(o.ntiles), I32(o.tile_e), I32(o.tile_m0), I32(o.nbig), I32(o.big_e), I32(o.big_m0), I32(o.nsmall), I32(o.small_e), I32(o.small_m0),
+                       I32(o.nmix), I32(o.mix_e), I32(o.mix_m0)};
     hipLaunchKernelGGL(k_pf_scan, dim3(1), dim3(DSGX_MAX_EXPERTS), 0, st, I32(o.bcnt), NB, E, I32(o.boff), I32(o.cnt), I32(o.off), tl);
     hipLaunchKernelGGL(k_pf_place, dim3(NB), dim3(256), 0, st, idx, w, T, topk, E, I32(o.off), I32(o.boff), bmask, L->desc, I32(o.perm),
                        I32(o.pickpos), I32(o.rpos), I32(o.re), F32(o.rk));
@@ -647,37 +668,42 @@ int dsgx_moe_prefill(const dsgx_layer_w* L, const uint16_t* x, const int* idx, c
   // same kernel) -> down (f32 a pick) -> ordered combine. Every GEMM runs twice: the 256-position tiles, then the
   // experts' remainders of up to 128 positions.
   if (H > 8192 || I > 8192) return fail(DSGX_EUNSUPPORTED, "moe_prefill: FP8 activations: hidden %d, intermediate %d (up to 8192)", H, I);
-  auto k_up1 = pf8::k_gemm<true, 1>, k_up2 = pf8::k_gemm<true, 2>, k_dn1 = pf8::k_gemm<false, 1>, k_dn2 = pf8::k_gemm<false, 2>;
-  for (const void* k : {(const void*)k_up1, (const void*)k_dn1})
-    if (int rc = allow_dynamic_lds(k, pf8::Shape<1>::kLds)) return rc;
+  void (*k_up)(pf8::Args) = pf8::k_gemm_mixed<true>;    // the routed experts: the merged list of both tile shapes
+  void (*k_dn)(pf8::Args) = pf8::k_gemm_mixed<false>;
+  void (*k_up2)(pf8::Args) = pf8::k_gemm<true, 2>;      // the shared expert: 256-position tiles
+  void (*k_dn2)(pf8::Args) = pf8::k_gemm<false, 2>;
+#ifdef DSGX_PF_DIAG
+  {  // diagnostic build: DSGX_PF_DIAG=<bits> switches parts of the kernels off (wrong results; for timing only)
+    const char* dv = std::getenv("DSGX_PF_DIAG");
+    switch (dv ? std::atoi(dv) : 0) {
+#define DSGX_DIAG_CASE(n) case n: k_up = pf8::k_gemm_mixed<true, n>, k_dn = pf8::k_gemm_mixed<false, n>, k_up2 = pf8::k_gemm<true, 2, n>, k_dn2 = pf8::k_gemm<false, 2, n>; break;
+      DSGX_DIAG_CASE(1) DSGX_DIAG_CASE(2) DSGX_DIAG_CASE(4) DSGX_DIAG_CASE(8) DSGX_DIAG_CASE(16) DSGX_DIAG_CASE(3) DSGX_DIAG_CASE(9) DSGX_DIAG_CASE(25)
+#undef DSGX_DIAG_CASE
+    }
+  }
+#endif
+  constexpr int kLdsMix = pf8::Shape<1>::kLds > pf8::Shape<2>::kLds ? pf8::Shape<1>::kLds : pf8::Shape<2>::kLds;
+  for (const void* k : {(const void*)k_up, (const void*)k_dn})
+    if (int rc = allow_dynamic_lds(k, kLdsMix)) return rc;
   for (const void* k : {(const void*)k_up2, (const void*)k_dn2})
     if (int rc = allow_dynamic_lds(k, pf8::Shape<2>::kLds)) return rc;
   pf8::Args g{};
   g.L = *L;
   const int NSU = I / (pf8::kWgRows / 2), NSD = H / pf8::kWgRows;
-  auto routed = [&](bool big) {
-    g.tile_e = I32(big ? o.big_e : o.small_e), g.tile_m0 = I32(big ? o.big_m0 : o.small_m0), g.ntiles = I32(big ? o.nbig : o.nsmall);
-    g.off = I32(o.off), g.nrows = P;
-  };
+  g.tile_e = I32(o.mix_e), g.tile_m0 = I32(o.mix_m0), g.ntiles = I32(o.nmix), g.off = I32(o.off), g.nrows = P;
   if (cfg.phases & (2 | 16)) {
     if (int rc = dsgx_act_quant(x, T, H, W + o.xq, F32(o.xs), stream)) return rc;
   }
   if (cfg.phases & 2) {
     g.aq = W + o.xq, g.as = F32(o.xs), g.gather = I32(o.perm);
     g.h = reinterpret_cast<uint16_t*>(W + o.h), g.hq = W + o.hq, g.hs = F32(o.hs), g.d = nullptr;
-    routed(true);
-    hipLaunchKernelGGL(k_up2, dim3(pf8::grid_of(o.max_big, NSU)), dim3(pf8::kThreads), pf8::Shape<2>::kLds, st, g);
-    routed(false);
-    hipLaunchKernelGGL(k_up1, dim3(pf8::grid_of(E, NSU)), dim3(pf8::kThreads), pf8::Shape<1>::kLds, st, g);
+    hipLaunchKernelGGL(k_up, dim3(pf8::grid_of(o.max_big + E, NSU)), dim3(pf8::kThreads), kLdsMix, st, g);
     DSGX_HIP(hipGetLastError());
   }
   if (cfg.phases & 4) {
     g.aq = W + o.hq, g.as = F32(o.hs), g.gather = nullptr;
     g.h = nullptr, g.hq = nullptr, g.hs = nullptr, g.d = F32(o.d);
-    routed(true);
-    hipLaunchKernelGGL(k_dn2, dim3(pf8::grid_of(o.max_big, NSD)), dim3(pf8::kThreads), pf8::Shape<2>::kLds, st, g);
-    routed(false);
-    hipLaunchKernelGGL(k_dn1, dim3(pf8::grid_of(E, NSD)), dim3(pf8::kThreads), pf8::Shape<1>::kLds, st, g);
+    hipLaunchKernelGGL(k_dn, dim3(pf8::grid_of(o.max_big + E, NSD)), dim3(pf8::kThreads), kLdsMix, st, g);
     DSGX_HIP(hipGetLastError());
   }
   if (cfg.phases & 8) {

@@ -105,24 +105,14 @@ __device__ __forceinline__ void wait_loads() {
 }
 __device__ __forceinline__ int swz(int r) { return (r & 7) ^ (r >> 3); }
 
-template <bool UP, int WP>
-__global__ void __launch_bounds__(kThreads) k_gemm(Args g) {
+// DIAG (diagnostic builds only; results are then wrong): 1 no loads after the first stages, 2 the MFMAs accumulate by
+// themselves (no scaled adds on the vector unit), 4 no workgroup barrier in the loop, 8 no MFMAs, 16 no fragment reads
+// after the first turn
+// one tile: expert e (-1: the shared expert), rows [m0, mend) of the activations' positions, row group ns
+template <bool UP, int WP, int DIAG>
+__device__ __forceinline__ void gemm_tile(const Args& g, uint8_t* smem, int e, int m0, int mend, int ns) {
   using S = Shape<WP>;
-  extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
   const int K = UP ? g.L.H : g.L.I, KB = K / 128;
-  const int NS = UP ? g.L.I / (kWgRows / 2) : g.L.H / kWgRows;
-  int tile, ns;
-  task_of(NS, tile, ns);
-  if (ns >= NS) return;
-  int e = -1, m0 = tile * S::kPos, mend = g.nrows;
-  if (g.tile_e) {
-    if (tile >= *g.ntiles) return;
-    e = g.tile_e[tile];
-    const int o = g.off[e];
-    m0 = o + g.tile_m0[tile], mend = g.off[e + 1];
-  } else if (m0 >= mend) {
-    return;
-  }
   if (mend > m0 + S::kPos) mend = m0 + S::kPos;  // (the tile's own rows)
   const uint8_t *wa, *wb;  // UP: gate, up; DOWN: down twice
   const float *sa, *sb;
@@ -236,12 +226,12 @@ __global__ void __launch_bounds__(kThreads) k_gemm(Args g) {
       // this wave's loads of block kb have landed (later blocks may be in flight); after the barrier everyone's have, and
       // everyone is done reading the stage of block kb - 1, which the loads of block kb + kStages - 1 now overwrite
       wait_loads<(S::kStages - 2) * S::kLoads>();
-      __syncthreads();
-      issue(kb + S::kStages - 1);
+      if (!(DIAG & 4)) __syncthreads();
+      if (!(DIAG & 1)) issue(kb + S::kStages - 1);
       if (NJ == 0) continue;
       const float wsa = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, wsa_l), kb & 63));
       const float wsb = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, wsb_l), kb & 63));
-      const uint8_t* st = smem + (size_t)(kb % S::kStages) * S::kStageBytes;
+      const uint8_t* st = smem + (size_t)(((DIAG & 16) ? 0 : kb) % S::kStages) * S::kStageBytes;
       const uint8_t* W = st + S::RA * rg * 2048;
       const uint8_t* X = st + S::kStageW + pg * 2048;
       const float* XS = reinterpret_cast<const float*>(st + S::kStageW + S::kStageX) + 16 * pg;
@@ -255,7 +245,13 @@ __global__ void __launch_bounds__(kThreads) k_gemm(Args g) {
         const float s0 = __fmul_rn(xv, wsa), s1 = __fmul_rn(xv, wsb);
 #pragma unroll
         for (int t = 0; t < S::RA; ++t) {
-          const v4f_t p = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fa[t], fb, v4f_t{0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
+          if (DIAG & 2) {
+            acc[t][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fa[t], fb, acc[t][j], 0, 0, 0, 0, 0, 0);
+            continue;
+          }
+          v4f_t p;
+          if (DIAG & 8) p = v4f_t{__builtin_bit_cast(float, fa[t][0] ^ fb[0]), __builtin_bit_cast(float, fa[t][1] ^ fb[3]), __builtin_bit_cast(float, fa[t][4] ^ fb[4]), __builtin_bit_cast(float, fa[t][7] ^ fb[7])};
+          else p = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fa[t], fb, v4f_t{0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
           const float sc = (UP && (t & 1)) ? s1 : s0;
 #pragma unroll
           for (int q = 0; q < 4; ++q) acc[t][j][q] = fmaf(sc, p[q], acc[t][j][q]);
@@ -351,6 +347,40 @@ __global__ void __launch_bounds__(kThreads) k_gemm(Args g) {
       }
     }
   }
+}
+
+// The shared expert (tile_e null: tiles of Shape<WP>::kPos rows over [0, nrows)) or one list of tiles of one shape.
+template <bool UP, int WP, int DIAG = 0>
+__global__ void __launch_bounds__(kThreads) k_gemm(Args g) {
+  extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+  const int NS = UP ? g.L.I / (kWgRows / 2) : g.L.H / kWgRows;
+  int tile, ns;
+  task_of(NS, tile, ns);
+  if (ns >= NS) return;
+  int e = -1, m0 = tile * Shape<WP>::kPos, mend = g.nrows;
+  if (g.tile_e) {
+    if (tile >= *g.ntiles) return;
+    e = g.tile_e[tile] & 0xFFFF;
+    const int o = g.off[e];
+    m0 = o + g.tile_m0[tile], mend = g.off[e + 1];
+  } else if (m0 >= mend) {
+    return;
+  }
+  gemm_tile<UP, WP, DIAG>(g, smem, e, m0, mend, ns);
+}
+// The routed experts' list of both shapes (bit 30 of tile_e: a 256-position tile), mixed so that the tiles that mostly
+// stream weights (the experts' small remainders) run beside the ones that mostly multiply.
+template <bool UP, int DIAG = 0>
+__global__ void __launch_bounds__(kThreads) k_gemm_mixed(Args g) {
+  extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+  const int NS = UP ? g.L.I / (kWgRows / 2) : g.L.H / kWgRows;
+  int tile, ns;
+  task_of(NS, tile, ns);
+  if (ns >= NS || tile >= *g.ntiles) return;
+  const int te = g.tile_e[tile], e = te & 0xFFFF;
+  const int m0 = g.off[e] + g.tile_m0[tile], mend = g.off[e + 1];
+  if (te >> 30) gemm_tile<UP, 2, DIAG>(g, smem, e, m0, mend, ns);
+  else gemm_tile<UP, 1, DIAG>(g, smem, e, m0, mend, ns);
 }
 
 }  // namespace pf8
