@@ -104,7 +104,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=64)
     ap.add_argument("--no-extra", action="store_true", help="only the headline workload")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
-    ap.add_argument("--workload", default="fp8_m1", help="headline workload: fp8_m1 | int4_m1; fp8_prefill | int4_prefill time only that prefill chunk")
+    ap.add_argument("--workload", default="fp8_m1", help="headline workload: fp8_m1 | int4_m1; fp8_prefill | int4_prefill time only that prefill chunk; gemv only the dense GEMVs")
     ap.add_argument("--variant", default="vector", choices=("vector", "mfma"),
                     help="the headline's decode kernels (dsgx_decode_cfg::up = 0 | 1); --no-extra then runs nothing else")
     args = ap.parse_args()
@@ -176,6 +176,18 @@ def main():
                           "roofline": {"bound": "mfma", "achieved": d["tflops_routed"], "peak": d["mfma_peak_tflops"], "unit": "TFLOP/s",
                                        "frac": d["mfma_frac"], "traffic": None},
                           "cpu_baseline": None, "extra": [d], "wall_s": round(time.time() - t_start, 1)}))
+        return
+    if args.workload == "gemv":
+        # only the dense GEMVs (for profiler runs): one line, the FP8 [2048 x 4096] row-1 call as the value
+        from dsgx10_amd.benchdata import gemv_bench
+        g = gemv_bench()
+        head = min((d for d in g if d["workload"].startswith("dense_fp8")), key=lambda d: d["us_per_call"])
+        print(json.dumps({"metric": "dense_gemv_us", "value": head["us_per_call"], "unit": "us", "n_gpus": 1, "steps": 64, "warmup": 4,
+                          "ms_per_step": head["us_per_call"] * 1e-3, "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+                          "dtype": "f32 sums of bf16 x bf16 products", "data": "synthetic", "config": {"workload": head["workload"], "rows_M": 1},
+                          "roofline": {"bound": "hbm", "achieved": head["bytes"] / head["us_per_call"] * 1e-3, "peak": 8000.0, "unit": "GB/s",
+                                       "frac": head["hbm_frac"], "traffic": None},
+                          "cpu_baseline": None, "extra": g, "wall_s": round(time.time() - t_start, 1)}))
         return
     head_fp8 = args.workload == "fp8_m1"
     log("generating the %s layer ..." % ("FP8 256-expert" if head_fp8 else "INT4 168-expert"))

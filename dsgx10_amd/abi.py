@@ -46,7 +46,7 @@ assert C.sizeof(MatDesc) == 64
 # every symbol include/dsgx.h declares
 SYMBOLS = [
     "dsgx_mat_bytes", "dsgx_mat_scale_off", "dsgx_mat_zp_off", "dsgx_route", "dsgx_decode_cfg_default",
-    "dsgx_decode_ws_bytes", "dsgx_decode_ws_flag_offset", "dsgx_decode_status", "dsgx_moe_decode", "dsgx_moe_decode_noalloc", "dsgx_finalize", "dsgx_prefill_cfg_default", "dsgx_prefill_ws_bytes",
+    "dsgx_decode_ws_bytes", "dsgx_decode_ws_flag_offset", "dsgx_decode_status", "dsgx_moe_decode", "dsgx_moe_decode_noalloc", "dsgx_finalize", "dsgx_add_norm", "dsgx_prefill_cfg_default", "dsgx_prefill_ws_bytes",
     "dsgx_moe_prefill", "dsgx_prefill_view_get", "dsgx_gemv", "dsgx_dequant_int4", "dsgx_probe_dequant_int4", "dsgx_probe_mfma_fp8",
     "dsgx_widen_fp8", "dsgx_act_quant", "dsgx_last_error", "dsgx_version", "dsgx_stream_read", "dsgx_stream_read_cfg", "dsgx_stream_copy",
 ]

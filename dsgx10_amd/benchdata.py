@@ -291,44 +291,47 @@ class DecodeBench:
 
 
 def gemv_bench(reps=64):
-    """the two dense GEMV configurations: FP8 [2048 x 4096] at 1 row, INT4 [1536 x 6144] at 1, 2, 4, 6 rows; weights rotate
-    over copies that exceed the caches"""
+    """the two dense GEMV configurations: FP8 [2048 x 4096] at 1 row, INT4 [1536 x 6144] at 1, 2, 4, 6 rows, and the router's
+    logits (BF16 [E x H], f32 out, 1 row), each with K unsplit and split over 2 and 4 waves; weights rotate over copies that
+    exceed the caches"""
     out = []
     g = torch.Generator(device="cuda")
     g.manual_seed(7)
-    for name, fmt, N, K, rows in (("dense_fp8_gemv_2048x4096", abi.FMT_FP8, 2048, 4096, (1,)),
-                                  ("dense_int4_gemv_1536x6144", abi.FMT_INT4, 1536, 6144, (1, 2, 4, 6))):
+    for name, fmt, N, K, rows, kind in (("dense_fp8_gemv_2048x4096", abi.FMT_FP8, 2048, 4096, (1,), abi.OUT_BF16),
+                                        ("dense_int4_gemv_1536x6144", abi.FMT_INT4, 1536, 6144, (1, 2, 4, 6), abi.OUT_BF16),
+                                        ("router_bf16_gemv_256x4096", abi.FMT_BF16, 256, 4096, (1,), abi.OUT_F32),
+                                        ("router_bf16_gemv_168x6144", abi.FMT_BF16, 168, 6144, (1,), abi.OUT_F32)):
         per = mat_bytes(fmt, N, K)
         copies = max(8, int(600e6 // per))
         mats = []
         for c in range(copies):
             w = torch.randn(N, K, generator=g, device="cuda") * 0.02
-            mats.append(fp8_quantize_gpu(w) if fmt == abi.FMT_FP8 else int4_quantize_gpu(w))
+            mats.append(fp8_quantize_gpu(w) if fmt == abi.FMT_FP8 else int4_quantize_gpu(w) if fmt == abi.FMT_INT4 else (w.to(torch.bfloat16), None))
         for M in rows:
             x = torch.randn(M, K, generator=g, device="cuda").to(torch.bfloat16)
-            y = torch.zeros(M, N, dtype=torch.bfloat16, device="cuda")
-
-            def one(c):
-                m = mats[c % copies]
-                seg = dict(fmt=fmt, w=m[0], s=m[1], zp=m[2] if len(m) > 2 else None, n=N, y=y, ldy=N)
-                lib.gemv(x, K, M, K, [seg], abi.OUT_BF16)
-            for c in range(4):
-                one(c)
-            torch.cuda.synchronize()
-            gr = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(gr):
-                for c in range(reps):
+            y = torch.zeros(M, N, dtype=torch.float32 if kind == abi.OUT_F32 else torch.bfloat16, device="cuda")
+            for sk in (1, 2, 4):
+                def one(c):
+                    m = mats[c % copies]
+                    seg = dict(fmt=fmt, w=m[0], s=m[1], zp=m[2] if len(m) > 2 else None, n=N, y=y, ldy=N)
+                    lib.gemv(x, K, M, K, [seg], kind, splitk=sk)
+                for c in range(4):
                     one(c)
-            gr.replay()
-            torch.cuda.synchronize()
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            e0.record()
-            gr.replay()
-            e1.record()
-            torch.cuda.synchronize()
-            us = e0.elapsed_time(e1) * 1e3 / reps
-            b = per + M * K * 2 + M * N * 2
-            out.append(dict(workload=name, M=M, us_per_call=us, bytes=b, hbm_frac=b / (us * 1e-6) / HBM_PEAK))
+                torch.cuda.synchronize()
+                gr = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(gr):
+                    for c in range(reps):
+                        one(c)
+                gr.replay()
+                torch.cuda.synchronize()
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                gr.replay()
+                e1.record()
+                torch.cuda.synchronize()
+                us = e0.elapsed_time(e1) * 1e3 / reps
+                b = per + M * K * 2 + M * N * y.element_size()
+                out.append(dict(workload=name, M=M, splitk=sk, us_per_call=us, bytes=b, hbm_frac=b / (us * 1e-6) / HBM_PEAK))
     return out
 
 

@@ -74,6 +74,66 @@ __global__ void __launch_bounds__(256) k_finalize(const float* __restrict__ R, c
   out[i] = (uint16_t)f32_to_bf16_bits(__fadd_rn(bf16_round(R[i]), bf16_round(S[i])));
 }
 
+// The residual add and the next layer's RMSNorm after an MoE (or MLP) step: the local half of the reference's
+// comm::glm::allreduce_add_norm / allreduce2_add_norm (engine/comm/glmcoll.h:34-62) at one rank, the norm as
+// engine/attn/prep.cu:12-66 (k_rmsnorm). One workgroup a row:
+//   sum        = part                                   (one partial: the reference's decision 8, yr already holds yr + ys)
+//              | bf16(bf16(part) + bf16(part2))         (two partials: the old combine, experts.h finalize)
+//   h          = bf16(f32(res) + sum)                   (the contract: the f32 sum rounded once, with the residual)
+//              | bf16(f32(res) + bf16(sum))             (round2: the sum rounded first)
+//   xn         = bf16(w * bf16(h * rstd)),  rstd = 1 / sqrt(mean(h^2) + eps)
+// mean(h^2) in f32 in a fixed order: a thread's H / 256 contiguous values in order, the wave by a butterfly, the waves in
+// order (the reference fixes an order too, its own: the statistics' order is not part of the contract).
+__global__ void __launch_bounds__(256) k_add_norm(const float* __restrict__ part, const float* __restrict__ part2, int H,
+                                                  const uint16_t* __restrict__ res, uint16_t* __restrict__ res_out,
+                                                  const uint16_t* __restrict__ w, float eps, uint16_t* __restrict__ xn, int round2) {
+  __shared__ float red[4];
+  const int row = blockIdx.x, tid = threadIdx.x, per = H / 256;  // (per a multiple of 8, at most 64: the host checks)
+  const size_t base = (size_t)row * H + (size_t)tid * per;
+  float hv[64];
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < 64; i += 8) {
+    if (i >= per) break;
+    const u32x4_t rq = *reinterpret_cast<const DSGX_GLOBAL u32x4_t*>((uintptr_t)(res + base + i));
+    uint32_t ho[4];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const float r = bf16_bits_to_f32(j & 1 ? rq[j >> 1] >> 16 : rq[j >> 1] & 0xFFFFu);
+      float s = part[base + i + j];
+      if (part2) s = __fadd_rn(bf16_round(s), bf16_round(part2[base + i + j])), s = bf16_round(s);
+      else if (round2) s = bf16_round(s);
+      const uint32_t hb = f32_to_bf16_bits(__fadd_rn(r, s));
+      const float h = bf16_bits_to_f32(hb);
+      hv[i + j] = h;
+      ss = __fadd_rn(ss, __fmul_rn(h, h));
+      if (j & 1) ho[j >> 1] |= hb << 16;
+      else ho[j >> 1] = hb;
+    }
+    if (res_out) *reinterpret_cast<u32x4_t*>(res_out + base + i) = u32x4_t{ho[0], ho[1], ho[2], ho[3]};
+  }
+  if (!xn) return;
+  ss = wave_sum(ss);
+  if ((tid & 63) == 0) red[tid >> 6] = ss;
+  __syncthreads();
+  const float tot = __fadd_rn(__fadd_rn(__fadd_rn(red[0], red[1]), red[2]), red[3]);
+  const float rstd = __fdiv_rn(1.f, __fsqrt_rn(__fadd_rn(__fdiv_rn(tot, (float)H), eps)));
+#pragma unroll
+  for (int i = 0; i < 64; i += 8) {
+    if (i >= per) break;
+    const u32x4_t wq = *reinterpret_cast<const DSGX_GLOBAL u32x4_t*>((uintptr_t)(w + (size_t)tid * per + i));
+    uint32_t o[4];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const float wv = bf16_bits_to_f32(j & 1 ? wq[j >> 1] >> 16 : wq[j >> 1] & 0xFFFFu);
+      const uint32_t b = f32_to_bf16_bits(__fmul_rn(wv, bf16_round(__fmul_rn(hv[i + j], rstd))));
+      if (j & 1) o[j >> 1] |= b << 16;
+      else o[j >> 1] = b;
+    }
+    *reinterpret_cast<u32x4_t*>(xn + base + i) = u32x4_t{o[0], o[1], o[2], o[3]};
+  }
+}
+
 // INT4 canonical tensors -> the contract's bf16 weight, one thread a group of 32 (the subtract-first form, exact for
 // every finite scale). hot: decode through the streaming kernels' own i4x8_to_bf16 instead (the probe the tests use to
 // pin the hot loop's arithmetic, as the reference's k_deq does: engine/experts/tests/test_experts.cu:217-235).
@@ -210,6 +270,16 @@ int dsgx_finalize(const float* R, const float* S, int n, uint16_t* out, void* st
   if (!R || !S || !out || n < 0) return fail(DSGX_EINVAL, "finalize: null argument or n %d", n);
   if (!n) return DSGX_OK;
   hipLaunchKernelGGL(k_finalize, dim3((n + 255) / 256), dim3(256), 0, static_cast<hipStream_t>(stream), R, S, n, out);
+  DSGX_HIP(hipGetLastError());
+  return DSGX_OK;
+}
+int dsgx_add_norm(const float* part, const float* part2, int M, int H, const uint16_t* res, uint16_t* res_out, const uint16_t* w,
+                  float eps, uint16_t* xn, int round2, void* stream) {
+  if (!part || !res || M < 1) return fail(DSGX_EINVAL, "add_norm: null partial or residual, or %d rows", M);
+  if (H < 2048 || H % 2048 || H > 16384) return fail(DSGX_EINVAL, "add_norm: hidden %d (a multiple of 2048 up to 16384)", H);
+  if (xn && !w) return fail(DSGX_EINVAL, "add_norm: the norm needs its weight");
+  if (!xn && !res_out) return fail(DSGX_EINVAL, "add_norm: no output");
+  hipLaunchKernelGGL(k_add_norm, dim3(M), dim3(256), 0, static_cast<hipStream_t>(stream), part, part2, H, res, res_out, w, eps, xn, round2);
   DSGX_HIP(hipGetLastError());
   return DSGX_OK;
 }

@@ -21,7 +21,7 @@ struct GemvSegDev {
 };
 struct GemvArgs {
   const uint16_t* x;
-  int ldx, K, nq, nsegk, nsegs, total_rows, out;
+  int ldx, K, nq, nsegk, nsegs, total_rows, out, splitk;
   GemvSegDev sg[kMaxSegs];
 };
 
@@ -46,7 +46,7 @@ __global__ void __launch_bounds__(256) k_gemv(GemvArgs a) {
   for (int r = 0; r < RB; ++r)
 #pragma unroll
     for (int m = 0; m < M; ++m) acc[r][m] = 0.f;
-  const uint8_t* dummy = reinterpret_cast<const uint8_t*>(a.x);  // where the loads past the last step go
+  const uint8_t* dummy = a.sg[0].m.w;  // where the loads past the last step go: the first KiB of the first matrix (always there)
   int lt = 0, lj = 0, lseg = 0;  // the load cursor: step, batch number of this wave, segment
   auto load = [&](Raw (&r)[RB]) {
     const bool ok = lt < nsteps;
@@ -105,6 +105,95 @@ __global__ void __launch_bounds__(256) k_gemv(GemvArgs a) {
   }
 }
 
+// Split-K (engine/attn/attn.h:119 of the reference: warps of a CTA share a tile's k range, for small N): a workgroup of
+// four waves holds 4 / SK row batches, the SK waves of a batch take the K segments slice, slice + SK, ... of its rows;
+// the waves' sums meet in LDS and the batch's first wave adds them in slice order (a fixed order, as the reference's
+// finish(), gemv.cu:138-151), then the epilogue of k_gemv. One batch a group and launch: this form is for matrices of
+// few rows, where whole-K waves would leave most of the chip idle and walk K in several dependent round trips.
+template <int FMT, int M, int RB, int SK>
+__global__ void __launch_bounds__(256) k_gemv_sk(GemvArgs a) {
+  extern __shared__ uint4 xs[];
+  __shared__ float part[4][RB * M];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  constexpr int GPW = 4 / SK;  // batches a workgroup
+  const int grp = wave / SK, slice = wave % SK;
+  const int nbatch = a.total_rows / RB;
+  const int batch = blockIdx.x * GPW + grp;
+  const bool live = batch < nbatch;
+  const int row = live ? batch * RB : 0;
+  int si = 0;
+#pragma unroll
+  for (int i = 1; i < kMaxSegs; ++i)
+    if (i < a.nsegs && row >= a.sg[i].row0) si = i;
+  const GemvSegDev& sg = a.sg[si];
+  const int nmine = live && slice < a.nsegk ? (a.nsegk - slice + SK - 1) / SK : 0;  // this wave's segments
+  constexpr int D = 4;
+  Raw w[D][RB];
+  float acc[RB][M];
+#pragma unroll
+  for (int r = 0; r < RB; ++r)
+#pragma unroll
+    for (int m = 0; m < M; ++m) acc[r][m] = 0.f;
+  const uint8_t* dummy = reinterpret_cast<const uint8_t*>(sg.m.w);  // (loads past the last step: the matrix's first bytes)
+  int lt = 0;
+  auto load = [&](Raw (&r)[RB]) {
+    const bool ok = lt < nmine;
+    const int seg = slice + (ok ? lt : 0) * SK;
+    ++lt;
+#pragma unroll
+    for (int i = 0; i < RB; ++i) load_raw<FMT, true>(r[i], sg.m, row - sg.row0 + i, seg, lane, a.K, acc[i][0], ok ? nullptr : dummy);
+  };
+#pragma unroll
+  for (int d = 0; d < D; ++d) load(w[d]);
+  stage_x<FmtT<FMT>::KL>(xs, a.x, a.ldx, M, a.K, a.nq * 8);
+  __syncthreads();
+  for (int t = 0; t < nmine; t += D) {
+#pragma unroll
+    for (int d = 0; d < D; ++d) {
+      if (t + d < nmine) step_dot<FMT, M, RB, true>(w[d], xs, a.nq, slice + (t + d) * SK, lane, acc, a.K);
+      load(w[d]);
+    }
+  }
+  // the wave's sums over its lanes, value (i, m) kept by lane i * M + m
+  float mine = 0.f;
+#pragma unroll
+  for (int i = 0; i < RB; ++i)
+#pragma unroll
+    for (int m = 0; m < M; ++m) {
+      const float v = wave_sum(acc[i][m]);
+      if (lane == i * M + m) mine = v;
+    }
+  if (lane < RB * M) part[wave][lane] = mine;
+  __syncthreads();
+  if (!live || slice != 0 || lane >= RB * M) return;
+  float sum = part[grp * SK][lane];
+#pragma unroll
+  for (int k = 1; k < SK; ++k) sum = __fadd_rn(sum, part[grp * SK + k][lane]);
+  const int r = lane / M, m = lane % M, n = row - sg.row0 + r;
+  if (a.out == DSGX_OUT_BF16) {
+    static_cast<uint16_t*>(sg.y)[(size_t)m * sg.ldy + n] = (uint16_t)f32_to_bf16_bits(sum);
+  } else if (a.out == DSGX_OUT_F32) {
+    static_cast<float*>(sg.y)[(size_t)m * sg.ldy + n] = sum;
+  } else if ((r & 1) == 0) {  // SwiGLU: row 2i gate, 2i + 1 up -> column i; the up row's sum sits M lanes further
+    float up = part[grp * SK][lane + M];
+#pragma unroll
+    for (int k = 1; k < SK; ++k) up = __fadd_rn(up, part[grp * SK + k][lane + M]);
+    static_cast<uint16_t*>(sg.y)[(size_t)m * sg.ldy + n / 2] = (uint16_t)swiglu_bits(bf16_round(sum), bf16_round(up));
+  }
+}
+
+template <int FMT, int M, int SK>
+int launch_gemv_sk(const GemvArgs& a, hipStream_t st) {
+  constexpr int RB = 2;
+  const size_t lds = (size_t)M * a.nq * 16;
+  const int nbatch = a.total_rows / RB, gpw = 4 / SK;
+  auto kern = k_gemv_sk<FMT, M, RB, SK>;
+  if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds)) return rc;
+  hipLaunchKernelGGL(kern, dim3((nbatch + gpw - 1) / gpw), dim3(256), lds, st, a);
+  DSGX_HIP(hipGetLastError());
+  return DSGX_OK;
+}
+
 template <int FMT, int M, int RB>
 int launch_gemv(const GemvArgs& a, hipStream_t st) {
   constexpr int D = 4;
@@ -123,6 +212,11 @@ int launch_gemv(const GemvArgs& a, hipStream_t st) {
 }
 template <int FMT, int M>
 int launch_gemv_rb(const GemvArgs& a, hipStream_t st) {
+  // split-K as asked for, where the rows are few enough for one batch a wave group and launch
+  if (a.splitk > 1 && a.total_rows / 2 <= 16 * num_cus_cached()) {
+    if (a.splitk == 2) return launch_gemv_sk<FMT, M, 2>(a, st);
+    return launch_gemv_sk<FMT, M, 4>(a, st);
+  }
   // few rows: two rows a wavefront so that the whole chip streams
   if (a.total_rows / 4 < 4 * num_cus_cached()) return launch_gemv<FMT, M, 2>(a, st);
   return launch_gemv<FMT, M, 4>(a, st);
@@ -149,9 +243,9 @@ int ilog2_exact(int v) {
 }
 
 // one launch: the segments of one format (gemv_one of the reference, gemv.cu:459-516)
-int gemv_one(int fmt, const uint16_t* x, int ldx, int rows, int K, const dsgx_gemv_seg* segs, int nseg, int out, hipStream_t st) {
+int gemv_one(int fmt, const uint16_t* x, int ldx, int rows, int K, const dsgx_gemv_seg* segs, int nseg, int out, int splitk, hipStream_t st) {
   GemvArgs a{};
-  a.x = x, a.ldx = ldx, a.K = K, a.out = out, a.nsegs = nseg;
+  a.x = x, a.ldx = ldx, a.K = K, a.out = out, a.nsegs = nseg, a.splitk = splitk;
   const int segk = fmt == DSGX_FMT_FP8_B128 ? 1024 : fmt == DSGX_FMT_INT4_G32 ? 2048 : 512;
   a.nsegk = (K + segk - 1) / segk;
   a.nq = a.nsegk * segk / 8;
@@ -221,7 +315,7 @@ extern "C" int dsgx_gemv(const uint16_t* x, int ldx, int rows, int K, const dsgx
         const size_t esz = out == DSGX_OUT_F32 ? 4 : 2;
         gg[i].y = static_cast<uint8_t*>(g[i].y) + (size_t)r0 * g[i].ldy * esz;
       }
-      const int rc = gemv_one(fmt, x + (size_t)r0 * ldx, ldx, nr, K, gg, n, out, st);
+      const int rc = gemv_one(fmt, x + (size_t)r0 * ldx, ldx, nr, K, gg, n, out, splitk, st);
       if (rc) return rc;
     }
   }

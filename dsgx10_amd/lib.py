@@ -44,6 +44,8 @@ def lib():
                                               C.c_void_p, C.c_void_p, C.c_void_p, C.POINTER(abi.DecodeCfg)]
         L.dsgx_decode_status.argtypes = [C.POINTER(abi.LayerW), C.c_void_p, C.c_void_p]
         L.dsgx_finalize.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p]
+        L.dsgx_add_norm.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_float,
+                                    C.c_void_p, C.c_int, C.c_void_p]
         L.dsgx_gemv.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.POINTER(abi.GemvSeg), C.c_int, C.c_int, C.c_int, C.c_void_p]
         for f in ("dsgx_dequant_int4", "dsgx_probe_dequant_int4"):
             getattr(L, f).argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_size_t, C.c_void_p]
@@ -116,6 +118,11 @@ def decode_status(layer_w, ws, stream=None):
 def finalize(R, S, n, out, stream=None):
     """out[i] = bf16(bf16(R[i]) + bf16(S[i])) for n = M * H values"""
     _check(lib().dsgx_finalize(_ptr(R), _ptr(S), n, _ptr(out), _stream(stream)))
+
+
+def add_norm(part, part2, M, H, res, res_out, w, eps, xn, round2=False, stream=None):
+    """h = bf16(f32(res) + sum) -> res_out; xn = bf16(w * bf16(h * rstd)): the local half of allreduce_add_norm"""
+    _check(lib().dsgx_add_norm(_ptr(part), _ptr(part2), M, H, _ptr(res), _ptr(res_out), _ptr(w), eps, _ptr(xn), int(round2), _stream(stream)))
 
 
 # ---- gx::moe_prefill --------------------------------------------------------------------------------------------------

@@ -152,6 +152,17 @@ DSGX_API int dsgx_moe_decode_noalloc(const dsgx_layer_w* L, const uint16_t* x, c
 /* out = bf16(bf16(R) + bf16(S)): gx::finalize (engine/experts/experts.h:146-147, decode.cu:591-598) */
 DSGX_API int dsgx_finalize(const float* R, const float* S, int n, uint16_t* out, void* stream);
 
+/* The residual add after the expert step and the next layer's RMSNorm, the local half of the reference's
+   comm::glm::allreduce_add_norm / allreduce2_add_norm (engine/comm/glmcoll.h:34-62; the norm: engine/attn/prep.cu:12-66),
+   M rows of H (a multiple of 2048, up to 16384):
+     sum = part, or with part2 bf16(bf16(part) + bf16(part2)) (the old combine of yr and ys)
+     h   = bf16(f32(res) + sum), the contract's single rounding (ref/glmref.py:269-276 add_residual); round2: the sum is
+           rounded to bf16 first (the engine's order before its decision 8)
+     xn  = bf16(w * bf16(h * rstd)), rstd = 1 / sqrt(mean(h^2) + eps), statistics in f32
+   res_out (may be res itself) receives h, xn the normed row for the next layer; either may be null. */
+DSGX_API int dsgx_add_norm(const float* part, const float* part2, int M, int H, const uint16_t* res, uint16_t* res_out,
+                           const uint16_t* w, float eps, uint16_t* xn, int round2, void* stream);
+
 /* ---- prefill: gx::moe_prefill (engine/experts/experts.h:149-193, prefill.cu:1056-1116) --------------------------- */
 typedef struct dsgx_prefill_cfg {
   int32_t shared;   /* run the fused shared expert (if the layer has one) */
@@ -186,8 +197,10 @@ typedef struct dsgx_gemv_seg {
   int32_t ldy;        /* y's row stride in elements */
 } dsgx_gemv_seg;
 /* y[r][n] = sum_k x[r][k] W[n][k]; x bf16 [rows][ldx], rows 1..16, K a multiple of 128 (INT4: of 256).
-   out: DSGX_OUT_*; SwiGLU: rows interleaved gate/up in pairs. splitk is accepted for signature parity and ignored
-   (K is always split over the 64 lanes of a wavefront and reduced by cross-lane shuffles). */
+   out: DSGX_OUT_*; SwiGLU: rows interleaved gate/up in pairs. splitk 1, 2 or 4 (engine/attn/attn.h:119): with 2 or 4 the
+   waves of a workgroup share a row pair's K range and their sums are added in a fixed order (for matrices of few rows,
+   e.g. the router's; ignored above 32 rows a CU, where whole-K waves already fill the chip). A given splitk always gives
+   the same bits; different values add in different orders. */
 DSGX_API int dsgx_gemv(const uint16_t* x, int ldx, int rows, int K, const dsgx_gemv_seg* segs, int nseg, int out,
                        int splitk, void* stream);
 /* glm::dequant_int4 (engine/attn/attn.h:154-158): the contract's bf16 weight [N][ld] from the canonical tensors */

@@ -673,4 +673,34 @@ ORC void orc_moe_prefill_fp8_row_range(const dsgx_layer_w* L, const dsgx_mat_des
   }
 }
 
+// The residual add and RMSNorm after the expert step: A/engine/comm/glmcoll.h:34-62 (allreduce_add_norm at one rank),
+// A/ref/glmref.py:225-228 (rms_norm), :269-276 (add_residual), A/engine/attn/prep.cu:26-34 (rstd and the two roundings).
+// res_out bf16 = the contract's h; xn from mean(h^2) summed in f64 (xn) and in f32 sequentially (xn32).
+ORC void orc_add_norm(const float* part, const float* part2, int M, int H, const uint16_t* res, const uint16_t* w, float eps,
+                      int round2, uint16_t* res_out, uint16_t* xn, uint16_t* xn32) {
+  for (int m = 0; m < M; ++m) {
+    std::vector<float> h(H);
+    double ss = 0;
+    float ss32 = 0.f;
+    for (int n = 0; n < H; ++n) {
+      const size_t i = (size_t)m * H + n;
+      float s = part[i];
+      if (part2) s = bfr(bfr(s) + bfr(part2[i]));
+      else if (round2) s = bfr(s);
+      const uint16_t hb = f2bf(bf2f(res[i]) + s);
+      if (res_out) res_out[i] = hb;
+      h[n] = bf2f(hb);
+      ss += (double)h[n] * h[n];
+      ss32 += h[n] * h[n];
+    }
+    for (int pass = 0; pass < 2; ++pass) {
+      uint16_t* out = pass ? xn32 : xn;
+      if (!out) continue;
+      const float tot = pass ? ss32 : (float)ss;
+      const float rstd = 1.f / sqrtf(tot / (float)H + eps);
+      for (int n = 0; n < H; ++n) out[(size_t)m * H + n] = f2bf(bf2f(w[n]) * bfr(h[n] * rstd));
+    }
+  }
+}
+
 ORC int orc_threads() { return omp_get_max_threads(); }

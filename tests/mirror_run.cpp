@@ -1,6 +1,6 @@
 // Test program: drives the C++ mirror headers (include/gx/experts.h, include/glm/attn.h) on the GPU the way the
 // reference's runner calls its operators (altar1-4xgx10-switchless/engine/model/model.cu:309-343): route -> moe_decode
-// (routing apart, then fused) -> finalize, plus one dense GEMV. Inputs are raw files written by
+// (routing apart, then fused) -> finalize, one dense GEMV with K split four ways, and the residual add + RMSNorm. Inputs are raw files written by
 // tests/test_gpu_mirror.py into a directory; outputs go back as raw files, and the test compares them bit for bit with
 // what the same calls give through the ctypes binding of the C ABI.
 //   mirror_run <dir> <fmt> <H> <I> <E> <topk> <M> <route scale> <up variant>
@@ -12,6 +12,7 @@
 #include <vector>
 
 #include "glm/attn.h"
+#include "glm/coll.h"
 #include "gx/experts.h"
 
 #define HIPOK(x)                                                          \
@@ -114,8 +115,13 @@ int main(int argc, char** argv) {
     seg.fmt = L.sh.g ? glm::WFmt::kFP8 : glm::WFmt::kBF16;
     seg.w = L.sh.g ? static_cast<const void*>(L.sh.g) : static_cast<const void*>(L.sh.bgu);
     seg.s = L.sh.gs, seg.n = gn, seg.y = gv, seg.ldy = gn;
-    glm::gemv(x, H, M, H, &seg, 1, glm::GemvOut::kF32, 1, st);
+    glm::gemv(x, H, M, H, &seg, 1, glm::GemvOut::kF32, 4, st);
   }
+  // the step's end (model.cu:343): h = bf16(resid16 + yr2) in place, xn = the next layer's RMSNorm of h
+  uint16_t* res16 = static_cast<uint16_t*>(upload(slurp(dir + "res16.bin")));
+  const uint16_t* normw = static_cast<const uint16_t*>(upload(slurp(dir + "normw.bin")));
+  uint16_t* xn = static_cast<uint16_t*>(dalloc((size_t)M * H * 2, 0xFF));
+  comm::glm::allreduce_add_norm(comm::DevChannel{}, yr2, M, H, res16, res16, normw, 1e-5f, xn, st);
   HIPOK(hipStreamSynchronize(st));
   dump(dir + "o_idx.bin", idx, (size_t)M * topk * 4);
   dump(dir + "o_w.bin", w, (size_t)M * topk * 4);
@@ -125,6 +131,8 @@ int main(int argc, char** argv) {
   dump(dir + "o_yr2.bin", yr2, (size_t)M * H * 4);
   dump(dir + "o_ys2.bin", ys2, (size_t)M * H * 4);
   if (gv) dump(dir + "o_gemv.bin", gv, (size_t)M * gn * 4);
+  dump(dir + "o_h.bin", res16, (size_t)M * H * 2);
+  dump(dir + "o_xn.bin", xn, (size_t)M * H * 2);
   std::printf("CHECK mirror_run ok  ws %zu bytes\n", wsb);
   return 0;
 }

@@ -242,6 +242,17 @@ def moe_prefill_fp8_row_range(hl, xrow, idx, sum_tol):
     return lo, hi
 
 
+def add_norm(part, part2, res, w, eps, round2=False):
+    """(res_out bf16, xn bf16 from f64 statistics, xn bf16 from sequential f32 statistics), each [M][H]"""
+    part = np.ascontiguousarray(part, np.float32)
+    M, H = part.shape
+    p2 = None if part2 is None else np.ascontiguousarray(part2, np.float32)
+    res, w = np.ascontiguousarray(res, np.uint16), np.ascontiguousarray(w, np.uint16)
+    ro, xn, xn32 = np.empty((M, H), np.uint16), np.empty((M, H), np.uint16), np.empty((M, H), np.uint16)
+    lib().orc_add_norm(_p(part), _p(p2), M, H, _p(res), _p(w), C.c_float(eps), int(round2), _p(ro), _p(xn), _p(xn32))
+    return ro, xn, xn32
+
+
 def finalize(R, S):
     R = np.ascontiguousarray(R, np.float32)
     S = np.ascontiguousarray(S, np.float32)

@@ -1,6 +1,6 @@
 """The C++ mirror headers on the GPU (marked gpu): tests/mirror_run (tests/mirror_run.cpp, compiled by
 dsgx10_amd.build against include/gx/experts.h and include/glm/attn.h) runs route -> moe_decode -> finalize, the fused
-form and a dense GEMV through the gx:: / glm:: forwarders; every output must equal, bit for bit, what the same calls
+form, a dense GEMV and the residual add + RMSNorm through the gx:: / glm:: / comm::glm:: forwarders; every output must equal, bit for bit, what the same calls
 give through the ctypes binding of the C ABI."""
 import os
 import subprocess
@@ -28,10 +28,12 @@ def test_cpp_mirrors_give_the_c_abi_bits(fmt, shared, scale, up):
     x, logits, _, _ = rows_and_routing(51, M, H, E, topk, scale)
     bias = orc.normal_f32(51, 3, (E,), 0.3)
     resid = orc.normal_f32(51, 4, (M, H), 1.0)
+    res16, normw = orc.normal_bf16(51, 5, (M, H), 1.0), orc.normal_bf16(51, 6, (H,), 1.0)
     with tempfile.TemporaryDirectory() as d:
         def put(name, a):
             np.ascontiguousarray(a).tofile(os.path.join(d, name + ".bin"))
         put("pool", hl.pool), put("desc", hl.desc), put("x", x), put("logits", logits), put("bias", bias), put("resid", resid)
+        put("res16", res16), put("normw", normw)
         if hl.shared_fp8 is not None:
             for n, (c, s) in zip("gud", hl.shared_fp8):
                 put("sh_" + n, c), put("sh_" + n + "s", s)
@@ -40,7 +42,7 @@ def test_cpp_mirrors_give_the_c_abi_bits(fmt, shared, scale, up):
         r = subprocess.run([EXE, d, str(fmt), str(H), str(I), str(E), str(topk), str(M), repr(scale), str(up)], capture_output=True, text=True, timeout=120)
         assert r.returncode == 0 and "CHECK mirror_run ok" in r.stdout, r.stdout + r.stderr
         got = {n: np.fromfile(os.path.join(d, "o_%s.bin" % n), dt) for n, dt in
-               (("idx", np.int32), ("w", np.uint32), ("yr", np.uint32), ("ys", np.uint32), ("out", np.uint16), ("yr2", np.uint32), ("ys2", np.uint32), ("gemv", np.uint32))}
+               (("idx", np.int32), ("w", np.uint32), ("yr", np.uint32), ("ys", np.uint32), ("out", np.uint16), ("yr2", np.uint32), ("ys2", np.uint32), ("gemv", np.uint32), ("h", np.uint16), ("xn", np.uint16))}
     # the same calls through ctypes
     dlog, dbias = gpu.dev(logits), gpu.dev(bias)
     gi, gw = gpu.empty(M * topk * 4), gpu.empty(M * topk * 4)
@@ -64,5 +66,10 @@ def test_cpp_mirrors_give_the_c_abi_bits(fmt, shared, scale, up):
         seg = dict(fmt=abi.FMT_FP8, w=gpu.dev(hl.shared_fp8[0][0]), s=gpu.dev(hl.shared_fp8[0][1]), n=gn, y=y, ldy=gn)
     else:
         seg = dict(fmt=abi.FMT_BF16, w=gpu.dev(hl.shared_bf16[0]), n=gn, y=y, ldy=gn)
-    lib.gemv(gpu.dev(x), H, M, H, [seg], abi.OUT_F32)
+    lib.gemv(gpu.dev(x), H, M, H, [seg], abi.OUT_F32, splitk=4)
     assert np.array_equal(got["gemv"], gpu.host(y, np.uint32, (-1,)))
+    # comm::glm::allreduce_add_norm at a world of one
+    r16, xn = gpu.dev(res16), gpu.empty(M * H * 2, 0)
+    lib.add_norm(gpu.dev(yr2), None, M, H, r16, r16, gpu.dev(normw), 1e-5, xn)
+    assert np.array_equal(got["h"], gpu.host(r16, np.uint16, (-1,))) and np.array_equal(got["xn"], gpu.host(xn, np.uint16, (-1,)))
+    assert np.array_equal(got["h"], orc.add_norm(yr2, None, res16, normw, 1e-5)[0].reshape(-1))

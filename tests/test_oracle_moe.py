@@ -2,6 +2,7 @@
 products on independently dequantised weights, the INT4 = BF16(dequantised) identity, batch invariance, and the
 expert-id order of the weighted sum."""
 import numpy as np
+import pytest
 import torch
 
 from dsgx10_amd import abi
@@ -164,6 +165,41 @@ def test_finalize():
     S = orc.normal_f32(0, 2, (64,), 1.0)
     want = (torch.from_numpy(R).to(torch.bfloat16) + torch.from_numpy(S).to(torch.bfloat16)).view(torch.int16).numpy().view(np.uint16)
     assert np.array_equal(orc.finalize(R, S), want)
+
+
+@pytest.mark.parametrize("mode", ["contract", "round2", "two_partials"])
+def test_add_norm_against_torch(mode):
+    """orc_add_norm against torch ops that spell the reference's python contract (ref/glmref.py:225-228 rms_norm, :269-276
+    add_residual; glmcoll.h:44-62 for the two older orders): h bit for bit (elementwise, no order involved); xn against
+    x * rsqrt(mean(x^2) + eps) rounded, times w rounded. torch's mean order and rsqrt differ from 1/sqrt of a sequential
+    sum in the last f32 bit, which can move a value across a bf16 boundary: at most 1 step on at most 0.1%.
+    Negative controls: a dropped rounding of the normalised value, and the norm of the unrounded sum, both differ."""
+    bf = torch.bfloat16
+    M, H, eps = 4, 2048, 1e-5
+    part = orc.normal_f32(3, 1, (M, H), 0.7)
+    part2 = orc.normal_f32(3, 2, (M, H), 0.3) if mode == "two_partials" else None
+    res, w = orc.normal_bf16(3, 3, (M, H), 1.5), orc.normal_bf16(3, 4, (H,), 1.0)
+    ro, xn, xn32 = orc.add_norm(part, part2, res, w, eps, round2=mode == "round2")
+    t = lambda a: torch.from_numpy(a)
+    tb = lambda a: torch.from_numpy(a.view(np.int16)).view(bf)
+    s = t(part)
+    if part2 is not None:
+        s = (s.to(bf) + t(part2).to(bf)).float()  # bf16 + bf16 in torch: the f32 sum rounded once
+    elif mode == "round2":
+        s = s.to(bf).float()
+    h = (tb(res).float() + s).to(bf)
+    assert np.array_equal(h.view(torch.int16).numpy().view(np.uint16), ro)
+    h32 = h.float()
+    n = (h32 * torch.rsqrt(h32.pow(2).mean(-1, keepdim=True) + eps)).to(bf)
+    want = (n.float() * tb(w).float()).to(bf).view(torch.int16).numpy().view(np.uint16)
+    for got in (xn, xn32):
+        assert (got == want).mean() >= 0.999
+        assert np.abs(got.astype(np.int32) - want.astype(np.int32)).max() <= 1
+    unrounded = ((h32 * torch.rsqrt(h32.pow(2).mean(-1, keepdim=True) + eps)) * tb(w).float()).to(bf).view(torch.int16).numpy().view(np.uint16)
+    assert (unrounded != xn).mean() > 0.01
+    hs = tb(res).float() + s
+    of_sum = ((hs * torch.rsqrt(hs.pow(2).mean(-1, keepdim=True) + eps)).to(bf).float() * tb(w).float()).to(bf).view(torch.int16).numpy().view(np.uint16)
+    assert (of_sum != xn).mean() > 0.01
 
 
 def test_prefill_fp8_row_range_brackets_h():
