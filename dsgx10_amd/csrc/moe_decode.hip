@@ -67,22 +67,46 @@ static int decode_variant(uint32_t fmt, int M, int H, int I) {
   return 0;
 }
 
-static size_t ws_h_bytes(const dsgx_layer_w* L) { return (size_t)(DSGX_MAX_UNION + 1) * DSGX_MAX_ROWS * L->I * 2; }
-// after h and the barrier words: the slot-partitioned down phase's slot table (kFacBytes) and its f32 results
-// [slot][8 rows][H]
-static constexpr size_t kFacBytes = (size_t)(8 + (DSGX_MAX_UNION + 1) * 8) * 4 + 192;  // (a multiple of 256)
-static size_t ws_part_bytes(const dsgx_layer_w* L) { return kFacBytes + (size_t)(DSGX_MAX_UNION + 1) * 8 * L->H * 4; }
+}  // extern "C"
+
+// The workspace: h [DSGX_MAX_UNION + 1 slots][DSGX_MAX_ROWS][I] | the barrier's words (kBarBytes) | the slot-partitioned down
+// phase's slot table (kFacBytes) and its f32 results [slot][8 rows][H]. I and H here are the LAYOUT's: the layer's own for a
+// caller's workspace; the built-in workspace is laid out for its largest shapes whatever the layer, so that every layer run
+// on it finds the barrier's words in one place (at an offset that moved with the layer, one layer's h or partial sums would
+// lie where another's counters are expected to be zero).
+struct WsLayout {
+  int I, H;
+  static constexpr size_t kFacBytes = (size_t)(8 + (DSGX_MAX_UNION + 1) * 8) * 4 + 192;  // (a multiple of 256)
+  constexpr size_t h_bytes() const { return (size_t)(DSGX_MAX_UNION + 1) * DSGX_MAX_ROWS * I * 2; }
+  constexpr size_t bar_off() const { return h_bytes(); }
+  constexpr size_t fac_off() const { return bar_off() + kBarBytes; }
+  constexpr size_t dpart_off() const { return fac_off() + kFacBytes; }
+  constexpr size_t bytes() const { return dpart_off() + (size_t)(DSGX_MAX_UNION + 1) * 8 * H * 4; }
+};
+static constexpr WsLayout kStaticLayout{DSGX_NOALLOC_MAX_I, DSGX_NOALLOC_MAX_H};
+static_assert(kStaticLayout.bytes() == kStaticWsBytes, "the built-in workspace's size");
+static int moe_decode_at(const dsgx_layer_w* L, const uint16_t* x, const int* idx, const float* w, int M, void* ws, const WsLayout& lay,
+                         float* yr, float* ys, void* stream, const dsgx_decode_cfg* cfg);
+
+extern "C" {
 size_t dsgx_decode_ws_bytes(const dsgx_layer_w* L) {
   if (!L || L->I <= 0 || L->H <= 0) return 0;
-  return ws_h_bytes(L) + kBarBytes + ws_part_bytes(L);
+  return WsLayout{L->I, L->H}.bytes();
 }
 size_t dsgx_decode_ws_flag_offset(const dsgx_layer_w* L) {
   if (!L || L->I <= 0) return 0;
-  return ws_h_bytes(L) + (size_t)(2 * kBarGroups + 1) * kBarLine * 4;
+  return WsLayout{L->I, L->H}.bar_off() + (size_t)(2 * kBarGroups + 1) * kBarLine * 4;
 }
 
 int dsgx_moe_decode(const dsgx_layer_w* L, const uint16_t* x, const int* idx, const float* w, int M, void* ws, float* yr, float* ys,
                     void* stream, const dsgx_decode_cfg* cfg) {
+  if (!L) return fail(DSGX_EINVAL, "moe_decode: null layer, x or workspace");
+  return moe_decode_at(L, x, idx, w, M, ws, WsLayout{L->I, L->H}, yr, ys, stream, cfg);
+}
+}  // extern "C"
+
+static int moe_decode_at(const dsgx_layer_w* L, const uint16_t* x, const int* idx, const float* w, int M, void* ws, const WsLayout& lay,
+                         float* yr, float* ys, void* stream, const dsgx_decode_cfg* cfg) {
   dsgx_decode_cfg c;
   if (cfg) c = *cfg;
   else dsgx_decode_cfg_default(&c);
@@ -127,16 +151,17 @@ int dsgx_moe_decode(const dsgx_layer_w* L, const uint16_t* x, const int* idx, co
     dsgx_decode_cfg c1 = c, c2 = c;
     c1.parts = c2.parts = c.parts & 3;
     if (c.logits) c2.logits = c.logits + (size_t)M1 * E;
-    if (int rc = dsgx_moe_decode(L, x, idx, w, M1, ws, yr, ys, stream, &c1)) return rc;
-    return dsgx_moe_decode(L, x + (size_t)M1 * H, idx ? idx + (size_t)M1 * topk : nullptr, w ? w + (size_t)M1 * topk : nullptr, M - M1, ws,
-                           yr ? yr + (size_t)M1 * H : nullptr, ys ? ys + (size_t)M1 * H : nullptr, stream, &c2);
+    if (int rc = moe_decode_at(L, x, idx, w, M1, ws, lay, yr, ys, stream, &c1)) return rc;
+    return moe_decode_at(L, x + (size_t)M1 * H, idx ? idx + (size_t)M1 * topk : nullptr, w ? w + (size_t)M1 * topk : nullptr, M - M1, ws, lay,
+                         yr ? yr + (size_t)M1 * H : nullptr, ys ? ys + (size_t)M1 * H : nullptr, stream, &c2);
   }
   DecodeArgs a{};
   a.x = x, a.M = M, a.idx = idx, a.w = w, a.logits = c.logits, a.bias = c.bias, a.route_scale = c.route_scale, a.score_fn = c.score_fn;
   a.L = *L, a.h = static_cast<uint16_t*>(ws), a.yr = yr, a.ys = ys, a.ysum = c.ysum;
-  a.bar = reinterpret_cast<int*>(static_cast<uint8_t*>(ws) + ws_h_bytes(L));
-  a.fac = reinterpret_cast<float*>(static_cast<uint8_t*>(ws) + ws_h_bytes(L) + kBarBytes);
-  a.dpart = reinterpret_cast<float*>(static_cast<uint8_t*>(ws) + ws_h_bytes(L) + kBarBytes + kFacBytes);
+  uint8_t* wsb = static_cast<uint8_t*>(ws);
+  a.bar = reinterpret_cast<int*>(wsb + lay.bar_off());
+  a.fac = reinterpret_cast<float*>(wsb + lay.fac_off());
+  a.dpart = reinterpret_cast<float*>(wsb + lay.dpart_off());
   a.spin_limit = 1 << 22;
 #ifdef DSGX_TRACE
   a.trace = g_trace_buf;
@@ -158,15 +183,17 @@ int dsgx_moe_decode(const dsgx_layer_w* L, const uint16_t* x, const int* idx, co
 }
 
 // ---- the barrier's error flag ------------------------------------------------------------------------------------------
+extern "C" {
 int dsgx_decode_status(const dsgx_layer_w* L, void* ws, void* stream) {
   if (!L || L->I <= 0 || L->H <= 0) return fail(DSGX_EINVAL, "decode_status: null or empty layer");
+  WsLayout lay{L->I, L->H};
   if (!ws) {
     void* p = nullptr;
     if (int rc = static_ws(&p)) return rc;
-    ws = p;
+    ws = p, lay = kStaticLayout;
   }
   hipStream_t st = static_cast<hipStream_t>(stream);
-  uint8_t* bar = static_cast<uint8_t*>(ws) + ws_h_bytes(L);
+  uint8_t* bar = static_cast<uint8_t*>(ws) + lay.bar_off();
   int flag = 0;
   DSGX_HIP(hipMemcpyAsync(&flag, bar + (size_t)(2 * kBarGroups + 1) * kBarLine * 4, 4, hipMemcpyDeviceToHost, st));
   DSGX_HIP(hipStreamSynchronize(st));
@@ -186,10 +213,9 @@ int dsgx_moe_decode_noalloc(const dsgx_layer_w* L, const uint16_t* x, const int*
   if (L->I < 1 || L->I > DSGX_NOALLOC_MAX_I || L->H < 1 || L->H > DSGX_NOALLOC_MAX_H)
     return fail(DSGX_EINVAL, "moe_decode_noalloc: hidden %d, intermediate %d exceed the built-in workspace (hidden <= %d, intermediate <= %d); "
                              "use dsgx_moe_decode with a workspace of dsgx_decode_ws_bytes()", L->H, L->I, DSGX_NOALLOC_MAX_H, DSGX_NOALLOC_MAX_I);
-  if (dsgx_decode_ws_bytes(L) > kStaticWsBytes) return fail(DSGX_EINVAL, "moe_decode_noalloc: the layer's workspace exceeds the built-in one");
   void* ws = nullptr;
   if (int rc = static_ws(&ws)) return rc;
-  return dsgx_moe_decode(L, x, idx, w, M, ws, yr, ys, stream, cfg);
+  return moe_decode_at(L, x, idx, w, M, ws, kStaticLayout, yr, ys, stream, cfg);
 }
 
 }  // extern "C"

@@ -740,37 +740,47 @@ constexpr int kBarGroups = 16, kBarLine = 32;
 constexpr size_t kBarBytes = (size_t)(2 * kBarGroups + 2) * kBarLine * 4;
 __device__ __forceinline__ int bar_load(int* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 __device__ __forceinline__ int grid_barrier_gen(int* bar) { return bar_load(bar + (kBarGroups + 1 + blockIdx.x % kBarGroups) * kBarLine); }
+// The two halves, both for one thread of the workgroup, after a workgroup barrier that follows every wave's wait for its own
+// h stores. arrive counts the workgroup in (and, as the very last, releases everyone: it then returns true); wait polls the
+// group's release word. Work placed between the two (the down phase's first loads) overlaps the counters' round trips.
+// (Measured alternatives, all slower: one counter that every waiter polls - the polls delay the arrivals' adds by
+// microseconds; no counter at all, every workgroup polling h itself at the memory side - 256 readers of the same few KiB
+// queue on its memory channels; an extra wave a workgroup that stages h in the background - its loads wait behind the
+// streaming waves' and it saw the first slot whole only when its workgroup's stream had ended.)
+__device__ __forceinline__ bool grid_barrier_arrive(int* bar, int my_gen) {
+  const int g = blockIdx.x % kBarGroups;
+  const int members = ((int)gridDim.x - g + kBarGroups - 1) / kBarGroups;
+  const int groups = min((int)gridDim.x, kBarGroups);
+  int* rel = bar + (kBarGroups + 1) * kBarLine;
+  if (__hip_atomic_fetch_add(bar + g * kBarLine, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == members - 1) {
+    __hip_atomic_store(bar + g * kBarLine, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (__hip_atomic_fetch_add(bar + kBarGroups * kBarLine, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == groups - 1) {
+      __hip_atomic_store(bar + kBarGroups * kBarLine, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      for (int i = 0; i < kBarGroups; ++i) __hip_atomic_store(rel + i * kBarLine, my_gen + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      return true;
+    }
+  }
+  return false;
+}
+__device__ __forceinline__ void grid_barrier_wait(int* bar, int my_gen, int spin_limit) {
+  const int g = blockIdx.x % kBarGroups;
+  int* rel = bar + (kBarGroups + 1) * kBarLine;
+  int spins = 0;
+  while (bar_load(rel + g * kBarLine) == my_gen) {
+    __builtin_amdgcn_s_sleep(8);
+    if (++spins > spin_limit) {
+      __hip_atomic_store(bar + (2 * kBarGroups + 1) * kBarLine, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      break;
+    }
+  }
+}
 __device__ __forceinline__ void grid_barrier(int* bar, int my_gen, int spin_limit) {
   // h was stored with device-scope write-through stores and every wave has waited for its own to complete (the
   // s_waitcnt vmcnt(0) that ends the gate/up phase), so after the workgroup barrier all of this workgroup's h is in
   // memory and no cache write-back or invalidate is needed around the counters (a device-scope fence would flush the
   // whole L2 here)
   __syncthreads();
-  if (threadIdx.x == 0) {
-    const int g = blockIdx.x % kBarGroups;
-    const int members = ((int)gridDim.x - g + kBarGroups - 1) / kBarGroups;
-    const int groups = min((int)gridDim.x, kBarGroups);
-    int* rel = bar + (kBarGroups + 1) * kBarLine;
-    bool released = false;
-    if (__hip_atomic_fetch_add(bar + g * kBarLine, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == members - 1) {
-      __hip_atomic_store(bar + g * kBarLine, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      if (__hip_atomic_fetch_add(bar + kBarGroups * kBarLine, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == groups - 1) {
-        __hip_atomic_store(bar + kBarGroups * kBarLine, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        for (int i = 0; i < kBarGroups; ++i) __hip_atomic_store(rel + i * kBarLine, my_gen + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        released = true;
-      }
-    }
-    if (!released) {
-      int spins = 0;
-      while (bar_load(rel + g * kBarLine) == my_gen) {
-        __builtin_amdgcn_s_sleep(8);
-        if (++spins > spin_limit) {
-          __hip_atomic_store(bar + (2 * kBarGroups + 1) * kBarLine, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          break;
-        }
-      }
-    }
-  }
+  if (threadIdx.x == 0 && !grid_barrier_arrive(bar, my_gen)) grid_barrier_wait(bar, my_gen, spin_limit);
   __syncthreads();
 }
 
@@ -786,7 +796,16 @@ __global__ void __launch_bounds__(DSGX_DECODE_THREADS) k_decode(DecodeArgs a, in
   const int H = a.L.H, GW = gridDim.x * (blockDim.x >> 6), gw = uni((int)(blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)));
   const int rpw = uni((H + GW - 1) / GW);
   const int n_lo = min(H, gw * rpw), n_hi = min(H, n_lo + rpw);
-  down_phase<FMT, SHFMT, M, DSGX_DOWND, RBD>(a, lds, S, spc, n_lo, n_hi, [&] { DSGX_MARK(5); grid_barrier(a.bar, S.gen, a.spin_limit); DSGX_MARK(6); });
+  // the workgroup is counted in before the down phase issues its first loads; it waits for the release after them
+  __shared__ int s_released;
+  __syncthreads();
+  if (threadIdx.x == 0) s_released = grid_barrier_arrive(a.bar, S.gen) ? 1 : 0;
+  down_phase<FMT, SHFMT, M, DSGX_DOWND, RBD>(a, lds, S, spc, n_lo, n_hi, [&] {
+    DSGX_MARK(5);
+    if (threadIdx.x == 0 && !s_released) grid_barrier_wait(a.bar, S.gen, a.spin_limit);
+    __syncthreads();
+    DSGX_MARK(6);
+  });
   DSGX_MARK(8);
 }
 template <int FMT, int SHFMT, int M>
