@@ -38,7 +38,7 @@ def log(*a):
 # HBM bytes a launch of the FP8 M=1 decode kernel (k_decode), from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs of this
 # script, each scaled by what the counter reads for a kernel of known size in the same run (profiles/): the algorithmic
 # bytes are 226,547,712
-LAYER_TRAFFIC_FP8_M1 = 231007642
+LAYER_TRAFFIC_FP8_M1 = 229050000
 
 
 def prefill_extra(gen, T, name, peak, check=True):
@@ -53,8 +53,17 @@ def prefill_extra(gen, T, name, peak, check=True):
              mfma_peak_tflops=peak / 1e12, mfma_frac=pb.flops_routed / t_routed / peak,
              phases_ms={n: pb.time(ph, sh) * 1e3 for n, ph, sh in (("bucket", 1, False), ("up", 2, False), ("down", 4, False),
                                                                       ("combine", 8, False), ("shared", 16, True))})
-    log("  %s T=%d: routed %.3f ms (%.0f TFLOP/s, %.1f%% of %.1f PFLOP/s), with shared %.3f ms" %
-        (name, T, d["ms_routed"], d["tflops_routed"], 100 * d["mfma_frac"], peak / 1e15, d["ms_with_shared"]))
+    # the other roofline: every picked expert's weights once, x in, yr out (a chunk of few rows an expert is bound by these)
+    import torch
+    picked = int((torch.bincount(pb.idx.reshape(-1).long(), minlength=gen.E) > 0).sum())
+    d["algorithmic_bytes_routed"] = picked * gen.expert_bytes + T * gen.H * (2 + 4)
+    d["hbm_bound_ms"] = d["algorithmic_bytes_routed"] / (HBM_PEAK_GBS * 1e9) * 1e3
+    d["mfma_bound_ms"] = pb.flops_routed / peak * 1e3
+    d["hbm_frac"] = d["hbm_bound_ms"] / d["ms_routed"]
+    d["bound"] = "hbm" if d["hbm_bound_ms"] > d["mfma_bound_ms"] else "mfma"
+    log("  %s T=%d: routed %.3f ms (%.0f TFLOP/s, %.1f%% of %.1f PFLOP/s; %.2f GB of weights and rows at least: %.1f%% of 8 TB/s), with shared %.3f ms" %
+        (name, T, d["ms_routed"], d["tflops_routed"], 100 * d["mfma_frac"], peak / 1e15, d["algorithmic_bytes_routed"] / 1e9,
+         100 * d["hbm_frac"], d["ms_with_shared"]))
     if check:
         d["gpu_vs_oracle"] = prefill_check_rows(pb)
         log("  %s: rows %s against the oracle: max-abs %.2e, rel-L2 %.2e" %
@@ -75,7 +84,10 @@ def prefill_check_rows(pb, nrows=4):
     cnt = torch.bincount(pb.idx.reshape(-1).long(), minlength=gen.E).cpu().numpy()
     idx_h = pb.idx.cpu().numpy()
     hot, cold = int(np.argmax(cnt)), int(np.argmin(np.where(cnt > 0, cnt, 1 << 30)))
-    rows = [int(np.nonzero((idx_h == hot).any(1))[0][-1]), int(np.nonzero((idx_h == cold).any(1))[0][0]), 0, T - 1][:nrows]
+    rows = []
+    for t in (int(np.nonzero((idx_h == hot).any(1))[0][-1]), int(np.nonzero((idx_h == cold).any(1))[0][0]), 0, T - 1, T // 2, T // 3):
+        if t not in rows and len(rows) < nrows:
+            rows.append(t)
     worst = dict(rows=rows, max_abs_err=0.0, rel_l2=0.0)
     for t in rows:
         experts = sorted(int(e) for e in idx_h[t])
@@ -173,8 +185,10 @@ def main():
                           "warmup": 1, "ms_per_step": d["ms_routed"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
                           "dtype": "fp8 (e4m3 x e4m3, f32 sums)" if fp8 else "bf16 (INT4 weights decoded to bf16, f32 sums)", "data": "synthetic",
                           "config": {"workload": d["workload"], "T": d["T"]},
-                          "roofline": {"bound": "mfma", "achieved": d["tflops_routed"], "peak": d["mfma_peak_tflops"], "unit": "TFLOP/s",
-                                       "frac": d["mfma_frac"], "traffic": None},
+                          "roofline": ({"bound": "hbm", "achieved": d["algorithmic_bytes_routed"] / d["ms_routed"] * 1e-6, "peak": HBM_PEAK_GBS,
+                                        "unit": "GB/s", "frac": d["hbm_frac"], "traffic": None, "mfma_frac": d["mfma_frac"]} if d["bound"] == "hbm" else
+                                       {"bound": "mfma", "achieved": d["tflops_routed"], "peak": d["mfma_peak_tflops"], "unit": "TFLOP/s",
+                                        "frac": d["mfma_frac"], "traffic": None, "hbm_frac": d["hbm_frac"]}),
                           "cpu_baseline": None, "extra": [d], "wall_s": round(time.time() - t_start, 1)}))
         return
     if args.workload == "gemv":
@@ -251,7 +265,7 @@ def main():
                                ("k_decode" if head_up == 0 else "k_decode_mfma + k_down_combine"),
                      "achieved": r["bytes_per_layer"] / (r["us_per_layer"] * 1e-6) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": r["layer_hbm_frac"], "traffic": LAYER_TRAFFIC_FP8_M1 if head_fp8 and head_up == 0 else None,
-                     "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of an earlier run of this command (profiles/), not measured in this run",
+                     "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of an earlier run of this command (profiles/k_decode_fp8_m1_one_launch.md), not measured in this run",
                      "bytes_per_launch": r["bytes_per_layer"], "avg_launch_us": r["us_per_layer"],
                      "gate_up_kernel_alone": {"kernel": "k_up" if head_up == 0 else "k_up_mfma", "avg_launch_us": r["up_us"],
                                               "bytes_per_launch": r["up_bytes"], "achieved": r["up_gbs"], "frac": r["up_frac"]},

@@ -396,4 +396,21 @@ __device__ __forceinline__ uint32_t swiglu_bits(float g, float u) {
   return f32_to_bf16_bits(__fmul_rn(sl, u));
 }
 
+// The same with the hardware's exponential and reciprocal (each within 1 ulp) in place of expf() and the IEEE division:
+// silu before its rounding to bf16 is within a few f32 ulp of the exact value (the reference's own expf() is specified to
+// 2 ulp), so the bf16 it rounds to differs from swiglu_bits' once in ~10^4 values, by one bf16 step. For the prefill
+// GEMMs' epilogues, where the exact form's ~20 extra instructions a value are a tenth of the kernel.
+__device__ __forceinline__ uint32_t swiglu_fast_bits(float g, float u) {
+  const float e = __builtin_amdgcn_exp2f(__fmul_rn(g, -1.44269504088896341f));
+  const float sl = bf16_round(__fmul_rn(g, __builtin_amdgcn_rcpf(__fadd_rn(1.f, e))));
+  return f32_to_bf16_bits(__fmul_rn(sl, u));
+}
+// v / d by d's reciprocal (r = rcp(d), within 1 ulp) and one correction step: the quotient rounded to nearest for every v
+// and d met here (normal numbers far from the format's ends; the IEEE sequence spends twice the instructions on scaling
+// for the ends). Checked against the division bit for bit in tests.
+__device__ __forceinline__ float div_by(float v, float d, float r) {
+  const float q = __fmul_rn(v, r);
+  return fmaf(fmaf(-q, d, v), r, q);
+}
+
 }  // namespace dsgx

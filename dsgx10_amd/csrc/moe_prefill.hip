@@ -133,7 +133,7 @@ struct TileLists {
   int *ntiles, *tile_e, *tile_m0;     // all rows in 128-position tiles
   int *nbig, *big_e, *big_m0;         // 256-position tiles
   int *nsmall, *small_e, *small_m0;   // the remainders of up to 128 positions
-  int *nmix, *mix_e, *mix_m0;         // both, merged evenly (expert | 1 << 30 for a 256-position tile)
+  int *nmix, *mix_e, *mix_m0;         // both, in expert order (expert | 1 << 30 for a 256-position tile)
 };
 __global__ void __launch_bounds__(DSGX_MAX_EXPERTS) k_pf_scan(const int* __restrict__ bcnt, int NB, int E, int* __restrict__ boff,
                                                               int* __restrict__ cnt, int* __restrict__ off, TileLists tl) {
@@ -167,18 +167,15 @@ __global__ void __launch_bounds__(DSGX_MAX_EXPERTS) k_pf_scan(const int* __restr
     if (nsmall) tl.small_e[sd[e] - 1] = e, tl.small_m0[sd[e] - 1] = (c / 256) * 256;
   }
   __syncthreads();
-  // The merged list: the small tiles (they mostly stream an expert's weights) spread evenly among the big ones (they
-  // mostly multiply), each kind in expert order: entry i of the small list goes in after floor(i nb / ns) big ones.
   const int nb = sc[DSGX_MAX_EXPERTS - 1], nsm = sd[DSGX_MAX_EXPERTS - 1];
-  __threadfence_block();
-  for (int i = e; i < nb; i += DSGX_MAX_EXPERTS) {
-    // small entries before big entry i: those j with floor(j nb / nsm) <= i, j < nsm
-    const int before = nsm ? min(nsm, (int)(((long)(i + 1) * nsm + nb - 1) / nb)) : 0;
-    tl.mix_e[i + before] = tl.big_e[i] | (1 << 30), tl.mix_m0[i + before] = tl.big_m0[i];
-  }
-  for (int j = e; j < nsm; j += DSGX_MAX_EXPERTS) {
-    const int before = (int)((long)j * nb / nsm);  // big entries before small entry j
-    tl.mix_e[j + before] = tl.small_e[j], tl.mix_m0[j + before] = tl.small_m0[j];
+  // The merged list, in expert order: an expert's 256-position tiles, then its remainder. Neighbours in the list run at
+  // about the same time on one XCD (pf8::task_of), so part of what an expert's tiles stream, each in full, comes out of
+  // that XCD's L2: 12% fewer bytes from HBM for gate/up, 19% for down, than with the remainders spread evenly among the
+  // big tiles (measured; the time differs by 1% only: the stream is not what bounds these launches).
+  if (e < E) {
+    const int p0 = (sc[e] - nbig) + (sd[e] - nsmall);
+    for (int i = 0; i < nbig; ++i) tl.mix_e[p0 + i] = e | (1 << 30), tl.mix_m0[p0 + i] = i * 256;
+    if (nsmall) tl.mix_e[p0 + nbig] = e, tl.mix_m0[p0 + nbig] = (c / 256) * 256;
   }
   if (e == 0) *tl.nmix = nb + nsm;
 }
@@ -677,7 +674,7 @@ int dsgx_moe_prefill(const dsgx_layer_w* L, const uint16_t* x, const int* idx, c
     const char* dv = std::getenv("DSGX_PF_DIAG");
     switch (dv ? std::atoi(dv) : 0) {
 #define DSGX_DIAG_CASE(n) case n: k_up = pf8::k_gemm_mixed<true, n>, k_dn = pf8::k_gemm_mixed<false, n>, k_up2 = pf8::k_gemm<true, 2, n>, k_dn2 = pf8::k_gemm<false, 2, n>; break;
-      DSGX_DIAG_CASE(1) DSGX_DIAG_CASE(2) DSGX_DIAG_CASE(4) DSGX_DIAG_CASE(8) DSGX_DIAG_CASE(16) DSGX_DIAG_CASE(3) DSGX_DIAG_CASE(9) DSGX_DIAG_CASE(25)
+      DSGX_DIAG_CASE(1) DSGX_DIAG_CASE(2) DSGX_DIAG_CASE(4) DSGX_DIAG_CASE(8) DSGX_DIAG_CASE(16) DSGX_DIAG_CASE(3) DSGX_DIAG_CASE(9) DSGX_DIAG_CASE(25) DSGX_DIAG_CASE(32) DSGX_DIAG_CASE(64)
 #undef DSGX_DIAG_CASE
     }
   }
