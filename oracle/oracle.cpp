@@ -10,8 +10,10 @@
 // pinned by closed forms, exhaustive checks, torch-CPU library routines and brute force in tests/test_oracle_*.py, and
 // orc_moe_prefill_fp8_row also by vectors from the reference's own torch kernels (tests/golden/prefill_fp8_expert.npz).
 //
-// Pinned: bf16 RNE, e4m3 decode/encode, INT4 dequant, FP8 quantiser and dequant, act_quant, router, union,
-// GEMV and MoE sums (f32 contract order, f64 and sum of |terms|). Parity unpinned: none of the functions here; the
+// Pinned: bf16 RNE, e4m3 decode/encode, INT4 dequant, FP8 quantiser and dequant, act_quant, router (the sigmoid and the
+// sqrt-softplus score, ids, ties, the weights' sum order), union, GEMV and MoE sums (f32 contract order, f64 and sum of
+// |terms|), the FP8-activation prefill row and the range it allows for h, the residual add + RMSNorm (orc_add_norm: against
+// torch's bf16 ops, with two negative controls). Parity unpinned: none of the functions here; the
 // INT4 *quantiser* (orc_int4_quantize_sym) has no reference counterpart at all (the reference never quantises INT4)
 // and is this build's own definition.
 //
