@@ -116,7 +116,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=64)
     ap.add_argument("--no-extra", action="store_true", help="only the headline workload")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
-    ap.add_argument("--workload", default="fp8_m1", help="headline workload: fp8_m1 | int4_m1; fp8_prefill | int4_prefill time only that prefill chunk; gemv only the dense GEMVs")
+    ap.add_argument("--workload", default="fp8_m1", help="headline workload: fp8_m1 | int4_m1; fp8_prefill | int4_prefill time only that prefill chunk; gemv only the dense GEMVs; chain only the layer chains")
     ap.add_argument("--variant", default="vector", choices=("vector", "mfma"),
                     help="the headline's decode kernels (dsgx_decode_cfg::up = 0 | 1); --no-extra then runs nothing else")
     args = ap.parse_args()
@@ -191,6 +191,20 @@ def main():
                                         "frac": d["mfma_frac"], "traffic": None, "hbm_frac": d["hbm_frac"]}),
                           "cpu_baseline": None, "extra": [d], "wall_s": round(time.time() - t_start, 1)}))
         return
+    if args.workload == "chain":
+        # only the layer chains (router GEMV -> experts -> add + norm, 128 layers a graph), FP8 then INT4
+        from dsgx10_amd.benchdata import ChainBench
+        ds = []
+        for cls in (Fp8LayerGen, Int4LayerGen):
+            g2 = cls(seed=0)
+            ds.append(ChainBench(g2, 1, 128).time())
+            log("  %s M=1: %.2f us a layer" % (ds[-1]["workload"], ds[-1]["us_per_layer"]))
+            del g2
+        print(json.dumps({"metric": "us_per_moe_layer_step", "value": ds[0]["us_per_layer"], "unit": "us", "n_gpus": 1, "steps": 128, "warmup": 4,
+                          "ms_per_step": ds[0]["us_per_layer"] * 1e-3, "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+                          "dtype": "f32 sums of bf16 x bf16 products", "data": "synthetic", "config": {"workload": ds[0]["workload"], "rows_M": 1},
+                          "roofline": None, "cpu_baseline": None, "extra": ds, "wall_s": round(time.time() - t_start, 1)}))
+        return
     if args.workload == "gemv":
         # only the dense GEMVs (for profiler runs): one line, the FP8 [2048 x 4096] row-1 call as the value
         from dsgx10_amd.benchdata import gemv_bench
@@ -235,8 +249,14 @@ def main():
                 extra.append(d)
                 del ob
         extra.append(prefill_extra(other, 2048, "int4_moe_prefill", 2.5e15, not args.no_cpu) if head_fp8 else prefill_extra(other, 8192, "fp8_moe_prefill", 5.0e15, not args.no_cpu))
+        from dsgx10_amd.benchdata import ChainBench, gemv_bench
+        for g2 in (gen, other):
+            cb = ChainBench(g2, 1, 128)
+            d = cb.time()
+            log("  %s M=1: %.2f us a layer (router GEMV + experts + add/norm, %d layers in one graph)" % (d["workload"], d["us_per_layer"], d["layers"]))
+            extra.append(d)
+            del cb
         del other
-        from dsgx10_amd.benchdata import gemv_bench
         extra += gemv_bench()
 
     out = {

@@ -290,6 +290,69 @@ class DecodeBench:
                     experts=experts)
 
 
+class ChainBench:
+    """The MoE half of a decode step as the reference's runner chains it (model.cu:309-343), layer after layer in one graph:
+    the router's logits by the BF16 GEMV (f32 out, K over 4 waves) from the normed row, the experts with the routing, the
+    shared expert and yr += ys fused in one launch, then the residual add and the next layer's RMSNorm, whose output is the
+    next layer's input. Every layer has its own router matrix and norm weight (rotating over copies that exceed the caches)
+    and routes by its own data, so the experts differ from layer to layer."""
+
+    def __init__(self, gen, M, layers, seed=99, up=-1):
+        self.gen, self.M, self.layers, self.up = gen, M, layers, up
+        g = torch.Generator(device="cuda")
+        g.manual_seed(seed)
+        H, E = gen.H, gen.E
+        self.nr = max(8, int(600e6 // (E * H * 2)))
+        self.router = [(torch.randn(E, H, generator=g, device="cuda") * 0.05).to(torch.bfloat16) for _ in range(self.nr)]
+        self.normw = [(1.0 + 0.1 * torch.randn(H, generator=g, device="cuda")).to(torch.bfloat16) for _ in range(self.nr)]
+        self.x0 = torch.randn(M, H, generator=g, device="cuda").to(torch.bfloat16)
+        self.xn = [torch.zeros(M, H, dtype=torch.bfloat16, device="cuda") for _ in range(2)]
+        self.res = torch.zeros(M, H, dtype=torch.bfloat16, device="cuda")
+        self.logits = torch.zeros(M, E, dtype=torch.float32, device="cuda")
+        self.yr = torch.zeros(M, H, dtype=torch.float32, device="cuda")
+        self.ys = torch.zeros(M, H, dtype=torch.float32, device="cuda")
+        self.lw = [gen.layer_w(c) for c in range(gen.NSH)]
+        self.ws = torch.zeros(lib.decode_ws_bytes(self.lw[0]), dtype=torch.uint8, device="cuda")
+
+    def layer(self, l):
+        g, M = self.gen, self.M
+        x, xo = self.xn[l & 1], self.xn[(l + 1) & 1]
+        seg = dict(fmt=abi.FMT_BF16, w=self.router[l % self.nr], s=None, zp=None, n=g.E, y=self.logits, ldy=g.E)
+        lib.gemv(x, g.H, M, g.H, [seg], abi.OUT_F32, splitk=4)
+        lib.moe_decode(self.lw[l % g.NSH], x, None, None, M, self.ws, self.yr, self.ys, logits=self.logits, route_scale=g.route_scale,
+                       ysum=True, up=self.up)
+        lib.add_norm(self.yr, None, M, g.H, self.res, self.res, self.normw[l % self.nr], 1e-5, xo)
+
+    def time(self):
+        def run():
+            for l in range(self.layers):
+                self.layer(l)
+        self.xn[0].copy_(self.x0)
+        self.res.zero_()
+        for l in range(4):
+            self.layer(l)
+        torch.cuda.synchronize()
+        self.xn[0].copy_(self.x0)
+        self.res.zero_()
+        gr = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(gr):
+            run()
+        gr.replay()
+        torch.cuda.synchronize()
+        self.xn[0].copy_(self.x0)
+        self.res.zero_()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        gr.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        lib.decode_status(self.lw[0], self.ws)
+        finite = bool(torch.isfinite(self.xn[self.layers & 1].float()).all())
+        return dict(workload=self.gen.name.replace("decode", "layer_chain"), M=self.M, layers=self.layers,
+                    launches_per_layer=["k_gemv_sk (router logits, f32, K over 4)", "k_decode / k_decode_mfma (+ its ordered sum)", "k_add_norm"],
+                    us_per_layer=e0.elapsed_time(e1) * 1e3 / self.layers, outputs_finite=finite)
+
+
 def gemv_bench(reps=64):
     """the two dense GEMV configurations: FP8 [2048 x 4096] at 1 row, INT4 [1536 x 6144] at 1, 2, 4, 6 rows, and the router's
     logits (BF16 [E x H], f32 out, 1 row), each with K unsplit and split over 2 and 4 waves; weights rotate over copies that
