@@ -335,7 +335,7 @@ __device__ __forceinline__ void mf_up_phase(Step<M>& S, const DecodeArgs& a, uin
   // Units are (slot, tile of 8 channels), numbered slot-major; workgroup g of G walks the units g, g + G, g + 2 G, ...
   // (with as many tiles a slot as workgroups that is one tile of every slot; with fewer, a narrow intermediate size, the
   // workgroups still share the slots' tiles evenly)
-  const int tiles = I / 8, g = blockIdx.x, G = gridDim.x;
+  const int tiles = I / 8;
   auto done = [&](int sl, int t, v4f_t sum) {
     const int pos = lane & 15, part = lane >> 4;
     if (pos >= M) return;
@@ -346,7 +346,7 @@ __device__ __forceinline__ void mf_up_phase(Step<M>& S, const DecodeArgs& a, uin
     uint16_t* dst = a.h + ((size_t)T.hslot * M + pos) * I + 8 * t + 2 * part;
     __hip_atomic_store((DSGX_GLOBAL uint32_t*)(uintptr_t)dst, h0 | (h1 << 16), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   };
-  auto run = [&](auto fmt_tag, int s0, int nslots) {  // slots s0 .. s0 + nslots - 1 in format F
+  auto run = [&](auto fmt_tag, int s0, int nslots, int g, int G) {  // slots s0 .. s0 + nslots - 1 in format F, by workgroup g of G
     constexpr int F = decltype(fmt_tag)::value;
     const int total = nslots * tiles;
     const int mine = uni(g < total ? (total - g + G - 1) / G : 0);  // this workgroup's units
@@ -364,12 +364,22 @@ __device__ __forceinline__ void mf_up_phase(Step<M>& S, const DecodeArgs& a, uin
                     [](int) { return 0u; }, fin, [] {});
   };
   const int nrouted = uni(S.n);
+  const int G = gridDim.x, g = blockIdx.x;
   if constexpr (SHFMT != 0 && SHFMT != FMT) {
-    run(std::integral_constant<int, SHFMT>{}, 0, 1);
-    __syncthreads();
-    if (nrouted > 0) run(std::integral_constant<int, FMT>{}, 1, nrouted);
+    // The shared slot in its own format: the first workgroups take it, the others the routed slots, both at once, so that a
+    // stream that waits for memory (BF16) and one that waits for the vector unit (INT4) share the chip instead of taking
+    // turns. The split goes by bytes, a routed byte counted kShCost times (its stream is that much slower a byte).
+#ifndef DSGX_MF_SHCOST
+#define DSGX_MF_SHCOST 2.0f
+#endif
+    constexpr float kShCost = DSGX_MF_SHCOST;
+    auto bpv = [](int f) { return f == DSGX_FMT_BF16 ? 2.f : f == DSGX_FMT_FP8_B128 ? 1.f : 0.5703f; };  // bytes a value
+    const float bsh = bpv(SHFMT), bro = kShCost * (float)nrouted * bpv(FMT);
+    const int nshw = uni(nrouted > 0 ? max(1, min(G - 1, (int)((float)G * bsh / (bsh + bro) + 0.5f))) : G);
+    if (g < nshw) run(std::integral_constant<int, SHFMT>{}, 0, 1, g, nshw);
+    else run(std::integral_constant<int, FMT>{}, 1, nrouted, g - nshw, G - nshw);
   } else {
-    if (nsh + nrouted > 0) run(std::integral_constant<int, FMT>{}, 0, nsh + nrouted);
+    if (nsh + nrouted > 0) run(std::integral_constant<int, FMT>{}, 0, nsh + nrouted, g, G);
   }
   // the wave's h stores are complete before it goes on to the grid barrier (see up_phase)
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
