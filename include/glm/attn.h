@@ -1,6 +1,6 @@
 // glm:: - the dense GEMV operators with the reference engine's names and argument order
 // (altar1-4xgx10-switchless/engine/attn/attn.h:59-158), forwarding to the C ABI in dsgx.h. Only the weight-streaming
-// GEMV and dequant_int4 are on this build's path; the attention side of attn.h is not mirrored.
+// GEMV, its many-row form gemm() and dequant_int4 are on this build's path; the attention side of attn.h is not mirrored.
 #pragma once
 #include <cstddef>
 #include <cstdint>
@@ -45,6 +45,36 @@ inline void gemv(const uint16_t* x, int ldx, int rows, int K, const GemvSeg* seg
     g[i].zp = a.zp, g[i].n = a.n, g[i].rs = a.rs, g[i].ks = a.ks, g[i].y = a.y, g[i].ldy = a.ldy;
   }
   DSGX_DIE_ON(dsgx_gemv(x, ldx, rows, K, g, nseg, (int)out, splitk, st));
+}
+// attn.h:141-157: the GEMM for prefill chunks (any number of rows), "every output equals gemv()'s at the same splitk bit
+// for bit". Here that holds by construction: the rows go through gemv() sixteen at a time (the weights are read once a
+// group of sixteen rows; a tiled MFMA GEMM for long chunks is the FP8 / INT4 prefill path of gx::moe_prefill, not this).
+// scratch (the reference's INT4 staging buffer) is not needed and ignored.
+inline void gemm(const uint16_t* x, int ldx, int rows, int K, const GemvSeg* segs, int nseg, GemvOut out, int splitk, void* st,
+                 bool pdl = false, uint16_t* scratch = nullptr, size_t scratch_elems = 0) {
+  (void)scratch, (void)scratch_elems;
+  if (nseg < 1 || nseg > kMaxSegs) die("gemm: K %d, %d segments", K, nseg);
+  const size_t esz = out == GemvOut::kF32 ? 4 : 2;
+  for (int r0 = 0; r0 < rows; r0 += kMaxRows) {
+    GemvSeg g[kMaxSegs];
+    for (int i = 0; i < nseg; ++i) {
+      g[i] = segs[i];
+      g[i].y = static_cast<uint8_t*>(segs[i].y) + (size_t)r0 * segs[i].ldy * esz;
+    }
+    gemv(x + (size_t)r0 * ldx, ldx, rows - r0 < kMaxRows ? rows - r0 : kMaxRows, K, g, nseg, out, splitk, st, pdl);
+  }
+}
+// attn.h:150-152: BF16 weights only (the router, the head): every segment taken as BF16 (kNone allowed)
+inline void gemm_bf16(const uint16_t* x, int ldx, int rows, int K, const GemvSeg* segs, int nseg, GemvOut out, int splitk, void* st,
+                      bool pdl = false) {
+  if (nseg < 1 || nseg > kMaxSegs) die("gemm_bf16: K %d, %d segments", K, nseg);
+  GemvSeg g[kMaxSegs];
+  for (int i = 0; i < nseg; ++i) {
+    g[i] = segs[i];
+    if (g[i].fmt != WFmt::kNone && g[i].fmt != WFmt::kBF16) die("gemm_bf16: segment %d is not BF16", i);
+    g[i].fmt = WFmt::kBF16;
+  }
+  gemm(x, ldx, rows, K, g, nseg, out, splitk, st, pdl);
 }
 // attn.h:154-158 (row-major output only; the tiled form is a GB10 layout)
 inline void dequant_int4(const void* packed, const void* scale, const void* zp, int N, int K, uint16_t* out, size_t ld, void* st,

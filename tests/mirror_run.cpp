@@ -115,7 +115,7 @@ int main(int argc, char** argv) {
     seg.fmt = L.sh.g ? glm::WFmt::kFP8 : glm::WFmt::kBF16;
     seg.w = L.sh.g ? static_cast<const void*>(L.sh.g) : static_cast<const void*>(L.sh.bgu);
     seg.s = L.sh.gs, seg.n = gn, seg.y = gv, seg.ldy = gn;
-    glm::gemv(x, H, M, H, &seg, 1, glm::GemvOut::kF32, 4, st);
+    glm::gemm(x, H, M, H, &seg, 1, glm::GemvOut::kF32, 4, st);  // (gemm() forwards its rows to gemv() sixteen at a time)
   }
   // the step's end (model.cu:343): h = bf16(resid16 + yr2) in place, xn = the next layer's RMSNorm of h
   uint16_t* res16 = static_cast<uint16_t*>(upload(slurp(dir + "res16.bin")));
