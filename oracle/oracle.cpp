@@ -13,7 +13,9 @@
 // Pinned: bf16 RNE, e4m3 decode/encode, INT4 dequant, FP8 quantiser and dequant, act_quant, router (the sigmoid and the
 // sqrt-softplus score, ids, ties, the weights' sum order), union, GEMV and MoE sums (f32 contract order, f64 and sum of
 // |terms|), the FP8-activation prefill row and the range it allows for h, the residual add + RMSNorm (orc_add_norm: against
-// torch's bf16 ops, with two negative controls). Parity unpinned: none of the functions here; the
+// torch's bf16 ops, with two negative controls), DeepSeek's MXFP4 x FP8 expert (codecs by closed forms, the scale byte by
+// brute force against f64 logarithms, the expert by vectors from the reference's torch kernels:
+// tests/golden/dsk_mxfp4_expert.npz). Parity unpinned: none of the functions here; the
 // INT4 *quantiser* (orc_int4_quantize_sym) has no reference counterpart at all (the reference never quantises INT4)
 // and is this build's own definition.
 //
@@ -703,6 +705,128 @@ ORC void orc_add_norm(const float* part, const float* part2, int M, int H, const
       for (int n = 0; n < H; ++n) out[(size_t)m * H + n] = f2bf(bf2f(w[n]) * bfr(h[n] * rstd));
     }
   }
+}
+
+// ---- DeepSeek's MXFP4 x FP8 decode MoE (D/engine/kernels/moe.cu, D/ref/inference/model.py:841-851, D/ref/torchref/kernel.py) --
+// e2m1: sign, two exponent bits, one mantissa bit (OCP MX): 0, 0.5, 1, 1.5, 2, 3, 4, 6 (D/ref/torchref/kernel.py:38-52's grid)
+ORC float orc_e2m1_value(int c) {
+  static const float mag[8] = {0.f, 0.5f, 1.f, 1.5f, 2.f, 3.f, 4.f, 6.f};
+  return (c & 8) ? -mag[c & 7] : mag[c & 7];
+}
+// ue8m0 byte -> 2^(b - 127) (D/engine/kernels/common.cuh:50-51; b >= 1)
+ORC float orc_ue8m0_value(int b) { return ldexpf(1.f, b - 127); }
+// The per-32 activation scale byte: 2^ceil(log2(amax / 448)) with amax clamped at 1e-4, from the f32 bits
+// (D/engine/kernels/common.cuh:53-60; D/ref/torchref/kernel.py:19-27 fast_round_scale)
+ORC int orc_act_scale_byte(float amax) {
+  const float v = std::max(amax, 1e-4f) * (1.0f / 448.0f);
+  uint32_t b;
+  memcpy(&b, &v, 4);
+  return (int)((b >> 23) & 0xFF) + ((b & 0x7FFFFF) != 0);
+}
+// act_quant with ue8m0 scales per 32 values (D/ref/torchref/kernel.py:56-78 with block 32 and scale_fmt set;
+// D/engine/kernels/common.cuh:62-66): q = e4m3_rne(clamp(x * 2^(127 - e), +-448))
+ORC void orc_act_quant_ue8m0(const uint16_t* x, int T, int K, uint8_t* q, uint8_t* s) {
+  const int KB = K / 32;
+  for (int t = 0; t < T; ++t)
+    for (int b = 0; b < KB; ++b) {
+      const uint16_t* p = x + (size_t)t * K + 32 * b;
+      float amax = 0.f;
+      for (int i = 0; i < 32; ++i) amax = std::max(amax, fabsf(bf2f(p[i])));
+      const int e = orc_act_scale_byte(amax);
+      s[(size_t)t * KB + b] = (uint8_t)e;
+      const float inv = ldexpf(1.f, 127 - e);
+      for (int i = 0; i < 32; ++i) q[(size_t)t * K + 32 * b + i] = f2e4m3(std::min(448.f, std::max(-448.f, bf2f(p[i]) * inv)));
+    }
+}
+// e4m3 codes with ue8m0 scales per 32 -> the values (exact in f32, and in bf16)
+ORC void orc_dequant_act_ue8m0(const uint8_t* q, const uint8_t* s, int T, int K, float* out) {
+  for (int t = 0; t < T; ++t)
+    for (int k = 0; k < K; ++k) out[(size_t)t * K + k] = e4m3f(q[(size_t)t * K + k]) * orc_ue8m0_value(s[(size_t)t * (K / 32) + k / 32]);
+}
+// MXFP4 weights: w u8 [N][K/2] (two e2m1, the low nibble the even k), s ue8m0 [N][K/32] -> f32 [N][K] (exact)
+// (D/ref/torchref/kernel.py:111-117 dequant_fp4_weight; D/engine/kernels/README.md L3's source form)
+ORC void orc_mxfp4_dequant(const uint8_t* w, const uint8_t* s, int N, int K, float* out) {
+  for (int n = 0; n < N; ++n)
+    for (int k = 0; k < K; ++k) {
+      const uint8_t b = w[(size_t)n * (K / 2) + k / 2];
+      out[(size_t)n * K + k] = orc_e2m1_value((k & 1) ? b >> 4 : b & 15) * orc_ue8m0_value(s[(size_t)n * (K / 32) + k / 32]);
+    }
+}
+// FP8 weights with ue8m0 scales per 32 x 32 block (the shared expert: D/engine/kernels/README.md L1; kernel.py:105-108)
+ORC void orc_fp8e_dequant(const uint8_t* w, const uint8_t* s, int N, int K, float* out) {
+  for (int n = 0; n < N; ++n)
+    for (int k = 0; k < K; ++k) out[(size_t)n * K + k] = e4m3f(w[(size_t)n * K + k]) * orc_ue8m0_value(s[(size_t)(n / 32) * (K / 32) + k / 32]);
+}
+// One expert's gate/up for M rows from dequantised weights w1, w3 f32 [I][H] and dequantised activations xd f32 [M][H]
+// (D/engine/kernels/moe.cu:519-528; model.py:841-850): gt = bf16(sum), up = bf16(sum), up clamped to +-limit, gt to <= limit,
+// h = gt / (1 + exp(-gt)) * up, routed: h = rw * h; hpre = bf16(h). h32: from f32 sums in k order; h64: from f64 sums;
+// lo / hi: the range when each sum moves by sum_tol * its sum of |terms|. rw null: the shared expert.
+static inline float dsk_h(float gs, float us, float limit, const float* rw) {
+  float gt = bfr(gs), up = bfr(us);
+  up = std::min(std::max(up, -limit), limit);
+  gt = std::min(gt, limit);
+  float h = gt / (1.0f + expf(-gt)) * up;
+  if (rw) h = *rw * h;
+  return bfr(h);
+}
+ORC void orc_dsk_up(const float* w1, const float* w3, const float* xd, int M, int H, int I, const float* rw, float limit, double sum_tol,
+                    uint16_t* h32, uint16_t* h64, float* lo, float* hi) {
+#pragma omp parallel for schedule(static)
+  for (int c = 0; c < I; ++c)
+    for (int m = 0; m < M; ++m) {
+      float gf = 0.f, uf = 0.f;
+      double gd = 0, ud = 0, gm = 0, um = 0;
+      for (int k = 0; k < H; ++k) {
+        const float x = xd[(size_t)m * H + k], a = w1[(size_t)c * H + k], b = w3[(size_t)c * H + k];
+        gf += a * x, uf += b * x;
+        gd += (double)a * x, ud += (double)b * x, gm += fabs((double)a * x), um += fabs((double)b * x);
+      }
+      const size_t i = (size_t)m * I + c;
+      const float* r = rw ? rw + m : nullptr;
+      if (h32) h32[i] = f2bf(dsk_h(gf, uf, limit, r));
+      const float hv = dsk_h((float)gd, (float)ud, limit, r);
+      if (h64) h64[i] = f2bf(hv);
+      if (lo || hi) {
+        float l = hv, hh = hv;
+        const double g0 = gd - sum_tol * gm, g1 = gd + sum_tol * gm, u0 = ud - sum_tol * um, u1 = ud + sum_tol * um;
+        const double gs[3] = {g0, g1, std::min(std::max(-1.2785, g0), g1)};  // (silu's minimum lies at -1.2785)
+        const double us[3] = {u0, u1, std::min(std::max(0.0, u0), u1)};
+        for (double gg : gs)
+          for (double uu : us) {
+            const float v = dsk_h((float)gg, (float)uu, limit, r);
+            l = std::min(l, v), hh = std::max(hh, v);
+          }
+        if (lo) lo[i] = l;
+        if (hi) hi[i] = hh;
+      }
+    }
+}
+// The expert's w2 from a given hpre bf16 [M][I] (moe.cu:529-534, 974-981): h quantised per 32 (e4m3, ue8m0), dotted with the
+// dequantised w2 f32 [H][I]; out32 the f32 sums in k order, out64 / mag the f64 sums and sums of |terms|; outb the bf16 the
+// fold adds (from the f32 sums). hq, hs receive the quantised h (may be null).
+ORC void orc_dsk_down(const float* w2, const uint16_t* hpre, int M, int H, int I, uint8_t* hq, uint8_t* hs, float* out32, double* out64,
+                      double* mag, uint16_t* outb) {
+  std::vector<uint8_t> q((size_t)M * I), sc((size_t)M * (I / 32));
+  orc_act_quant_ue8m0(hpre, M, I, q.data(), sc.data());
+  if (hq) memcpy(hq, q.data(), q.size());
+  if (hs) memcpy(hs, sc.data(), sc.size());
+  std::vector<float> hd((size_t)M * I);
+  orc_dequant_act_ue8m0(q.data(), sc.data(), M, I, hd.data());
+#pragma omp parallel for schedule(static)
+  for (int n = 0; n < H; ++n)
+    for (int m = 0; m < M; ++m) {
+      float f = 0.f;
+      double d = 0, a = 0;
+      for (int k = 0; k < I; ++k) {
+        const float w = w2[(size_t)n * I + k], h = hd[(size_t)m * I + k];
+        f += w * h, d += (double)w * h, a += fabs((double)w * h);
+      }
+      const size_t i = (size_t)m * H + n;
+      if (out32) out32[i] = f;
+      if (out64) out64[i] = d;
+      if (mag) mag[i] = a;
+      if (outb) outb[i] = f2bf(f);
+    }
 }
 
 ORC int orc_threads() { return omp_get_max_threads(); }

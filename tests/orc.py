@@ -268,3 +268,76 @@ def set_f32_only(on):
 
 def threads():
     return lib().orc_threads()
+
+
+# ---- DeepSeek's MXFP4 x FP8 expert ---------------------------------------------------------------------------------------
+def e2m1_table():
+    lib().orc_e2m1_value.restype = C.c_float
+    return np.array([lib().orc_e2m1_value(i) for i in range(16)], np.float32)
+
+
+def ue8m0_value(b):
+    lib().orc_ue8m0_value.restype = C.c_float
+    return lib().orc_ue8m0_value(int(b))
+
+
+def act_scale_byte(amax):
+    return lib().orc_act_scale_byte(C.c_float(amax))
+
+
+def act_quant_ue8m0(x):
+    """x bf16 bits [T][K] -> (e4m3 codes u8 [T][K], ue8m0 bytes u8 [T][K/32])"""
+    x = np.ascontiguousarray(x, np.uint16)
+    T, K = x.shape
+    q, s = np.empty((T, K), np.uint8), np.empty((T, K // 32), np.uint8)
+    lib().orc_act_quant_ue8m0(_p(x), T, K, _p(q), _p(s))
+    return q, s
+
+
+def dequant_act_ue8m0(q, s):
+    q, s = np.ascontiguousarray(q, np.uint8), np.ascontiguousarray(s, np.uint8)
+    T, K = q.shape
+    o = np.empty((T, K), np.float32)
+    lib().orc_dequant_act_ue8m0(_p(q), _p(s), T, K, _p(o))
+    return o
+
+
+def mxfp4_dequant(w, s):
+    """w u8 [N][K/2], s ue8m0 [N][K/32] -> f32 [N][K]"""
+    w, s = np.ascontiguousarray(w, np.uint8), np.ascontiguousarray(s, np.uint8)
+    N, K = w.shape[0], w.shape[1] * 2
+    o = np.empty((N, K), np.float32)
+    lib().orc_mxfp4_dequant(_p(w), _p(s), N, K, _p(o))
+    return o
+
+
+def fp8e_dequant(w, s):
+    """e4m3 codes u8 [N][K], ue8m0 [N/32][K/32] -> f32 [N][K]"""
+    w, s = np.ascontiguousarray(w, np.uint8), np.ascontiguousarray(s, np.uint8)
+    N, K = w.shape
+    o = np.empty((N, K), np.float32)
+    lib().orc_fp8e_dequant(_p(w), _p(s), N, K, _p(o))
+    return o
+
+
+def dsk_up(w1, w3, xd, rw=None, limit=10.0, sum_tol=2e-5, want_range=True):
+    """dequantised w1, w3 f32 [I][H], xd f32 [M][H], rw f32 [M] or None (the shared expert) -> dict h32, h64 (bf16 bits), lo, hi"""
+    w1, w3, xd = (np.ascontiguousarray(a, np.float32) for a in (w1, w3, xd))
+    I, H = w1.shape
+    M = xd.shape[0]
+    r = None if rw is None else np.ascontiguousarray(rw, np.float32)
+    h32, h64 = np.empty((M, I), np.uint16), np.empty((M, I), np.uint16)
+    lo, hi = (np.empty((M, I), np.float32), np.empty((M, I), np.float32)) if want_range else (None, None)
+    lib().orc_dsk_up(_p(w1), _p(w3), _p(xd), M, H, I, _p(r), C.c_float(limit), C.c_double(sum_tol), _p(h32), _p(h64), _p(lo), _p(hi))
+    return dict(h32=h32, h64=h64, lo=lo, hi=hi)
+
+
+def dsk_down(w2, hpre):
+    """dequantised w2 f32 [H][I], hpre bf16 bits [M][I] -> dict hq, hs, out32, out64, mag, outb (bf16 bits)"""
+    w2, hpre = np.ascontiguousarray(w2, np.float32), np.ascontiguousarray(hpre, np.uint16)
+    H, I = w2.shape
+    M = hpre.shape[0]
+    o = dict(hq=np.empty((M, I), np.uint8), hs=np.empty((M, I // 32), np.uint8), out32=np.empty((M, H), np.float32),
+             out64=np.empty((M, H), np.float64), mag=np.empty((M, H), np.float64), outb=np.empty((M, H), np.uint16))
+    lib().orc_dsk_down(_p(w2), _p(hpre), M, H, I, _p(o["hq"]), _p(o["hs"]), _p(o["out32"]), _p(o["out64"]), _p(o["mag"]), _p(o["outb"]))
+    return o
