@@ -3,6 +3,7 @@ import ctypes as C
 
 FMT_REF_NVFP4, FMT_REF_INT4, FMT_REF_BF16 = 0, 2, 3
 FMT_FP8, FMT_INT4, FMT_BF16 = 16, 18, 19
+FMT_MXFP4, FMT_FP8E = 20, 21  # DeepSeek's routed experts; their shared expert (ue8m0 scales per 32 x 32)
 OUT_BF16, OUT_F32, OUT_SWIGLU = 0, 1, 2
 MAX_ROWS, MAX_TOPK, MAX_UNION, SH_SLOT, MAX_EXPERTS, MAX_CHUNK = 16, 8, 128, 128, 512, 8192
 OK, EINVAL, EFORMAT, EUNSUPPORTED, EHIP, ETIMEOUT = 0, 1, 2, 3, 4, 5
@@ -20,6 +21,10 @@ class SharedW(C.Structure):
 class LayerW(C.Structure):
     _fields_ = [("pool", C.c_void_p), ("desc", C.c_void_p), ("sh", SharedW), ("fmt", C.c_uint32),
                 ("H", C.c_int32), ("I", C.c_int32), ("E", C.c_int32), ("topk", C.c_int32)]
+
+
+class DskCfg(C.Structure):
+    _fields_ = [("swiglu_limit", C.c_float), ("logits", C.c_void_p), ("bias", C.c_void_p), ("route_scale", C.c_float), ("parts", C.c_int32)]
 
 
 class DecodeCfg(C.Structure):
@@ -46,7 +51,7 @@ assert C.sizeof(MatDesc) == 64
 # every symbol include/dsgx.h declares
 SYMBOLS = [
     "dsgx_mat_bytes", "dsgx_mat_scale_off", "dsgx_mat_zp_off", "dsgx_route", "dsgx_decode_cfg_default",
-    "dsgx_decode_ws_bytes", "dsgx_decode_ws_flag_offset", "dsgx_decode_status", "dsgx_moe_decode", "dsgx_moe_decode_noalloc", "dsgx_finalize", "dsgx_add_norm", "dsgx_prefill_cfg_default", "dsgx_prefill_ws_bytes",
+    "dsgx_decode_ws_bytes", "dsgx_decode_ws_flag_offset", "dsgx_decode_status", "dsgx_moe_decode", "dsgx_moe_decode_noalloc", "dsgx_finalize", "dsgx_add_norm", "dsgx_dsk_cfg_default", "dsgx_dsk_moe", "dsgx_prefill_cfg_default", "dsgx_prefill_ws_bytes",
     "dsgx_moe_prefill", "dsgx_prefill_view_get", "dsgx_gemv", "dsgx_dequant_int4", "dsgx_probe_dequant_int4", "dsgx_probe_mfma_fp8",
     "dsgx_widen_fp8", "dsgx_act_quant", "dsgx_last_error", "dsgx_version", "dsgx_stream_read", "dsgx_stream_read_cfg", "dsgx_stream_copy",
 ]

@@ -11,7 +11,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 SO = os.path.join(CSRC, "libdsgx.so")
-SOURCES = ["abi.hip", "route.hip", "gemv.hip", "moe_decode.hip", "moe_decode_fp8.hip", "moe_decode_int4.hip", "moe_decode_int4_mfma.hip",
+SOURCES = ["abi.hip", "route.hip", "gemv.hip", "moe_decode.hip", "moe_decode_fp8.hip", "moe_decode_int4.hip", "moe_decode_int4_mfma.hip", "moe_decode_mxfp4_mfma.hip",
            "moe_decode_bf16.hip", "moe_prefill.hip"]
 # -packed-fp32-ops off: hipcc -O3 otherwise forms v_pk_*_f32 from scalar float code
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden", "-ffp-contract=off",

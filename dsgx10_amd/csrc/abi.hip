@@ -225,7 +225,8 @@ const char* dsgx_version(void) { return "dsgx10_amd 0.1 (gfx950)"; }
 size_t dsgx_mat_scale_off(uint32_t fmt, int N, int K) {
   if (N <= 0 || K <= 0) return 0;
   if (fmt == DSGX_FMT_FP8_B128) return align256((size_t)N * K);
-  if (fmt == DSGX_FMT_INT4_G32) return align256((size_t)N * K / 2);
+  if (fmt == DSGX_FMT_INT4_G32 || fmt == DSGX_FMT_MXFP4_G32) return align256((size_t)N * K / 2);
+  if (fmt == DSGX_FMT_FP8_B32E) return align256((size_t)N * K);
   return 0;
 }
 size_t dsgx_mat_zp_off(uint32_t fmt, int N, int K) {
@@ -238,6 +239,8 @@ size_t dsgx_mat_bytes(uint32_t fmt, int N, int K) {
   if (fmt == DSGX_FMT_INT4_G32)
     return (K % 32 || N % 8) ? 0 : align256((size_t)N * K / 2) + align256((size_t)N * (K / 32) * 2) + align256((size_t)(N / 8) * (K / 32) * 4);
   if (fmt == DSGX_FMT_BF16) return align256((size_t)N * K * 2);
+  if (fmt == DSGX_FMT_MXFP4_G32) return K % 32 ? 0 : align256((size_t)N * K / 2) + align256((size_t)N * (K / 32));
+  if (fmt == DSGX_FMT_FP8_B32E) return (K % 32 || N % 32) ? 0 : align256((size_t)N * K) + align256((size_t)(N / 32) * (K / 32));
   return 0;
 }
 

@@ -77,8 +77,13 @@ struct DecodeArgs {
   unsigned long long* trace;
 #endif
   int spin_limit;
+  // DeepSeek's expert arithmetic (variant 1 only; moe_decode_mfma.cuh): gate and up clamped, the routing weight applied
+  // before w2, h quantised per 32 on its way into the down phase, every expert's output rounded to bf16 before the fold
+  int dsk;
+  float dsk_limit;
 };
 
+int launch_decode_mxfp4_mfma(const DecodeArgs& a, int parts, bool shared_fp8e, hipStream_t st);  // MXFP4 experts (+ FP8_B32E shared)
 int launch_decode_fp8(const DecodeArgs& a, int parts, bool shared, hipStream_t st);
 int launch_decode_fp8_mfma(const DecodeArgs& a, int parts, bool shared, hipStream_t st);  // variant 1 (moe_decode_mfma.cuh)
 int launch_decode_int4(const DecodeArgs& a, int parts, bool shared_bf16, hipStream_t st);
@@ -162,8 +167,8 @@ template <int FMT>
 __device__ __forceinline__ MatRef mat_ref(const uint8_t* base, int N, int K, float s2) {
   MatRef m;
   m.w = base, m.s = nullptr, m.s2 = s2, m.pad = 0;
-  if (FMT == DSGX_FMT_FP8_B128) m.s = base + al256d((size_t)N * K);
-  else if (FMT == DSGX_FMT_INT4_G32) m.s = base + al256d((size_t)N * K / 2);
+  if (FMT == DSGX_FMT_FP8_B128 || FMT == DSGX_FMT_FP8_B32E) m.s = base + al256d((size_t)N * K);
+  else if (FMT == DSGX_FMT_INT4_G32 || FMT == DSGX_FMT_MXFP4_G32) m.s = base + al256d((size_t)N * K / 2);
   return m;
 }
 template <int FMT>
@@ -717,12 +722,17 @@ __global__ void __launch_bounds__(256) k_down_combine(DecodeArgs a) {
     }
 #pragma unroll
     for (int j = 0; j < B; ++j)
-      if (s0 + j < nrouted) acc = fmaf(f[j], v[j], acc);
+      if (s0 + j < nrouted) {
+        // DeepSeek's fold: the outputs of the experts the row picked (their routing weight, never zero, went in before
+        // w2), each rounded to bf16, added in expert-id order (ds41f engine/kernels/moe.cu:974-981)
+        if (a.dsk) acc = f[j] != 0.f ? __fadd_rn(acc, bf16_round(v[j])) : acc;
+        else acc = fmaf(f[j], v[j], acc);
+      }
   }
   float sv = 0.f;
-  if (SH) a.ys[i] = sv = a.dpart[i];
+  if (SH) a.ys[i] = sv = a.dsk ? bf16_round(a.dpart[i]) : a.dpart[i];
   else if (a.ysum) sv = a.ys[i];
-  if (a.ysum) acc = __fadd_rn(acc, sv);
+  if (a.ysum || (a.dsk && SH)) acc = __fadd_rn(acc, sv);  // (DeepSeek: the shared expert last, always)
   a.yr[i] = acc;
 }
 

@@ -32,7 +32,7 @@ constexpr int kMfD = DSGX_MFD;    // ring depth in steps
 // Bytes between activation rows in LDS beyond their length, by the routed experts' format: the lanes of one MFMA
 // operand read (position l % 16, k part l / 16) 16 bytes each, parts 16 bytes apart (FP8, BF16: rows 64 bytes apart
 // mod 256 spread four rows over the banks) or 128 bytes apart (INT4: rows 16 bytes apart spread eight).
-__host__ __device__ constexpr int mf_pad(int fmt) { return fmt == DSGX_FMT_INT4_G32 ? 16 : 64; }
+__host__ __device__ constexpr int mf_pad(int fmt) { return fmt == DSGX_FMT_INT4_G32 || fmt == DSGX_FMT_MXFP4_G32 ? 16 : 64; }
 constexpr int kMfThreads = 512;   // eight waves a workgroup, one workgroup a CU
 constexpr int kMfWaves = kMfThreads / 64;
 
@@ -43,6 +43,9 @@ template <int FMT> struct MfFmt;
 template <> struct MfFmt<DSGX_FMT_FP8_B128> { static constexpr int STEPK = 128, MINSTEPS = 4; };
 template <> struct MfFmt<DSGX_FMT_INT4_G32> { static constexpr int STEPK = 256, MINSTEPS = 8; };
 template <> struct MfFmt<DSGX_FMT_BF16> { static constexpr int STEPK = 64, MINSTEPS = 8; };
+// MXFP4: INT4's bytes and k map (a lane's 16 bytes are one scale group of 32 values); FP8_B32E: FP8's
+template <> struct MfFmt<DSGX_FMT_MXFP4_G32> { static constexpr int STEPK = 256, MINSTEPS = 8; };
+template <> struct MfFmt<DSGX_FMT_FP8_B32E> { static constexpr int STEPK = 128, MINSTEPS = 4; };
 
 // The slices of K: a power of two (1 .. 8) that divides the steps of K, `minsteps` steps or more a slice where K allows
 // (fewer steps between two workgroup barriers cost more than they spread). With ns < 8 slices, 8 / ns groups of waves
@@ -80,6 +83,45 @@ __device__ __forceinline__ void mf_stage_rows(uint8_t* lds, const uint16_t* src,
 // the 256 zero bytes that the lanes of positions beyond the step's rows read (a step's fragments lie within 208 bytes)
 __device__ __forceinline__ void mf_zero_bytes(uint8_t* at) {
   if (threadIdx.x < 16) *reinterpret_cast<uint4*>(at + 16 * threadIdx.x) = make_uint4(0, 0, 0, 0);
+}
+
+// e2m1 x 8 (one 32-bit word, value i at bits 4 i) times the power of two sc -> exact bf16 values
+__device__ __forceinline__ void fp4x8_to_bf16(uint32_t w, float sc, uint32_t (&o)[4]) {
+  o[0] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, sc, 0));
+  o[1] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, sc, 1));
+  o[2] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, sc, 2));
+  o[3] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, sc, 3));
+}
+// act_quant in place on `rows` staged rows of K bf16 values (row stride rs bytes): per 32 values the ue8m0 scale byte
+// e = exponent of max(amax, 1e-4) / 448 rounded up to a power of two (ds41f engine/kernels/common.cuh:53-66), the values
+// to e4m3 (round to nearest even) and back: x -> e4m3(x * 2^(127 - e)) * 2^(e - 127), a thread a group
+__device__ __forceinline__ void mf_quant_rows(uint8_t* lds, int rows, int K, size_t rs) {
+  const int G = K / 32;
+  for (int i = threadIdx.x; i < rows * G; i += blockDim.x) {
+    uint32_t* p = reinterpret_cast<uint32_t*>(lds + (size_t)(i / G) * rs + (size_t)(i % G) * 64);
+    uint32_t v[16];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const u32x4_t q = *reinterpret_cast<const u32x4_t*>(p + 4 * j);
+      v[4 * j] = q.x, v[4 * j + 1] = q.y, v[4 * j + 2] = q.z, v[4 * j + 3] = q.w;
+    }
+    float amax = 0.f;
+#pragma unroll
+    for (int j = 0; j < 16; ++j) amax = fmaxf(amax, fmaxf(fabsf(bf16_bits_to_f32(v[j] & 0xFFFFu)), fabsf(bf16_bits_to_f32(v[j] >> 16))));
+    const uint32_t b = __float_as_uint(__fmul_rn(fmaxf(amax, 1e-4f), 1.0f / 448.0f));
+    const uint32_t e = ((b >> 23) & 0xFFu) + ((b & 0x7FFFFFu) != 0 ? 1u : 0u);
+    const float inv = __uint_as_float((254u - e) << 23), sc = __uint_as_float(e << 23);
+#pragma unroll
+    for (int j = 0; j < 16; j += 2) {
+      auto qf = [&](uint32_t bits) { return fminf(448.f, fmaxf(-448.f, __fmul_rn(bf16_bits_to_f32(bits), inv))); };
+      uint32_t c = __builtin_amdgcn_cvt_pk_fp8_f32(qf(v[j] & 0xFFFFu), qf(v[j] >> 16), 0, false);
+      c = __builtin_amdgcn_cvt_pk_fp8_f32(qf(v[j + 1] & 0xFFFFu), qf(v[j + 1] >> 16), c, true);
+      v[j] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(c, sc, false));
+      v[j + 1] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(c, sc, true));
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) *reinterpret_cast<u32x4_t*>(p + 4 * j) = u32x4_t{v[4 * j], v[4 * j + 1], v[4 * j + 2], v[4 * j + 3]};
+  }
 }
 
 // What a lane needs to walk a unit: set per unit by the caller's `open`. The weight loads are row-major (lane l: rows
@@ -134,14 +176,16 @@ __device__ __forceinline__ void mf_stream(uint8_t* smem, size_t rows_bytes, uint
   // LDS offsets. The row-major writes stay whole 128-byte rows; a row's eight 16-byte pieces are exchanged so that the
   // MFMA-order reads (16 lanes: 16 rows, one k part) touch every bank once: by (row / 2) % 8 for FP8's reads of 8 bytes,
   // by row % 8 for the reads of 16 bytes.
-  constexpr int RSH = FMT == DSGX_FMT_FP8_B128 ? 1 : 0;
-  int wr_off[2], rd_off[FMT == DSGX_FMT_FP8_B128 ? 4 : 2];
+  constexpr bool F8 = FMT == DSGX_FMT_FP8_B128 || FMT == DSGX_FMT_FP8_B32E;   // 8-byte fragment reads, four MFMAs a 128-k step
+  constexpr bool G32 = FMT == DSGX_FMT_INT4_G32 || FMT == DSGX_FMT_MXFP4_G32;  // a lane's 16 bytes = one scale group of 32 values
+  constexpr int RSH = F8 ? 1 : 0;
+  int wr_off[2], rd_off[F8 ? 4 : 2];
 #pragma unroll
   for (int h = 0; h < 2; ++h) wr_off[h] = (8 * h + r8) * 128 + ((q ^ (((8 * h + r8) >> RSH) & 7)) * 16);
-  if constexpr (FMT == DSGX_FMT_FP8_B128) {
+  if constexpr (F8) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) rd_off[j] = r16 * 128 + (((2 * j + (part >> 1)) ^ ((r16 >> 1) & 7)) * 16) + 8 * (part & 1);
-  } else if constexpr (FMT == DSGX_FMT_INT4_G32) {  // pieces 2 part, 2 part + 1: two scale groups
+  } else if constexpr (G32) {  // pieces 2 part, 2 part + 1: two scale groups
 #pragma unroll
     for (int j = 0; j < 2; ++j) rd_off[j] = r16 * 128 + (((2 * part + j) ^ (r16 & 7)) * 16);
   } else {  // pieces part, 4 + part: the lane's 8 k of the step's two MFMAs
@@ -150,7 +194,7 @@ __device__ __forceinline__ void mf_stream(uint8_t* smem, size_t rows_bytes, uint
   }
   const bool live = r16 < M;  // positions beyond the step's rows read the zero bytes
   // the lane's activations: row r16 from k0 + (FP8, BF16: 8 part; INT4: 64 part)
-  constexpr int XPART = FMT == DSGX_FMT_INT4_G32 ? 64 : 8;
+  constexpr int XPART = G32 ? 64 : 8;
   const uint32_t xl = (uint32_t)(r16 * rs) + (uint32_t)(k0 + XPART * part) * 2;
   // xp: the lane's activations of the step at hand (the fragments' offsets within a step are immediates); the lanes of
   // positions beyond the step's rows stay on the zero bytes
@@ -175,6 +219,10 @@ __device__ __forceinline__ void mf_stream(uint8_t* smem, size_t rows_bytes, uint
     } else if constexpr (FMT == DSGX_FMT_INT4_G32) {
       e.s = ldg_u32(cur.sp + (size_t)lstep * 16);
       e.z = *(const DSGX_GLOBAL u32x2_t*)(uintptr_t)(cur.zp + (size_t)lstep * 32);
+    } else if constexpr (FMT == DSGX_FMT_MXFP4_G32) {  // the two groups' ue8m0 bytes (8 groups a row and step)
+      e.s = *(const DSGX_GLOBAL uint16_t*)(uintptr_t)(cur.sp + (size_t)lstep * 8);
+    } else if constexpr (FMT == DSGX_FMT_FP8_B32E) {   // the step's four k blocks' ue8m0 bytes of the lane's row block
+      e.s = ldg_u32(cur.sp + (size_t)lstep * 4);
     }
     if (++lstep == steps) {
       lstep = 0;
@@ -204,6 +252,32 @@ __device__ __forceinline__ void mf_stream(uint8_t* smem, size_t rows_bytes, uint
       const float s1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane((int)e.s, 1));
       acc[0] = fmaf(s0, part_sum[0], acc[0]), acc[1] = fmaf(s1, part_sum[1], acc[1]);
       acc[2] = fmaf(s0, part_sum[2], acc[2]), acc[3] = fmaf(s1, part_sum[3], acc[3]);
+    } else if constexpr (FMT == DSGX_FMT_FP8_B32E) {
+      // e4m3 * 2^(scale - 127) is a bf16 value: the scale goes into the conversion and the MFMAs accumulate over K
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const uint2 wq = *reinterpret_cast<const uint2*>(W + rd_off[j]);
+        const float sc = __uint_as_float(((e.s >> (8 * j)) & 0xFFu) << 23);
+        uint32_t o[4];
+        o[0] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(wq.x, sc, false));
+        o[1] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(wq.x, sc, true));
+        o[2] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(wq.y, sc, false));
+        o[3] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(wq.y, sc, true));
+        acc = mfma(o, 32 * j, acc);
+      }
+    } else if constexpr (FMT == DSGX_FMT_MXFP4_G32) {
+      // e2m1 * 2^(scale - 127) is a bf16 value too: two values an instruction (v_cvt_scalef32_pk_bf16_fp4)
+#pragma unroll
+      for (int jj = 0; jj < 2; ++jj) {
+        const u32x4_t pc = *reinterpret_cast<const u32x4_t*>(W + rd_off[jj]);
+        const float sc = __uint_as_float(((e.s >> (8 * jj)) & 0xFFu) << 23);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          uint32_t o[4];
+          fp4x8_to_bf16(pc[j], sc, o);
+          acc = mfma(o, 32 * jj + 8 * j, acc);
+        }
+      }
     } else if constexpr (FMT == DSGX_FMT_INT4_G32) {
 #pragma unroll
       for (int jj = 0; jj < 2; ++jj) {
@@ -279,6 +353,15 @@ __device__ __forceinline__ MfUnit mf_open_up(const Slot& T, int t, int H, int I,
     q.wp = ((r8 & 1) ? uw : gw) + (size_t)(8 * t + (r8 >> 1)) * H + k0 + p8 * 16;
     q.half = (size_t)4 * H;  // row 8 + r is gate / up (the same parity) of channel 4 further
     q.sp = ((lane & 1) ? us : gs) + ((size_t)((8 * t) >> 7) * (H >> 7) + (k0 >> 7)) * 4;
+  } else if constexpr (F == DSGX_FMT_FP8_B32E) {
+    q.wp = ((r8 & 1) ? uw : gw) + (size_t)(8 * t + (r8 >> 1)) * H + k0 + p8 * 16;
+    q.half = (size_t)4 * H;
+    q.sp = ((r16 & 1) ? us : gs) + (size_t)((8 * t) >> 5) * (H >> 5) + (k0 >> 5);  // the lane's own row (MFMA order): gate or up
+  } else if constexpr (F == DSGX_FMT_MXFP4_G32) {
+    const int G = H >> 5;
+    q.wp = ((r8 & 1) ? uw : gw) + (size_t)(8 * t + (r8 >> 1)) * (H >> 1) + (k0 >> 1) + p8 * 16;
+    q.half = (size_t)4 * (H >> 1);
+    q.sp = ((r16 & 1) ? us : gs) + (size_t)(8 * t + (r16 >> 1)) * G + (size_t)(k0 >> 5) + 2 * part;
   } else if constexpr (F == DSGX_FMT_INT4_G32) {
     const int G = H >> 5;
     q.wp = ((r8 & 1) ? uw : gw) + (size_t)(8 * t + (r8 >> 1)) * (H >> 1) + (k0 >> 1) + p8 * 16;
@@ -305,6 +388,15 @@ __device__ __forceinline__ MfUnit mf_open_down(const Slot& T, int t, int H, int 
     q.wp = dw + (size_t)(16 * t + r8) * I + k0 + p8 * 16;
     q.half = (size_t)8 * I;
     q.sp = ds + ((size_t)((16 * t) >> 7) * (I >> 7) + (k0 >> 7)) * 4;
+  } else if constexpr (F == DSGX_FMT_FP8_B32E) {
+    q.wp = dw + (size_t)(16 * t + r8) * I + k0 + p8 * 16;
+    q.half = (size_t)8 * I;
+    q.sp = ds + (size_t)((16 * t) >> 5) * (I >> 5) + (k0 >> 5);
+  } else if constexpr (F == DSGX_FMT_MXFP4_G32) {
+    const int G = I >> 5;
+    q.wp = dw + (size_t)(16 * t + r8) * (I >> 1) + (k0 >> 1) + p8 * 16;
+    q.half = (size_t)8 * (I >> 1);
+    q.sp = ds + (size_t)(16 * t + r16) * G + (size_t)(k0 >> 5) + 2 * part;
   } else if constexpr (F == DSGX_FMT_INT4_G32) {
     const int G = I >> 5;
     q.wp = dw + (size_t)(16 * t + r8) * (I >> 1) + (k0 >> 1) + p8 * 16;
@@ -341,8 +433,24 @@ __device__ __forceinline__ void mf_up_phase(Step<M>& S, const DecodeArgs& a, uin
     if (pos >= M) return;
     const Slot& T = S.slots[sl];
     const float sg = T.g.s2, su = T.u.s2;
-    const uint32_t h0 = swiglu_bits(bf16_round(__fmul_rn(sum[0], sg)), bf16_round(__fmul_rn(sum[1], su)));
-    const uint32_t h1 = swiglu_bits(bf16_round(__fmul_rn(sum[2], sg)), bf16_round(__fmul_rn(sum[3], su)));
+    uint32_t h0, h1;
+    if (a.dsk) {
+      // ds41f engine/kernels/moe.cu:519-528: gate and up rounded to bf16, up clamped to +-limit and gate from above,
+      // silu(gate) * up, times the row's routing weight (routed slots), rounded to bf16; quantised per 32 when the down
+      // phase stages it
+      auto hd = [&](float gs, float us) {
+        float gt = bf16_round(gs), up = bf16_round(us);
+        up = fminf(fmaxf(up, -a.dsk_limit), a.dsk_limit);
+        gt = fminf(gt, a.dsk_limit);
+        float h = __fmul_rn(__fdiv_rn(gt, __fadd_rn(1.f, expf(-gt))), up);
+        if (!T.shared) h = __fmul_rn(S.wslot[sl - nsh][pos], h);
+        return f32_to_bf16_bits(h);
+      };
+      h0 = hd(sum[0], sum[1]), h1 = hd(sum[2], sum[3]);
+    } else {
+      h0 = swiglu_bits(bf16_round(__fmul_rn(sum[0], sg)), bf16_round(__fmul_rn(sum[1], su)));
+      h1 = swiglu_bits(bf16_round(__fmul_rn(sum[2], sg)), bf16_round(__fmul_rn(sum[3], su)));
+    }
     uint16_t* dst = a.h + ((size_t)T.hslot * M + pos) * I + 8 * t + 2 * part;
     __hip_atomic_store((DSGX_GLOBAL uint32_t*)(uintptr_t)dst, h0 | (h1 << 16), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   };
@@ -372,8 +480,8 @@ __device__ __forceinline__ void mf_up_phase(Step<M>& S, const DecodeArgs& a, uin
 #ifndef DSGX_MF_SHCOST
 #define DSGX_MF_SHCOST 2.0f
 #endif
-    constexpr float kShCost = DSGX_MF_SHCOST;
-    auto bpv = [](int f) { return f == DSGX_FMT_BF16 ? 2.f : f == DSGX_FMT_FP8_B128 ? 1.f : 0.5703f; };  // bytes a value
+    constexpr float kShCost = FMT == DSGX_FMT_INT4_G32 ? DSGX_MF_SHCOST : 1.f;  // (only the INT4 stream waits for the vector unit)
+    auto bpv = [](int f) { return f == DSGX_FMT_BF16 ? 2.f : f == DSGX_FMT_FP8_B128 || f == DSGX_FMT_FP8_B32E ? 1.f : 0.5703f; };  // bytes a value
     const float bsh = bpv(SHFMT), bro = kShCost * (float)nrouted * bpv(FMT);
     const int nshw = uni(nrouted > 0 ? max(1, min(G - 1, (int)((float)G * bsh / (bsh + bro) + 0.5f))) : G);
     if (g < nshw) run(std::integral_constant<int, SHFMT>{}, 0, 1, g, nshw);
@@ -426,6 +534,10 @@ __device__ __forceinline__ void mf_down_phase(Step<M>& S, const DecodeArgs& a, u
         mf_stage_rows<FUSED>(mf_smem + (size_t)j * M * rs, a.h + (size_t)S.slots[sl0 + j].hslot * M * I, I, M, I, pad);
       mf_zero_bytes(mf_smem + (size_t)2 * M * rs);
       __syncthreads();
+      if (a.dsk) {  // w2's input is act_quant(h): e4m3 with a ue8m0 scale per 32 values (moe.cu:529-534), again bf16 values
+        mf_quant_rows(mf_smem, nss * M, I, rs);
+        __syncthreads();
+      }
     };
     const int ns = mf_slices(I, MfFmt<F>::STEPK, MfFmt<F>::MINSTEPS), KS = I / ns, k0 = (wave % ns) * KS;
     auto open = [&](int u) {

@@ -23,6 +23,8 @@ def mat_bytes(fmt, N, K):
         return _al256(N * K // 2) + _al256(N * (K // 32) * 2) + _al256((N // 8) * (K // 32) * 4)
     if fmt == abi.FMT_BF16:
         return _al256(N * K * 2)
+    if fmt == abi.FMT_MXFP4:
+        return _al256(N * K // 2) + _al256(N * (K // 32))
     raise ValueError("format %r is not FP8_B128 (16), INT4_G32 (18) or BF16 (19)" % (fmt,))
 
 
@@ -45,6 +47,11 @@ def mat_blob(fmt, parts):
         N, K = w.shape
         assert w.dtype == np.uint16
         chunks = [w]
+    elif fmt == abi.FMT_MXFP4:  # e2m1 pairs u8 [N][K/2] (low nibble the even k), ue8m0 u8 [N][K/32]
+        packed, scale = parts
+        N, K = packed.shape[0], packed.shape[1] * 2
+        assert packed.dtype == np.uint8 and scale.dtype == np.uint8 and scale.shape == (N, K // 32)
+        chunks = [packed, scale]
     else:
         raise ValueError("format %r" % (fmt,))
     out = np.zeros(mat_bytes(fmt, N, K), np.uint8)

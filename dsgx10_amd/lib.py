@@ -43,6 +43,8 @@ def lib():
         L.dsgx_moe_decode_noalloc.argtypes = [C.POINTER(abi.LayerW), C.c_void_p, C.c_void_p, C.c_void_p, C.c_int,
                                               C.c_void_p, C.c_void_p, C.c_void_p, C.POINTER(abi.DecodeCfg)]
         L.dsgx_decode_status.argtypes = [C.POINTER(abi.LayerW), C.c_void_p, C.c_void_p]
+        L.dsgx_dsk_moe.argtypes = [C.POINTER(abi.LayerW), C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
+                                   C.c_void_p, C.c_void_p, C.POINTER(abi.DskCfg)]
         L.dsgx_finalize.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p]
         L.dsgx_add_norm.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_float,
                                     C.c_void_p, C.c_int, C.c_void_p]
@@ -107,6 +109,13 @@ def moe_decode(layer_w, x, idx, w, M, ws, yr, ys, stream=None, parts=3, ysum=Fal
         return
     _check(lib().dsgx_moe_decode(C.byref(layer_w), _ptr(x), _ptr(idx), _ptr(w), M, _ptr(ws), _ptr(yr), _ptr(ys),
                                  _stream(stream), C.byref(cfg)))
+
+
+def dsk_moe(layer_w, xq, xs, idx, w, M, ws, y, ys, stream=None, limit=10.0, logits=None, bias=None, route_scale=1.0, parts=3):
+    """DeepSeek's decode MoE (dsk::moe / moe_routed): MXFP4 experts + FP8 shared expert, rows given as act_quant(x)"""
+    cfg = abi.DskCfg(limit, _ptr(logits), _ptr(bias), route_scale, parts)
+    _check(lib().dsgx_dsk_moe(C.byref(layer_w), _ptr(xq), _ptr(xs), M, _ptr(idx), _ptr(w), _ptr(ws), _ptr(y), _ptr(ys), _stream(stream),
+                              C.byref(cfg)))
 
 
 def decode_status(layer_w, ws, stream=None):

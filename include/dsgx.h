@@ -50,7 +50,14 @@ enum {
      W(n,k) = bf16_rne((u - u_z) * s)       (engine/experts/layout.h:24-42, docs/model.md:111-195) */
   DSGX_FMT_INT4_G32 = 18,
   /* bf16 bits [N][K] row-major */
-  DSGX_FMT_BF16 = 19
+  DSGX_FMT_BF16 = 19,
+  /* OCP MXFP4, the routed experts of DeepSeek's layers: e2m1 pairs u8 [N][K/2] row-major (the low nibble the even k),
+     then (256-byte aligned) ue8m0 scales u8 [N][K/32]: W(n,k) = e2m1(nibble) * 2^(S[n][k/32] - 127)
+     (ds41f-4xgx10-switchless/engine/kernels/README.md, L3's source form; ref/torchref/kernel.py:111-117). K a multiple of 256. */
+  DSGX_FMT_MXFP4_G32 = 20,
+  /* FP8 e4m3fn codes u8 [N][K] row-major, then (256-byte aligned) ue8m0 scales u8 [N/32][K/32], one a 32 x 32 block
+     (the same layers' shared expert: README.md L1's source form; kernel.py:105-108 with block 32) */
+  DSGX_FMT_FP8_B32E = 21
 };
 
 /* Bytes of one [N][K] matrix in a format, parts laid as above (0 for an unknown tag or a bad shape).
@@ -151,6 +158,27 @@ DSGX_API int dsgx_moe_decode_noalloc(const dsgx_layer_w* L, const uint16_t* x, c
                                      float* ys, void* stream, const dsgx_decode_cfg* cfg);
 /* out = bf16(bf16(R) + bf16(S)): gx::finalize (engine/experts/experts.h:146-147, decode.cu:591-598) */
 DSGX_API int dsgx_finalize(const float* R, const float* S, int n, uint16_t* out, void* stream);
+
+/* ---- DeepSeek's decode MoE: dsk::moe / dsk::moe_routed (ds41f-4xgx10-switchless/engine/kernels/dsk.h:199-241) ------------
+   L: MXFP4_G32 experts (pool + descriptors as for the other formats; desc.s2 = 1) and, optionally, the FP8 shared expert
+   in L->sh.g / u / d (e4m3 [I][H], [I][H], [H][I]) with its ue8m0 scales per 32 x 32 block in L->sh.gs / us / ds (the three
+   pointers then address BYTES [N/32][K/32], not floats). xq, xs = act_quant(x): e4m3 [M][H] and ue8m0 [M][H/32]. idx, w
+   [M][topk] from the router, or cfg->logits (+ bias): the sqrt-softplus router runs inside the kernel.
+   Arithmetic (engine/kernels/moe.cu:519-534, 974-981; ref/inference/model.py:841-851): per expert gate, up = bf16(f32 sums of
+   the block-scaled products), up clamped to +-limit and gate from above, h = bf16(w_row * (silu(gate) * up)) (no weight for
+   the shared expert), h quantised like x, the expert's w2 output rounded to bf16; y = the f32 sum of the picked experts'
+   outputs in expert-id order, then the shared expert's. y f32 [M][H] the sum, ys f32 [M][H] the shared expert's bf16
+   output alone. ws: dsgx_decode_ws_bytes(L), zeroed once. M <= 16 (9-16: two passes). */
+typedef struct dsgx_dsk_cfg {
+  float swiglu_limit;   /* 10 */
+  const float* logits;  /* fused routing (moe_routed): f32 [M][E]; idx, w are then not read */
+  const float* bias;
+  float route_scale;
+  int32_t parts;        /* 1 gate/up only, 2 down only, 3 both (bench) */
+} dsgx_dsk_cfg;
+DSGX_API void dsgx_dsk_cfg_default(dsgx_dsk_cfg* cfg);
+DSGX_API int dsgx_dsk_moe(const dsgx_layer_w* L, const uint8_t* xq, const uint8_t* xs, int M, const int* idx, const float* w, void* ws,
+                          float* y, float* ys, void* stream, const dsgx_dsk_cfg* cfg);
 
 /* The residual add after the expert step and the next layer's RMSNorm, the local half of the reference's
    comm::glm::allreduce_add_norm / allreduce2_add_norm (engine/comm/glmcoll.h:34-62; the norm: engine/attn/prep.cu:12-66),
