@@ -116,7 +116,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=64)
     ap.add_argument("--no-extra", action="store_true", help="only the headline workload")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
-    ap.add_argument("--workload", default="fp8_m1", help="headline workload: fp8_m1 | int4_m1; fp8_prefill | int4_prefill time only that prefill chunk; gemv only the dense GEMVs; chain only the layer chains")
+    ap.add_argument("--workload", default="fp8_m1", help="headline workload: fp8_m1 | int4_m1; fp8_prefill | int4_prefill time only that prefill chunk; gemv only the dense GEMVs; chain only the layer chains; dsk only the MXFP4 layer")
     ap.add_argument("--variant", default="vector", choices=("vector", "mfma"),
                     help="the headline's decode kernels (dsgx_decode_cfg::up = 0 | 1); --no-extra then runs nothing else")
     args = ap.parse_args()
@@ -191,6 +191,22 @@ def main():
                                         "frac": d["mfma_frac"], "traffic": None, "hbm_frac": d["hbm_frac"]}),
                           "cpu_baseline": None, "extra": [d], "wall_s": round(time.time() - t_start, 1)}))
         return
+    if args.workload == "dsk":
+        # only DeepSeek's MXFP4 layer (dsgx_dsk_moe, routing fused), M = 1, 2, 4, 8
+        from dsgx10_amd.benchdata import DskBench, DskLayerGen
+        dg = DskLayerGen(seed=0)
+        ds = []
+        for M in (1, 2, 4, 8):
+            ds.append(DskBench(dg, M, 128).time())
+            log("  %s M=%d: %.2f us/layer (%.1f%% of 8 TB/s)" % (ds[-1]["workload"], M, ds[-1]["us_per_layer"], 100 * ds[-1]["hbm_frac"]))
+        print(json.dumps({"metric": "us_per_moe_layer", "value": ds[0]["us_per_layer"], "unit": "us", "n_gpus": 1, "steps": 128, "warmup": 4,
+                          "ms_per_step": ds[0]["us_per_layer"] * 1e-3, "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+                          "dtype": "f32 sums of exact bf16 x bf16 products (MXFP4 / e4m3 values times power-of-two scales)", "data": "synthetic",
+                          "config": {"workload": ds[0]["workload"], "rows_M": 1},
+                          "roofline": {"bound": "hbm", "achieved": ds[0]["bytes"] / ds[0]["us_per_layer"] * 1e-3, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                                       "frac": ds[0]["hbm_frac"], "traffic": None},
+                          "cpu_baseline": None, "extra": ds, "wall_s": round(time.time() - t_start, 1)}))
+        return
     if args.workload == "chain":
         # only the layer chains (router GEMV -> experts -> add + norm, 128 layers a graph), FP8 then INT4
         from dsgx10_amd.benchdata import ChainBench
@@ -249,7 +265,7 @@ def main():
                 extra.append(d)
                 del ob
         extra.append(prefill_extra(other, 2048, "int4_moe_prefill", 2.5e15, not args.no_cpu) if head_fp8 else prefill_extra(other, 8192, "fp8_moe_prefill", 5.0e15, not args.no_cpu))
-        from dsgx10_amd.benchdata import ChainBench, gemv_bench
+        from dsgx10_amd.benchdata import ChainBench, DskBench, DskLayerGen, gemv_bench
         for g2 in (gen, other):
             cb = ChainBench(g2, 1, 128)
             d = cb.time()
@@ -257,6 +273,12 @@ def main():
             extra.append(d)
             del cb
         del other
+        dg = DskLayerGen(seed=0)
+        for M in (1, 8):
+            d = DskBench(dg, M, 128).time()
+            log("  %s M=%d: %.2f us/layer (%.1f%% of 8 TB/s)" % (d["workload"], M, d["us_per_layer"], 100 * d["hbm_frac"]))
+            extra.append(d)
+        del dg
         extra += gemv_bench()
 
     out = {

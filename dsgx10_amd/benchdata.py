@@ -290,6 +290,104 @@ class DecodeBench:
                     experts=experts)
 
 
+class DskLayerGen(_LayerGen):
+    """DeepSeek's MoE layer (ds41f-4xgx10-switchless/engine/kernels/dsk.h:199-241) at its unsharded shape: hidden 5120,
+    intermediate 2304 (the reference's 576 a rank x 4), 256 MXFP4 experts, top-6 by the sqrt-softplus router, one FP8 shared
+    expert with ue8m0 scales per 32 x 32; random e2m1 codes and scale bytes (the values' statistics do not change the bytes
+    streamed)."""
+    name = "dsk_mxfp4_moe_decode"
+    fmt, H, I, E, topk, route_scale, NSH = abi.FMT_MXFP4, 5120, 2304, 256, 6, 1.5, 16
+
+    def __init__(self, seed=0):
+        g = torch.Generator(device="cuda")
+        g.manual_seed(seed + 2)
+        H, I, E = self.H, self.I, self.E
+        per = [mat_bytes(self.fmt, I, H), mat_bytes(self.fmt, I, H), mat_bytes(self.fmt, H, I)]
+        self.expert_bytes = sum(per)
+        self.pool = torch.zeros(E * self.expert_bytes, dtype=torch.uint8, device="cuda")
+        desc = np.zeros(E * 3, DESC_DTYPE)
+        o = 0
+        for e in range(E):
+            for j in range(3):
+                N, K = (I, H) if j < 2 else (H, I)
+                d = desc[e * 3 + j]
+                d["off"], d["s2"], d["fmt"] = o, 1.0, self.fmt
+                _put(self.pool, o, torch.randint(0, 256, (N, K // 2), generator=g, device="cuda", dtype=torch.uint8))
+                _put(self.pool, o + _al256(N * K // 2), torch.randint(114, 120, (N, K // 32), generator=g, device="cuda", dtype=torch.uint8))
+                o += per[j]
+        self.desc = torch.from_numpy(desc.view(np.uint8).reshape(-1)).cuda()
+        self.shared = []
+        for c in range(self.NSH):
+            mats = []
+            for j in range(3):
+                N, K = (I, H) if j < 2 else (H, I)
+                codes = (torch.randn(N, K, generator=g, device="cuda") * 40.0).clamp(-448, 448).to(torch.float8_e4m3fn).view(torch.uint8)
+                mats.append((codes, torch.randint(110, 116, (N // 32, K // 32), generator=g, device="cuda", dtype=torch.uint8)))
+            self.shared.append(mats)
+        self.shared_bytes = 3 * (H * I + (H // 32) * (I // 32))
+
+    def _set_shared(self, L, c):
+        (gc, gs), (uc, us), (dc, ds) = self.shared[c]
+        L.sh.g, L.sh.u, L.sh.d = gc.data_ptr(), uc.data_ptr(), dc.data_ptr()
+        L.sh.gs, L.sh.us, L.sh.ds = gs.data_ptr(), us.data_ptr(), ds.data_ptr()
+
+    def layer_bytes(self, U):
+        return U * self.expert_bytes + self.shared_bytes
+
+
+class DskBench:
+    """`steps` decode steps of M rows through dsgx_dsk_moe with the routing fused (dsk::moe_routed): step s routes logits[s]"""
+
+    def __init__(self, gen, M, steps, seed=77):
+        self.gen, self.M, self.steps = gen, M, steps
+        g = torch.Generator(device="cuda")
+        g.manual_seed(seed)
+        x = torch.randn(M, gen.H, generator=g, device="cuda") * 1.5
+        blk = x.view(M, gen.H // 32, 32)
+        v = blk.abs().amax(-1).clamp_min(1e-4) * torch.tensor(1.0 / 448.0, device="cuda")
+        bits = v.view(torch.int32)
+        e = ((bits >> 23) & 0xFF) + ((bits & 0x7FFFFF) != 0).to(torch.int32)
+        self.xs = e.to(torch.uint8).contiguous()
+        self.xq = (blk * torch.ldexp(torch.ones_like(v), (127 - e).float())[..., None]).clamp(-448, 448).to(torch.float8_e4m3fn).view(torch.uint8).reshape(M, gen.H).contiguous()
+        self.logits = torch.randn(steps, M, gen.E, generator=g, device="cuda")
+        idx = torch.zeros(steps, M, gen.topk, dtype=torch.int32, device="cuda")
+        w = torch.zeros(steps, M, gen.topk, dtype=torch.float32, device="cuda")
+        for s in range(steps):
+            lib.route(self.logits[s], None, idx[s], w[s], gen.route_scale, score_fn=1)
+        torch.cuda.synchronize()
+        self.union_sizes = np.array([len(np.unique(idx[s].cpu().numpy())) for s in range(steps)])
+        self.layers = [gen.layer_w(c) for c in range(gen.NSH)]
+        self.ws = torch.zeros(lib.decode_ws_bytes(self.layers[0]), dtype=torch.uint8, device="cuda")
+        self.y = torch.zeros(M, gen.H, dtype=torch.float32, device="cuda")
+        self.ys = torch.zeros(M, gen.H, dtype=torch.float32, device="cuda")
+
+    def step(self, s, parts=3):
+        g = self.gen
+        lib.dsk_moe(self.layers[s % g.NSH], self.xq, self.xs, None, None, self.M, self.ws, self.y, self.ys, logits=self.logits[s],
+                    route_scale=g.route_scale, parts=parts)
+
+    def time(self, parts=3):
+        for s in range(4):
+            self.step(s, parts)
+        torch.cuda.synchronize()
+        gr = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(gr):
+            for s in range(self.steps):
+                self.step(s, parts)
+        gr.replay()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        gr.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        lib.decode_status(self.layers[0], self.ws)
+        us = e0.elapsed_time(e1) * 1e3 / self.steps
+        b = float(np.mean([self.gen.layer_bytes(u) for u in self.union_sizes]))
+        return dict(workload=self.gen.name, M=self.M, variant="mfma", us_per_layer=us, bytes=b, hbm_frac=b / (us * 1e-6) / HBM_PEAK,
+                    outputs_finite=bool(torch.isfinite(self.y).all()))
+
+
 class ChainBench:
     """The MoE half of a decode step as the reference's runner chains it (model.cu:309-343), layer after layer in one graph:
     the router's logits by the BF16 GEMV (f32 out, K over 4 waves) from the normed row, the experts with the routing, the
