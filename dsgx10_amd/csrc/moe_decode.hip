@@ -15,7 +15,7 @@ extern "C" unsigned long long* dsgx_trace_buf() { return g_trace_buf; }
 
 // The workspace of dsgx_moe_decode_noalloc: a device array of the library itself, sized for the largest layer that entry
 // point takes (h of 129 slots x 16 rows x DSGX_NOALLOC_MAX_I, the barrier's words, the slot-partitioned down phase's
-// table and its f32 [129][8][DSGX_NOALLOC_MAX_H] results: 33.8 MB on every GPU the library runs on, zero when the
+// table and its f32 [129][8][DSGX_NOALLOC_MAX_H] results: 34.0 MB on every GPU the library runs on, zero when the
 // module loads, which is the barrier's initial state). In host code the array's name is not a device address: the
 // address is asked for once a device (static_ws) and only that pointer is used.
 static constexpr size_t kStaticWsBytes = (size_t)(DSGX_MAX_UNION + 1) * DSGX_MAX_ROWS * DSGX_NOALLOC_MAX_I * 2 + dsgx::kBarBytes +

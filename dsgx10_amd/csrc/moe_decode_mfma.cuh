@@ -225,8 +225,10 @@ __device__ __forceinline__ void mf_stream(uint8_t* smem, size_t rows_bytes, uint
       e.s = ldg_u32(cur.sp + (size_t)lstep * 4);
     }
     if (++lstep == steps) {
-      lstep = 0;
-      if (++lu < mine) cur = open(lu * ng + grp);  // (past the end the ring re-reads the last unit: unused)
+      // past the end the ring keeps re-reading the last step (unused, and still in the caches: re-reading the last unit
+      // from its start fetched it from memory again, 2 KB a step and wave)
+      if (lu + 1 < mine) lstep = 0, cur = open(++lu * ng + grp);
+      else lstep = steps - 1;
     }
   };
   const uint32_t zsh = cur.zsh;  // (the same for every unit of a stream)

@@ -148,7 +148,7 @@ DSGX_API int dsgx_moe_decode(const dsgx_layer_w* L, const uint16_t* x, const int
 /* dsgx_moe_decode on a workspace inside the library, for callers that cannot allocate device memory (code under HIP graph
    capture, serving loops and harnesses that forbid hipMalloc): no workspace argument, no allocation of any kind. It has
    no counterpart in the reference, whose moe_decode always takes the caller's workspace. The workspace is one array of
-   33.8 MB on every GPU the library runs on, held until the process ends; it fits layers with hidden <= DSGX_NOALLOC_MAX_H
+   34.0 MB on every GPU the library runs on, held until the process ends; it fits layers with hidden <= DSGX_NOALLOC_MAX_H
    and intermediate <= DSGX_NOALLOC_MAX_I (larger ones: DSGX_EINVAL). All calls on a GPU share it: calls that overlap on
    one GPU (two streams) race; stream-ordered calls are fine (h and the barrier's words are rewritten by every step).
    Same arguments, bits and errors as dsgx_moe_decode otherwise. */
