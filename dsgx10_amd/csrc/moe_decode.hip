@@ -70,7 +70,7 @@ static int decode_variant(uint32_t fmt, int M, int H, int I) {
 }  // extern "C"
 
 // The workspace: h [DSGX_MAX_UNION + 1 slots][DSGX_MAX_ROWS][I] | the barrier's words (kBarBytes) | the slot-partitioned down
-// phase's slot table (kFacBytes) and its f32 results [slot][8 rows][H] | dsgx_dsk_moe's dequantised rows. I and H here are the LAYOUT's: the layer's own for a
+// phase's slot table (kFacBytes) and its f32 results [slot][8 rows][H] | a reserved row buffer [16][H] bf16. I and H here are the LAYOUT's: the layer's own for a
 // caller's workspace; the built-in workspace is laid out for its largest shapes whatever the layer, so that every layer run
 // on it finds the barrier's words in one place (at an offset that moved with the layer, one layer's h or partial sums would
 // lie where another's counters are expected to be zero).
@@ -81,13 +81,20 @@ struct WsLayout {
   constexpr size_t bar_off() const { return h_bytes(); }
   constexpr size_t fac_off() const { return bar_off() + kBarBytes; }
   constexpr size_t dpart_off() const { return fac_off() + kFacBytes; }
-  constexpr size_t xdeq_off() const { return dpart_off() + (size_t)(DSGX_MAX_UNION + 1) * 8 * H * 4; }  // dsgx_dsk_moe: the rows as bf16
+  constexpr size_t xdeq_off() const { return dpart_off() + (size_t)(DSGX_MAX_UNION + 1) * 8 * H * 4; }  // (reserved)
   constexpr size_t bytes() const { return xdeq_off() + (size_t)DSGX_MAX_ROWS * H * 2; }
 };
 static constexpr WsLayout kStaticLayout{DSGX_NOALLOC_MAX_I, DSGX_NOALLOC_MAX_H};
 static_assert(kStaticLayout.bytes() == kStaticWsBytes, "the built-in workspace's size");
+// DeepSeek's entry point: the rows as e4m3 codes with a ue8m0 scale per 32 values (x then only names the workspace's row buffer)
+struct DskIn {
+  int on = 0;
+  float limit = 0.f;
+  const uint8_t* xq = nullptr;
+  const uint8_t* xs = nullptr;
+};
 static int moe_decode_at(const dsgx_layer_w* L, const uint16_t* x, const int* idx, const float* w, int M, void* ws, const WsLayout& lay,
-                         float* yr, float* ys, void* stream, const dsgx_decode_cfg* cfg, int dsk = 0, float dsk_limit = 0.f);
+                         float* yr, float* ys, void* stream, const dsgx_decode_cfg* cfg, DskIn dsk = DskIn{});
 
 extern "C" {
 size_t dsgx_decode_ws_bytes(const dsgx_layer_w* L) {
@@ -107,7 +114,7 @@ int dsgx_moe_decode(const dsgx_layer_w* L, const uint16_t* x, const int* idx, co
 }  // extern "C"
 
 static int moe_decode_at(const dsgx_layer_w* L, const uint16_t* x, const int* idx, const float* w, int M, void* ws, const WsLayout& lay,
-                         float* yr, float* ys, void* stream, const dsgx_decode_cfg* cfg, int dsk, float dsk_limit) {
+                         float* yr, float* ys, void* stream, const dsgx_decode_cfg* cfg, DskIn dsk) {
   dsgx_decode_cfg c;
   if (cfg) c = *cfg;
   else dsgx_decode_cfg_default(&c);
@@ -124,10 +131,10 @@ static int moe_decode_at(const dsgx_layer_w* L, const uint16_t* x, const int* id
   if (c.down == 1 && c.parts == 3) c.parts = 3 | 4;  // variant 1: the two phases as two launches
   if (L->fmt == DSGX_FMT_REF_NVFP4 || L->fmt == DSGX_FMT_REF_INT4 || L->fmt == DSGX_FMT_REF_BF16)
     return fail(DSGX_EFORMAT, "moe_decode: layer expert format %u names a GB10 block tiling; repack to FP8_B128 (16), INT4_G32 (18) or BF16 (19)", L->fmt);
-  if (L->fmt == DSGX_FMT_MXFP4_G32 && !dsk)
+  if (L->fmt == DSGX_FMT_MXFP4_G32 && !dsk.on)
     return fail(DSGX_EFORMAT, "moe_decode: MXFP4 experts follow DeepSeek's expert arithmetic: dsgx_dsk_moe");
-  if (dsk && L->fmt != DSGX_FMT_MXFP4_G32) return fail(DSGX_EFORMAT, "dsk_moe: layer expert format %u is not MXFP4_G32 (20)", L->fmt);
-  if (dsk) c.up = 1;  // (the MFMA kernels are the ones built for it)
+  if (dsk.on && L->fmt != DSGX_FMT_MXFP4_G32) return fail(DSGX_EFORMAT, "dsk_moe: layer expert format %u is not MXFP4_G32 (20)", L->fmt);
+  if (dsk.on) c.up = 1;  // (the MFMA kernels are the ones built for it)
   if (L->fmt != DSGX_FMT_FP8_B128 && L->fmt != DSGX_FMT_INT4_G32 && L->fmt != DSGX_FMT_BF16 && L->fmt != DSGX_FMT_MXFP4_G32)
     return fail(DSGX_EFORMAT, "moe_decode: layer expert format %u is not FP8_B128 (16), INT4_G32 (18) or BF16 (19)", L->fmt);
   if (!L->pool || !L->desc) return fail(DSGX_EINVAL, "moe_decode: null pool or descriptors");
@@ -156,9 +163,11 @@ static int moe_decode_at(const dsgx_layer_w* L, const uint16_t* x, const int* id
     dsgx_decode_cfg c1 = c, c2 = c;
     c1.parts = c2.parts = c.parts & 3;
     if (c.logits) c2.logits = c.logits + (size_t)M1 * E;
-    if (int rc = moe_decode_at(L, x, idx, w, M1, ws, lay, yr, ys, stream, &c1, dsk, dsk_limit)) return rc;
+    if (int rc = moe_decode_at(L, x, idx, w, M1, ws, lay, yr, ys, stream, &c1, dsk)) return rc;
+    DskIn dsk2 = dsk;
+    if (dsk.xq) dsk2.xq = dsk.xq + (size_t)M1 * H, dsk2.xs = dsk.xs + (size_t)M1 * (H / 32);
     return moe_decode_at(L, x + (size_t)M1 * H, idx ? idx + (size_t)M1 * topk : nullptr, w ? w + (size_t)M1 * topk : nullptr, M - M1, ws, lay,
-                         yr ? yr + (size_t)M1 * H : nullptr, ys ? ys + (size_t)M1 * H : nullptr, stream, &c2, dsk, dsk_limit);
+                         yr ? yr + (size_t)M1 * H : nullptr, ys ? ys + (size_t)M1 * H : nullptr, stream, &c2, dsk2);
   }
   DecodeArgs a{};
   a.x = x, a.M = M, a.idx = idx, a.w = w, a.logits = c.logits, a.bias = c.bias, a.route_scale = c.route_scale, a.score_fn = c.score_fn;
@@ -167,7 +176,7 @@ static int moe_decode_at(const dsgx_layer_w* L, const uint16_t* x, const int* id
   a.bar = reinterpret_cast<int*>(wsb + lay.bar_off());
   a.fac = reinterpret_cast<float*>(wsb + lay.fac_off());
   a.dpart = reinterpret_cast<float*>(wsb + lay.dpart_off());
-  a.dsk = dsk, a.dsk_limit = dsk_limit;
+  a.dsk = dsk.on, a.dsk_limit = dsk.limit, a.dsk_xq = dsk.xq, a.dsk_xs = dsk.xs;
   a.spin_limit = 1 << 22;
 #ifdef DSGX_TRACE
   a.trace = g_trace_buf;
@@ -193,24 +202,6 @@ static int moe_decode_at(const dsgx_layer_w* L, const uint16_t* x, const int* id
 }
 
 // ---- DeepSeek's decode MoE: dsk::moe / dsk::moe_routed (ds41f-4xgx10-switchless/engine/kernels/dsk.h:199-241) -----------------
-namespace {
-// e4m3 codes with a ue8m0 scale per 32 values -> the values as bf16 (exact), a thread eight values
-__global__ void __launch_bounds__(256) k_dsk_dequant_rows(const uint8_t* __restrict__ q, const uint8_t* __restrict__ s, int n8, int K,
-                                                          uint16_t* __restrict__ out) {
-  const int i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= n8) return;
-  const size_t e0 = (size_t)i * 8;
-  const uint2 c = *reinterpret_cast<const uint2*>(q + e0);
-  const float sc = __uint_as_float((uint32_t)s[(e0 / K) * (K / 32) + (e0 % K) / 32] << 23);
-  u32x4_t o;
-  o.x = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(c.x, sc, false));
-  o.y = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(c.x, sc, true));
-  o.z = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(c.y, sc, false));
-  o.w = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(c.y, sc, true));
-  *reinterpret_cast<u32x4_t*>(out + e0) = o;
-}
-}  // namespace
-
 extern "C" {
 void dsgx_dsk_cfg_default(dsgx_dsk_cfg* c) {
   if (!c) return;
@@ -231,13 +222,10 @@ int dsgx_dsk_moe(const dsgx_layer_w* L, const uint8_t* xq, const uint8_t* xs, in
   if ((uintptr_t)xq & 7) return fail(DSGX_EINVAL, "dsk_moe: the rows' codes must be 8-byte aligned");
   const WsLayout lay{L->I, L->H};
   uint16_t* xd = reinterpret_cast<uint16_t*>(static_cast<uint8_t*>(ws) + lay.xdeq_off());
-  const int n8 = M * L->H / 8;
-  hipLaunchKernelGGL(k_dsk_dequant_rows, dim3((n8 + 255) / 256), dim3(256), 0, static_cast<hipStream_t>(stream), xq, xs, n8, L->H, xd);
-  DSGX_HIP(hipGetLastError());
   dsgx_decode_cfg d;
   dsgx_decode_cfg_default(&d);
   d.up = 1, d.parts = c.parts, d.logits = c.logits, d.bias = c.bias, d.route_scale = c.route_scale, d.score_fn = 1;
-  return moe_decode_at(L, xd, idx, w, M, ws, lay, y, ys, stream, &d, 1, c.swiglu_limit);
+  return moe_decode_at(L, xd, idx, w, M, ws, lay, y, ys, stream, &d, DskIn{1, c.swiglu_limit, xq, xs});
 }
 }  // extern "C"
 

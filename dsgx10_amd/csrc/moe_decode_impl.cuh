@@ -81,6 +81,8 @@ struct DecodeArgs {
   // before w2, h quantised per 32 on its way into the down phase, every expert's output rounded to bf16 before the fold
   int dsk;
   float dsk_limit;
+  const uint8_t* dsk_xq;  // the rows as e4m3 codes [M][H] with ue8m0 scales [M][H / 32] (x is then not read)
+  const uint8_t* dsk_xs;
 };
 
 int launch_decode_mxfp4_mfma(const DecodeArgs& a, int parts, bool shared_fp8e, hipStream_t st);  // MXFP4 experts (+ FP8_B32E shared)
@@ -705,20 +707,28 @@ __global__ void __launch_bounds__(DSGX_DECODE_THREADS) k_down_part(DecodeArgs a,
 // yr[m][n] = the slots' dots chained in slot (expert id) order, acc = fma(s2 w, dot, acc); ys = the shared slot's dot
 template <int M, bool SH>
 __global__ void __launch_bounds__(256) k_down_combine(DecodeArgs a) {
-  const int H = a.L.H, nrouted = reinterpret_cast<const int*>(a.fac)[0];
+  const int H = a.L.H;
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= M * H) return;
   const int m = i / H;
   const float* d = a.dpart + (size_t)(SH ? 1 : 0) * M * H + i;
   float acc = 0.f;
-  // sixteen slots' loads in flight together (past the end: the last slot again, unused), then their adds in slot order
+  // sixteen slots' loads in flight together (past the end: the last slot again, unused), then their adds in slot order. The
+  // first sixteen are loaded before the slot count is known (the buffers hold that many slots whatever the step: stale
+  // values past the count are not used), so that a step with up to sixteen slots takes one memory round trip, not two.
   constexpr int B = 16;
-  for (int s0 = 0; s0 < nrouted; s0 += B) {
-    float v[B], f[B];
+  static_assert(B <= DSGX_MAX_UNION, "the first batch lies within the buffers");
+  float v[B], f[B];
 #pragma unroll
-    for (int j = 0; j < B; ++j) {
-      const int s = min(s0 + j, nrouted - 1);
-      v[j] = d[(size_t)s * M * H], f[j] = a.fac[8 + s * 8 + m];
+  for (int j = 0; j < B; ++j) v[j] = d[(size_t)j * M * H], f[j] = a.fac[8 + j * 8 + m];
+  const int nrouted = reinterpret_cast<const int*>(a.fac)[0];
+  for (int s0 = 0; s0 < nrouted; s0 += B) {
+    if (s0 > 0) {
+#pragma unroll
+      for (int j = 0; j < B; ++j) {
+        const int s = min(s0 + j, nrouted - 1);
+        v[j] = d[(size_t)s * M * H], f[j] = a.fac[8 + s * 8 + m];
+      }
     }
 #pragma unroll
     for (int j = 0; j < B; ++j)

@@ -80,6 +80,23 @@ __device__ __forceinline__ void mf_stage_rows(uint8_t* lds, const uint16_t* src,
     }
   }
 }
+// The same from DeepSeek's quantised rows: e4m3 codes q [M][K] with a ue8m0 scale s [M][K / 32] per 32 values, widened
+// exactly (code x 2^(scale - 127) is a bf16 value), a thread eight values at a time
+__device__ __forceinline__ void mf_stage_rows_q(uint8_t* lds, const uint8_t* q, const uint8_t* s, int M, int K, int pad) {
+  const int nq = K / 8, total = M * nq;
+  const size_t rs = (size_t)K * 2 + pad;
+  for (int i = threadIdx.x; i < total; i += blockDim.x) {
+    const int m = i / nq, c = i - m * nq;
+    const uint2 w = *reinterpret_cast<const uint2*>(q + (size_t)m * K + 8 * c);
+    const float sc = __uint_as_float((uint32_t)s[(size_t)m * (K / 32) + c / 4] << 23);
+    u32x4_t o;
+    o.x = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w.x, sc, false));
+    o.y = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w.x, sc, true));
+    o.z = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w.y, sc, false));
+    o.w = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w.y, sc, true));
+    *reinterpret_cast<u32x4_t*>(lds + (size_t)m * rs + 16 * c) = o;
+  }
+}
 // the 256 zero bytes that the lanes of positions beyond the step's rows read (a step's fragments lie within 208 bytes)
 __device__ __forceinline__ void mf_zero_bytes(uint8_t* at) {
   if (threadIdx.x < 16) *reinterpret_cast<uint4*>(at + 16 * threadIdx.x) = make_uint4(0, 0, 0, 0);
@@ -423,7 +440,8 @@ __device__ __forceinline__ void mf_up_phase(Step<M>& S, const DecodeArgs& a, uin
   const uint32_t lane = threadIdx.x & 63;
   const int wave = uni((int)(threadIdx.x >> 6));
   constexpr int pad = mf_pad(FMT);
-  mf_stage_rows<false>(mf_smem, a.x, H, M, H, pad);
+  if (a.dsk_xq) mf_stage_rows_q(mf_smem, a.dsk_xq, a.dsk_xs, M, H, pad);
+  else mf_stage_rows<false>(mf_smem, a.x, H, M, H, pad);
   mf_zero_bytes(mf_smem + (size_t)M * ((size_t)H * 2 + pad));
   __syncthreads();
   // Units are (slot, tile of 8 channels), numbered slot-major; workgroup g of G walks the units g, g + G, g + 2 G, ...
