@@ -314,6 +314,23 @@ __device__ __forceinline__ uint32_t wave_min_u32(uint32_t v) {
   return min(r[0], r[1]);
 }
 
+// wave-wide maximum of unsigned ints, valid in every lane
+__device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
+  v = max(v, dpp_mov<0xB1>(v));
+  v = max(v, dpp_mov<0x4E>(v));
+  v = max(v, dpp_mov<0x141>(v));
+  v = max(v, dpp_mov<0x140>(v));
+  auto r = __builtin_amdgcn_permlane16_swap(v, v, false, false);
+  v = max(r[0], r[1]);
+  r = __builtin_amdgcn_permlane32_swap(v, v, false, false);
+  return max(r[0], r[1]);
+}
+// a float's bits as an unsigned int of the same order (no NaNs; -0 does not occur: a score is never negative zero)
+__device__ __forceinline__ uint32_t f32_order_bits(float f) {
+  const uint32_t b = __float_as_uint(f);
+  return (b & 0x80000000u) ? ~b : (b | 0x80000000u);
+}
+
 // One row by one wavefront: experts e = lane + 64 j, j < NJ (E <= 64 NJ). Lane k < topk gets pick k's expert and
 // weight (route_warp of the reference, engine/experts/formats.cuh:207-247, at 64 lanes): descending key (float
 // compares), ties to the lower id; the sum in the butterfly order ((p0+p4)+(p2+p6))+((p1+p5)+(p3+p7)), absent places
@@ -335,15 +352,18 @@ __device__ __forceinline__ void route_fetch(const float* __restrict__ row, int E
 template <int NJ>
 __device__ __forceinline__ void route_row_nj(const float (&logit)[kRouteRJ], const float (&bias)[kRouteRJ], int E, int topk, float scale,
                                              int score_fn, int lane, int& id_out, float& w_out) {
-  constexpr float kDead = -__builtin_inff();
-  float s[NJ], key[NJ];
+  // The keys are compared as unsigned ints of the floats' order (f32_order_bits): the wave-wide maximum is then one
+  // instruction a step, a third of the float form's (which re-canonicalises its operands). 0 is below every key.
+  constexpr uint32_t kDead = 0u;
+  float s[NJ];
+  uint32_t key[NJ];
   int jj[NJ];
 #pragma unroll
   for (int j = 0; j < NJ; ++j) {
     s[j] = 0.f, key[j] = kDead, jj[j] = j;  // an empty place never wins
     if (lane + kWave * j < E) {
       s[j] = route_score(logit[j], score_fn);
-      key[j] = __fadd_rn(s[j], bias[j]);
+      key[j] = f32_order_bits(__fadd_rn(s[j], bias[j]));
     }
   }
   // odd-even transposition: NJ passes of adjacent exchanges, strictly-greater only (equal keys keep their j order)
@@ -352,7 +372,8 @@ __device__ __forceinline__ void route_row_nj(const float (&logit)[kRouteRJ], con
 #pragma unroll
     for (int j = pass & 1; j + 1 < NJ; j += 2) {
       const bool sw = key[j + 1] > key[j];
-      const float k0 = key[j], s0 = s[j];
+      const uint32_t k0 = key[j];
+      const float s0 = s[j];
       const int j0 = jj[j];
       key[j] = sw ? key[j + 1] : k0, s[j] = sw ? s[j + 1] : s0, jj[j] = sw ? jj[j + 1] : j0;
       key[j + 1] = sw ? k0 : key[j + 1], s[j + 1] = sw ? s0 : s[j + 1], jj[j + 1] = sw ? j0 : jj[j + 1];
@@ -362,7 +383,7 @@ __device__ __forceinline__ void route_row_nj(const float (&logit)[kRouteRJ], con
   int my_id = 0;
 #pragma unroll 1
   for (int k = 0; k < topk; ++k) {
-    const float top = wave_max_f32(key[0]);
+    const uint32_t top = wave_max_u32(key[0]);
     const uint64_t hit = __ballot(key[0] == top);
     int wl = __builtin_ctzll(hit);
     if (hit & (hit - 1)) wl = wave_min_u32(key[0] == top ? (uint32_t)(lane + kWave * jj[0]) : 0xFFFFFFFFu) & (kWave - 1);

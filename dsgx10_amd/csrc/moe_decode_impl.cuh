@@ -105,8 +105,8 @@ struct Slot {
 };
 template <int M>
 struct Step {
+  alignas(16) uint32_t mask[DSGX_MAX_EXPERTS / 32];  // the picked experts (read 16 bytes at a time)
   int n;                               // distinct picked experts
-  uint32_t mask[DSGX_MAX_EXPERTS / 32];
   int ri[M * DSGX_MAX_TOPK];
   float rw[M * DSGX_MAX_TOPK];
   float wslot[M * DSGX_MAX_TOPK][M];   // per slot the rows' routing weights (0: the row did not pick it)
@@ -225,10 +225,23 @@ __device__ __forceinline__ void resolve(Step<M>& S, const DecodeArgs& a, int rw,
     return;
   }
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+  // the mask in every lane's registers (four 16-byte reads in flight together, not a chain of dependent ones)
+  constexpr int NW = DSGX_MAX_EXPERTS / 32;
+  static_assert(NW % 4 == 0, "the mask is read 16 bytes at a time");
+  uint32_t mk[NW];
+#pragma unroll
+  for (int j = 0; j < NW; j += 4) {
+    const u32x4_t q = *reinterpret_cast<const u32x4_t*>(&S.mask[j]);
+    mk[j] = q.x, mk[j + 1] = q.y, mk[j + 2] = q.z, mk[j + 3] = q.w;
+  }
   for (int i = lane; i < ne; i += kWave) {
     const int e = S.ri[i];
-    int r = __popc(S.mask[e >> 5] & ((1u << (e & 31)) - 1));
-    for (int j = 0; j < (e >> 5); ++j) r += __popc(S.mask[j]);
+    int r = 0;  // the picks below e: its slot
+#pragma unroll
+    for (int j = 0; j < NW; ++j) {
+      const uint32_t below = j < (e >> 5) ? 0xFFFFFFFFu : j == (e >> 5) ? (1u << (e & 31)) - 1 : 0u;
+      r += __popc(mk[j] & below);
+    }
     S.wslot[r][i / topk] = S.rw[i];
     // the routed slot (rows that picked the same expert write the same values)
     Slot t;
@@ -242,7 +255,8 @@ __device__ __forceinline__ void resolve(Step<M>& S, const DecodeArgs& a, int rw,
   }
   if (lane == 0) {
     int n = 0;
-    for (int j = 0; j < DSGX_MAX_EXPERTS / 32; ++j) n += __popc(S.mask[j]);
+#pragma unroll
+    for (int j = 0; j < NW; ++j) n += __popc(mk[j]);
     S.n = n;
   }
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
