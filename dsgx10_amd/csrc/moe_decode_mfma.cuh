@@ -346,18 +346,11 @@ __device__ __forceinline__ void mf_stream(uint8_t* smem, size_t rows_bytes, uint
   if (ns > 1 && mine < rounds) __syncthreads();  // (the last round has no unit for this group)
 }
 
-template <int FMT, int SHFMT, int M>
-__device__ __forceinline__ void mf_setup(Step<M>& S, const DecodeArgs& a) {
-  constexpr int NR = resolver_waves<M>();
-  const int wave = uni((int)(threadIdx.x >> 6)), nw = blockDim.x >> 6;
-  ResolveRegs rr;
-  if (wave >= nw - NR) resolve_fetch(S, a, wave - (nw - NR), NR, rr);
-  prep<FMT, SHFMT, M>(S, a);
-  __syncthreads();
-  if (wave >= nw - NR) resolve<FMT, SHFMT, M>(S, a, wave - (nw - NR), NR, rr);
-  __syncthreads();
-}
-
+// UP: the launch has a gate/up phase: the activation rows are staged with the set-up's other loads, and with a shared
+// expert in another format (INT4 or MXFP4 experts) its first tiles - tile g by workgroup g - stream while the routing is
+// being resolved (mf_shared_early), when nothing else could.
+template <int FMT, int SHFMT, int M, bool UP>
+__device__ __forceinline__ void mf_setup(Step<M>& S, const DecodeArgs& a, uint8_t* mf_smem);
 // A unit of a gate/up matrix pair in format F: tile t = channels 8 t .. 8 t + 7, unit rows 2 c and 2 c + 1 gate and up of
 // channel 8 t + c. (BF16: the shared expert's interleaved matrix, whose rows already come in this order.)
 template <int F>
@@ -431,6 +424,110 @@ __device__ __forceinline__ MfUnit mf_open_down(const Slot& T, int t, int H, int 
   return q;
 }
 
+// The gate/up epilogue of a unit's complete sums (v4f of lane l: gate, up of channel 8 t + 2 (l / 16) and of the next,
+// activation row l % 16): SwiGLU and the store of h
+template <int SHFMT, int M>
+__device__ __forceinline__ void mf_up_store(Step<M>& S, const DecodeArgs& a, int sl, int t, v4f_t sum, uint32_t lane) {
+  constexpr int nsh = SHFMT != 0 ? 1 : 0;
+  const int I = a.L.I;
+  const int pos = lane & 15, part = lane >> 4;
+  if (pos >= M) return;
+  const Slot& T = S.slots[sl];
+  const float sg = T.g.s2, su = T.u.s2;
+  uint32_t h0, h1;
+  if (a.dsk) {
+    // ds41f engine/kernels/moe.cu:519-528: gate and up rounded to bf16, up clamped to +-limit and gate from above,
+    // silu(gate) * up, times the row's routing weight (routed slots), rounded to bf16; quantised per 32 when the down
+    // phase stages it
+    auto hd = [&](float gs, float us) {
+      float gt = bf16_round(gs), up = bf16_round(us);
+      up = fminf(fmaxf(up, -a.dsk_limit), a.dsk_limit);
+      gt = fminf(gt, a.dsk_limit);
+      float h = __fmul_rn(__fdiv_rn(gt, __fadd_rn(1.f, expf(-gt))), up);
+      if (!T.shared) h = __fmul_rn(S.wslot[sl - nsh][pos], h);
+      return f32_to_bf16_bits(h);
+    };
+    h0 = hd(sum[0], sum[1]), h1 = hd(sum[2], sum[3]);
+  } else {
+    h0 = swiglu_bits(bf16_round(__fmul_rn(sum[0], sg)), bf16_round(__fmul_rn(sum[1], su)));
+    h1 = swiglu_bits(bf16_round(__fmul_rn(sum[2], sg)), bf16_round(__fmul_rn(sum[3], su)));
+  }
+  uint16_t* dst = a.h + ((size_t)T.hslot * M + pos) * I + 8 * t + 2 * part;
+  __hip_atomic_store((DSGX_GLOBAL uint32_t*)(uintptr_t)dst, h0 | (h1 << 16), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// The shared expert's gate/up tile `blockIdx.x` (if there is one) between the set-up's two barriers, by the waves that do
+// not resolve the routing (the first four at most): a wave a K slice at a time, the slices of mf_slices as in the main
+// stream, their sums left in LDS; mf_shared_early_finish, after the second barrier, adds them in slice order and stores h:
+// the bits of the main stream. No workgroup barrier inside (mf_stream with one slice a unit has none).
+#ifndef DSGX_MF_EARLY
+#define DSGX_MF_EARLY 1
+#endif
+__host__ __device__ inline int mf_early_tiles(int I, int G) { return DSGX_MF_EARLY ? (I / 8 < G ? I / 8 : G) : 0; }
+template <int FMT, int SHFMT, int M>
+__device__ __forceinline__ void mf_shared_early(Step<M>& S, const DecodeArgs& a, uint8_t* mf_smem) {
+  constexpr int F = SHFMT, pad = mf_pad(FMT);
+  const int H = a.L.H, I = a.L.I, t = blockIdx.x;
+  if (t >= mf_early_tiles(I, gridDim.x)) return;
+  const uint32_t lane = threadIdx.x & 63;
+  const int wave = uni((int)(threadIdx.x >> 6));
+  const int ns = mf_slices(H, MfFmt<F>::STEPK, MfFmt<F>::MINSTEPS), KS = H / ns, act = ns < 4 ? ns : 4;
+  if (wave >= act) return;
+  const size_t rows_bytes = mf_rows_bytes(M, H, pad);
+  float* red = reinterpret_cast<float*>(mf_smem + rows_bytes + kMfWaves * 2048);
+  // mf_stream's unit u of this wave (u = wave, wave + 8, ...) is K slice wave + act (u / 8)
+  auto slice_of = [&](int u) { return (u & 7) + act * (u >> 3); };
+  auto open = [&](int u) { return mf_open_up<F>(S.slots[0], t, H, I, slice_of(u) * KS, lane); };
+  auto xoff = [&](int u) { return (uint32_t)(slice_of(u) * KS * 2); };
+  auto fin = [&](int u, v4f_t sum) {
+    const int pos = lane & 15, part = lane >> 4;
+    if (pos < M) *reinterpret_cast<v4f_t*>(red + ((size_t)slice_of(u) * 4 * M + part * M + pos) * 4) = sum;
+  };
+  mf_stream<F, M>(mf_smem, rows_bytes, (uint32_t)(M * ((size_t)H * 2 + pad)), pad, H, 0, 1, kMfWaves * (ns / act), KS / MfFmt<F>::STEPK, open, xoff, fin,
+                  [] {});
+}
+template <int FMT, int SHFMT, int M>
+__device__ __forceinline__ void mf_shared_early_finish(Step<M>& S, const DecodeArgs& a, uint8_t* mf_smem) {
+  constexpr int F = SHFMT, pad = mf_pad(FMT);
+  const int H = a.L.H, I = a.L.I, t = blockIdx.x;
+  if (t >= mf_early_tiles(I, gridDim.x) || threadIdx.x >= 64) return;
+  const uint32_t lane = threadIdx.x;
+  const int ns = mf_slices(H, MfFmt<F>::STEPK, MfFmt<F>::MINSTEPS);
+  const float* red = reinterpret_cast<const float*>(mf_smem + mf_rows_bytes(M, H, pad) + kMfWaves * 2048);
+  const int pos = lane & 15, part = lane >> 4;
+  v4f_t sum = {0.f, 0.f, 0.f, 0.f};
+  if (pos < M)
+    for (int w = 0; w < ns; ++w) sum += *reinterpret_cast<const v4f_t*>(red + ((size_t)w * 4 * M + part * M + pos) * 4);
+  mf_up_store<SHFMT, M>(S, a, 0, t, sum, lane);
+}
+template <int FMT, int SHFMT, int M, bool UP>
+__device__ __forceinline__ void mf_setup(Step<M>& S, const DecodeArgs& a, uint8_t* mf_smem) {
+  constexpr int NR = resolver_waves<M>();
+#ifndef DSGX_MF_EARLY_SAME
+#define DSGX_MF_EARLY_SAME 1
+#endif
+  constexpr bool EARLY = UP && SHFMT != 0 && (SHFMT != FMT || DSGX_MF_EARLY_SAME);
+  const int wave = uni((int)(threadIdx.x >> 6)), nw = blockDim.x >> 6;
+  ResolveRegs rr;
+  if (wave >= nw - NR) resolve_fetch(S, a, wave - (nw - NR), NR, rr);
+  prep<FMT, SHFMT, M>(S, a);
+  if constexpr (UP) {
+    constexpr int pad = mf_pad(FMT);
+    const int H = a.L.H;
+    if (a.dsk_xq) mf_stage_rows_q(mf_smem, a.dsk_xq, a.dsk_xs, M, H, pad);
+    else mf_stage_rows<false>(mf_smem, a.x, H, M, H, pad);
+    mf_zero_bytes(mf_smem + (size_t)M * ((size_t)H * 2 + pad));
+  }
+  __syncthreads();
+  if (wave >= nw - NR) resolve<FMT, SHFMT, M>(S, a, wave - (nw - NR), NR, rr);
+  else if constexpr (EARLY) mf_shared_early<FMT, SHFMT, M>(S, a, mf_smem);
+  __syncthreads();
+  if constexpr (EARLY) {
+    mf_shared_early_finish<FMT, SHFMT, M>(S, a, mf_smem);
+    __syncthreads();  // (the slices' sums are read: the main stream reuses their LDS)
+  }
+}
+
 // SHFMT: 0 (no fused shared expert), FMT (slot 0 streams with the routed slots) or another format (slot 0 first, in a
 // stream of its own)
 template <int FMT, int SHFMT, int M>
@@ -440,52 +537,25 @@ __device__ __forceinline__ void mf_up_phase(Step<M>& S, const DecodeArgs& a, uin
   const uint32_t lane = threadIdx.x & 63;
   const int wave = uni((int)(threadIdx.x >> 6));
   constexpr int pad = mf_pad(FMT);
-  if (a.dsk_xq) mf_stage_rows_q(mf_smem, a.dsk_xq, a.dsk_xs, M, H, pad);
-  else mf_stage_rows<false>(mf_smem, a.x, H, M, H, pad);
-  mf_zero_bytes(mf_smem + (size_t)M * ((size_t)H * 2 + pad));
-  __syncthreads();
+  // (the activation rows are in LDS: mf_setup)
   // Units are (slot, tile of 8 channels), numbered slot-major; workgroup g of G walks the units g, g + G, g + 2 G, ...
   // (with as many tiles a slot as workgroups that is one tile of every slot; with fewer, a narrow intermediate size, the
   // workgroups still share the slots' tiles evenly)
   const int tiles = I / 8;
-  auto done = [&](int sl, int t, v4f_t sum) {
-    const int pos = lane & 15, part = lane >> 4;
-    if (pos >= M) return;
-    const Slot& T = S.slots[sl];
-    const float sg = T.g.s2, su = T.u.s2;
-    uint32_t h0, h1;
-    if (a.dsk) {
-      // ds41f engine/kernels/moe.cu:519-528: gate and up rounded to bf16, up clamped to +-limit and gate from above,
-      // silu(gate) * up, times the row's routing weight (routed slots), rounded to bf16; quantised per 32 when the down
-      // phase stages it
-      auto hd = [&](float gs, float us) {
-        float gt = bf16_round(gs), up = bf16_round(us);
-        up = fminf(fmaxf(up, -a.dsk_limit), a.dsk_limit);
-        gt = fminf(gt, a.dsk_limit);
-        float h = __fmul_rn(__fdiv_rn(gt, __fadd_rn(1.f, expf(-gt))), up);
-        if (!T.shared) h = __fmul_rn(S.wslot[sl - nsh][pos], h);
-        return f32_to_bf16_bits(h);
-      };
-      h0 = hd(sum[0], sum[1]), h1 = hd(sum[2], sum[3]);
-    } else {
-      h0 = swiglu_bits(bf16_round(__fmul_rn(sum[0], sg)), bf16_round(__fmul_rn(sum[1], su)));
-      h1 = swiglu_bits(bf16_round(__fmul_rn(sum[2], sg)), bf16_round(__fmul_rn(sum[3], su)));
-    }
-    uint16_t* dst = a.h + ((size_t)T.hslot * M + pos) * I + 8 * t + 2 * part;
-    __hip_atomic_store((DSGX_GLOBAL uint32_t*)(uintptr_t)dst, h0 | (h1 << 16), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  };
-  auto run = [&](auto fmt_tag, int s0, int nslots, int g, int G) {  // slots s0 .. s0 + nslots - 1 in format F, by workgroup g of G
+  auto done = [&](int sl, int t, v4f_t sum) { mf_up_store<SHFMT, M>(S, a, sl, t, sum, lane); };
+  // slots s0 .. s0 + nslots - 1 in format F, from the first slot's tile t0 on, by workgroup g of G
+  auto run = [&](auto fmt_tag, int s0, int nslots, int g, int G, int t0) {
     constexpr int F = decltype(fmt_tag)::value;
-    const int total = nslots * tiles;
+    const int total = nslots * tiles - t0;
     const int mine = uni(g < total ? (total - g + G - 1) / G : 0);  // this workgroup's units
     if (mine == 0) return;  // (the same for every wave of the workgroup)
     const int ns = mf_slices(H, MfFmt<F>::STEPK, MfFmt<F>::MINSTEPS), KS = H / ns, k0 = (wave % ns) * KS;
     auto open = [&](int u) {
-      const int q = g + u * G, sl = uni(q / tiles);
+      const int q = t0 + g + u * G, sl = uni(q / tiles);
       return mf_open_up<F>(S.slots[s0 + sl], q - sl * tiles, H, I, k0, lane);
     };
     auto fin = [&](int u, v4f_t sum) {
-      const int q = g + u * G, sl = uni(q / tiles);
+      const int q = t0 + g + u * G, sl = uni(q / tiles);
       done(s0 + sl, q - sl * tiles, sum);
     };
     mf_stream<F, M>(mf_smem, mf_rows_bytes(M, H, pad), (uint32_t)(M * ((size_t)H * 2 + pad)), pad, H, k0, ns, mine, KS / MfFmt<F>::STEPK, open,
@@ -502,12 +572,15 @@ __device__ __forceinline__ void mf_up_phase(Step<M>& S, const DecodeArgs& a, uin
 #endif
     constexpr float kShCost = FMT == DSGX_FMT_INT4_G32 ? DSGX_MF_SHCOST : 1.f;  // (only the INT4 stream waits for the vector unit)
     auto bpv = [](int f) { return f == DSGX_FMT_BF16 ? 2.f : f == DSGX_FMT_FP8_B128 || f == DSGX_FMT_FP8_B32E ? 1.f : 0.5703f; };  // bytes a value
-    const float bsh = bpv(SHFMT), bro = kShCost * (float)nrouted * bpv(FMT);
-    const int nshw = uni(nrouted > 0 ? max(1, min(G - 1, (int)((float)G * bsh / (bsh + bro) + 0.5f))) : G);
-    if (g < nshw) run(std::integral_constant<int, SHFMT>{}, 0, 1, g, nshw);
-    else run(std::integral_constant<int, FMT>{}, 1, nrouted, g - nshw, G - nshw);
+    // (the shared slot's first tiles were done while the routing was being resolved: mf_shared_early)
+    const int t0 = mf_early_tiles(I, G);
+    const float bsh = bpv(SHFMT) * (float)(tiles - t0) / (float)tiles, bro = kShCost * (float)nrouted * bpv(FMT);
+    const int nshw = uni(t0 == tiles ? 0 : nrouted > 0 ? max(1, min(G - 1, (int)((float)G * bsh / (bsh + bro) + 0.5f))) : G);
+    if (g < nshw) run(std::integral_constant<int, SHFMT>{}, 0, 1, g, nshw, t0);
+    else if (nrouted > 0) run(std::integral_constant<int, FMT>{}, 1, nrouted, g - nshw, G - nshw, 0);
   } else {
-    if (nsh + nrouted > 0) run(std::integral_constant<int, FMT>{}, 0, nsh + nrouted, g, G);
+    const int t0 = nsh && DSGX_MF_EARLY_SAME ? mf_early_tiles(I, G) : 0;
+    if (nsh + nrouted > 0) run(std::integral_constant<int, FMT>{}, 0, nsh + nrouted, g, G, t0);
   }
   // the wave's h stores are complete before it goes on to the grid barrier (see up_phase)
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -588,14 +661,14 @@ template <int FMT, int SHFMT, int M>
 __global__ void __launch_bounds__(kMfThreads) k_up_mfma(DecodeArgs a) {
   extern __shared__ uint8_t mf_smem[];
   __shared__ Step<M> S;
-  mf_setup<FMT, SHFMT, M>(S, a);
+  mf_setup<FMT, SHFMT, M, true>(S, a, mf_smem);
   mf_up_phase<FMT, SHFMT, M>(S, a, mf_smem);
 }
 template <int FMT, int SHFMT, int M>
 __global__ void __launch_bounds__(kMfThreads) k_down_mfma(DecodeArgs a) {
   extern __shared__ uint8_t mf_smem[];
   __shared__ Step<M> S;
-  mf_setup<FMT, SHFMT, M>(S, a);
+  mf_setup<FMT, SHFMT, M, false>(S, a, mf_smem);
   mf_down_phase<FMT, SHFMT, M, false>(S, a, mf_smem);
 }
 // Both phases in one launch, a grid barrier between them (every workgroup resident: one a CU); the step's set-up runs once
@@ -604,7 +677,7 @@ __global__ void __launch_bounds__(kMfThreads) k_decode_mfma(DecodeArgs a) {
   extern __shared__ uint8_t mf_smem[];
   __shared__ Step<M> S;
   if (threadIdx.x == 0) S.gen = grid_barrier_gen(a.bar);
-  mf_setup<FMT, SHFMT, M>(S, a);
+  mf_setup<FMT, SHFMT, M, true>(S, a, mf_smem);
   mf_up_phase<FMT, SHFMT, M>(S, a, mf_smem);
   mf_down_phase<FMT, SHFMT, M, true>(S, a, mf_smem);
 }
