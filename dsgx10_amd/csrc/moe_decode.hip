@@ -113,6 +113,49 @@ int dsgx_moe_decode(const dsgx_layer_w* L, const uint16_t* x, const int* idx, co
 }
 }  // extern "C"
 
+// up = DSGX_UP_PREFILL_ORDER (the reference's kUpPrefillOrder, experts.h:111-113, 138): the rows go through the prefill
+// kernels as a chunk of M rows (bf16 activations), so yr and ys are moe_prefill's bit for bit - for callers that verify
+// drafted tokens against a prefill of the same rows. The chunk's intermediates take the h part of the workspace (in
+// dsgx_prefill_view's layout, not the decode step's slots); the barrier's words behind it are left alone.
+namespace {
+__global__ void __launch_bounds__(256) k_ysum(float* __restrict__ yr, const float* __restrict__ ys, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) yr[i] = __fadd_rn(yr[i], ys[i]);
+}
+}  // namespace
+static int decode_by_prefill(const dsgx_layer_w* L, const uint16_t* x, const int* idx, const float* w, int M, void* ws, const WsLayout& lay,
+                             float* yr, float* ys, void* stream, const dsgx_decode_cfg& c, bool dsk) {
+  if (dsk) return fail(DSGX_EUNSUPPORTED, "dsk_moe: no prefill-order variant");
+  if (c.parts != 3) return fail(DSGX_EUNSUPPORTED, "moe_decode: the prefill-order variant runs both phases (parts 3), not %d", c.parts);
+  if (!yr) return fail(DSGX_EINVAL, "moe_decode: null yr");
+  if (L->E < 1 || L->E > DSGX_MAX_EXPERTS || L->topk < 1 || L->topk > DSGX_MAX_TOPK || L->topk > L->E)
+    return fail(DSGX_EINVAL, "moe_decode: E %d, top-k %d", L->E, L->topk);
+  const size_t pick_bytes = (size_t)DSGX_MAX_ROWS * DSGX_MAX_TOPK * 4, need = dsgx_prefill_ws_bytes(L, M);
+  if (need == 0) return DSGX_EINVAL;  // (dsgx_prefill_ws_bytes has said why)
+  const size_t tail = (need + 255) / 256 * 256;
+  if (tail + 2 * pick_bytes > lay.bar_off())
+    return fail(DSGX_EUNSUPPORTED, "moe_decode: the prefill-order variant needs %zu bytes of the workspace's %zu in front of the barrier's words", tail + 2 * pick_bytes,
+                lay.bar_off());
+  uint8_t* W = static_cast<uint8_t*>(ws);
+  if (c.logits) {  // the routing's picks behind the chunk's intermediates
+    int* ri = reinterpret_cast<int*>(W + tail);
+    float* rw = reinterpret_cast<float*>(W + tail + pick_bytes);
+    if (int rc = dsgx_route(c.logits, c.bias, M, L->E, L->topk, c.route_scale, c.score_fn, ri, rw, stream)) return rc;
+    idx = ri, w = rw;
+  }
+  dsgx_prefill_cfg p;
+  dsgx_prefill_cfg_default(&p);
+  p.act_fp8 = 0;
+  if (int rc = dsgx_moe_prefill(L, x, idx, w, M, ws, yr, ys, stream, &p)) return rc;
+  if (c.ysum) {
+    if (!ys) return fail(DSGX_EINVAL, "moe_decode: ysum without ys");
+    const int n = M * L->H;
+    hipLaunchKernelGGL(k_ysum, dim3((n + 255) / 256), dim3(256), 0, static_cast<hipStream_t>(stream), yr, ys, n);
+    DSGX_HIP(hipGetLastError());
+  }
+  return DSGX_OK;
+}
+
 static int moe_decode_at(const dsgx_layer_w* L, const uint16_t* x, const int* idx, const float* w, int M, void* ws, const WsLayout& lay,
                          float* yr, float* ys, void* stream, const dsgx_decode_cfg* cfg, DskIn dsk) {
   dsgx_decode_cfg c;
@@ -124,6 +167,7 @@ static int moe_decode_at(const dsgx_layer_w* L, const uint16_t* x, const int* id
   if (!c.logits && (!idx || !w)) return fail(DSGX_EINVAL, "moe_decode: idx and w, or logits");
   if (c.post) return fail(DSGX_EUNSUPPORTED, "moe_decode: posted outputs need the reference's ring; one GPU has none");
   if (c.parts < 1 || c.parts > 3) return fail(DSGX_EINVAL, "moe_decode: parts %d", c.parts);
+  if (c.up == DSGX_UP_PREFILL_ORDER) return decode_by_prefill(L, x, idx, w, M, ws, lay, yr, ys, stream, c, dsk.on != 0);
   if (c.up < -1 || c.up > 1 || c.down < 0 || c.down > 1) return fail(DSGX_EINVAL, "moe_decode: up variant %d / down variant %d", c.up, c.down);
   if (c.up == -1) c.up = c.down == 1 ? 0 : decode_variant(L->fmt, M, L->H, L->I);  // (the two-launch form is the vector-unit kernels')
   if (c.up == 1 && L->fmt != DSGX_FMT_FP8_B128 && L->fmt != DSGX_FMT_INT4_G32 && L->fmt != DSGX_FMT_MXFP4_G32)

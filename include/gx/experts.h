@@ -73,9 +73,9 @@ inline void route(const float* logits, const float* bias, int M, int* idx, float
 
 // ---- decode (experts.h:104-147) -----------------------------------------------------------------------------------
 // The reference's variant numbers name its launch shapes (decode.cu:624-698); here up / down are this build's variants
-// (dsgx_decode_cfg). kUpPrefillOrder (experts.h:111-113,138: decode = prefill bit for bit) has no counterpart yet and is
-// refused by name rather than mapped to something else.
-constexpr int kUpPrefillOrder = 6;
+// (dsgx_decode_cfg). kUpPrefillOrder (experts.h:111-113,138: decode = prefill bit for bit) keeps its number and its
+// promise: the rows go through the prefill kernels (DSGX_UP_PREFILL_ORDER).
+constexpr int kUpPrefillOrder = DSGX_UP_PREFILL_ORDER;
 struct DecodeCfg {
   int up = -1, down = 0;   // up -1: the faster variant for the layer's format and the row count
   int up_ctas_per_sm = 0;  // accepted, unused: the grid is sized to the chip
@@ -95,7 +95,6 @@ inline size_t decode_ws_bytes(const LayerW& L) { const dsgx_layer_w c = L.c(); r
 inline size_t decode_ws_bytes() { return decode_ws_bytes(LayerW()); }
 inline void moe_decode(const LayerW& L, const uint16_t* x, const int* idx, const float* w, int M, void* ws, float* yr, float* ys,
                        void* st, const DecodeCfg& cfg = DecodeCfg()) {
-  if (cfg.up == kUpPrefillOrder) die("moe_decode: up variant %d (decode in the prefill kernels' order of adds) is not built", cfg.up);
   const dsgx_layer_w c = L.c();
   dsgx_decode_cfg d;
   dsgx_decode_cfg_default(&d);

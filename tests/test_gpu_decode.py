@@ -230,3 +230,43 @@ def test_decode_variant1_narrow_shapes_and_fp8_shared_beside_int4(fmt, H, I, E, 
     if fmt == abi.FMT_INT4 and shared == "fp8":
         with pytest.raises(lib.DsgxError):
             gpu.decode_layer(dl, x[:1], idx[:1], w[:1], 1, up=0)
+
+
+@pytest.mark.parametrize("fmt,H,I,E,topk,shared,scale", [(abi.FMT_FP8, 2048, 1024, 32, 8, "fp8", 1.0), (abi.FMT_INT4, 2048, 2048, 16, 8, "bf16", 2.5),
+                                                       (abi.FMT_FP8, 1024, 1024, 8, 2, None, 1.0)],
+                         ids=["fp8", "int4", "fp8-no-shared"])
+def test_decode_prefill_order_variant(fmt, H, I, E, topk, shared, scale):
+    """cfg.up = 6 (the reference's kUpPrefillOrder, experts.h:111-113, 138: "their h, yr and ys equal moe_prefill's bit for
+    bit"): the decode call's yr and ys are dsgx_moe_prefill's of the same rows (bf16 activations), at 1, 5 and 16 rows,
+    with the picks given and with the routing fused; ysum adds ys once; the outputs meet the decode oracle's bar like any
+    variant's, and the step's barrier words survive (a fused step on the same workspace follows)."""
+    hl, dl = _layer(fmt, H, I, E, topk, 4, shared)
+    x, logits, idx, w = rows_and_routing(29, 16, H, E, topk, scale)
+    ws = gpu.empty(lib.decode_ws_bytes(dl.w), 0)
+    for M in (1, 5, 16):
+        yr, ys, _ = gpu.decode_layer(dl, x[:M], idx[:M], w[:M], M, ws=ws, up=abi.UP_PREFILL_ORDER)
+        pws = gpu.empty(lib.prefill_ws_bytes(dl.w, M), 0)
+        pyr, pys = gpu.empty(M * H * 4, 0xFF), gpu.empty(M * H * 4, 0xFF)
+        lib.moe_prefill(dl.w, gpu.dev(x[:M]), gpu.dev(idx[:M]), gpu.dev(w[:M]), M, pws, pyr, pys, act_fp8=False)
+        assert np.array_equal(yr.view(np.uint32), gpu.host(pyr, np.uint32, (M, H)))
+        if hl.has_shared:
+            assert np.array_equal(ys.view(np.uint32), gpu.host(pys, np.uint32, (M, H)))
+        # the decode oracle's bar
+        uni = orc.union(idx[:M], E)
+        up = orc.moe_up(hl, x[:M], uni)
+        full = orc.moe_down(hl, up["h32"], idx[:M], w[:M], uni)
+        assert rel_l2(yr, full["yr32"]) < 1e-3 and np.abs(yr - full["yr32"]).max() < 2e-2
+        if hl.has_shared:
+            assert rel_l2(ys, full["ys32"]) < 1e-3
+        # the routing fused, and ysum
+        yl, sl, _ = gpu.decode_layer(dl, x[:M], None, None, M, ws=ws, up=abi.UP_PREFILL_ORDER, logits=gpu.dev(logits[:M]), route_scale=scale)
+        assert np.array_equal(yl.view(np.uint32), yr.view(np.uint32))
+        if hl.has_shared:
+            ysum, _, _ = gpu.decode_layer(dl, x[:M], idx[:M], w[:M], M, ws=ws, up=abi.UP_PREFILL_ORDER, ysum=True)
+            assert np.array_equal(ysum, yr + ys)
+    # the default step on the same workspace afterwards
+    y0, s0, _ = gpu.decode_layer(dl, x[:3], idx[:3], w[:3], 3, ws=ws)
+    y1, s1, _ = gpu.decode_layer(dl, x[:3], idx[:3], w[:3], 3)
+    assert np.array_equal(y0.view(np.uint32), y1.view(np.uint32)) and np.array_equal(s0.view(np.uint32), s1.view(np.uint32))
+    with pytest.raises(lib.DsgxError):
+        gpu.decode_layer(dl, x[:1], idx[:1], w[:1], 1, ws=ws, up=abi.UP_PREFILL_ORDER, parts=1)

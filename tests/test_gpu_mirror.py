@@ -19,7 +19,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 EXE = os.path.join(ROOT, "tests", "mirror_run")
 
 
-@pytest.mark.parametrize("fmt,shared,scale,up", [(abi.FMT_FP8, "fp8", 1.0, -1), (abi.FMT_FP8, "fp8", 1.0, 0), (abi.FMT_INT4, "bf16", 2.5, 1)])
+@pytest.mark.parametrize("fmt,shared,scale,up", [(abi.FMT_FP8, "fp8", 1.0, -1), (abi.FMT_FP8, "fp8", 1.0, 0), (abi.FMT_INT4, "bf16", 2.5, 1), (abi.FMT_FP8, "fp8", 1.0, abi.UP_PREFILL_ORDER)])
 def test_cpp_mirrors_give_the_c_abi_bits(fmt, shared, scale, up):
     assert os.path.exists(EXE), "tests/mirror_run is not built (python -m dsgx10_amd.build)"
     H, I, E, topk, M = 2048, 2048, 32, 8, 3
