@@ -46,7 +46,15 @@ __global__ void __launch_bounds__(256) k_gemv(GemvArgs a) {
   for (int r = 0; r < RB; ++r)
 #pragma unroll
     for (int m = 0; m < M; ++m) acc[r][m] = 0.f;
-  const uint8_t* dummy = a.sg[0].m.w;  // where the loads past the last step go: the first KiB of the first matrix (always there)
+  // where the loads past the last step go: the first 16 bytes of this wave's first row (cached; a line of its own, not one
+  // that every wave of the launch reads)
+  const uint8_t* dummy;
+  {
+    const int row = min(gw * RB, a.total_rows - 1);
+    int si;
+    locate(row, si);
+    dummy = a.sg[si].m.w + (size_t)(row - a.sg[si].row0) * FmtT<FMT>::row_bytes(a.K);
+  }
   int lt = 0, lj = 0, lseg = 0;  // the load cursor: step, batch number of this wave, segment
   auto load = [&](Raw (&r)[RB]) {
     const bool ok = lt < nsteps;
@@ -134,7 +142,8 @@ __global__ void __launch_bounds__(256) k_gemv_sk(GemvArgs a) {
   for (int r = 0; r < RB; ++r)
 #pragma unroll
     for (int m = 0; m < M; ++m) acc[r][m] = 0.f;
-  const uint8_t* dummy = reinterpret_cast<const uint8_t*>(sg.m.w);  // (loads past the last step: the matrix's first bytes)
+  // (loads past the last step: the first 16 bytes of this wave's row)
+  const uint8_t* dummy = reinterpret_cast<const uint8_t*>(sg.m.w) + (size_t)(row - sg.row0) * FmtT<FMT>::row_bytes(a.K);
   int lt = 0;
   auto load = [&](Raw (&r)[RB]) {
     const bool ok = lt < nmine;

@@ -345,14 +345,18 @@ __device__ __forceinline__ void up_body(const DecodeArgs& a, const uint4* xs, co
   };
   RowSrc src[RB];
   int lsl = 0, lp = 0, lseg = 0;
-  bool lvalid = true;
+  bool lvalid = true, opened = false;
   auto open = [&]() {  // the next batch of this wave: the claim issued a batch ago; then claims the one after
     const int k = uni(pending);
     claim();
     if (k >= nk && !resolved) nk = batches_of(wait_nsl()), resolved = true;
     lvalid = k < nk;
-    const int b = lvalid ? g + k * G : 0;  // past the end the ring keeps loading: the first rows of the first slot (cached)
-    lsl = uni(b / nb_e), lp = b - lsl * nb_e, lseg = 0;
+    lseg = 0;
+    // past the end the ring keeps loading: 16 bytes of the wave's last rows (cached, and other lines than the other waves')
+    if (!lvalid && opened) return;
+    opened = true;
+    const int b = lvalid ? g + k * G : 0;
+    lsl = uni(b / nb_e), lp = b - lsl * nb_e;
     const Slot& S = slots[lsl];
     MatRef gr{}, ur{};
     gr.w = uni(S.g.w), gr.s = uni(S.g.s), ur.w = uni(S.u.w), ur.s = uni(S.u.s);
@@ -368,7 +372,7 @@ __device__ __forceinline__ void up_body(const DecodeArgs& a, const uint4* xs, co
       else lseg = 0;
     }
 #pragma unroll
-    for (int i = 0; i < RB; ++i) load_row<FMT>(r[i], src[i], lseg, lane, 7, acc[i][0]);
+    for (int i = 0; i < RB; ++i) load_row<FMT>(r[i], src[i], lvalid ? lseg : 0, lvalid ? lane : 0u, 7, acc[i][0]);
     sl = lsl, p = lp, seg = lvalid ? lseg : -1;
     ++lseg;
   };
@@ -507,17 +511,22 @@ __device__ __forceinline__ void down_phase(const DecodeArgs& a, uint4* hs, Step<
   };
   open(nsub > 0 ? 0 : -1, 0);
   auto load = [&](Raw (&r)[RB]) {
+    // past the wave's last step the ring keeps loading: 16 bytes of its last rows (cached; other lines than other waves')
+    const bool lv = lsub < nsub;
+    const int sg = lv ? lseg : 0;
+    const uint32_t ll = lv ? lane : 0u;
 #pragma unroll
     for (int i = 0; i < RB; ++i) {
-      if (lsh) load_row<SF>(r[i], src[i], lseg, lane, 7, acc[i][0]);
-      else load_row<FMT>(r[i], src[i], lseg, lane, 7, acc[i][0]);
+      if (lsh) load_row<SF>(r[i], src[i], sg, ll, 7, acc[i][0]);
+      else load_row<FMT>(r[i], src[i], sg, ll, 7, acc[i][0]);
     }
-    if (++lseg == (ls < nsh ? segs_s : segs_r)) {
+    if (lv && ++lseg == (ls < nsh ? segs_s : segs_r)) {
       lseg = 0;
       if (++ls == nsl) ls = 0, ++lsub;
-      // past the wave's last step the ring keeps loading: the first rows of every slot in turn (the same for all waves)
-      open(lsub < nsub ? lsub : -1, ls);
-      lsh = kMixed && ls < nsh;
+      if (lsub < nsub) {
+        open(lsub, ls);
+        lsh = kMixed && ls < nsh;
+      }
     }
   };
 #pragma unroll

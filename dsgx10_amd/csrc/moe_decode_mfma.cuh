@@ -225,6 +225,7 @@ __device__ __forceinline__ void mf_stream(uint8_t* smem, size_t rows_bytes, uint
   };
   Entry ring[kMfD];
   int lu = 0, lstep = 0, cu = 0, cstep = 0;
+  bool ltail = false;
   MfUnit cur = open(grp);
   v4f_t acc = {0.f, 0.f, 0.f, 0.f};
   auto load = [&](Entry& e) {
@@ -241,11 +242,22 @@ __device__ __forceinline__ void mf_stream(uint8_t* smem, size_t rows_bytes, uint
     } else if constexpr (FMT == DSGX_FMT_FP8_B32E) {   // the step's four k blocks' ue8m0 bytes of the lane's row block
       e.s = ldg_u32(cur.sp + (size_t)lstep * 4);
     }
-    if (++lstep == steps) {
-      // past the end the ring keeps re-reading the last step (unused, and still in the caches: re-reading the last unit
-      // from its start fetched it from memory again, 2 KB a step and wave)
-      if (lu + 1 < mine) lstep = 0, cur = open(++lu * ng + grp);
-      else lstep = steps - 1;
+    if (!ltail && ++lstep == steps) {
+      lstep = 0;
+      if (lu + 1 < mine) {
+        cur = open(++lu * ng + grp);
+      } else if constexpr (FMT == DSGX_FMT_INT4_G32) {
+        lstep = steps - 1;  // (the INT4 stream waits for the vector unit, not for these loads: whole last steps, measured)
+      } else {
+        // Past the end the ring keeps loading (unused): every lane the first lane's 16 bytes of the last step, which are
+        // still cached - one line a load, and other lines than the other waves'. (Re-reading the last unit from its start
+        // fetched it from memory again, 2 KB a step and wave; whole steps of cached lines still cost the L2 their bytes.)
+        ltail = true;
+        const size_t last = (size_t)(steps - 1);
+        cur.wp = uni(cur.wp + last * 128), cur.half = 0;
+        if constexpr (FMT == DSGX_FMT_FP8_B128 || FMT == DSGX_FMT_FP8_B32E) cur.sp = uni(cur.sp + last * 4);
+        else if constexpr (FMT == DSGX_FMT_MXFP4_G32) cur.sp = uni(cur.sp + last * 8);
+      }
     }
   };
   const uint32_t zsh = cur.zsh;  // (the same for every unit of a stream)

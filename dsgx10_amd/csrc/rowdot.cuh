@@ -52,7 +52,7 @@ __device__ __forceinline__ void load_raw(Raw& r, const MatDev& m, int n, int seg
   const uint8_t* wp = m.w + (size_t)n * F::row_bytes(K) + F::row_bytes(k0);
   const uint8_t* ap = nullptr;
   if constexpr (FMT == DSGX_FMT_FP8_B128) ap = m.s + ((size_t)(n >> m.lrs) * m.srow + (k0 >> m.lks)) * 4;
-  if (dummy) wp = dummy + lane * 16, ap = dummy;
+  if (dummy) wp = ap = dummy;  // (every lane the same 16 bytes: one cache line a load)
   r.v = ldg_stream(pin_after(wp, pin));
   if constexpr (FMT == DSGX_FMT_FP8_B128) {
     r.aux = ldg_u32(ap);
