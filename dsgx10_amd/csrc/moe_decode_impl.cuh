@@ -346,6 +346,8 @@ __device__ __forceinline__ void up_body(const DecodeArgs& a, const uint4* xs, co
   RowSrc src[RB];
   int lsl = 0, lp = 0, lseg = 0;
   bool lvalid = true, opened = false;
+  // (the INT4 stream waits for the vector unit, where the lane offset's select costs more than the tail's cache lines)
+  constexpr bool kTailLine = FMT != DSGX_FMT_INT4_G32;
   auto open = [&]() {  // the next batch of this wave: the claim issued a batch ago; then claims the one after
     const int k = uni(pending);
     claim();
@@ -353,7 +355,7 @@ __device__ __forceinline__ void up_body(const DecodeArgs& a, const uint4* xs, co
     lvalid = k < nk;
     lseg = 0;
     // past the end the ring keeps loading: 16 bytes of the wave's last rows (cached, and other lines than the other waves')
-    if (!lvalid && opened) return;
+    if (kTailLine && !lvalid && opened) return;  // (INT4: the first rows of the first slot, the same for all waves: L1 hits)
     opened = true;
     const int b = lvalid ? g + k * G : 0;
     lsl = uni(b / nb_e), lp = b - lsl * nb_e;
@@ -372,7 +374,7 @@ __device__ __forceinline__ void up_body(const DecodeArgs& a, const uint4* xs, co
       else lseg = 0;
     }
 #pragma unroll
-    for (int i = 0; i < RB; ++i) load_row<FMT>(r[i], src[i], lvalid ? lseg : 0, lvalid ? lane : 0u, 7, acc[i][0]);
+    for (int i = 0; i < RB; ++i) load_row<FMT>(r[i], src[i], lvalid ? lseg : 0, kTailLine && !lvalid ? 0u : lane, 7, acc[i][0]);
     sl = lsl, p = lp, seg = lvalid ? lseg : -1;
     ++lseg;
   };
@@ -513,18 +515,20 @@ __device__ __forceinline__ void down_phase(const DecodeArgs& a, uint4* hs, Step<
   auto load = [&](Raw (&r)[RB]) {
     // past the wave's last step the ring keeps loading: 16 bytes of its last rows (cached; other lines than other waves')
     const bool lv = lsub < nsub;
-    const int sg = lv ? lseg : 0;
-    const uint32_t ll = lv ? lane : 0u;
+    const int sg = lv || FMT == DSGX_FMT_INT4_G32 ? lseg : 0;
+    const uint32_t ll = lv || FMT == DSGX_FMT_INT4_G32 ? lane : 0u;  // (INT4: the select costs its stream more than it saves)
 #pragma unroll
     for (int i = 0; i < RB; ++i) {
       if (lsh) load_row<SF>(r[i], src[i], sg, ll, 7, acc[i][0]);
       else load_row<FMT>(r[i], src[i], sg, ll, 7, acc[i][0]);
     }
-    if (lv && ++lseg == (ls < nsh ? segs_s : segs_r)) {
+    if ((lv || FMT == DSGX_FMT_INT4_G32) && ++lseg == (ls < nsh ? segs_s : segs_r)) {
       lseg = 0;
       if (++ls == nsl) ls = 0, ++lsub;
-      if (lsub < nsub) {
-        open(lsub, ls);
+      // (INT4, past the end: the first rows of every slot in turn, the same for all waves - L1 hits; its stream waits
+      // for the vector unit, where a select a load costs more than those lines)
+      if (lsub < nsub || FMT == DSGX_FMT_INT4_G32) {
+        open(lsub < nsub ? lsub : -1, ls);
         lsh = kMixed && ls < nsh;
       }
     }
@@ -660,15 +664,20 @@ __device__ __forceinline__ void down_part_body(const DecodeArgs& a, uint4* hs, c
     int lsub = 0, lseg = 0, csub = 0, cseg = 0;
     RowSrc src[RB];
     auto open = [&](int sub) {
-      const int n0 = (ta + wave + min(sub, nsub - 1) * nw) * RB;  // (past the end: the last sub-batch again, unused)
+      const int n0 = (ta + wave + sub * nw) * RB;
 #pragma unroll
       for (int i = 0; i < RB; ++i) src[i] = row_src<F>(dm, min(n0 + i, H - 1), I);
     };
     open(0);
     auto load = [&](Raw (&r)[RB]) {
+      // past the end the ring keeps loading (unused): 16 bytes of the wave's last rows, one cache line a load
+      const bool lv = lsub < nsub;
 #pragma unroll
-      for (int i = 0; i < RB; ++i) load_row<F>(r[i], src[i], lseg, lane, 7, acc[i][0]);
-      if (++lseg == segs) lseg = 0, open(++lsub);
+      for (int i = 0; i < RB; ++i) load_row<F>(r[i], src[i], lv ? lseg : 0, lv ? lane : 0u, 7, acc[i][0]);
+      if (lv && ++lseg == segs) {
+        lseg = 0;
+        if (++lsub < nsub) open(lsub);
+      }
     };
     auto compute = [&](const Raw (&r)[RB]) {
       step_dot<F, M, RB>(r, hs, nq, cseg, lane, acc);
