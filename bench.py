@@ -38,7 +38,7 @@ def log(*a):
 # HBM bytes a launch of the FP8 M=1 decode kernel (k_decode), from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs of this
 # script, each scaled by what the counter reads for a kernel of known size in the same run (profiles/): the algorithmic
 # bytes are 226,547,712
-LAYER_TRAFFIC_FP8_M1 = 229050000
+LAYER_TRAFFIC_FP8_M1 = 229540000
 
 
 def prefill_extra(gen, T, name, peak, check=True):
