@@ -671,14 +671,14 @@ __device__ __forceinline__ void mf_down_phase(Step<M>& S, const DecodeArgs& a, u
 
 template <int FMT, int SHFMT, int M>
 __global__ void __launch_bounds__(kMfThreads) k_up_mfma(DecodeArgs a) {
-  extern __shared__ uint8_t mf_smem[];
+  extern __shared__ __attribute__((aligned(16))) uint8_t mf_smem[];  // (read and written 16 bytes at a time)
   __shared__ Step<M> S;
   mf_setup<FMT, SHFMT, M, true>(S, a, mf_smem);
   mf_up_phase<FMT, SHFMT, M>(S, a, mf_smem);
 }
 template <int FMT, int SHFMT, int M>
 __global__ void __launch_bounds__(kMfThreads) k_down_mfma(DecodeArgs a) {
-  extern __shared__ uint8_t mf_smem[];
+  extern __shared__ __attribute__((aligned(16))) uint8_t mf_smem[];  // (read and written 16 bytes at a time)
   __shared__ Step<M> S;
   mf_setup<FMT, SHFMT, M, false>(S, a, mf_smem);
   mf_down_phase<FMT, SHFMT, M, false>(S, a, mf_smem);
@@ -686,7 +686,7 @@ __global__ void __launch_bounds__(kMfThreads) k_down_mfma(DecodeArgs a) {
 // Both phases in one launch, a grid barrier between them (every workgroup resident: one a CU); the step's set-up runs once
 template <int FMT, int SHFMT, int M>
 __global__ void __launch_bounds__(kMfThreads) k_decode_mfma(DecodeArgs a) {
-  extern __shared__ uint8_t mf_smem[];
+  extern __shared__ __attribute__((aligned(16))) uint8_t mf_smem[];  // (read and written 16 bytes at a time)
   __shared__ Step<M> S;
   if (threadIdx.x == 0) S.gen = grid_barrier_gen(a.bar);
   mf_setup<FMT, SHFMT, M, true>(S, a, mf_smem);
