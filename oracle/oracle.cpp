@@ -677,6 +677,39 @@ ORC void orc_moe_prefill_fp8_row_range(const dsgx_layer_w* L, const dsgx_mat_des
   }
 }
 
+// h of one chunk row with every gate and up sum moved inside the reference's own tolerance on such sums: each f64 sum S
+// becomes S + sum_eps * r * sum|terms|, r uniform in [-1, 1) from mix64 (seed, slot, channel, gate / up). What a correct
+// evaluation of the contract that adds its products in another order (or on another unit) may produce; sum_eps = 0 gives
+// the h of the f64 sums. h_out bf16 [topk in expert-id order (+ 1, the shared expert's)][I]. (The rule of the lo / hi
+// range above, A/engine/experts/tests/test_experts.cu:366-407, sampled instead of bracketed.)
+ORC void orc_moe_prefill_fp8_row_h_perturbed(const dsgx_layer_w* L, const dsgx_mat_desc* desc, const uint16_t* x, const int* idx,
+                                             double sum_eps, uint64_t seed, uint16_t* h_out) {
+  const int H = L->H, I = L->I, topk = L->topk;
+  std::vector<uint8_t> xq(H);
+  std::vector<float> xs(H / 128), g, u;
+  std::vector<double> g64, gm, u64, um;
+  orc_act_quant(x, 1, H, xq.data(), xs.data());
+  int ord[8];
+  for (int k = 0; k < topk; ++k) ord[k] = k;
+  std::sort(ord, ord + topk, [&](int a, int b) { return idx[a] < idx[b]; });
+  const int nsl = topk + (sh_fp8(L) ? 1 : 0);
+  const uint64_t key = stream_key(seed, 0x5045525455ull);
+  for (int s = 0; s < nsl; ++s) {
+    const bool sh = s == topk;
+    const int e = sh ? -1 : idx[ord[s]];
+    const Mat G = sh ? shared_mat(L, 0) : expert_mat(L, desc, e, 0);
+    const Mat Uw = sh ? shared_mat(L, 1) : expert_mat(L, desc, e, 1);
+    fp8_row_qdot(G, xq.data(), xs.data(), g, &g64, &gm);
+    fp8_row_qdot(Uw, xq.data(), xs.data(), u, &u64, &um);
+    for (int c = 0; c < I; ++c) {
+      const uint64_t at = 2 * ((uint64_t)s * I + c);
+      const double rg = (double)(mix64(key + at) >> 11) * 0x1p-52 - 1.0, ru = (double)(mix64(key + at + 1) >> 11) * 0x1p-52 - 1.0;
+      const double gg = (g64[c] + sum_eps * rg * gm[c]) * (double)G.s2, uu = (u64[c] + sum_eps * ru * um[c]) * (double)Uw.s2;
+      h_out[(size_t)s * I + c] = f2bf(silu_mul(bfr((float)gg), bfr((float)uu)));
+    }
+  }
+}
+
 // The residual add and RMSNorm after the expert step: A/engine/comm/glmcoll.h:34-62 (allreduce_add_norm at one rank),
 // A/ref/glmref.py:225-228 (rms_norm), :269-276 (add_residual), A/engine/attn/prep.cu:26-34 (rstd and the two roundings).
 // res_out bf16 = the contract's h; xn from mean(h^2) summed in f64 (xn) and in f32 sequentially (xn32).

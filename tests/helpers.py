@@ -78,3 +78,35 @@ def check_outputs(got, ref, bf16_rel=True, stress=False):
     # although the f32 values agree within the bar)
     if bf16_rel:
         assert rel_l2(g16, r16) <= 1e-3
+
+
+def zipf_picks(T, E, topk, s=1.1, seed=4321):
+    """top-k distinct experts a row drawn (without replacement) from a Zipf(s) popularity over a seeded permutation of the
+    experts: the k largest of log p + Gumbel noise; uniform weights 1 / top-k (the bench's prefill input)"""
+    rng = np.random.default_rng(seed)
+    logp = -s * np.log(rng.permutation(E) + 1.0)
+    idx = np.argsort(-(logp[None, :] + rng.gumbel(size=(T, E))), axis=1, kind="stable")[:, :topk]
+    return np.ascontiguousarray(idx, np.int32), np.full((T, topk), 1.0 / topk, np.float32)
+
+
+def prefill_fp8_spread(hl, x, idx, w, rows, eps_list=(0.0, 2e-6, 2e-5, 1e-4)):
+    """How far two correct evaluations of the FP8-activation prefill contract lie apart END TO END on the rows given:
+    the oracle's f32-contract evaluation against evaluations whose gate and up sums are the f64 sums moved by
+    eps * r * sum|terms| (r uniform in [-1, 1); eps = 0: the f64 sums themselves), each then re-quantised to e4m3 and put
+    through the same down projection. Returns {eps: dict(h_equal, rel_r, rel_s, max_abs)} against the f32 contract's
+    outputs: the reference tolerates 2e-5 on such sums for h and 1e-4 for outputs (test_experts.cu:352-407)."""
+    base = [orc.moe_prefill_fp8_row(hl, x[t], idx[t], w[t]) for t in rows]
+    ref_r, ref_s = np.stack([o["yr"] for o in base]), np.stack([o["ys"] for o in base])
+    out = {}
+    for eps in eps_list:
+        got_r, got_s, same, total = [], [], 0, 0
+        for o, t in zip(base, rows):
+            hp = orc.moe_prefill_fp8_row_h_perturbed(hl, x[t], idx[t], eps, seed=1000 + t)
+            same += int((hp == o["h"]).sum())
+            total += hp.size
+            o2 = orc.moe_prefill_fp8_row(hl, x[t], idx[t], w[t], h_in=hp)
+            got_r.append(o2["yr"]), got_s.append(o2["ys"])
+        got_r, got_s = np.stack(got_r), np.stack(got_s)
+        out[eps] = dict(h_equal=same / total, rel_r=rel_l2(got_r, ref_r), rel_s=rel_l2(got_s, ref_s),
+                        max_abs=float(max(np.abs(got_r - ref_r).max(), np.abs(got_s - ref_s).max())))
+    return out

@@ -242,6 +242,18 @@ def moe_prefill_fp8_row_range(hl, xrow, idx, sum_tol):
     return lo, hi
 
 
+def moe_prefill_fp8_row_h_perturbed(hl, xrow, idx, sum_eps, seed=0):
+    """h bf16 [topk in expert-id order (+ 1)][I] with every gate and up sum moved by sum_eps * r * its sum of |terms|,
+    r uniform in [-1, 1) (seeded); sum_eps = 0: the h of the f64 sums"""
+    xrow = np.ascontiguousarray(xrow, np.uint16)
+    idx = np.ascontiguousarray(idx, np.int32)
+    n = hl.topk + (1 if hl.has_shared else 0)
+    h = np.empty((n, hl.I), np.uint16)
+    Lw, desc = hl.host_layer_w()
+    lib().orc_moe_prefill_fp8_row_h_perturbed(C.byref(Lw), _p(desc), _p(xrow), _p(idx), C.c_double(sum_eps), C.c_uint64(seed), _p(h))
+    return h
+
+
 def add_norm(part, part2, res, w, eps, round2=False):
     """(res_out bf16, xn bf16 from f64 statistics, xn bf16 from sequential f32 statistics), each [M][H]"""
     part = np.ascontiguousarray(part, np.float32)

@@ -16,13 +16,7 @@ from tests.test_gpu_decode import _check_step
 pytestmark = pytest.mark.gpu
 
 
-def zipf_picks(T, E, topk, s=1.1, seed=4321):
-    """top-k distinct experts a row drawn (without replacement) from a Zipf(s) popularity over a seeded permutation of the
-    experts: the k largest of log p + Gumbel noise; uniform weights 1 / top-k (the bench's prefill input)"""
-    rng = np.random.default_rng(seed)
-    logp = -s * np.log(rng.permutation(E) + 1.0)
-    idx = np.argsort(-(logp[None, :] + rng.gumbel(size=(T, E))), axis=1, kind="stable")[:, :topk]
-    return np.ascontiguousarray(idx, np.int32), np.full((T, topk), 1.0 / topk, np.float32)
+zipf_picks = helpers.zipf_picks
 
 
 def _run_prefill(hl, dl, x, idx, w, **kw):
