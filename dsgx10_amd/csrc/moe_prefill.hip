@@ -575,6 +575,7 @@ void dsgx_prefill_cfg_default(dsgx_prefill_cfg* c) {
   c->shared = 1;
   c->phases = 31;
   c->act_fp8 = 1;
+  c->fast_act = 0;
 }
 
 static int prefill_check(const dsgx_layer_w* L, int T, const char* who) {
@@ -686,6 +687,7 @@ int dsgx_moe_prefill(const dsgx_layer_w* L, const uint16_t* x, const int* idx, c
     if (int rc = allow_dynamic_lds(k, pf8::Shape<2>::kLds)) return rc;
   pf8::Args g{};
   g.L = *L;
+  g.fast_act = cfg.fast_act;
   const int NSU = I / (pf8::kWgRows / 2), NSD = H / pf8::kWgRows;
   g.tile_e = I32(o.mix_e), g.tile_m0 = I32(o.mix_m0), g.ntiles = I32(o.nmix), g.off = I32(o.off), g.nrows = P;
   if (cfg.phases & (2 | 16)) {

@@ -68,6 +68,7 @@ struct Args {
   const int* ntiles;
   const int* off;
   int nrows;           // shared expert: T
+  int fast_act;        // UP: SwiGLU by the hardware's exp2 / rcp instead of expf() and the IEEE division
   dsgx_layer_w L;
   uint16_t* h;         // UP: h bf16 [position][I]
   uint8_t* hq;         // UP: h quantised, e4m3 [position][I]
@@ -293,6 +294,7 @@ __device__ __forceinline__ void gemm_tile(const Args& g, uint8_t* smem, int e, i
     // lanes a position: h to memory as whole lines, act_quant over the 128 channels (the scale block of the down
     // projection: amax clamped at 1e-4, scale = amax * f32(1 / 448), e4m3 codes of h / scale clamped to +-448).
     const int I = g.L.I;
+    const bool fast = uni(g.fast_act) != 0;
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       if (j >= nj) break;
@@ -301,8 +303,10 @@ __device__ __forceinline__ void gemm_tile(const Args& g, uint8_t* smem, int e, i
       for (int b = 0; b < S::RA / 2; ++b) {
         uint32_t hb[4];
 #pragma unroll
-        for (int q = 0; q < 4; ++q)
-          hb[q] = swiglu_fast_bits(bf16_round(__fmul_rn(acc[2 * b][j][q], s2a)), bf16_round(__fmul_rn(acc[2 * b + 1][j][q], s2b)));
+        for (int q = 0; q < 4; ++q) {
+          const float gv = bf16_round(__fmul_rn(acc[2 * b][j][q], s2a)), uv = bf16_round(__fmul_rn(acc[2 * b + 1][j][q], s2b));
+          hb[q] = fast ? swiglu_fast_bits(gv, uv) : swiglu_bits(gv, uv);
+        }
         const int ch = 16 * (S::RA / 2 * rg + b) + 4 * part;  // first of the lane's four channels (of the workgroup's 128)
         const int piece = (ch >> 3) ^ (p & 15);
         *reinterpret_cast<uint2*>(smem + p * 256 + piece * 16 + (ch & 4) * 2) = make_uint2(hb[0] | (hb[1] << 16), hb[2] | (hb[3] << 16));

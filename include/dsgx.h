@@ -203,6 +203,10 @@ typedef struct dsgx_prefill_cfg {
   int32_t act_fp8;  /* FP8 layers: 1 = quantise activations per row and 128 k to e4m3 and run the fp8 MFMA
                        (ds41f-4xgx10-switchless/ref/torchref/kernel.py:56-77, ref/inference/kernel.py:207-274);
                        0 = bf16 activations, weights widened to bf16 (the altar-1 contract) */
+  int32_t fast_act; /* FP8 activations only. 0 (the default): SwiGLU with expf() and the IEEE division, as the decode kernels
+                       and the reference compute it (engine/experts/decode.cu:110-113); 1: the hardware's exponential and
+                       reciprocal (each within 1 ulp; h then differs from the exact form's in about one value in 10^4, by one
+                       bf16 step), for callers that trade that for the epilogue's time */
 } dsgx_prefill_cfg;
 DSGX_API void dsgx_prefill_cfg_default(dsgx_prefill_cfg* cfg);
 DSGX_API size_t dsgx_prefill_ws_bytes(const dsgx_layer_w* L, int T);

@@ -353,3 +353,21 @@ def dsk_down(w2, hpre):
              out64=np.empty((M, H), np.float64), mag=np.empty((M, H), np.float64), outb=np.empty((M, H), np.uint16))
     lib().orc_dsk_down(_p(w2), _p(hpre), M, H, I, _p(o["hq"]), _p(o["hs"]), _p(o["out32"]), _p(o["out64"]), _p(o["mag"]), _p(o["outb"]))
     return o
+
+
+def mfma_fp8_k128(a, b):
+    """the oracle's statement of gfx950's v_mfma_f32_16x16x128_f8f6f4 block sum: e4m3 codes a [R][128], b [S][128] in
+    register order -> f32 [R][S]"""
+    a, b = np.ascontiguousarray(a, np.uint8), np.ascontiguousarray(b, np.uint8)
+    lib().orc_mfma_fp8_k128.restype = C.c_float
+    out = np.empty((a.shape[0], b.shape[0]), np.float32)
+    for i in range(a.shape[0]):
+        for j in range(b.shape[0]):
+            out[i, j] = lib().orc_mfma_fp8_k128(C.c_void_p(a[i].ctypes.data), C.c_void_p(b[j].ctypes.data))
+    return out
+
+
+def set_fp8_block_rule(rule):
+    """0: a 128-k block's products are added sequentially in f32 (the contract as the reference's CPU stand-in states it);
+    1: by the gfx950 matrix unit's rule (orc_mfma_fp8_k128) in the prefill kernels' k map"""
+    lib().orc_set_fp8_block_rule(int(rule))
