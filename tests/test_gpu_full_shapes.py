@@ -84,42 +84,54 @@ def test_prefill_fp8_at_the_benchmark_shape():
     off, perm, rpos, re, v = _buckets(dl, ws, idx, T, E, topk)
     rows, cnt = _sample_rows(off, perm, T)
     assert cnt.max() > 4 * 128 and np.median(cnt) < 128, "the draw should give multi-tile hot experts and sub-tile cold ones"
-    nh = nbad = 0
+    nh = nbad = nbits = 0
     worst_sum = 0.0
-    ref_r, ref_s, got_r, got_s = [], [], [], []
-    for t in rows:
-        o = orc.moe_prefill_fp8_row(hl, x[t], idx[t], w[t])
-        mine = np.concatenate([_h_rows(ws, v.h, T * topk, I, rpos[t]), _h_rows(ws, v.hsh, T, I, [t])])
-        # (1) h: most values equal, every one inside the range the contract allows when the gate and up sums move by
-        # 1e-4 of their sums of |terms| (the reference's tolerance on such sums, test_experts.cu:352-361, which is also
-        # what the e4m3 MFMA's own additions are good for: test_mfma_fp8_accuracy)
-        nbad += int((mine != o["h"]).sum())
-        nh += mine.size
-        lo, hi = orc.moe_prefill_fp8_row_range(hl, x[t], idx[t], 1e-4)
-        hv = orc.bf16_to_f32(mine)
-        far = ~((hv >= lo[:mine.shape[0]]) & (hv <= hi[:mine.shape[0]]))
-        assert far.sum() == 0, (t, int(far.sum()), float(np.abs(hv - orc.bf16_to_f32(o["h"])).max()))
-        # (2) down + combine from the GPU's own h: the reference's GEMV tolerance and the benchmark's bar
-        o2 = orc.moe_prefill_fp8_row(hl, x[t], idx[t], w[t], h_in=mine)
-        for got, r64, mag, r32 in ((yr[t], o2["yr64"], o2["yrmag"], o2["yr"]), (ys[t], o2["ys64"], o2["ysmag"], o2["ys"])):
-            worst, bad = helpers.check_sums(got, r64, mag)
-            worst_sum = max(worst_sum, worst)
-            assert bad == 0, (t, worst)
-            helpers.check_outputs(got, r32, bf16_rel=False)
-        ref_r.append(o["yr"]), ref_s.append(o["ys"]), got_r.append(yr[t]), got_s.append(ys[t])
-    assert nbad <= 0.05 * nh, (nbad, nh)
-    # (3) end to end against the oracle's own h on the sampled rows. Two correct evaluations of this contract do not
-    # agree to the benchmark's 1e-3 / 2e-2 here: ~2% of the gate and up sums fall on the other side of a bf16 rounding
-    # (the MFMA's additions against the oracle's f32 ones), one such h in sixteen then moves a whole e4m3 step (6-12% of
-    # its value) when h is quantised for the down projection, and at this shape the outputs are of order 1-3. The bar
-    # is held stage by stage in (2); end to end the sampled rows stay within 3e-3 / 6e-2 (measured: 1.3e-3 routed,
-    # 2.4e-3 shared, max-abs 3.9e-2).
-    e2e_r, e2e_s = helpers.rel_l2(np.stack(got_r), np.stack(ref_r)), helpers.rel_l2(np.stack(got_s), np.stack(ref_s))
-    mx = max(np.abs(np.stack(got_r) - np.stack(ref_r)).max(), np.abs(np.stack(got_s) - np.stack(ref_s)).max())
-    print("fp8 prefill T=8192: %d rows sampled, h equal %.2f%%, staged |err|/sum|terms| %.2e, end-to-end rel-L2 routed %.2e shared %.2e, max-abs %.2e"
-          % (len(rows), 100 - 100.0 * nbad / nh, worst_sum, e2e_r, e2e_s, mx))
-    assert e2e_r <= 3e-3 and e2e_s <= 3e-3 and mx <= 6e-2
-    # (4) a row's bits do not depend on the chunk: a slice of rows as a chunk of its own
+    ref_r, ref_s, got_r, got_s, seq_r, seq_s = [], [], [], [], [], []
+    orc.set_fp8_block_rule(1)   # the oracle adds each 128-k block by the matrix unit's rule (tests/test_oracle_mfma.py)
+    try:
+        for n, t in enumerate(rows):
+            o = orc.moe_prefill_fp8_row(hl, x[t], idx[t], w[t])
+            mine = np.concatenate([_h_rows(ws, v.h, T * topk, I, rpos[t]), _h_rows(ws, v.hsh, T, I, [t])])
+            # (1) h: the same sums on both sides, so it differs only where the device's expf() and the host's round silu to
+            # different bf16 values, by one step; the reference asks 98.5% of a prefill chunk (test_prefill.inc:183-186)
+            nbad += int((mine != o["h"]).sum())
+            nh += mine.size
+            hv, hr = orc.bf16_to_f32(mine).astype(np.float64), orc.bf16_to_f32(o["h"]).astype(np.float64)
+            step = 2.0 ** (np.floor(np.log2(np.maximum(np.abs(hr), 2.0 ** -100))) - 7)
+            assert np.all(np.abs(hv - hr) <= step), (t, float(np.abs(hv - hr).max()))
+            # (2) down + combine from the GPU's own h: the reference's GEMV tolerance against exact sums, and every f32
+            # output bit against the oracle's (same block sums, same order of adds)
+            o2 = orc.moe_prefill_fp8_row(hl, x[t], idx[t], w[t], h_in=mine)
+            for got, r64, mag, r32 in ((yr[t], o2["yr64"], o2["yrmag"], o2["yr"]), (ys[t], o2["ys64"], o2["ysmag"], o2["ys"])):
+                worst, bad = helpers.check_sums(got, r64, mag)
+                worst_sum = max(worst_sum, worst)
+                assert bad == 0, (t, worst)
+                nbits += int((got.view(np.uint32) != r32.view(np.uint32)).sum())
+            ref_r.append(o["yr"]), ref_s.append(o["ys"]), got_r.append(yr[t]), got_s.append(ys[t])
+            if n < 12:
+                orc.set_fp8_block_rule(0)
+                o0 = orc.moe_prefill_fp8_row(hl, x[t], idx[t], w[t])
+                orc.set_fp8_block_rule(1)
+                seq_r.append(o0["yr"]), seq_s.append(o0["ys"])
+    finally:
+        orc.set_fp8_block_rule(0)
+    assert nbad <= 0.002 * nh, (nbad, nh)
+    assert nbits == 0, nbits
+    # (3) end to end against the oracle's own h on the sampled rows: the benchmark's bar (relative L2 1e-3, max-abs 2e-2,
+    # on the f32 outputs and their bf16 roundings)
+    G_r, G_s, R_r, R_s = np.stack(got_r), np.stack(got_s), np.stack(ref_r), np.stack(ref_s)
+    e2e_r, e2e_s = helpers.rel_l2(G_r, R_r), helpers.rel_l2(G_s, R_s)
+    mx = max(np.abs(G_r - R_r).max(), np.abs(G_s - R_s).max())
+    # (4) for the record, against the contract with sequential f32 block sums (the reference's CPU stand-in): the matrix
+    # unit's own additions move a sum by ~1.5e-6 of its sum of |terms|, and evaluations that far apart differ by 2-3e-3 end
+    # to end once h is re-quantised to e4m3 (tests/test_oracle_moe.py measures that spread on this chunk's rows)
+    s_r, s_s = helpers.rel_l2(G_r[:12], np.stack(seq_r)), helpers.rel_l2(G_s[:12], np.stack(seq_s))
+    print("fp8 prefill T=8192: %d rows sampled, h equal %.3f%%, staged |err|/sum|terms| %.2e, end-to-end rel-L2 routed %.2e shared %.2e, max-abs %.2e; "
+          "against sequential f32 block sums: routed %.2e shared %.2e" % (len(rows), 100 - 100.0 * nbad / nh, worst_sum, e2e_r, e2e_s, mx, s_r, s_s))
+    helpers.check_outputs(G_r, R_r)
+    helpers.check_outputs(G_s, R_s)
+    assert s_r <= 6e-3 and s_s <= 6e-3
+    # (5) a row's bits do not depend on the chunk: a slice of rows as a chunk of its own
     a, b = 4000, 4100
     yr2, ys2, _ = _run_prefill(hl, dl, x[a:b], idx[a:b], w[a:b])
     assert np.array_equal(yr[a:b].view(np.uint32), yr2.view(np.uint32)) and np.array_equal(ys[a:b].view(np.uint32), ys2.view(np.uint32))
