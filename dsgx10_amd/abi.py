@@ -28,6 +28,11 @@ class DskCfg(C.Structure):
     _fields_ = [("swiglu_limit", C.c_float), ("logits", C.c_void_p), ("bias", C.c_void_p), ("route_scale", C.c_float), ("parts", C.c_int32)]
 
 
+class DskWeights(C.Structure):
+    _fields_ = [(n, C.c_void_p) for n in ("w1", "s1", "w3", "s3", "w2", "s2", "sh_w1", "sh_s1", "sh_w3", "sh_s3", "sh_w2", "sh_s2")] + \
+               [(n, C.c_int32) for n in ("H", "I", "E", "topk")]
+
+
 class DecodeCfg(C.Structure):
     _fields_ = [("up", C.c_int32), ("down", C.c_int32), ("parts", C.c_int32), ("ysum", C.c_int32),
                 ("logits", C.c_void_p), ("bias", C.c_void_p), ("route_scale", C.c_float), ("score_fn", C.c_int32),
@@ -52,7 +57,7 @@ assert C.sizeof(MatDesc) == 64
 # every symbol include/dsgx.h declares
 SYMBOLS = [
     "dsgx_mat_bytes", "dsgx_mat_scale_off", "dsgx_mat_zp_off", "dsgx_route", "dsgx_decode_cfg_default",
-    "dsgx_decode_ws_bytes", "dsgx_decode_ws_flag_offset", "dsgx_decode_status", "dsgx_moe_decode", "dsgx_moe_decode_noalloc", "dsgx_finalize", "dsgx_add_norm", "dsgx_dsk_cfg_default", "dsgx_dsk_moe", "dsgx_prefill_cfg_default", "dsgx_prefill_ws_bytes",
+    "dsgx_decode_ws_bytes", "dsgx_decode_ws_flag_offset", "dsgx_decode_status", "dsgx_moe_decode", "dsgx_moe_decode_noalloc", "dsgx_finalize", "dsgx_add_norm", "dsgx_dsk_cfg_default", "dsgx_dsk_moe", "dsgx_dsk_ws_bytes", "dsgx_dsk_moe_stacked", "dsgx_prefill_cfg_default", "dsgx_prefill_ws_bytes",
     "dsgx_moe_prefill", "dsgx_prefill_view_get", "dsgx_gemv", "dsgx_dequant_int4", "dsgx_probe_dequant_int4", "dsgx_probe_mfma_fp8",
     "dsgx_widen_fp8", "dsgx_act_quant", "dsgx_last_error", "dsgx_version", "dsgx_stream_read", "dsgx_stream_read_cfg", "dsgx_stream_copy",
 ]

@@ -63,14 +63,16 @@ def build_mirror_run(force=False):
     """tests/mirror_run: the test program that drives the C++ mirror headers on the GPU (host code only; it links the
     library just built and finds it relative to its own place)"""
     root = os.path.dirname(HERE)
-    src, exe = os.path.join(root, "tests", "mirror_run.cpp"), os.path.join(root, "tests", "mirror_run")
-    if not os.path.exists(src):
-        return None
     inc = os.path.join(root, "include")
     hdrs = [os.path.join(dp, f) for dp, _, fs in os.walk(inc) for f in fs]
-    if force or _stale(exe, [src, SO] + hdrs):
-        subprocess.check_call(["hipcc", "-std=c++17", "-O1", "-Wall", "-I", inc, src, "-o", exe, "-L", CSRC, "-ldsgx",
-                               "-Wl,-rpath,$ORIGIN/../dsgx10_amd/csrc"])
+    exe = None
+    for name in ("mirror_run", "mirror_run_dsk"):
+        src, exe = os.path.join(root, "tests", name + ".cpp"), os.path.join(root, "tests", name)
+        if not os.path.exists(src):
+            continue
+        if force or _stale(exe, [src, SO] + hdrs):
+            subprocess.check_call(["hipcc", "-std=c++17", "-O1", "-Wall", "-I", inc, src, "-o", exe, "-L", CSRC, "-ldsgx",
+                                   "-Wl,-rpath,$ORIGIN/../dsgx10_amd/csrc"])
     return exe
 
 

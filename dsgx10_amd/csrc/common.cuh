@@ -284,9 +284,45 @@ __device__ __forceinline__ float route_sigmoid(float l) {
   const float e = ldexpf(p, (int)n);
   return __fdiv_rn(1.f, __fadd_rn(1.f, e));
 }
+// softplus(l) = log1p(exp(l)) for l <= 20, again from IEEE operations only (the reference's log1pf(expf(l)),
+// ds41f-4xgx10-switchless/engine/kernels/common.cuh:281, depends on the math library): exp by the sigmoid's reduction and
+// polynomial; log1p(e) = log(u) e / (u - 1) with u = 1 + e; log by u = 2^k (1 + f), sqrt(1/2) < 1 + f < sqrt(2),
+// s = f / (2 + f), log(1 + f) = f - f^2/2 + s (f^2/2 + R(s^2)), R the degree-7 minimax of fdlibm's e_logf.c. Every
+// operation is written out and rounded on its own, so the host oracle's copy gives the same bits.
+__device__ __forceinline__ float route_softplus(float l) {
+  if (l < -87.f) l = -87.f;
+  const float n = rintf(__fmul_rn(l, 1.44269504f));
+  float r = fmaf(-n, 0.693145751953125f, l);
+  r = fmaf(-n, 1.428606765330187e-06f, r);
+  float p = 1.f / 5040;
+  p = fmaf(p, r, 1.f / 720);
+  p = fmaf(p, r, 1.f / 120);
+  p = fmaf(p, r, 1.f / 24);
+  p = fmaf(p, r, 1.f / 6);
+  p = fmaf(p, r, 0.5f);
+  p = fmaf(p, r, 1.f);
+  p = fmaf(p, r, 1.f);
+  const float e = ldexpf(p, (int)n);
+  const float u = __fadd_rn(1.f, e);
+  if (u == 1.f) return e;
+  uint32_t ix = __float_as_uint(u);
+  int k = (int)(ix >> 23) - 127;
+  ix &= 0x007fffffu;
+  const uint32_t i = (ix + (0x95f64u << 3)) & 0x800000u;
+  ix |= i ^ 0x3f800000u;
+  k += (int)(i >> 23);
+  const float f = __fsub_rn(__uint_as_float(ix), 1.f), dk = (float)k;
+  const float s_ = __fdiv_rn(f, __fadd_rn(2.f, f)), z = __fmul_rn(s_, s_), w = __fmul_rn(z, z);
+  const float t1 = __fmul_rn(w, __fadd_rn(0.40000000596f, __fmul_rn(w, __fadd_rn(0.22222198546f, __fmul_rn(w, 0.15313838422f)))));
+  const float t2 = __fmul_rn(z, __fadd_rn(0.66666668653f, __fmul_rn(w, __fadd_rn(0.28571429849f, __fmul_rn(w, __fadd_rn(0.18183572590f, __fmul_rn(w, 0.14798198640f)))))));
+  const float R = __fadd_rn(t2, t1), hfsq = __fmul_rn(__fmul_rn(0.5f, f), f);
+  const float inner = __fadd_rn(__fmul_rn(s_, __fadd_rn(hfsq, R)), __fmul_rn(dk, 9.0580006145e-06f));
+  const float lg = __fsub_rn(__fmul_rn(dk, 0.69313812256f), __fsub_rn(__fsub_rn(hfsq, inner), f));
+  return __fmul_rn(lg, __fdiv_rn(e, __fsub_rn(u, 1.f)));
+}
 __device__ __forceinline__ float route_score(float l, int score_fn) {
   if (score_fn == 0) return route_sigmoid(l);
-  return sqrtf(l > 20.f ? l : log1pf(expf(l)));  // DeepSeek's sqrt(softplus): libm-dependent, not promised bit-exact
+  return sqrtf(l > 20.f ? l : route_softplus(l));  // DeepSeek's sqrt(softplus); sqrtf is the correctly rounded root (__fsqrt_rn is not)
 }
 // wave-wide maximum of floats (no NaNs), valid in every lane
 template <int CTRL>

@@ -83,6 +83,9 @@ struct WsLayout {
   constexpr size_t dpart_off() const { return fac_off() + kFacBytes; }
   constexpr size_t xdeq_off() const { return dpart_off() + (size_t)(DSGX_MAX_UNION + 1) * 8 * H * 4; }  // (reserved)
   constexpr size_t bytes() const { return xdeq_off() + (size_t)DSGX_MAX_ROWS * H * 2; }
+  // dsgx_dsk_moe_stacked's workspace: the same, then the shared expert's output rows f32 [DSGX_MAX_ROWS][H]
+  constexpr size_t dsk_ys_off() const { return (bytes() + 255) / 256 * 256; }
+  constexpr size_t dsk_bytes() const { return dsk_ys_off() + (size_t)DSGX_MAX_ROWS * H * 4; }
 };
 static constexpr WsLayout kStaticLayout{DSGX_NOALLOC_MAX_I, DSGX_NOALLOC_MAX_H};
 static_assert(kStaticLayout.bytes() == kStaticWsBytes, "the built-in workspace's size");
@@ -92,6 +95,9 @@ struct DskIn {
   float limit = 0.f;
   const uint8_t* xq = nullptr;
   const uint8_t* xs = nullptr;
+  const dsgx_dsk_weights* stacked = nullptr;  // experts stacked by id in their own tensors (no pool, no descriptors)
+  int* idx_out = nullptr;                     // fused routing: the selection, for the caller
+  float* wts_out = nullptr;
 };
 static int moe_decode_at(const dsgx_layer_w* L, const uint16_t* x, const int* idx, const float* w, int M, void* ws, const WsLayout& lay,
                          float* yr, float* ys, void* stream, const dsgx_decode_cfg* cfg, DskIn dsk = DskIn{});
@@ -181,7 +187,7 @@ static int moe_decode_at(const dsgx_layer_w* L, const uint16_t* x, const int* id
   if (dsk.on) c.up = 1;  // (the MFMA kernels are the ones built for it)
   if (L->fmt != DSGX_FMT_FP8_B128 && L->fmt != DSGX_FMT_INT4_G32 && L->fmt != DSGX_FMT_BF16 && L->fmt != DSGX_FMT_MXFP4_G32)
     return fail(DSGX_EFORMAT, "moe_decode: layer expert format %u is not FP8_B128 (16), INT4_G32 (18) or BF16 (19)", L->fmt);
-  if (!L->pool || !L->desc) return fail(DSGX_EINVAL, "moe_decode: null pool or descriptors");
+  if (!dsk.stacked && (!L->pool || !L->desc)) return fail(DSGX_EINVAL, "moe_decode: null pool or descriptors");
   const int H = L->H, I = L->I;
   if (L->E < 1 || L->E > DSGX_MAX_EXPERTS || L->topk < 1 || L->topk > DSGX_MAX_TOPK || L->topk > L->E)
     return fail(DSGX_EINVAL, "moe_decode: E %d, top-k %d", L->E, L->topk);
@@ -210,6 +216,7 @@ static int moe_decode_at(const dsgx_layer_w* L, const uint16_t* x, const int* id
     if (int rc = moe_decode_at(L, x, idx, w, M1, ws, lay, yr, ys, stream, &c1, dsk)) return rc;
     DskIn dsk2 = dsk;
     if (dsk.xq) dsk2.xq = dsk.xq + (size_t)M1 * H, dsk2.xs = dsk.xs + (size_t)M1 * (H / 32);
+    if (dsk.idx_out) dsk2.idx_out = dsk.idx_out + (size_t)M1 * topk, dsk2.wts_out = dsk.wts_out + (size_t)M1 * topk;
     return moe_decode_at(L, x + (size_t)M1 * H, idx ? idx + (size_t)M1 * topk : nullptr, w ? w + (size_t)M1 * topk : nullptr, M - M1, ws, lay,
                          yr ? yr + (size_t)M1 * H : nullptr, ys ? ys + (size_t)M1 * H : nullptr, stream, &c2, dsk2);
   }
@@ -221,6 +228,14 @@ static int moe_decode_at(const dsgx_layer_w* L, const uint16_t* x, const int* id
   a.fac = reinterpret_cast<float*>(wsb + lay.fac_off());
   a.dpart = reinterpret_cast<float*>(wsb + lay.dpart_off());
   a.dsk = dsk.on, a.dsk_limit = dsk.limit, a.dsk_xq = dsk.xq, a.dsk_xs = dsk.xs;
+  a.idx_out = c.logits ? dsk.idx_out : nullptr, a.wts_out = c.logits ? dsk.wts_out : nullptr;
+  if (const dsgx_dsk_weights* W = dsk.stacked) {
+    const size_t gu = (size_t)I * H, dn = (size_t)H * I;
+    a.stk_w[0] = W->w1, a.stk_w[1] = W->w3, a.stk_w[2] = W->w2;
+    a.stk_s[0] = W->s1, a.stk_s[1] = W->s3, a.stk_s[2] = W->s2;
+    a.stk_wb[0] = a.stk_wb[1] = gu / 2, a.stk_wb[2] = dn / 2;
+    a.stk_sb[0] = a.stk_sb[1] = gu / 32, a.stk_sb[2] = dn / 32;
+  }
   a.spin_limit = 1 << 22;
 #ifdef DSGX_TRACE
   a.trace = g_trace_buf;
@@ -270,6 +285,42 @@ int dsgx_dsk_moe(const dsgx_layer_w* L, const uint8_t* xq, const uint8_t* xs, in
   dsgx_decode_cfg_default(&d);
   d.up = 1, d.parts = c.parts, d.logits = c.logits, d.bias = c.bias, d.route_scale = c.route_scale, d.score_fn = 1;
   return moe_decode_at(L, xd, idx, w, M, ws, lay, y, ys, stream, &d, DskIn{1, c.swiglu_limit, xq, xs});
+}
+size_t dsgx_dsk_ws_bytes(int H, int I) {
+  if (H <= 0 || I <= 0) return 0;
+  return WsLayout{I, H}.dsk_bytes();
+}
+int dsgx_dsk_moe_stacked(const dsgx_dsk_weights* W, const uint8_t* xq, const uint8_t* xs, int M, const int* idx, const float* w, void* ws,
+                         float* y, void* stream, const dsgx_dsk_cfg* cfg, int* idx_out, float* wts_out) {
+  dsgx_dsk_cfg c;
+  if (cfg) c = *cfg;
+  else dsgx_dsk_cfg_default(&c);
+  if (!W || !xq || !xs || !ws || !y) return fail(DSGX_EINVAL, "dsk_moe_stacked: null weights, rows, workspace or output");
+  if (!W->w1 || !W->s1 || !W->w3 || !W->s3 || !W->w2 || !W->s2) return fail(DSGX_EINVAL, "dsk_moe_stacked: the routed experts need w1, s1, w3, s3, w2, s2");
+  const bool sh = W->sh_w1 != nullptr;
+  if (sh && (!W->sh_s1 || !W->sh_w3 || !W->sh_s3 || !W->sh_w2 || !W->sh_s2)) return fail(DSGX_EINVAL, "dsk_moe_stacked: the shared expert needs all of sh_w1 ... sh_s2");
+  if (M < 1 || M > DSGX_MAX_ROWS) return fail(DSGX_EINVAL, "dsk_moe_stacked: M=%d", M);
+  if (W->H <= 0 || W->H % 256 || W->I <= 0 || W->I % 256) return fail(DSGX_EINVAL, "dsk_moe_stacked: hidden %d, intermediate %d (multiples of 256)", W->H, W->I);
+  if (!(c.swiglu_limit > 0.f)) return fail(DSGX_EINVAL, "dsk_moe_stacked: swiglu_limit %g", (double)c.swiglu_limit);
+  if (((uintptr_t)xq & 7) || (((uintptr_t)W->w1 | (uintptr_t)W->w3 | (uintptr_t)W->w2) & 15))
+    return fail(DSGX_EINVAL, "dsk_moe_stacked: the rows' codes must be 8-byte aligned, the weight tensors 16-byte aligned");
+  if ((idx_out == nullptr) != (wts_out == nullptr)) return fail(DSGX_EINVAL, "dsk_moe_stacked: idx_out and wts_out go together");
+  dsgx_layer_w L{};
+  L.pool = W->w1, L.desc = nullptr, L.fmt = DSGX_FMT_MXFP4_G32, L.H = W->H, L.I = W->I, L.E = W->E, L.topk = W->topk;
+  if (sh) {
+    L.sh.g = W->sh_w1, L.sh.u = W->sh_w3, L.sh.d = W->sh_w2;
+    L.sh.gs = reinterpret_cast<const float*>(W->sh_s1), L.sh.us = reinterpret_cast<const float*>(W->sh_s3), L.sh.ds = reinterpret_cast<const float*>(W->sh_s2);
+  }
+  const WsLayout lay{L.I, L.H};
+  uint8_t* wsb = static_cast<uint8_t*>(ws);
+  uint16_t* xd = reinterpret_cast<uint16_t*>(wsb + lay.xdeq_off());
+  float* ys = reinterpret_cast<float*>(wsb + lay.dsk_ys_off());
+  dsgx_decode_cfg d;
+  dsgx_decode_cfg_default(&d);
+  d.up = 1, d.parts = c.parts, d.logits = c.logits, d.bias = c.bias, d.route_scale = c.route_scale, d.score_fn = 1;
+  DskIn in{1, c.swiglu_limit, xq, xs};
+  in.stacked = W, in.idx_out = idx_out, in.wts_out = wts_out;
+  return moe_decode_at(&L, xd, idx, w, M, ws, lay, y, ys, stream, &d, in);
 }
 }  // extern "C"
 

@@ -83,6 +83,14 @@ struct DecodeArgs {
   float dsk_limit;
   const uint8_t* dsk_xq;  // the rows as e4m3 codes [M][H] with ue8m0 scales [M][H / 32] (x is then not read)
   const uint8_t* dsk_xs;
+  // Experts stacked by expert id in six tensors of their own (dsk::MoeWeights, ds41f-4xgx10-switchless/engine/kernels/
+  // dsk.h:199-209) instead of a pool with descriptors: matrix j (gate, up, down) of expert e at stk_w[j] + e stk_wb[j], its
+  // scales at stk_s[j] + e stk_sb[j]. stk_w[0] null: the layer's descriptors.
+  const uint8_t* stk_w[3];
+  const uint8_t* stk_s[3];
+  size_t stk_wb[3], stk_sb[3];
+  int* idx_out;     // fused routing: the selection is also written here (idx_out / wts_out of dsk::moe_routed, dsk.h:239-241)
+  float* wts_out;
 };
 
 int launch_decode_mxfp4_mfma(const DecodeArgs& a, int parts, bool shared_fp8e, hipStream_t st);  // MXFP4 experts (+ FP8_B32E shared)
@@ -136,7 +144,7 @@ __device__ __forceinline__ void prep(Step<M>& S, const DecodeArgs& a) {
   // (loads past the end re-read the last descriptor: unconditional loads into named registers stay in flight together)
   const DSGX_GLOBAL u32x4_t* d = (const DSGX_GLOBAL u32x4_t*)(uintptr_t)a.L.desc;
   u32x4_t* tab = reinterpret_cast<u32x4_t*>(S.dtab);
-  const int nd = a.L.E * 3, bd = blockDim.x;
+  const int nd = a.stk_w[0] ? 0 : a.L.E * 3, bd = blockDim.x;  // (stacked experts are addressed by their id alone)
   for (int i0 = tid; i0 < nd; i0 += 3 * bd) {
     const int i1 = i0 + bd, i2 = i1 + bd;
     const u32x4_t v0 = d[(size_t)i0 * 4], v1 = d[(size_t)min(i1, nd - 1) * 4], v2 = d[(size_t)min(i2, nd - 1) * 4];
@@ -214,6 +222,7 @@ __device__ __forceinline__ void resolve(Step<M>& S, const DecodeArgs& a, int rw,
     if (lane < topk) {
       S.ri[row * topk + lane] = id, S.rw[row * topk + lane] = w;
       atomicOr(&S.mask[id >> 5], 1u << (id & 31));
+      if (a.idx_out && blockIdx.x == 0) a.idx_out[row * topk + lane] = id, a.wts_out[row * topk + lane] = w;
     }
   }
   DSGX_MARKW(9);
@@ -246,6 +255,7 @@ __device__ __forceinline__ void resolve(Step<M>& S, const DecodeArgs& a, int rw,
     // the routed slot (rows that picked the same expert write the same values)
     Slot t;
     auto ref = [&](int which, int N, int K) {
+      if (a.stk_w[0]) return MatRef{a.stk_w[which] + (size_t)e * a.stk_wb[which], a.stk_s[which] + (size_t)e * a.stk_sb[which], 1.f, 0};
       const uint4 d = S.dtab[e * 3 + which];
       return mat_ref<FMT>(a.L.pool + (((uint64_t)d.y << 32) | d.x), N, K, __uint_as_float(d.z));
     };

@@ -118,6 +118,19 @@ def dsk_moe(layer_w, xq, xs, idx, w, M, ws, y, ys, stream=None, limit=10.0, logi
                               C.byref(cfg)))
 
 
+def dsk_ws_bytes(H, I):
+    lib().dsgx_dsk_ws_bytes.restype = C.c_size_t
+    return lib().dsgx_dsk_ws_bytes(H, I)
+
+
+def dsk_moe_stacked(weights, xq, xs, idx, w, M, ws, y, stream=None, limit=10.0, logits=None, bias=None, route_scale=1.0, parts=3, idx_out=None,
+                    wts_out=None):
+    """dsk::moe / moe_routed on experts stacked by id (abi.DskWeights); the shared expert's rows stay in ws (dsk_ws_bytes)"""
+    cfg = abi.DskCfg(limit, _ptr(logits), _ptr(bias), route_scale, parts)
+    _check(lib().dsgx_dsk_moe_stacked(C.byref(weights), _ptr(xq), _ptr(xs), M, _ptr(idx), _ptr(w), _ptr(ws), _ptr(y), _stream(stream),
+                                      C.byref(cfg), _ptr(idx_out), _ptr(wts_out)))
+
+
 def decode_status(layer_w, ws, stream=None):
     """waits for the stream; raises DsgxError(ETIMEOUT) if a fused decode step gave up at its grid barrier since the last
     check (ws None: the library's own workspace)"""

@@ -184,6 +184,22 @@ typedef struct dsgx_dsk_cfg {
 DSGX_API void dsgx_dsk_cfg_default(dsgx_dsk_cfg* cfg);
 DSGX_API int dsgx_dsk_moe(const dsgx_layer_w* L, const uint8_t* xq, const uint8_t* xs, int M, const int* idx, const float* w, void* ws,
                           float* y, float* ys, void* stream, const dsgx_dsk_cfg* cfg);
+/* The same layer as the reference hands it over: dsk::MoeWeights (engine/kernels/dsk.h:199-209), the routed experts stacked
+   by expert id in six tensors (expert e at e times the per-expert size) and the FP8 shared expert in six more, all in the
+   row-major forms of DSGX_FMT_MXFP4_G32 / DSGX_FMT_FP8_B32E (not the reference's GB10 lane tilings):
+     w1, w3 e2m1 pairs [E][I][H/2]; s1, s3 ue8m0 [E][I][H/32]; w2 [E][H][I/2]; s2 [E][H][I/32];
+     sh_w1, sh_w3 e4m3 [I][H]; sh_s1, sh_s3 ue8m0 [I/32][H/32]; sh_w2 [H][I]; sh_s2 [H/32][I/32] (sh_w1 null: no shared expert).
+   dsgx_dsk_moe_stacked is dsk::moe (idx, w given) and dsk::moe_routed (cfg->logits given; idx_out / wts_out [M][topk],
+   optional, then receive the router's selection, dsk.h:234-241): y f32 [M][H] as dsgx_dsk_moe's. The shared expert's rows
+   stay inside the workspace (the reference keeps them in shared memory): ws of dsgx_dsk_ws_bytes(H, I), zeroed once. */
+typedef struct dsgx_dsk_weights {
+  const uint8_t *w1, *s1, *w3, *s3, *w2, *s2;
+  const uint8_t *sh_w1, *sh_s1, *sh_w3, *sh_s3, *sh_w2, *sh_s2;
+  int32_t H, I, E, topk;
+} dsgx_dsk_weights;
+DSGX_API size_t dsgx_dsk_ws_bytes(int H, int I);
+DSGX_API int dsgx_dsk_moe_stacked(const dsgx_dsk_weights* W, const uint8_t* xq, const uint8_t* xs, int M, const int* idx, const float* w,
+                                  void* ws, float* y, void* stream, const dsgx_dsk_cfg* cfg, int* idx_out, float* wts_out);
 
 /* The residual add after the expert step and the next layer's RMSNorm, the local half of the reference's
    comm::glm::allreduce_add_norm / allreduce2_add_norm (engine/comm/glmcoll.h:34-62; the norm: engine/attn/prep.cu:12-66),

@@ -1,8 +1,19 @@
-// dsk:: - the DeepSeek engine's MoE operator names (ds41f-4xgx10-switchless/engine/kernels/dsk.h:171-241,268-295) over
-// the C ABI in dsgx.h. Two layer kinds: the reference's own - MXFP4 routed experts + FP8 shared expert with ue8m0 scales,
-// FP8-quantised rows, its expert arithmetic (MoeWeights::mx: a dsgx_layer_w of MXFP4_G32 matrices in the checkpoint's
-// row-major form; the reference's tiled L3 tensors w1 / s1 ... are a GB10 lane order and are refused, never reinterpreted)
-// - and the FP8 e4m3 / 128 x 128 block-scaled configuration with bf16 rows (MoeWeights::fp8).
+// dsk:: - the DeepSeek engine's MoE operators (ds41f-4xgx10-switchless/engine/kernels/dsk.h:171-241, 268-295) with the
+// reference's names, argument lists and defaults, over the C ABI in dsgx.h. A caller written against the reference's
+// header compiles against this one: cudaStream_t becomes a HIP stream (taken as void*), device pointers stay as they are.
+//
+// What differs, and why:
+//  - Layouts. The reference's MoeWeights tensors are re-laid at load time for the GB10 lane map (tile_fp4 / tile_fp8, dsk.h:
+//    177-180). Here the load-time step keeps the checkpoint's row-major form (DSGX_FMT_MXFP4_G32 / DSGX_FMT_FP8_B32E), which
+//    is the coalesced streaming layout on gfx950: tile_fp4 / tile_fp8 below are plain copies, so a loader that calls them
+//    and stacks the results by expert id, as the reference's does, produces what these operators read.
+//  - Shapes. The reference compiles its shapes in (hidden 5120, intermediate 576 a rank at TP = 4, top-6). They are runtime
+//    values here, set once with dsk::set_shape (default: the whole layer on one GPU, hidden 5120, intermediate 2304,
+//    256 routed experts, top-6); moe_workspace_bytes() and moe() read them.
+//  - The 1-bit scale code (ScaleCode, dsk.h:181-198) is accepted and must be empty: scales are read as stored.
+//  - moe_prefill on MXFP4 layers runs the chunk through the decode operator sixteen rows at a time: the bits the reference
+//    promises ("the same result as moe()", dsk.h:284-286), not yet a grouped GEMM.
+// The FP8 e4m3 / 128 x 128 block-scaled configuration (bf16 rows, a dsgx_layer_w) is served by the overloads at the end.
 #pragma once
 #include <cstddef>
 #include <cstdint>
@@ -11,76 +22,140 @@
 
 namespace dsk {
 
-// dsk.h:171-176: scores sqrt(softplus(l)), top-k of scores + bias, weights = scores / (sum + 1e-20) * route_scale
-inline void router_topk(const float* logits, const float* bias, int M, int E, int* idx, float* wts, float route_scale, void* st,
-                        int topk = 6, int score_fn = 1) {
-  DSGX_DIE_ON(dsgx_route(logits, bias, M, E, topk, route_scale, score_fn, idx, wts, st));
+constexpr int kLowRows = 8;    // dsk.h:22-27
+constexpr int kMaxRows = 16;
+constexpr int kTopK = 6;
+constexpr int kMaxUnion = kMaxRows * kTopK;
+constexpr int row_budget(int M) { return M <= kLowRows ? kLowRows : kMaxRows; }
+
+struct Shape {
+  int dim = 5120, inter = 2304, experts = 256, topk = kTopK;
+};
+inline Shape& shape() {
+  static Shape s;
+  return s;
+}
+inline void set_shape(int dim, int inter, int experts, int topk = kTopK) { shape() = Shape{dim, inter, experts, topk}; }
+
+// dsk.h:171-176: scores sqrt(softplus(l)), top-6 of scores + bias (descending), weights = scores / (sum + 1e-20) * route_scale
+inline void router_topk(const float* logits, const float* bias, int M, int E, int* idx, float* wts, float route_scale, void* st) {
+  DSGX_DIE_ON(dsgx_route(logits, bias, M, E, shape().topk, route_scale, 1, idx, wts, st));
 }
 
-// dsk.h:199-209 keeps MXFP4 fields; this build takes the layer as a dsgx_layer_w of FP8_B128 matrices.
+// dsk.h:177-180 (tile_fp4) and its FP8 twin: the load-time re-layout. Row-major is this build's layout, so both copy:
+// w [N][K/2] (e2m1 pairs, low nibble first), s [N][K/32] -> wt, st of the same sizes; FP8: w [N][K], s [N/32][K/32].
+inline void tile_fp4(const uint8_t* w, const uint8_t* s, uint8_t* wt, uint8_t* st, int N, int K, void* stream) {
+  DSGX_DIE_ON(dsgx_stream_copy(w, wt, (size_t)N * K / 2, stream));
+  DSGX_DIE_ON(dsgx_stream_copy(s, st, (size_t)N * K / 32, stream));
+}
+inline void tile_fp8(const uint8_t* w, const uint8_t* s, uint8_t* wt, uint8_t* st, int N, int K, void* stream) {
+  DSGX_DIE_ON(dsgx_stream_copy(w, wt, (size_t)N * K, stream));
+  DSGX_DIE_ON(dsgx_stream_copy(s, st, (size_t)(N / 32) * (K / 32), stream));
+}
+
+// dsk.h:181-198: the reference's 1-bit code of the scale tensors, a GB10 bandwidth saving. Accepted empty only.
+struct ScaleCode {
+  const uint32_t* code = nullptr;
+  uint32_t base4 = 0;
+};
+
+// dsk.h:199-209. Routed experts stacked by expert id ([E][rows][...]: expert e at e times the per-expert size): w1, w3
+// [inter][dim] and w2 [dim][inter] MXFP4 with their ue8m0 scales; the shared expert FP8 with [N/32][K/32] scales.
 struct MoeWeights {
-  const uint8_t *w1 = nullptr, *s1 = nullptr, *w3 = nullptr, *s3 = nullptr, *w2 = nullptr, *s2 = nullptr;  // tiled L3: refused
-  const dsgx_layer_w* fp8 = nullptr;  // the FP8-128 layer (routed pool + descriptors + fused shared expert)
-  const dsgx_layer_w* mx = nullptr;   // the MXFP4_G32 layer (pool + descriptors; sh.g/u/d + sh.gs/us/ds as ue8m0 bytes: FP8_B32E)
+  const uint8_t *w1, *s1, *w3, *s3, *w2, *s2;
+  const uint8_t *sh_w1, *sh_s1, *sh_w3, *sh_s3, *sh_w2, *sh_s2;
+  ScaleCode c1{}, c3{}, c2{};
 };
+
+// dsk.h:211-223. The variants name the reference's GB10 launch shapes; one implementation serves them all here.
 struct MoeCfg {
-  int up = 0, down = 0;
+  int up = 0, down = 4;
+  int up_grid = 0;
   bool pdl = true;
-  int phases = 3;
+  int phases = 3;  // bit 0: moe_up, bit 1: moe_down (benchmarks)
+  bool dyn = false;
+  int up16 = 4, down16 = 2;
 };
-inline size_t moe_workspace_bytes(const MoeWeights& w) { return w.mx ? dsgx_decode_ws_bytes(w.mx) : w.fp8 ? dsgx_decode_ws_bytes(w.fp8) : 0; }
-// y [M][H] f32 = sum over each row's picks in expert-id order + the shared expert (dsk.h:226-233). x is bf16 here
-// (the FP8-128 decode contract keeps bf16 activations); ys is scratch for the shared expert's output.
-inline void moe(const uint16_t* x, int M, const int* idx, const float* wts, const MoeWeights& w, void* ws, float* y, float* ys,
+
+namespace detail {
+inline dsgx_dsk_weights c_weights(const MoeWeights& w, const char* who) {
+  if (w.c1.code || w.c3.code || w.c2.code) die("%s: the 1-bit scale code is a GB10 format; pass the scales as stored (ScaleCode empty)", who);
+  const Shape& s = shape();
+  return dsgx_dsk_weights{w.w1, w.s1, w.w3, w.s3, w.w2, w.s2, w.sh_w1, w.sh_s1, w.sh_w3, w.sh_s3, w.sh_w2, w.sh_s2, s.dim, s.inter, s.experts, s.topk};
+}
+}  // namespace detail
+
+// dsk.h:225
+inline size_t moe_workspace_bytes() { return dsgx_dsk_ws_bytes(shape().dim, shape().inter); }
+
+// dsk.h:226-233: y [M][dim] f32 = the sum over each row's picks, in expert-id order, of bf16(expert(x) * weight), plus the
+// shared expert. xq / xs = act_quant(x); idx / wts [M][6] from the router; ws of moe_workspace_bytes(), zeroed once.
+inline void moe(const uint8_t* xq, const uint8_t* xs, int M, const int* idx, const float* wts, const MoeWeights& w, void* ws, float* y,
                 MoeCfg cfg, void* st) {
-  if (w.w1 || w.w2 || w.w3) die("dsk::moe: bf16 rows go with an FP8_B128 layer (MoeWeights::fp8); MXFP4 layers take act_quant(x)");
-  if (!w.fp8) die("dsk::moe: no layer");
+  const dsgx_dsk_weights c = detail::c_weights(w, "dsk::moe");
+  dsgx_dsk_cfg d;
+  dsgx_dsk_cfg_default(&d);
+  d.parts = cfg.phases;
+  DSGX_DIE_ON(dsgx_dsk_moe_stacked(&c, xq, xs, M, idx, wts, ws, y, st, &d, nullptr, nullptr));
+}
+// dsk.h:234-241: the same with router_topk's selection inside the kernel; idx_out / wts_out [M][6] (optional) receive it
+inline void moe_routed(const uint8_t* xq, const uint8_t* xs, int M, const float* logits, const float* bias, int E, float route_scale,
+                       const MoeWeights& w, void* ws, float* y, MoeCfg cfg, void* st, int* idx_out = nullptr, float* wts_out = nullptr) {
+  if (E != shape().experts) die("dsk::moe_routed: %d logits a row for a layer of %d experts (dsk::set_shape)", E, shape().experts);
+  if ((idx_out == nullptr) != (wts_out == nullptr)) die("dsk::moe_routed: idx_out and wts_out go together");
+  const dsgx_dsk_weights c = detail::c_weights(w, "dsk::moe_routed");
+  dsgx_dsk_cfg d;
+  dsgx_dsk_cfg_default(&d);
+  d.parts = cfg.phases, d.logits = logits, d.bias = bias, d.route_scale = route_scale;
+  DSGX_DIE_ON(dsgx_dsk_moe_stacked(&c, xq, xs, M, nullptr, nullptr, ws, y, st, &d, idx_out, wts_out));
+}
+
+// dsk.h:284-295. The chunk goes through moe() sixteen rows at a time: ws needs moe()'s workspace only.
+struct MoePCfg {
+  int phases = 31;
+  void* side = nullptr;   // accepted, unused
+  int col0 = 0, cols = 0; // must be 0: all columns
+};
+inline size_t moe_prefill_workspace_bytes(int M, int E) {
+  (void)M, (void)E;
+  return moe_workspace_bytes();
+}
+inline void moe_prefill(const uint8_t* xq, const uint8_t* xs, int M, const int* idx, const float* wts, int E, const MoeWeights& w, void* ws,
+                        float* y, void* st, MoePCfg cfg = MoePCfg{}) {
+  if (E != shape().experts) die("dsk::moe_prefill: E %d for a layer of %d experts (dsk::set_shape)", E, shape().experts);
+  if (cfg.phases != 31 || cfg.col0 || cfg.cols) die("dsk::moe_prefill: phases %d, columns [%d, +%d): the whole step only", cfg.phases, cfg.col0, cfg.cols);
+  const Shape& s = shape();
+  for (int m0 = 0; m0 < M; m0 += kMaxRows) {
+    const int m = M - m0 < kMaxRows ? M - m0 : kMaxRows;
+    moe(xq + (size_t)m0 * s.dim, xs + (size_t)m0 * (s.dim / 32), m, idx + (size_t)m0 * s.topk, wts + (size_t)m0 * s.topk, w, ws,
+        y + (size_t)m0 * s.dim, MoeCfg{}, st);
+  }
+}
+
+// ---- the FP8 e4m3 / 128 x 128 block-scaled configuration: bf16 rows, a dsgx_layer_w (pool + descriptors + fused shared expert) ----
+inline size_t moe_workspace_bytes(const dsgx_layer_w& L) { return dsgx_decode_ws_bytes(&L); }
+// y = the routed sum + the shared expert's rows; ys: scratch f32 [M][H] for the latter
+inline void moe(const uint16_t* x, int M, const int* idx, const float* wts, const dsgx_layer_w& L, void* ws, float* y, float* ys, MoeCfg cfg,
+                void* st) {
   dsgx_decode_cfg d;
   dsgx_decode_cfg_default(&d);
   d.parts = cfg.phases, d.ysum = 1;
-  DSGX_DIE_ON(dsgx_moe_decode(w.fp8, x, idx, wts, M, ws, y, ys, st, &d));
+  DSGX_DIE_ON(dsgx_moe_decode(&L, x, idx, wts, M, ws, y, ys, st, &d));
 }
-// dsk.h:226-233, the reference's own form: xq / xs = act_quant(x) (e4m3 [M][H], ue8m0 [M][H / 32]), MXFP4 experts, the
-// shared expert last. ys: scratch f32 [M][H] (receives the shared expert's output; the reference keeps it in shared memory).
-inline void moe(const uint8_t* xq, const uint8_t* xs, int M, const int* idx, const float* wts, const MoeWeights& w, void* ws, float* y,
-                MoeCfg cfg, void* st, float* ys, float swiglu_limit = 10.f) {
-  if (w.w1 || w.w2 || w.w3) die("dsk::moe: the tiled MXFP4 tensors are a GB10 lane order; pass the layer in row-major form (MoeWeights::mx)");
-  if (!w.mx) die("dsk::moe: no MXFP4 layer");
-  dsgx_dsk_cfg d;
-  dsgx_dsk_cfg_default(&d);
-  d.parts = cfg.phases, d.swiglu_limit = swiglu_limit;
-  DSGX_DIE_ON(dsgx_dsk_moe(w.mx, xq, xs, M, idx, wts, ws, y, ys, st, &d));
-}
-// dsk.h:234-241: the same with router_topk's selection inside the kernels
-inline void moe_routed(const uint8_t* xq, const uint8_t* xs, int M, const float* logits, const float* bias, int E, float route_scale,
-                       const MoeWeights& w, void* ws, float* y, MoeCfg cfg, void* st, float* ys, float swiglu_limit = 10.f) {
-  if (w.w1 || w.w2 || w.w3) die("dsk::moe_routed: the tiled MXFP4 tensors are a GB10 lane order; pass the layer in row-major form (MoeWeights::mx)");
-  if (!w.mx) die("dsk::moe_routed: no MXFP4 layer");
-  if (E != w.mx->E) die("dsk::moe_routed: %d logits a row for a layer of %d experts", E, w.mx->E);
-  dsgx_dsk_cfg d;
-  dsgx_dsk_cfg_default(&d);
-  d.parts = cfg.phases, d.swiglu_limit = swiglu_limit, d.logits = logits, d.bias = bias, d.route_scale = route_scale;
-  DSGX_DIE_ON(dsgx_dsk_moe(w.mx, xq, xs, M, nullptr, nullptr, ws, y, ys, st, &d));
-}
-// the router's selection fused in (dsk.h:234-241), FP8-128 layers
-inline void moe_routed(const uint16_t* x, int M, const float* logits, const float* bias, float route_scale, const MoeWeights& w,
-                       void* ws, float* y, float* ys, MoeCfg cfg, void* st, int score_fn = 0) {
-  if (w.w1 || w.w2 || w.w3) die("dsk::moe_routed: MXFP4 experts are not built on this path; pass an FP8_B128 layer");
-  if (!w.fp8) die("dsk::moe_routed: no layer");
+inline void moe_routed(const uint16_t* x, int M, const float* logits, const float* bias, float route_scale, const dsgx_layer_w& L, void* ws,
+                       float* y, float* ys, MoeCfg cfg, void* st, int score_fn = 0) {
   dsgx_decode_cfg d;
   dsgx_decode_cfg_default(&d);
   d.parts = cfg.phases, d.ysum = 1, d.logits = logits, d.bias = bias, d.route_scale = route_scale, d.score_fn = score_fn;
-  DSGX_DIE_ON(dsgx_moe_decode(w.fp8, x, nullptr, nullptr, M, ws, y, ys, st, &d));
+  DSGX_DIE_ON(dsgx_moe_decode(&L, x, nullptr, nullptr, M, ws, y, ys, st, &d));
 }
-inline size_t moe_prefill_workspace_bytes(const MoeWeights& w, int M) { return w.fp8 ? dsgx_prefill_ws_bytes(w.fp8, M) : 0; }
-inline void moe_prefill(const uint16_t* x, int M, const int* idx, const float* wts, const MoeWeights& w, void* ws, float* y, float* ys,
-                        void* st, int phases = 31) {
-  if (w.w1 || w.w2 || w.w3) die("dsk::moe_prefill: MXFP4 experts are not built on this path; pass an FP8_B128 layer");
-  if (!w.fp8) die("dsk::moe_prefill: no layer");
+inline size_t moe_prefill_workspace_bytes(const dsgx_layer_w& L, int M) { return dsgx_prefill_ws_bytes(&L, M); }
+inline void moe_prefill(const uint16_t* x, int M, const int* idx, const float* wts, const dsgx_layer_w& L, void* ws, float* y, float* ys, void* st,
+                        int phases = 31) {
   dsgx_prefill_cfg p;
   dsgx_prefill_cfg_default(&p);
   p.phases = phases;
-  DSGX_DIE_ON(dsgx_moe_prefill(w.fp8, x, idx, wts, M, ws, y, ys, st, &p));
+  DSGX_DIE_ON(dsgx_moe_prefill(&L, x, idx, wts, M, ws, y, ys, st, &p));
 }
 
 }  // namespace dsk

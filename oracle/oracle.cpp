@@ -265,7 +265,44 @@ static inline float route_sum(const float* p, int k) {
 }
 // A/engine/experts/tests/testdata.h:339-355 (route_ref) with E, top-k and the scale as arguments; bias may be null.
 // score_fn 1: sqrt(softplus(l)), softplus as torch's (l > 20 ? l : log1p(exp(l))): D/engine/kernels/common.cuh:261-315.
-static inline float route_score(float v, int score_fn) { return score_fn == 0 ? route_sigmoid(v) : sqrtf(v > 20.f ? v : log1pf(expf(v))); }
+// softplus(l) = log1p(exp(l)) for l <= 20 from IEEE operations only (+, -, *, /, fma, rint, ldexp on normal numbers), so
+// that the CPU and the GPU give the same bits, as route_sigmoid does for the sigmoid: the reference's own form
+// log1pf(expf(l)) (common.cuh:281) depends on the math library. exp: the sigmoid's reduction and polynomial. log1p(e):
+// u = 1 + e; log(u) e / (u - 1) (the rounding of 1 + e cancels), log by the classic reduction u = 2^k (1 + f),
+// sqrt(1/2) < 1 + f < sqrt(2), s = f / (2 + f), log(1 + f) = f - f^2/2 + s (f^2/2 + R(s^2)) with the degree-7 minimax R of
+// e_logf.c (Sun's fdlibm). Logits below -87 are taken as -87 (a score of 1e-19 either way).
+static inline float route_softplus(float l) {
+  if (l < -87.f) l = -87.f;
+  const float n = rintf(l * 1.44269504f);
+  float r = fmaf(-n, 0.693145751953125f, l);
+  r = fmaf(-n, 1.428606765330187e-06f, r);
+  float p = 1.f / 5040;
+  p = fmaf(p, r, 1.f / 720);
+  p = fmaf(p, r, 1.f / 120);
+  p = fmaf(p, r, 1.f / 24);
+  p = fmaf(p, r, 1.f / 6);
+  p = fmaf(p, r, 0.5f);
+  p = fmaf(p, r, 1.f);
+  p = fmaf(p, r, 1.f);
+  const float e = ldexpf(p, (int)n);
+  const float u = 1.f + e;
+  if (u == 1.f) return e;
+  uint32_t ix; memcpy(&ix, &u, 4);
+  int k = (int)(ix >> 23) - 127;
+  ix &= 0x007fffffu;
+  const uint32_t i = (ix + (0x95f64u << 3)) & 0x800000u;   // mantissa above sqrt(2): halve it, k + 1
+  ix |= i ^ 0x3f800000u;
+  k += (int)(i >> 23);
+  float m; memcpy(&m, &ix, 4);
+  const float f = m - 1.f, dk = (float)k;
+  const float s_ = f / (2.f + f), z = s_ * s_, w = z * z;
+  const float t1 = w * (0.40000000596f + w * (0.22222198546f + w * 0.15313838422f));
+  const float t2 = z * (0.66666668653f + w * (0.28571429849f + w * (0.18183572590f + w * 0.14798198640f)));
+  const float R = t2 + t1, hfsq = 0.5f * f * f;
+  const float lg = dk * 0.69313812256f - ((hfsq - (s_ * (hfsq + R) + dk * 9.0580006145e-06f)) - f);
+  return lg * (e / (u - 1.f));
+}
+static inline float route_score(float v, int score_fn) { return score_fn == 0 ? route_sigmoid(v) : sqrtf(v > 20.f ? v : route_softplus(v)); }
 ORC float orc_route_score(float l, int score_fn) { return route_score(l, score_fn); }
 ORC void orc_route(const float* l, const float* bias, int M, int E, int topk, float scale, int score_fn, int* idx, float* w) {
   std::vector<float> s(E), key(E);

@@ -36,8 +36,21 @@ int main() {
   gx::DecodeCfg dc;
   gx::PrefillCfg pc;
   glm::GemvSeg seg;
-  dsk::MoeWeights mw;
-  bad += dc.parts != 3 || !pc.shared || seg.rs != 128 || mw.fp8 != nullptr, ++n;
+  dsk::MoeWeights mw{};
+  dsk::MoeCfg mc;
+  bad += dc.parts != 3 || !pc.shared || seg.rs != 128 || mw.sh_w1 != nullptr || mw.c1.code != nullptr || mc.phases != 3 || mc.down != 4, ++n;
+  // the reference's argument lists (ds41f-4xgx10-switchless/engine/kernels/dsk.h:171-176, 225-241, 284-295): these initialisations
+  // only compile if the mirror declares exactly them
+  void (*p_topk)(const float*, const float*, int, int, int*, float*, float, void*) = &dsk::router_topk;
+  size_t (*p_ws)() = &dsk::moe_workspace_bytes;
+  void (*p_moe)(const uint8_t*, const uint8_t*, int, const int*, const float*, const dsk::MoeWeights&, void*, float*, dsk::MoeCfg, void*) = &dsk::moe;
+  void (*p_routed)(const uint8_t*, const uint8_t*, int, const float*, const float*, int, float, const dsk::MoeWeights&, void*, float*, dsk::MoeCfg,
+                   void*, int*, float*) = &dsk::moe_routed;
+  size_t (*p_pws)(int, int) = &dsk::moe_prefill_workspace_bytes;
+  void (*p_pf)(const uint8_t*, const uint8_t*, int, const int*, const float*, int, const dsk::MoeWeights&, void*, float*, void*, dsk::MoePCfg) =
+      &dsk::moe_prefill;
+  bad += !p_topk || !p_ws || !p_moe || !p_routed || !p_pws || !p_pf, ++n;
+  bad += dsk::kTopK != 6 || dsk::row_budget(9) != 16 || dsk::shape().dim != 5120, ++n;
   bad += gx::decode_ws_bytes(L) < (size_t)(128 + 1) * 16 * 512 * 2 + 256, ++n;  // h as decode.cu:33-35, then the counters
   std::printf("CHECK mirror headers %s  %d wrong of %d\n", bad ? "FAIL" : "ok", bad, n);
   return bad != 0;

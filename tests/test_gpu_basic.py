@@ -136,14 +136,19 @@ def test_route_ids_and_weight_bits(E, topk, scale):
     assert np.array_equal(gi, ri) and np.array_equal(gw.view(np.uint32), rw.view(np.uint32))
 
 
-def test_route_sqrt_softplus_close():
-    # DeepSeek's score function goes through libm on both sides: ids equal where the margin allows, weights to 1e-6
+def test_route_sqrt_softplus_bits():
+    """DeepSeek's score sqrt(softplus(l)) is built from IEEE operations only on both sides (as the sigmoid is): ids and
+    weight bits equal the oracle's, on random rows, on rows with a bias, on logits across the whole range incl. both sides of
+    the switch at 20, and on engineered ties"""
     l = orc.normal_f32(3, 2, (16, 384), 1.0)
-    ri, rw = orc.route(l, None, 6, 1.5, score_fn=1)
-    gi, gw = _route_gpu(l, None, 6, 1.5, score_fn=1)
-    assert (gi != ri).mean() < 0.02
-    same = gi == ri
-    assert np.allclose(gw[same], rw[same], rtol=2e-6, atol=0)
+    wide = np.linspace(-95, 30, 16 * 384, dtype=np.float32).reshape(16, 384)[:, ::-1].copy()
+    ties = l.copy()
+    ties[:, 7] = ties[:, 300] = ties[:, 301] = 3.25   # a three-way tie at the top: lower ids first
+    bias = orc.normal_f32(3, 9, (384,), 0.1)
+    for logits, b in ((l, None), (l * 4, bias), (wide, None), (ties, None), (ties, bias)):
+        ri, rw = orc.route(logits, b, 6, 1.5, score_fn=1)
+        gi, gw = _route_gpu(logits, b, 6, 1.5, score_fn=1)
+        assert np.array_equal(gi, ri) and np.array_equal(gw.view(np.uint32), rw.view(np.uint32))
 
 
 def test_finalize_bits():

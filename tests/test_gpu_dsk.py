@@ -95,3 +95,35 @@ def test_dsk_moe_against_oracle(H, I, E, M, shared, fused):
     print("dsk moe H=%d I=%d M=%d: h equal %.2f%%, end-to-end rel-L2 %.2e max-abs %.2e (|y| max %.2f)"
           % (H, I, M, 100 - 100.0 * nbad / nh, rl2, np.abs(y - ref).max(), np.abs(ref).max()))
     assert rl2 <= 3e-3
+
+
+@pytest.mark.parametrize("M", [12, 16])
+def test_dsk_moe_nine_to_sixteen_rows(M):
+    """9-16 rows run as two passes of the kernels built for eight (dsk.h:211-223's up16 / down16 range): every row's bits are
+    what the row gives in a call of its own, whose parity with the oracle the test above holds; routing fused and apart"""
+    H, I, E, topk = 2048, 768, 32, 6
+    hl = _layer(22, H, I, E, topk, 5, True)
+    dl = hl.upload()
+    x = orc.normal_bf16(22, 1, (M, H), 1.5)
+    xq, xs = orc.act_quant_ue8m0(x)
+    logits, bias = orc.normal_f32(22, 2, (M, E), 1.0), orc.normal_f32(22, 3, (E,), 0.2)
+    idx, w = orc.route(logits, bias, topk, 1.5, score_fn=1)
+    ws = gpu.empty(lib.decode_ws_bytes(dl.w), 0)
+
+    def run(rows, fused):
+        n = len(rows)
+        y, ys = gpu.empty(n * H * 4, 0xFF), gpu.empty(n * H * 4, 0xFF)
+        if fused:
+            lib.dsk_moe(dl.w, gpu.dev(xq[rows]), gpu.dev(xs[rows]), None, None, n, ws, y, ys, logits=gpu.dev(logits[rows]), bias=gpu.dev(bias), route_scale=1.5)
+        else:
+            lib.dsk_moe(dl.w, gpu.dev(xq[rows]), gpu.dev(xs[rows]), gpu.dev(idx[rows]), gpu.dev(w[rows]), n, ws, y, ys)
+        lib.decode_status(dl.w, ws)
+        return gpu.host(y, np.uint32, (n, H)), gpu.host(ys, np.uint32, (n, H))
+    all_rows = list(range(M))
+    y, ys = run(all_rows, False)
+    yf, ysf = run(all_rows, True)
+    assert np.array_equal(y, yf) and np.array_equal(ys, ysf)
+    for m in (0, 7, 8, M - 1):
+        y1, ys1 = run([m], False)
+        assert np.array_equal(y[m], y1[0]) and np.array_equal(ys[m], ys1[0]), m
+    assert np.isfinite(y.view(np.float32)).all()

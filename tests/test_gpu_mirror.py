@@ -73,3 +73,45 @@ def test_cpp_mirrors_give_the_c_abi_bits(fmt, shared, scale, up):
     lib.add_norm(gpu.dev(yr2), None, M, H, r16, r16, gpu.dev(normw), 1e-5, xn)
     assert np.array_equal(got["h"], gpu.host(r16, np.uint16, (-1,))) and np.array_equal(got["xn"], gpu.host(xn, np.uint16, (-1,)))
     assert np.array_equal(got["h"], orc.add_norm(yr2, None, res16, normw, 1e-5)[0].reshape(-1))
+
+
+@pytest.mark.parametrize("H,I,E,M,shared", [(1024, 512, 16, 3, True), (2048, 768, 32, 12, True), (1024, 256, 8, 16, False)])
+def test_dsk_mirror_gives_the_c_abi_bits(H, I, E, M, shared):
+    """include/dsk/dsk.h with the reference's own argument lists (tests/mirror_run_dsk.cpp): experts stacked by id after
+    tile_fp4 / tile_fp8, router_topk -> moe, moe_routed with idx_out / wts_out, moe_prefill; against dsgx_route and dsgx_dsk_moe
+    on a pooled layer of the same weights (whose parity with the oracle tests/test_gpu_dsk.py holds), bit for bit. 12 and 16 rows
+    take two passes of the kernels."""
+    from tests.test_gpu_dsk import _layer
+    exe = os.path.join(ROOT, "tests", "mirror_run_dsk")
+    assert os.path.exists(exe), "tests/mirror_run_dsk is not built (python -m dsgx10_amd.build)"
+    topk, scale = 6, 1.5
+    hl = _layer(33, H, I, E, topk, 5, shared)
+    dl = hl.upload()
+    x = orc.normal_bf16(33, 1, (M, H), 1.5)
+    xq, xs = orc.act_quant_ue8m0(x)
+    logits, bias = orc.normal_f32(33, 2, (M, E), 1.0), orc.normal_f32(33, 3, (E,), 0.2)
+    with tempfile.TemporaryDirectory() as d:
+        def put(name, a):
+            np.ascontiguousarray(a).tofile(os.path.join(d, name + ".bin"))
+        for j, n in enumerate(("1", "3", "2")):
+            put("w" + n, np.stack([hl.experts[int(hl.emap[e])][j][0] for e in range(E)]))
+            put("s" + n, np.stack([hl.experts[int(hl.emap[e])][j][1] for e in range(E)]))
+            if shared:
+                put("sh_w" + n, hl.shared_fp8[j][0]), put("sh_s" + n, hl.shared_fp8[j][1])
+        put("xq", xq), put("xs", xs), put("logits", logits), put("bias", bias)
+        r = subprocess.run([exe, d, str(H), str(I), str(E), str(M), repr(scale), str(int(shared))], capture_output=True, text=True, timeout=120)
+        assert r.returncode == 0 and "CHECK mirror_run_dsk ok" in r.stdout, r.stdout + r.stderr
+        got = {n: np.fromfile(os.path.join(d, "o_%s.bin" % n), dt) for n, dt in
+               (("idx", np.int32), ("w", np.uint32), ("idx2", np.int32), ("w2", np.uint32), ("y", np.uint32), ("y2", np.uint32), ("y3", np.uint32))}
+    idx, w = orc.route(logits, bias, topk, scale, score_fn=1)
+    for k in ("idx", "idx2"):
+        assert np.array_equal(got[k], idx.reshape(-1)), k
+    for k in ("w", "w2"):
+        assert np.array_equal(got[k], w.view(np.uint32).reshape(-1)), k
+    ws = gpu.empty(lib.decode_ws_bytes(dl.w), 0)
+    y, ys = gpu.empty(M * H * 4, 0xFF), gpu.empty(M * H * 4, 0xFF)
+    lib.dsk_moe(dl.w, gpu.dev(xq), gpu.dev(xs), gpu.dev(idx), gpu.dev(w), M, ws, y, ys)
+    want = gpu.host(y, np.uint32, (-1,))
+    assert np.isfinite(want.view(np.float32)).all()
+    for k in ("y", "y2", "y3"):
+        assert np.array_equal(got[k], want), (k, int((got[k] != want).sum()))
