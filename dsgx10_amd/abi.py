@@ -6,7 +6,8 @@ FMT_FP8, FMT_INT4, FMT_BF16 = 16, 18, 19
 FMT_MXFP4, FMT_FP8E = 20, 21  # DeepSeek's routed experts; their shared expert (ue8m0 scales per 32 x 32)
 OUT_BF16, OUT_F32, OUT_SWIGLU = 0, 1, 2
 MAX_ROWS, MAX_TOPK, MAX_UNION, SH_SLOT, MAX_EXPERTS, MAX_CHUNK = 16, 8, 128, 128, 512, 8192
-UP_PREFILL_ORDER = 6  # dsgx_decode_cfg.up: the rows through the prefill kernels (gx::kUpPrefillOrder)
+UP_PREFILL_ORDER = 6  # dsgx_decode_cfg.up: the rows through the prefill kernels (gx::kUpPrefillOrder), bf16 activations
+UP_PREFILL_ORDER_ACT_FP8 = 7  # ... with FP8 activations (the default prefill of FP8 layers)
 OK, EINVAL, EFORMAT, EUNSUPPORTED, EHIP, ETIMEOUT = 0, 1, 2, 3, 4, 5
 NOALLOC_MAX_H, NOALLOC_MAX_I = 6144, 2048
 

@@ -151,7 +151,9 @@ static int decode_by_prefill(const dsgx_layer_w* L, const uint16_t* x, const int
   }
   dsgx_prefill_cfg p;
   dsgx_prefill_cfg_default(&p);
-  p.act_fp8 = 0;
+  p.act_fp8 = c.up == DSGX_UP_PREFILL_ORDER_ACT_FP8 ? 1 : 0;
+  if (p.act_fp8 && L->fmt != DSGX_FMT_FP8_B128)
+    return fail(DSGX_EUNSUPPORTED, "moe_decode: up = %d pairs with a prefill on FP8 activations, which FP8_B128 layers have (format %u)", c.up, L->fmt);
   if (int rc = dsgx_moe_prefill(L, x, idx, w, M, ws, yr, ys, stream, &p)) return rc;
   if (c.ysum) {
     if (!ys) return fail(DSGX_EINVAL, "moe_decode: ysum without ys");
@@ -173,7 +175,7 @@ static int moe_decode_at(const dsgx_layer_w* L, const uint16_t* x, const int* id
   if (!c.logits && (!idx || !w)) return fail(DSGX_EINVAL, "moe_decode: idx and w, or logits");
   if (c.post) return fail(DSGX_EUNSUPPORTED, "moe_decode: posted outputs need the reference's ring; one GPU has none");
   if (c.parts < 1 || c.parts > 3) return fail(DSGX_EINVAL, "moe_decode: parts %d", c.parts);
-  if (c.up == DSGX_UP_PREFILL_ORDER) return decode_by_prefill(L, x, idx, w, M, ws, lay, yr, ys, stream, c, dsk.on != 0);
+  if (c.up == DSGX_UP_PREFILL_ORDER || c.up == DSGX_UP_PREFILL_ORDER_ACT_FP8) return decode_by_prefill(L, x, idx, w, M, ws, lay, yr, ys, stream, c, dsk.on != 0);
   if (c.up < -1 || c.up > 1 || c.down < 0 || c.down > 1) return fail(DSGX_EINVAL, "moe_decode: up variant %d / down variant %d", c.up, c.down);
   if (c.up == -1) c.up = c.down == 1 ? 0 : decode_variant(L->fmt, M, L->H, L->I);  // (the two-launch form is the vector-unit kernels')
   if (c.up == 1 && L->fmt != DSGX_FMT_FP8_B128 && L->fmt != DSGX_FMT_INT4_G32 && L->fmt != DSGX_FMT_MXFP4_G32)

@@ -110,6 +110,7 @@ DSGX_API int dsgx_route(const float* logits, const float* bias, int M, int E, in
 
 /* ---- decode: gx::moe_decode (engine/experts/experts.h:104-147, decode.cu:708-730) ------------------------------- */
 #define DSGX_UP_PREFILL_ORDER 6 /* gx::kUpPrefillOrder (engine/experts/experts.h:138) */
+#define DSGX_UP_PREFILL_ORDER_ACT_FP8 7 /* the same against a prefill on FP8 activations (dsgx_prefill_cfg::act_fp8 = 1, its default) */
 typedef struct dsgx_decode_cfg {
   int32_t up, down;        /* kernel variants (the reference's DecodeCfg::up / down choose among its launch shapes too).
                               up -1 (the default): the faster of the two below for the layer's format and row count
@@ -118,9 +119,12 @@ typedef struct dsgx_decode_cfg {
                               the same in any batch within a variant; the two variants differ in the order of the f32 adds
                               inside a dot product, so a caller that needs a row's bits not to depend on the row count
                               names the variant. up DSGX_UP_PREFILL_ORDER (6, the reference's kUpPrefillOrder): the rows go
-                              through the prefill kernels (bf16 activations) and yr, ys are dsgx_moe_prefill's of the same rows bit
-                              for bit; parts 3 only; the workspace then holds the chunk's intermediates (dsgx_prefill_view's
-                              layout) instead of the step's h slots. down (with up 0) 0: both phases in one persistent
+                              through the prefill kernels with bf16 activations and yr, ys are bit for bit those of
+                              dsgx_moe_prefill with act_fp8 = 0 on the same rows; up DSGX_UP_PREFILL_ORDER_ACT_FP8 (7; FP8_B128
+                              layers): with FP8 activations, the bits of dsgx_moe_prefill's DEFAULT configuration (act_fp8 = 1) - a
+                              caller that verifies drafted tokens against a prefill names the one its prefill uses. Both: parts 3
+                              only; the workspace then holds the chunk's intermediates (dsgx_prefill_view's layout) instead of the
+                              step's h slots. down (with up 0) 0: both phases in one persistent
                               kernel; 1: two launches */
   int32_t parts;           /* 1 up only, 2 down only, 3 both (bench) */
   int32_t ysum;            /* 1: yr += ys in f32 after the routed experts (experts.h:132-136) */

@@ -5,6 +5,7 @@ h against the f64 reference (bit-exact share and the f32-sum range), the outputs
 batch invariance, determinism, ys untouched without a fused shared expert, fused routing, ysum."""
 import numpy as np
 import pytest
+import torch
 
 from dsgx10_amd import abi, lib
 from tests import gpu, orc
@@ -270,3 +271,43 @@ def test_decode_prefill_order_variant(fmt, H, I, E, topk, shared, scale):
     assert np.array_equal(y0.view(np.uint32), y1.view(np.uint32)) and np.array_equal(s0.view(np.uint32), s1.view(np.uint32))
     with pytest.raises(lib.DsgxError):
         gpu.decode_layer(dl, x[:1], idx[:1], w[:1], 1, ws=ws, up=abi.UP_PREFILL_ORDER, parts=1)
+    # the pairing with a prefill on FP8 activations (the default prefill of FP8 layers) has a name of its own
+    if fmt == abi.FMT_FP8:
+        for M in (1, 7):
+            yr, ys, _ = gpu.decode_layer(dl, x[:M], idx[:M], w[:M], M, ws=ws, up=abi.UP_PREFILL_ORDER_ACT_FP8)
+            pws = gpu.empty(lib.prefill_ws_bytes(dl.w, M), 0)
+            pyr, pys = gpu.empty(M * H * 4, 0xFF), gpu.empty(M * H * 4, 0xFF)
+            lib.moe_prefill(dl.w, gpu.dev(x[:M]), gpu.dev(idx[:M]), gpu.dev(w[:M]), M, pws, pyr, pys)
+            assert np.array_equal(yr.view(np.uint32), gpu.host(pyr, np.uint32, (M, H)))
+            if hl.has_shared:
+                assert np.array_equal(ys.view(np.uint32), gpu.host(pys, np.uint32, (M, H)))
+    else:
+        with pytest.raises(lib.DsgxError):
+            gpu.decode_layer(dl, x[:1], idx[:1], w[:1], 1, ws=ws, up=abi.UP_PREFILL_ORDER_ACT_FP8)
+
+
+def test_decode_status_reports_a_timeout_and_repairs_the_workspace():
+    """dsgx_decode_status's ETIMEOUT branch, driven from the host (no kernel waits for anything): the error flag and
+    the barrier's counters are overwritten as a step that gave up would leave them; the status call reports ETIMEOUT once,
+    puts the words back, and the next fused steps on that workspace give the bits of a fresh one."""
+    H, I, E, topk = 2048, 1024, 16, 4
+    hl, dl = _layer(abi.FMT_FP8, H, I, E, topk, 4, "fp8")
+    x, logits, idx, w = rows_and_routing(31, 2, H, E, topk, 1.0)
+    want = gpu.decode_layer(dl, x, idx, w, 2)
+    ws = gpu.empty(lib.decode_ws_bytes(dl.w), 0)
+    off = lib.decode_ws_flag_offset(dl.w)
+    bar0 = (abi.MAX_UNION + 1) * abi.MAX_ROWS * I * 2   # the barrier's words follow h
+    assert bar0 < off < bar0 + 4352
+    got = gpu.decode_layer(dl, x, idx, w, 2, ws=ws)
+    lib.decode_status(dl.w, ws)
+    for rep in range(2):
+        gpu.view(ws, ws.data_ptr() + bar0, off + 4 - bar0).view(torch.int32).fill_(0x01010101)   # counters, release words, flag
+        torch.cuda.synchronize()
+        with pytest.raises(lib.DsgxError) as ei:
+            lib.decode_status(dl.w, ws)
+        assert ei.value.code == abi.ETIMEOUT
+        lib.decode_status(dl.w, ws)   # reported once; the workspace is usable again
+        for _ in range(2):
+            got = gpu.decode_layer(dl, x, idx, w, 2, ws=ws)
+            assert np.array_equal(got[0].view(np.uint32), want[0].view(np.uint32)) and np.array_equal(got[1].view(np.uint32), want[1].view(np.uint32))
+        lib.decode_status(dl.w, ws)
