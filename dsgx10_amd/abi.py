@@ -48,6 +48,11 @@ class PrefillView(C.Structure):
     _fields_ = [(n, C.c_void_p) for n in ("rpos", "re", "h", "hsh", "off", "perm")]
 
 
+class NormIn(C.Structure):
+    _fields_ = [("part", C.c_void_p), ("part2", C.c_void_p), ("res", C.c_void_p), ("res_out", C.c_void_p), ("w", C.c_void_p), ("eps", C.c_float),
+                ("xn", C.c_void_p), ("round2", C.c_int32)]
+
+
 class GemvSeg(C.Structure):
     _fields_ = [("fmt", C.c_int32), ("w", C.c_void_p), ("s", C.c_void_p), ("zp", C.c_void_p), ("n", C.c_int32),
                 ("rs", C.c_int32), ("ks", C.c_int32), ("y", C.c_void_p), ("ldy", C.c_int32)]
@@ -60,5 +65,5 @@ SYMBOLS = [
     "dsgx_mat_bytes", "dsgx_mat_scale_off", "dsgx_mat_zp_off", "dsgx_route", "dsgx_decode_cfg_default",
     "dsgx_decode_ws_bytes", "dsgx_decode_ws_flag_offset", "dsgx_decode_status", "dsgx_moe_decode", "dsgx_moe_decode_noalloc", "dsgx_finalize", "dsgx_add_norm", "dsgx_dsk_cfg_default", "dsgx_dsk_moe", "dsgx_dsk_ws_bytes", "dsgx_dsk_moe_stacked", "dsgx_prefill_cfg_default", "dsgx_prefill_ws_bytes",
     "dsgx_moe_prefill", "dsgx_prefill_view_get", "dsgx_gemv", "dsgx_dequant_int4", "dsgx_probe_dequant_int4", "dsgx_probe_mfma_fp8",
-    "dsgx_widen_fp8", "dsgx_act_quant", "dsgx_last_error", "dsgx_version", "dsgx_stream_read", "dsgx_stream_read_cfg", "dsgx_stream_copy",
+    "dsgx_widen_fp8", "dsgx_act_quant", "dsgx_last_error", "dsgx_version", "dsgx_stream_read", "dsgx_stream_read_cfg", "dsgx_stream_copy", "dsgx_add_norm_gemv", "dsgx_fill_normal", "dsgx_launch_floor",
 ]

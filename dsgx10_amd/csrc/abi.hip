@@ -6,6 +6,7 @@
 #include <unordered_map>
 
 #include "abi_internal.h"
+#include "addnorm.cuh"
 #include "common.cuh"
 
 namespace dsgx {
@@ -67,6 +68,33 @@ __global__ void __launch_bounds__(256) k_stream_copy(const uint4* __restrict__ s
   for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += stride) d[i] = s[i];
 }
 
+// N(0, sigma): splitmix64 keyed by (seed, tensor, index) -> Box-Muller in f64 (the oracle's generator; the reference's mix64,
+// engine/experts/formats.cuh:131-136)
+__device__ __forceinline__ uint64_t mix64(uint64_t x) {
+  x += 0x9E3779B97F4A7C15ull;
+  x = (x ^ (x >> 30)) * 0xBF58476D1CE4E5B9ull;
+  x = (x ^ (x >> 27)) * 0x94D049BB133111EBull;
+  return x ^ (x >> 31);
+}
+__global__ void __launch_bounds__(256) k_fill_normal(uint64_t key, size_t n, double sigma, void* out, int bf16) {
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+    const uint64_t h1 = mix64(key + 2 * i), h2 = mix64(key + 2 * i + 1);
+    const double u1 = (double)((h1 >> 11) + 1) * 0x1p-53, u2 = (double)(h2 >> 11) * 0x1p-53;
+    const float v = (float)(sigma * (sqrt(-2.0 * log(u1)) * cos(6.283185307179586476925286766559 * u2)));
+    if (bf16) static_cast<uint16_t*>(out)[i] = (uint16_t)f32_to_bf16_bits(v);
+    else static_cast<float*>(out)[i] = v;
+  }
+}
+__global__ void __launch_bounds__(64) k_floor_empty() {}
+__global__ void __launch_bounds__(64) k_floor_chain(const uint32_t* __restrict__ p, uint32_t* __restrict__ sink) {
+  const uint32_t l = threadIdx.x;
+  const u32x4_t a = *reinterpret_cast<const DSGX_GLOBAL u32x4_t*>((uintptr_t)(p + 4 * l));
+  const uint32_t at = ((a.x ^ a.y) & 0xFFFu) * 4u;  // (a 16-byte slot within the first 64 KiB, known only when the first load is back)
+  const u32x4_t b = *reinterpret_cast<const DSGX_GLOBAL u32x4_t*>((uintptr_t)(p + at));
+  if (l == 0) *sink = b.x ^ b.w;
+}
+
 // out = bf16(bf16(R) + bf16(S)) (engine/experts/decode.cu:591-598 of the reference)
 __global__ void __launch_bounds__(256) k_finalize(const float* __restrict__ R, const float* __restrict__ S, int n, uint16_t* __restrict__ out) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
@@ -74,64 +102,13 @@ __global__ void __launch_bounds__(256) k_finalize(const float* __restrict__ R, c
   out[i] = (uint16_t)f32_to_bf16_bits(__fadd_rn(bf16_round(R[i]), bf16_round(S[i])));
 }
 
-// The residual add and the next layer's RMSNorm after an MoE (or MLP) step: the local half of the reference's
-// comm::glm::allreduce_add_norm / allreduce2_add_norm (engine/comm/glmcoll.h:34-62) at one rank, the norm as
-// engine/attn/prep.cu:12-66 (k_rmsnorm). One workgroup a row:
-//   sum        = part                                   (one partial: the reference's decision 8, yr already holds yr + ys)
-//              | bf16(bf16(part) + bf16(part2))         (two partials: the old combine, experts.h finalize)
-//   h          = bf16(f32(res) + sum)                   (the contract: the f32 sum rounded once, with the residual)
-//              | bf16(f32(res) + bf16(sum))             (round2: the sum rounded first)
-//   xn         = bf16(w * bf16(h * rstd)),  rstd = 1 / sqrt(mean(h^2) + eps)
-// mean(h^2) in f32 in a fixed order: a thread's H / 256 contiguous values in order, the wave by a butterfly, the waves in
-// order (the reference fixes an order too, its own: the statistics' order is not part of the contract).
-__global__ void __launch_bounds__(256) k_add_norm(const float* __restrict__ part, const float* __restrict__ part2, int H,
-                                                  const uint16_t* __restrict__ res, uint16_t* __restrict__ res_out,
-                                                  const uint16_t* __restrict__ w, float eps, uint16_t* __restrict__ xn, int round2) {
+// The residual add and the next layer's RMSNorm after an MoE (or MLP) step, one workgroup a row (addnorm.cuh)
+__global__ void __launch_bounds__(256) k_add_norm(NormIn a, int H) {
   __shared__ float red[4];
-  const int row = blockIdx.x, tid = threadIdx.x, per = H / 256;  // (per a multiple of 8, at most 64: the host checks)
-  const size_t base = (size_t)row * H + (size_t)tid * per;
-  float hv[64];
-  float ss = 0.f;
-#pragma unroll
-  for (int i = 0; i < 64; i += 8) {
-    if (i >= per) break;
-    const u32x4_t rq = *reinterpret_cast<const DSGX_GLOBAL u32x4_t*>((uintptr_t)(res + base + i));
-    uint32_t ho[4];
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const float r = bf16_bits_to_f32(j & 1 ? rq[j >> 1] >> 16 : rq[j >> 1] & 0xFFFFu);
-      float s = part[base + i + j];
-      if (part2) s = __fadd_rn(bf16_round(s), bf16_round(part2[base + i + j])), s = bf16_round(s);
-      else if (round2) s = bf16_round(s);
-      const uint32_t hb = f32_to_bf16_bits(__fadd_rn(r, s));
-      const float h = bf16_bits_to_f32(hb);
-      hv[i + j] = h;
-      ss = __fadd_rn(ss, __fmul_rn(h, h));
-      if (j & 1) ho[j >> 1] |= hb << 16;
-      else ho[j >> 1] = hb;
-    }
-    if (res_out) *reinterpret_cast<u32x4_t*>(res_out + base + i) = u32x4_t{ho[0], ho[1], ho[2], ho[3]};
-  }
-  if (!xn) return;
-  ss = wave_sum(ss);
-  if ((tid & 63) == 0) red[tid >> 6] = ss;
-  __syncthreads();
-  const float tot = __fadd_rn(__fadd_rn(__fadd_rn(red[0], red[1]), red[2]), red[3]);
-  const float rstd = __fdiv_rn(1.f, __fsqrt_rn(__fadd_rn(__fdiv_rn(tot, (float)H), eps)));
-#pragma unroll
-  for (int i = 0; i < 64; i += 8) {
-    if (i >= per) break;
-    const u32x4_t wq = *reinterpret_cast<const DSGX_GLOBAL u32x4_t*>((uintptr_t)(w + (size_t)tid * per + i));
-    uint32_t o[4];
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const float wv = bf16_bits_to_f32(j & 1 ? wq[j >> 1] >> 16 : wq[j >> 1] & 0xFFFFu);
-      const uint32_t b = f32_to_bf16_bits(__fmul_rn(wv, bf16_round(__fmul_rn(hv[i + j], rstd))));
-      if (j & 1) o[j >> 1] |= b << 16;
-      else o[j >> 1] = b;
-    }
-    *reinterpret_cast<u32x4_t*>(xn + base + i) = u32x4_t{o[0], o[1], o[2], o[3]};
-  }
+  const int row = blockIdx.x;
+  add_norm_row(a, row, H, red, a.xn != nullptr,
+               [&](int q, u32x4_t v) { if (a.res_out) *reinterpret_cast<u32x4_t*>(a.res_out + (size_t)row * H + 8 * q) = v; },
+               [&](int q, u32x4_t v) { *reinterpret_cast<u32x4_t*>(a.xn + (size_t)row * H + 8 * q) = v; });
 }
 
 // INT4 canonical tensors -> the contract's bf16 weight, one thread a group of 32 (the subtract-first form, exact for
@@ -269,6 +246,33 @@ int dsgx_stream_copy(const void* src, void* dst, size_t n, void* stream) {
   DSGX_HIP(hipGetLastError());
   return DSGX_OK;
 }
+int dsgx_fill_normal(uint64_t seed, uint64_t tid, size_t n, double sigma, void* out, int bf16, void* stream) {
+  if (!out) return fail(DSGX_EINVAL, "fill_normal: null output");
+  if (!n) return DSGX_OK;
+  const uint64_t key = [&] {  // stream_key of the oracle: mix64(seed * 0x100000001B3 + tid)
+    uint64_t x = seed * 0x100000001B3ull + tid;
+    x += 0x9E3779B97F4A7C15ull;
+    x = (x ^ (x >> 30)) * 0xBF58476D1CE4E5B9ull;
+    x = (x ^ (x >> 27)) * 0x94D049BB133111EBull;
+    return x ^ (x >> 31);
+  }();
+  const size_t blocks = (n + 255) / 256;
+  hipLaunchKernelGGL(k_fill_normal, dim3((unsigned)(blocks < 65536 ? blocks : 65536)), dim3(256), 0, static_cast<hipStream_t>(stream), key, n, sigma, out, bf16);
+  DSGX_HIP(hipGetLastError());
+  return DSGX_OK;
+}
+int dsgx_launch_floor(int kind, const void* p, void* sink, void* stream) {
+  if (kind == 0) {
+    hipLaunchKernelGGL(k_floor_empty, dim3(1), dim3(64), 0, static_cast<hipStream_t>(stream));
+  } else if (kind == 1) {
+    if (!p || !sink || ((uintptr_t)p & 15)) return fail(DSGX_EINVAL, "launch_floor: a 16-byte aligned buffer of 64 KiB and a sink are needed");
+    hipLaunchKernelGGL(k_floor_chain, dim3(1), dim3(64), 0, static_cast<hipStream_t>(stream), static_cast<const uint32_t*>(p), static_cast<uint32_t*>(sink));
+  } else {
+    return fail(DSGX_EINVAL, "launch_floor: kind %d", kind);
+  }
+  DSGX_HIP(hipGetLastError());
+  return DSGX_OK;
+}
 int dsgx_finalize(const float* R, const float* S, int n, uint16_t* out, void* stream) {
   if (!R || !S || !out || n < 0) return fail(DSGX_EINVAL, "finalize: null argument or n %d", n);
   if (!n) return DSGX_OK;
@@ -282,7 +286,7 @@ int dsgx_add_norm(const float* part, const float* part2, int M, int H, const uin
   if (H < 2048 || H % 2048 || H > 16384) return fail(DSGX_EINVAL, "add_norm: hidden %d (a multiple of 2048 up to 16384)", H);
   if (xn && !w) return fail(DSGX_EINVAL, "add_norm: the norm needs its weight");
   if (!xn && !res_out) return fail(DSGX_EINVAL, "add_norm: no output");
-  hipLaunchKernelGGL(k_add_norm, dim3(M), dim3(256), 0, static_cast<hipStream_t>(stream), part, part2, H, res, res_out, w, eps, xn, round2);
+  hipLaunchKernelGGL(k_add_norm, dim3(M), dim3(256), 0, static_cast<hipStream_t>(stream), NormIn{part, part2, res, res_out, w, xn, eps, round2}, H);
   DSGX_HIP(hipGetLastError());
   return DSGX_OK;
 }

@@ -8,6 +8,7 @@
 // One wavefront owns RB rows of W and the whole of K (rowdot.cuh); the grid is sized to the chip and walks the row
 // batches round-robin. The order of the adds inside a dot product is not the reference's (not part of its contract).
 #include "abi_internal.h"
+#include "addnorm.cuh"
 #include "rowdot.cuh"
 
 namespace dsgx {
@@ -23,11 +24,34 @@ struct GemvArgs {
   const uint16_t* x;
   int ldx, K, nq, nsegk, nsegs, total_rows, out, splitk;
   GemvSegDev sg[kMaxSegs];
+  NormIn norm;  // norm.part set: the rows are not read from x but made here, xn = RMSNorm(bf16(res + part)) (dsgx_add_norm_gemv)
 };
+
+// The activation rows into LDS: from x, or (fused add + norm) computed by this workgroup from the partial sums and the
+// residual - every workgroup makes all M rows for itself (M H values: a few KB from L2), workgroup 0 also writes the new
+// residual and the normed rows to memory for the kernels that follow.
+template <int KL, int M>
+__device__ __forceinline__ void stage_rows(uint4* xs, const GemvArgs& a, float* red) {
+  if (!a.norm.part) {
+    stage_x<KL>(xs, a.x, a.ldx, M, a.K, a.nq * 8);
+    return;
+  }
+  const bool writer = blockIdx.x == 0;
+  const int H = a.K;
+#pragma unroll 1
+  for (int m = 0; m < M; ++m)
+    add_norm_row(a.norm, m, H, red, true,
+                 [&](int q, u32x4_t v) { if (writer && a.norm.res_out) *reinterpret_cast<u32x4_t*>(a.norm.res_out + (size_t)m * H + 8 * q) = v; },
+                 [&](int q, u32x4_t v) {
+                   xs[(size_t)m * a.nq + xchunk_index<KL>(q)] = make_uint4(v.x, v.y, v.z, v.w);
+                   if (writer && a.norm.xn) *reinterpret_cast<u32x4_t*>(a.norm.xn + (size_t)m * H + 8 * q) = v;
+                 });
+}
 
 template <int FMT, int M, int RB, int D>
 __global__ void __launch_bounds__(256) k_gemv(GemvArgs a) {
   extern __shared__ uint4 xs[];
+  __shared__ float red[4];
   const int lane = threadIdx.x & 63;
   const int gw = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6), GW = gridDim.x * (blockDim.x >> 6);
   const int nbatch = a.total_rows / RB;
@@ -102,7 +126,7 @@ __global__ void __launch_bounds__(256) k_gemv(GemvArgs a) {
   // first product (these calls are a few microseconds long: latency is most of them)
 #pragma unroll
   for (int d = 0; d < D; ++d) load(w[d]);
-  stage_x<FmtT<FMT>::KL>(xs, a.x, a.ldx, M, a.K, a.nq * 8);
+  stage_rows<FmtT<FMT>::KL, M>(xs, a, red);
   __syncthreads();
   for (int t = 0; t < nsteps; t += D) {
 #pragma unroll
@@ -122,6 +146,7 @@ template <int FMT, int M, int RB, int SK>
 __global__ void __launch_bounds__(256) k_gemv_sk(GemvArgs a) {
   extern __shared__ uint4 xs[];
   __shared__ float part[4][RB * M];
+  __shared__ float red[4];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   constexpr int GPW = 4 / SK;  // batches a workgroup
   const int grp = wave / SK, slice = wave % SK;
@@ -154,7 +179,7 @@ __global__ void __launch_bounds__(256) k_gemv_sk(GemvArgs a) {
   };
 #pragma unroll
   for (int d = 0; d < D; ++d) load(w[d]);
-  stage_x<FmtT<FMT>::KL>(xs, a.x, a.ldx, M, a.K, a.nq * 8);
+  stage_rows<FmtT<FMT>::KL, M>(xs, a, red);
   __syncthreads();
   for (int t = 0; t < nmine; t += D) {
 #pragma unroll
@@ -252,9 +277,11 @@ int ilog2_exact(int v) {
 }
 
 // one launch: the segments of one format (gemv_one of the reference, gemv.cu:459-516)
-int gemv_one(int fmt, const uint16_t* x, int ldx, int rows, int K, const dsgx_gemv_seg* segs, int nseg, int out, int splitk, hipStream_t st) {
+int gemv_one(int fmt, const uint16_t* x, int ldx, int rows, int K, const dsgx_gemv_seg* segs, int nseg, int out, int splitk, hipStream_t st,
+             const NormIn* norm = nullptr) {
   GemvArgs a{};
   a.x = x, a.ldx = ldx, a.K = K, a.out = out, a.nsegs = nseg, a.splitk = splitk;
+  if (norm) a.norm = *norm;
   const int segk = fmt == DSGX_FMT_FP8_B128 ? 1024 : fmt == DSGX_FMT_INT4_G32 ? 2048 : 512;
   a.nsegk = (K + segk - 1) / segk;
   a.nq = a.nsegk * segk / 8;
@@ -329,4 +356,23 @@ extern "C" int dsgx_gemv(const uint16_t* x, int ldx, int rows, int K, const dsgx
     }
   }
   return DSGX_OK;
+}
+
+// The residual add + RMSNorm of dsgx_add_norm as the GEMV's prologue: x = the normed rows, made inside the GEMV kernel.
+extern "C" int dsgx_add_norm_gemv(const dsgx_norm_in* n, int rows, int K, const dsgx_gemv_seg* segs, int nseg, int out, int splitk, void* stream) {
+  if (!n || !n->part || !n->res || !n->w) return fail(DSGX_EINVAL, "add_norm_gemv: the partial sums, the residual and the norm's weight are needed");
+  if (rows < 1 || rows > 8) return fail(DSGX_EUNSUPPORTED, "add_norm_gemv: %d rows (1..8; more: dsgx_add_norm, then dsgx_gemv)", rows);
+  if (K < 2048 || K % 2048 || K > 16384) return fail(DSGX_EINVAL, "add_norm_gemv: hidden %d (a multiple of 2048 up to 16384)", K);
+  if (n->res_out == n->res) return fail(DSGX_EINVAL, "add_norm_gemv: res_out must not be res (every workgroup reads the residual while one writes the new one)");
+  if (!segs || nseg < 1 || nseg > kMaxSegs) return fail(DSGX_EINVAL, "add_norm_gemv: %d segments", nseg);
+  if (splitk != 1 && splitk != 2 && splitk != 4) return fail(DSGX_EINVAL, "add_norm_gemv: splitk %d", splitk);
+  if (out != DSGX_OUT_BF16 && out != DSGX_OUT_F32 && out != DSGX_OUT_SWIGLU) return fail(DSGX_EINVAL, "add_norm_gemv: output kind %d", out);
+  const int f = segs[0].fmt;
+  if (f != DSGX_FMT_BF16 && f != DSGX_FMT_INT4_G32 && f != DSGX_FMT_FP8_B128) return fail(DSGX_EFORMAT, "add_norm_gemv: no supported weight format (%d)", f);
+  for (int i = 0; i < nseg; ++i) {
+    if (segs[i].fmt != f) return fail(DSGX_EUNSUPPORTED, "add_norm_gemv: the segments of one call share a format (one launch)");
+    if (segs[i].n < 8 || segs[i].n % 8) return fail(DSGX_EINVAL, "add_norm_gemv: segment %d has %d rows", i, segs[i].n);
+  }
+  const NormIn ni{n->part, n->part2, n->res, n->res_out, n->w, n->xn, n->eps, n->round2};
+  return gemv_one(f, nullptr, K, rows, K, segs, nseg, out, splitk, static_cast<hipStream_t>(stream), &ni);
 }

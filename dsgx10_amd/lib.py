@@ -57,6 +57,13 @@ def lib():
         L.dsgx_stream_read_cfg.argtypes = [C.c_void_p, C.c_size_t, C.c_void_p, C.c_int, C.c_int, C.c_void_p]
         L.dsgx_stream_copy.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]
         L.dsgx_probe_mfma_fp8.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p]
+        L.dsgx_dsk_ws_bytes.restype = C.c_size_t
+        L.dsgx_dsk_ws_bytes.argtypes = [C.c_int, C.c_int]
+        L.dsgx_dsk_moe_stacked.argtypes = [C.POINTER(abi.DskWeights), C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
+                                           C.c_void_p, C.POINTER(abi.DskCfg), C.c_void_p, C.c_void_p]
+        L.dsgx_add_norm_gemv.argtypes = [C.POINTER(abi.NormIn), C.c_int, C.c_int, C.POINTER(abi.GemvSeg), C.c_int, C.c_int, C.c_int, C.c_void_p]
+        L.dsgx_fill_normal.argtypes = [C.c_uint64, C.c_uint64, C.c_size_t, C.c_double, C.c_void_p, C.c_int, C.c_void_p]
+        L.dsgx_launch_floor.argtypes = [C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]
         if hasattr(L, "dsgx_moe_prefill"):
             L.dsgx_prefill_ws_bytes.restype = C.c_size_t
             L.dsgx_prefill_ws_bytes.argtypes = [C.POINTER(abi.LayerW), C.c_int]
@@ -119,7 +126,6 @@ def dsk_moe(layer_w, xq, xs, idx, w, M, ws, y, ys, stream=None, limit=10.0, logi
 
 
 def dsk_ws_bytes(H, I):
-    lib().dsgx_dsk_ws_bytes.restype = C.c_size_t
     return lib().dsgx_dsk_ws_bytes(H, I)
 
 
@@ -172,6 +178,25 @@ def gemv(x, ldx, rows, K, segs, out, splitk=1, stream=None):
         arr[i] = abi.GemvSeg(g["fmt"], _ptr(g["w"]), _ptr(g.get("s")), _ptr(g.get("zp")), g["n"], g.get("rs", 128),
                              g.get("ks", 128), _ptr(g["y"]), g["ldy"])
     _check(lib().dsgx_gemv(_ptr(x), ldx, rows, K, arr, len(segs), out, splitk, _stream(stream)))
+
+
+def add_norm_gemv(part, part2, res, res_out, w, eps, xn, rows, K, segs, out, splitk=1, round2=False, stream=None):
+    """dsgx_add_norm as the prologue of the GEMV that reads its rows: y = W RMSNorm(bf16(res + part)); res_out, xn optional"""
+    arr = (abi.GemvSeg * len(segs))()
+    for i, g in enumerate(segs):
+        arr[i] = abi.GemvSeg(g["fmt"], _ptr(g["w"]), _ptr(g.get("s")), _ptr(g.get("zp")), g["n"], g.get("rs", 128),
+                             g.get("ks", 128), _ptr(g["y"]), g["ldy"])
+    n = abi.NormIn(_ptr(part), _ptr(part2), _ptr(res), _ptr(res_out), _ptr(w), eps, _ptr(xn), int(round2))
+    _check(lib().dsgx_add_norm_gemv(C.byref(n), rows, K, arr, len(segs), out, splitk, _stream(stream)))
+
+
+def fill_normal(seed, tid, n, sigma, out, bf16=False, stream=None):
+    """out[i] = N(0, sigma) value i of tensor `tid` under `seed` (the oracle's generator), f32 or bf16 bits"""
+    _check(lib().dsgx_fill_normal(C.c_uint64(seed), C.c_uint64(tid), C.c_size_t(n), C.c_double(sigma), _ptr(out), int(bf16), _stream(stream)))
+
+
+def launch_floor(kind, buf=None, sink=None, stream=None):
+    _check(lib().dsgx_launch_floor(kind, _ptr(buf), _ptr(sink), _stream(stream)))
 
 
 def dequant_int4(packed, scale, zp, N, K, out, ld=None, stream=None, probe=False):

@@ -260,6 +260,24 @@ typedef struct dsgx_gemv_seg {
    the same bits; different values add in different orders. */
 DSGX_API int dsgx_gemv(const uint16_t* x, int ldx, int rows, int K, const dsgx_gemv_seg* segs, int nseg, int out,
                        int splitk, void* stream);
+/* dsgx_add_norm fused into the GEMV that reads its output: y = W xn with xn made inside the GEMV kernel (every workgroup
+   computes the M normed rows for itself from part, res and w - a few KB out of L2 - and workgroup 0 writes res_out and xn for
+   the kernels that follow). One launch where the reference's step has two (allreduce_add_norm, then the router's or the next
+   projection's gemv: engine/model/model.cu:309-352): same bits as dsgx_add_norm followed by dsgx_gemv. rows 1..8, K = the
+   hidden size (a multiple of 2048), the segments of one format; res_out must not alias res. */
+typedef struct dsgx_norm_in {
+  const float* part;
+  const float* part2;      /* may be null */
+  const uint16_t* res;
+  uint16_t* res_out;       /* may be null */
+  const uint16_t* w;
+  float eps;
+  uint16_t* xn;            /* may be null */
+  int32_t round2;
+} dsgx_norm_in;
+DSGX_API int dsgx_add_norm_gemv(const dsgx_norm_in* n, int rows, int K, const dsgx_gemv_seg* segs, int nseg, int out, int splitk,
+                                void* stream);
+
 /* glm::dequant_int4 (engine/attn/attn.h:154-158): the contract's bf16 weight [N][ld] from the canonical tensors */
 DSGX_API int dsgx_dequant_int4(const void* packed, const void* scale, const void* zp, int N, int K, uint16_t* out,
                                size_t ld, void* stream);
@@ -289,6 +307,14 @@ DSGX_API const char* dsgx_version(void);
 DSGX_API int dsgx_stream_read(const void* p, size_t n, void* sink, void* stream);
 /* The same with the launch shape given: workgroups (of 256 threads) a CU and 16-byte loads in flight a lane (2, 4, 8, 16). */
 DSGX_API int dsgx_stream_read_cfg(const void* p, size_t n, void* sink, int wgs_per_cu, int unroll, void* stream);
+/* Seeded N(0, sigma) values, the generator the tests' oracle uses (splitmix64 of the reference, engine/experts/formats.cuh:
+   131-136, keyed by (seed, tensor id, index) -> Box-Muller in f64): value i of tensor `tid` under `seed`. out: n values as
+   f32 (bf16 = 0) or bf16 bits (bf16 = 1). For benchmark inputs made on the GPU. */
+DSGX_API int dsgx_fill_normal(uint64_t seed, uint64_t tid, size_t n, double sigma, void* out, int bf16, void* stream);
+/* What a launch costs with nothing in it, for the latency-bound calls' floor: kind 0 an empty kernel of one wavefront;
+   kind 1 one wavefront doing two dependent 16-byte loads from p (at least 64 KiB; the second address comes out of the
+   first's data) and one store to sink - the dependency chain of the smallest GEMV (activations, then weights, then y). */
+DSGX_API int dsgx_launch_floor(int kind, const void* p, void* sink, void* stream);
 /* A plain copy kernel (the reference for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE counters). */
 DSGX_API int dsgx_stream_copy(const void* src, void* dst, size_t n, void* stream);
 
