@@ -45,7 +45,7 @@ def prefill_extra(gen, T, name, peak, check=True):
     """a prefill chunk of the benchmark: T rows, top-8 experts drawn from a Zipf(1.1) popularity, uniform weights; FP8
     weights and activations on the e4m3 MFMA (peak 5 PFLOP/s), or INT4 weights decoded to bf16 on the bf16 MFMA
     (2.5 PFLOP/s); TFLOP/s over the useful multiply-adds of the routed experts (T * 8 * 3 * I * H * 2)"""
-    from dsgx10_amd.benchdata import PrefillBench
+    from benchdata import PrefillBench
     pb = PrefillBench(gen, T)
     t_routed, t_all = pb.time(15, False), pb.time(31, True)
     d = dict(workload=name, T=T, zipf_s=1.1, ms_routed=t_routed * 1e3, ms_with_shared=t_all * 1e3,
@@ -66,10 +66,29 @@ def prefill_extra(gen, T, name, peak, check=True):
          100 * d["hbm_frac"], d["ms_with_shared"]))
     if check:
         d["gpu_vs_oracle"] = prefill_check_rows(pb)
-        log("  %s: rows %s against the oracle: max-abs %.2e, rel-L2 %.2e" %
-            (name, d["gpu_vs_oracle"]["rows"], d["gpu_vs_oracle"]["max_abs_err"], d["gpu_vs_oracle"]["rel_l2"]))
+        log("  %s: rows %s against the oracle: max-abs %.2e, rel-L2 %.2e%s" %
+            (name, d["gpu_vs_oracle"]["rows"], d["gpu_vs_oracle"]["max_abs_err"], d["gpu_vs_oracle"]["rel_l2"],
+             "; against the oracle with sequential f32 block sums (the spread of correct evaluations): rel-L2 %.2e" % d["gpu_vs_oracle"]["vs_sequential_block_sums_rel_l2"]
+             if "vs_sequential_block_sums_rel_l2" in d["gpu_vs_oracle"] else ""))
     del pb
     return d
+
+
+def chain_entries(gen, layers=96):
+    """the layer chains of one format at one row: the MoE half alone (router GEMV + experts + add + norm) and the whole chain
+    with the dense projections, each with the add + norms as launches of their own and fused into the GEMVs that read them"""
+    from benchdata import ChainBench
+    out = []
+    for moe_only in (True, False):
+        cb = ChainBench(gen, 1, layers, moe_only=moe_only)
+        for fused in (False, True):
+            d = cb.time(fused)
+            log("  %s M=1 (add + norm %s): %.2f us a layer [%.2f .. %.2f] (%d layers in one graph, %.1f%% of 8 TB/s over %.0f MB)" %
+                (d["workload"], "fused" if fused else "apart", d["us_per_layer"], d["us_per_layer_min"], d["us_per_layer_max"], d["layers"],
+                 100 * d["hbm_frac"], d["bytes_per_layer"] / 1e6))
+            out.append(d)
+        del cb
+    return out
 
 
 def prefill_check_rows(pb, nrows=4):
@@ -88,7 +107,7 @@ def prefill_check_rows(pb, nrows=4):
     for t in (int(np.nonzero((idx_h == hot).any(1))[0][-1]), int(np.nonzero((idx_h == cold).any(1))[0][0]), 0, T - 1, T // 2, T // 3):
         if t not in rows and len(rows) < nrows:
             rows.append(t)
-    worst = dict(rows=rows, max_abs_err=0.0, rel_l2=0.0)
+    worst = dict(rows=rows, max_abs_err=0.0, rel_l2=0.0, oracle="C++ oracle; FP8 activations: each 128-k block added by the e4m3 MFMA's rule" if gen.fmt == abi.FMT_FP8 else "C++ oracle (decode contract row by row)")
     for t in rows:
         experts = sorted(int(e) for e in idx_h[t])
         hl = gen.host_sublayer(experts, 0)
@@ -96,8 +115,19 @@ def prefill_check_rows(pb, nrows=4):
         x = pb.x[t:t + 1].view(torch.int16).cpu().numpy().view(np.uint16)
         w = pb.w[t:t + 1].cpu().numpy()
         if gen.fmt == abi.FMT_FP8:
+            # the contract's oracle with each 128-k block added by the matrix unit's rule (pinned by tests/golden/mfma_fp8_k128.npz:
+            # what the e4m3 MFMA computes) ...
+            orc.set_fp8_block_rule(1)
             o = orc.moe_prefill_fp8_row(hl, x[0], li, w[0])
+            orc.set_fp8_block_rule(0)
             ref = [o["yr"], o["ys"]]
+            # ... and with sequential f32 block sums (the reference's CPU stand-in): two correct evaluations whose sums differ by
+            # ~1.5e-6 of their sums of |terms|, apart by what h's re-quantisation to e4m3 makes of that
+            o0 = orc.moe_prefill_fp8_row(hl, x[0], li, w[0])
+            for got, r in zip((pb.yr[t].cpu().numpy(), pb.ys[t].cpu().numpy()), (o0["yr"], o0["ys"])):
+                worst["vs_sequential_block_sums_rel_l2"] = max(worst.get("vs_sequential_block_sums_rel_l2", 0.0),
+                                                               float(np.sqrt(((got - r).astype(np.float64) ** 2).sum() / max((r.astype(np.float64) ** 2).sum(), 1e-300))))
+                worst["vs_sequential_block_sums_max_abs"] = max(worst.get("vs_sequential_block_sums_max_abs", 0.0), float(np.abs(got - r).max()))
         else:
             uni = np.arange(len(experts), dtype=np.int32)
             up = orc.moe_up(hl, x, uni, want_range=False)
@@ -127,7 +157,7 @@ def main():
 
     import torch
     from dsgx10_amd import abi, lib
-    from dsgx10_amd.benchdata import DecodeBench, Fp8LayerGen, Int4LayerGen
+    from benchdata import DecodeBench, Fp8LayerGen, Int4LayerGen
 
     if not torch.cuda.is_available():
         print("bench.py: no GPU", file=sys.stderr)
@@ -193,7 +223,7 @@ def main():
         return
     if args.workload == "dsk":
         # only DeepSeek's MXFP4 layer (dsgx_dsk_moe, routing fused), M = 1, 2, 4, 8
-        from dsgx10_amd.benchdata import DskBench, DskLayerGen
+        from benchdata import DskBench, DskLayerGen
         dg = DskLayerGen(seed=0)
         ds = []
         for M in (1, 2, 4, 8):
@@ -209,12 +239,11 @@ def main():
         return
     if args.workload == "chain":
         # only the layer chains (router GEMV -> experts -> add + norm, 128 layers a graph), FP8 then INT4
-        from dsgx10_amd.benchdata import ChainBench
+        from benchdata import ChainBench
         ds = []
         for cls in (Fp8LayerGen, Int4LayerGen):
             g2 = cls(seed=0)
-            ds.append(ChainBench(g2, 1, 128).time())
-            log("  %s M=1: %.2f us a layer" % (ds[-1]["workload"], ds[-1]["us_per_layer"]))
+            ds += chain_entries(g2)
             del g2
         print(json.dumps({"metric": "us_per_moe_layer_step", "value": ds[0]["us_per_layer"], "unit": "us", "n_gpus": 1, "steps": 128, "warmup": 4,
                           "ms_per_step": ds[0]["us_per_layer"] * 1e-3, "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
@@ -223,7 +252,7 @@ def main():
         return
     if args.workload == "gemv":
         # only the dense GEMVs (for profiler runs): one line, the FP8 [2048 x 4096] row-1 call as the value
-        from dsgx10_amd.benchdata import gemv_bench
+        from benchdata import gemv_bench
         g = gemv_bench()
         head = min((d for d in g if d["workload"].startswith("dense_fp8")), key=lambda d: d["us_per_call"])
         print(json.dumps({"metric": "dense_gemv_us", "value": head["us_per_call"], "unit": "us", "n_gpus": 1, "steps": 64, "warmup": 4,
@@ -265,13 +294,9 @@ def main():
                 extra.append(d)
                 del ob
         extra.append(prefill_extra(other, 2048, "int4_moe_prefill", 2.5e15, not args.no_cpu) if head_fp8 else prefill_extra(other, 8192, "fp8_moe_prefill", 5.0e15, not args.no_cpu))
-        from dsgx10_amd.benchdata import ChainBench, DskBench, DskLayerGen, gemv_bench
+        from benchdata import ChainBench, DskBench, DskLayerGen, gemv_bench
         for g2 in (gen, other):
-            cb = ChainBench(g2, 1, 128)
-            d = cb.time()
-            log("  %s M=1: %.2f us a layer (router GEMV + experts + add/norm, %d layers in one graph)" % (d["workload"], d["us_per_layer"], d["layers"]))
-            extra.append(d)
-            del cb
+            extra += chain_entries(g2)
         del other
         dg = DskLayerGen(seed=0)
         for M in (1, 8):
@@ -293,13 +318,13 @@ def main():
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "f32",
-        "data": "synthetic (torch-seeded N(0,0.02) weights quantised on the GPU, N(0,1) bf16 rows and f32 logits)",
+        "data": "synthetic (seeded splitmix64 / Box-Muller values: N(0,0.02) weights quantised on the GPU, N(0,1) bf16 rows and f32 logits)",
         "config": {"workload": gen.describe(1), "arithmetic": "f32 sums of bf16 x bf16 products (weights decoded to bf16 in registers)", "rows_M": 1, "steps_route_different_experts": True,
                    "bytes_per_layer": r["bytes_per_layer"], "layer_hbm_frac_of_8TBs": r["layer_hbm_frac"],
                    "variant": args.variant,
                    "kernels_per_step": ["k_decode (routing + gate/up + SwiGLU + down + weighted sum, one persistent launch)"] if head_up == 0 else
                                        ["k_decode_mfma (routing + gate/up + SwiGLU + down, one persistent launch)", "k_down_combine (weighted sum in expert order)"],
-                   "timed_as": "one HIP graph of all steps, one replay"},
+                   "timed_as": "one HIP graph of all steps; the median of 7 replays", "us_min_max_of_replays": [r["us_per_layer_min"], r["us_per_layer_max"]]},
         # the kernel(s) of the timed step: the algorithmic bytes of a layer (every weight byte of the picked experts and the
         # shared expert once, scales included) over the step's time in the timed graph (HIP events on the launch stream)
         "roofline": {"bound": "hbm",

@@ -1,4 +1,7 @@
-"""Synthetic layers and timing loops for bench.py (GPU side only; torch is the allocator and RNG).
+"""Synthetic layers and timing loops for bench.py (GPU side only; torch is the allocator).
+
+Values come from the generator the tests' oracle uses (splitmix64 keyed by seed, tensor id and index -> Box-Muller), made
+on the GPU by the library's fill kernel (dsgx_fill_normal).
 
 The layers have the benchmark's full shapes: weights ~ N(0, 0.02) quantised on the GPU with the reference's FP8
 quantiser (per 128 x 128 block: scale = amax * f32(1/448), e4m3 round-to-nearest-even;
@@ -9,14 +12,43 @@ import ctypes as C
 import numpy as np
 import torch
 
-from . import abi, lib
-from .layer import DESC_DTYPE, HostLayer, mat_bytes
+from dsgx10_amd import abi, lib
+from dsgx10_amd.layer import DESC_DTYPE, HostLayer, mat_bytes
 
 HBM_PEAK = 8.0e12
 
 
 def _al256(n):
     return (n + 255) // 256 * 256
+
+
+class Seeded:
+    """N(0, sigma) tensors on the GPU from the oracle's generator: tensor number `tid` counts up with every draw"""
+
+    def __init__(self, seed):
+        self.seed, self.tid = seed, 0
+
+    def normal(self, shape, sigma=1.0, dtype=torch.float32):
+        n = int(np.prod(shape))
+        out = torch.empty(shape, dtype=dtype, device="cuda")
+        assert dtype in (torch.float32, torch.bfloat16)
+        lib.fill_normal(self.seed, self.tid, n, sigma, out, bf16=dtype == torch.bfloat16)
+        self.tid += 1
+        return out
+
+
+def time_graph(gr, reps=7):
+    """seconds a replay: the median of `reps` replays, each between its own pair of events (and the fastest and slowest)"""
+    torch.cuda.synchronize()
+    ts = []
+    for _ in range(reps):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        gr.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        ts.append(e0.elapsed_time(e1) * 1e-3)
+    return float(np.median(ts)), float(min(ts)), float(max(ts))
 
 
 def fp8_quantize_gpu(w):
@@ -77,8 +109,7 @@ class Fp8LayerGen(_LayerGen):
     fmt, H, I, E, topk, route_scale, NSH = abi.FMT_FP8, 4096, 2048, 256, 8, 1.0, 16
 
     def __init__(self, seed=0):
-        g = torch.Generator(device="cuda")
-        g.manual_seed(seed)
+        g = Seeded(seed)
         H, I, E = self.H, self.I, self.E
         per = [mat_bytes(self.fmt, I, H), mat_bytes(self.fmt, I, H), mat_bytes(self.fmt, H, I)]
         self.expert_bytes = sum(per)
@@ -88,7 +119,7 @@ class Fp8LayerGen(_LayerGen):
         for e in range(E):
             for j in range(3):
                 N, K = (I, H) if j < 2 else (H, I)
-                codes, scale = fp8_quantize_gpu(torch.randn(N, K, generator=g, device="cuda") * 0.02)
+                codes, scale = fp8_quantize_gpu(g.normal((N, K), 0.02))
                 d = desc[e * 3 + j]
                 d["off"], d["s2"], d["fmt"] = o, 1.0, self.fmt
                 _put(self.pool, o, codes)
@@ -100,7 +131,7 @@ class Fp8LayerGen(_LayerGen):
             mats = []
             for j in range(3):
                 N, K = (I, H) if j < 2 else (H, I)
-                mats.append(fp8_quantize_gpu(torch.randn(N, K, generator=g, device="cuda") * 0.02))
+                mats.append(fp8_quantize_gpu(g.normal((N, K), 0.02)))
             self.shared.append(mats)
         self.shared_bytes = self.expert_bytes
 
@@ -143,8 +174,7 @@ class Int4LayerGen(_LayerGen):
     fmt, H, I, E, topk, route_scale, NSH = abi.FMT_INT4, 6144, 2048, 168, 8, 2.5, 8
 
     def __init__(self, seed=0):
-        g = torch.Generator(device="cuda")
-        g.manual_seed(seed + 1)
+        g = Seeded(seed + 1)
         H, I, E = self.H, self.I, self.E
         per = [mat_bytes(self.fmt, I, H), mat_bytes(self.fmt, I, H), mat_bytes(self.fmt, H, I)]
         self.expert_bytes = sum(per)
@@ -154,7 +184,7 @@ class Int4LayerGen(_LayerGen):
         for e in range(E):
             for j in range(3):
                 N, K = (I, H) if j < 2 else (H, I)
-                words, s, zp = int4_quantize_gpu(torch.randn(N, K, generator=g, device="cuda") * 0.02)
+                words, s, zp = int4_quantize_gpu(g.normal((N, K), 0.02))
                 d = desc[e * 3 + j]
                 d["off"], d["s2"], d["fmt"] = o, 1.0, self.fmt
                 _put(self.pool, o, words)
@@ -164,8 +194,7 @@ class Int4LayerGen(_LayerGen):
         self.desc = torch.from_numpy(desc.view(np.uint8).reshape(-1)).cuda()
         self.shared = []
         for c in range(self.NSH):
-            bgu = (torch.randn(2 * I, H, generator=g, device="cuda") * 0.02).to(torch.bfloat16)
-            bd = (torch.randn(H, I, generator=g, device="cuda") * 0.02).to(torch.bfloat16)
+            bgu, bd = g.normal((2 * I, H), 0.02, torch.bfloat16), g.normal((H, I), 0.02, torch.bfloat16)
             self.shared.append((bgu, bd))
         self.shared_bytes = 3 * H * I * 2
 
@@ -209,10 +238,9 @@ class DecodeBench:
     def __init__(self, gen, M, steps, seed=1234, up=0):
         """up: the decode variant (dsgx_decode_cfg::up): 0 the vector-unit kernels, 1 the MFMA kernels"""
         self.gen, self.M, self.steps, self.up = gen, M, steps, up
-        g = torch.Generator(device="cuda")
-        g.manual_seed(seed)
-        self.x = torch.randn(M, gen.H, generator=g, device="cuda").to(torch.bfloat16)
-        self.logits = torch.randn(steps, M, gen.E, generator=g, device="cuda")
+        g = Seeded(seed)
+        self.x = g.normal((M, gen.H), 1.0, torch.bfloat16)
+        self.logits = g.normal((steps, M, gen.E), 1.0)
         self.idx = torch.zeros(steps, M, gen.topk, dtype=torch.int32, device="cuda")
         self.w = torch.zeros(steps, M, gen.topk, dtype=torch.float32, device="cuda")
         self.layers = [gen.layer_w(c) for c in range(gen.NSH)]
@@ -243,15 +271,6 @@ class DecodeBench:
             fn()
         return gr
 
-    def _time_graph(self, gr, reps=1):
-        torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        for _ in range(reps):
-            gr.replay()
-        e1.record()
-        torch.cuda.synchronize()
-        return e0.elapsed_time(e1) * 1e-3 / reps
 
     def time_layer(self, warmup):
         for s in range(warmup):
@@ -259,17 +278,17 @@ class DecodeBench:
         torch.cuda.synchronize()
         gr = self._graph(lambda: [self.step(s) for s in range(self.steps)])
         gr.replay()  # untimed: uploads the graph
-        sec = self._time_graph(gr)
+        sec, lo, hi = time_graph(gr)
         us = sec / self.steps * 1e6
         bytes_ = float(np.mean([self.gen.layer_bytes(u) for u in self.union_sizes]))
-        return dict(us_per_layer=us, bytes_per_layer=bytes_, layer_hbm_frac=bytes_ / (us * 1e-6) / HBM_PEAK,
-                    mean_union=float(self.union_sizes.mean()))
+        return dict(us_per_layer=us, us_per_layer_min=lo / self.steps * 1e6, us_per_layer_max=hi / self.steps * 1e6, replays=7,
+                    bytes_per_layer=bytes_, layer_hbm_frac=bytes_ / (us * 1e-6) / HBM_PEAK, mean_union=float(self.union_sizes.mean()))
 
     def time_up_kernel(self):
         """the dominant kernel alone: `steps` launches of the gate/up kernel back to back in one graph"""
         gr = self._graph(lambda: [self.step(s, parts=1, route=False) for s in range(self.steps)])
         gr.replay()
-        sec = self._time_graph(gr)
+        sec = time_graph(gr)[0]
         us = sec / self.steps * 1e6
         b = float(np.mean([self.gen.up_bytes(u) for u in self.union_sizes]))
         gbs = b / (us * 1e-6) / 1e9
@@ -340,16 +359,15 @@ class DskBench:
 
     def __init__(self, gen, M, steps, seed=77):
         self.gen, self.M, self.steps = gen, M, steps
-        g = torch.Generator(device="cuda")
-        g.manual_seed(seed)
-        x = torch.randn(M, gen.H, generator=g, device="cuda") * 1.5
+        g = Seeded(seed)
+        x = g.normal((M, gen.H), 1.5)
         blk = x.view(M, gen.H // 32, 32)
         v = blk.abs().amax(-1).clamp_min(1e-4) * torch.tensor(1.0 / 448.0, device="cuda")
         bits = v.view(torch.int32)
         e = ((bits >> 23) & 0xFF) + ((bits & 0x7FFFFF) != 0).to(torch.int32)
         self.xs = e.to(torch.uint8).contiguous()
         self.xq = (blk * torch.ldexp(torch.ones_like(v), (127 - e).float())[..., None]).clamp(-448, 448).to(torch.float8_e4m3fn).view(torch.uint8).reshape(M, gen.H).contiguous()
-        self.logits = torch.randn(steps, M, gen.E, generator=g, device="cuda")
+        self.logits = g.normal((steps, M, gen.E), 1.0)
         idx = torch.zeros(steps, M, gen.topk, dtype=torch.int32, device="cuda")
         w = torch.zeros(steps, M, gen.topk, dtype=torch.float32, device="cuda")
         for s in range(steps):
@@ -375,89 +393,120 @@ class DskBench:
             for s in range(self.steps):
                 self.step(s, parts)
         gr.replay()
-        torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        gr.replay()
-        e1.record()
-        torch.cuda.synchronize()
+        us = time_graph(gr)[0] * 1e6 / self.steps
         lib.decode_status(self.layers[0], self.ws)
-        us = e0.elapsed_time(e1) * 1e3 / self.steps
         b = float(np.mean([self.gen.layer_bytes(u) for u in self.union_sizes]))
         return dict(workload=self.gen.name, M=self.M, variant="mfma", us_per_layer=us, bytes=b, hbm_frac=b / (us * 1e-6) / HBM_PEAK,
                     outputs_finite=bool(torch.isfinite(self.y).all()))
 
 
 class ChainBench:
-    """The MoE half of a decode step as the reference's runner chains it (model.cu:309-343), layer after layer in one graph:
-    the router's logits by the BF16 GEMV (f32 out, K over 4 waves) from the normed row, the experts with the routing, the
-    shared expert and yr += ys fused in one launch, then the residual add and the next layer's RMSNorm, whose output is the
-    next layer's input. Every layer has its own router matrix and norm weight (rotating over copies that exceed the caches)
-    and routes by its own data, so the experts differ from layer to layer."""
+    """A decode layer's dense projections and MoE step as the reference's runner chains them (model.cu:229-352; the sequence
+    is dsgx10_amd/chain.py's), layer after layer in one graph: x-projection (BF16, K over 4), q_b and o_proj (the layer's
+    format: INT4 or FP8 128 x 128), the add + norms, the router's logits (BF16, f32 out, K over 4) and the experts with the
+    routing, the shared expert and yr += ys fused. Shapes: the whole layer on one GPU (GLM / altar-1: hidden 6144, x-projection
+    2752 rows, q_lora 2048, 64 heads x 256; the FP8 layer: hidden 4096, 2112, 1536, 64 x 256). Every layer rotates over
+    weight sets that together exceed the caches and routes by its own data. fused: each add + norm inside the GEMV that
+    reads it (the router's: 6 launches a layer, 7 with the MFMA variant's ordered sum) or as launches of their own (7 / 8)."""
 
-    def __init__(self, gen, M, layers, seed=99, up=-1):
-        self.gen, self.M, self.layers, self.up = gen, M, layers, up
-        g = torch.Generator(device="cuda")
-        g.manual_seed(seed)
+    def __init__(self, gen, M, layers, seed=99, up=-1, moe_only=False):
+        from dsgx10_amd.chain import LayerChain
+        self.gen, self.M, self.layers, self.up, self.moe_only = gen, M, layers, up, moe_only
+        g = Seeded(seed)
         H, E = gen.H, gen.E
-        self.nr = max(8, int(600e6 // (E * H * 2)))
-        self.router = [(torch.randn(E, H, generator=g, device="cuda") * 0.05).to(torch.bfloat16) for _ in range(self.nr)]
-        self.normw = [(1.0 + 0.1 * torch.randn(H, generator=g, device="cuda")).to(torch.bfloat16) for _ in range(self.nr)]
-        self.x0 = torch.randn(M, H, generator=g, device="cuda").to(torch.bfloat16)
-        self.xn = [torch.zeros(M, H, dtype=torch.bfloat16, device="cuda") for _ in range(2)]
-        self.res = torch.zeros(M, H, dtype=torch.bfloat16, device="cuda")
-        self.logits = torch.zeros(M, E, dtype=torch.float32, device="cuda")
-        self.yr = torch.zeros(M, H, dtype=torch.float32, device="cuda")
-        self.ys = torch.zeros(M, H, dtype=torch.float32, device="cuda")
-        self.lw = [gen.layer_w(c) for c in range(gen.NSH)]
-        self.ws = torch.zeros(lib.decode_ws_bytes(self.lw[0]), dtype=torch.uint8, device="cuda")
+        fp8 = gen.fmt == abi.FMT_FP8
+        self.XR, self.QL, self.NQ = (2112, 1536, 16384) if fp8 else (2752, 2048, 16384)
+        XR, QL, NQ = self.XR, self.QL, self.NQ
+        quant = fp8_quantize_gpu if fp8 else int4_quantize_gpu
 
-    def layer(self, l):
-        g, M = self.gen, self.M
-        x, xo = self.xn[l & 1], self.xn[(l + 1) & 1]
-        seg = dict(fmt=abi.FMT_BF16, w=self.router[l % self.nr], s=None, zp=None, n=g.E, y=self.logits, ldy=g.E)
-        lib.gemv(x, g.H, M, g.H, [seg], abi.OUT_F32, splitk=4)
-        lib.moe_decode(self.lw[l % g.NSH], x, None, None, M, self.ws, self.yr, self.ys, logits=self.logits, route_scale=g.route_scale,
-                       ysum=True, up=self.up)
-        lib.add_norm(self.yr, None, M, g.H, self.res, self.res, self.normw[l % self.nr], 1e-5, xo)
+        def mat(N, K):
+            t = quant(g.normal((N, K), 0.02))
+            return dict(fmt=gen.fmt, w=t[0], s=t[1], zp=t[2] if len(t) > 2 else None)
+        self.nsets = 4
+        lw = [gen.layer_w(c) for c in range(gen.NSH)]
+        self.ws = torch.zeros(lib.decode_ws_bytes(lw[0]), dtype=torch.uint8, device="cuda")
+        self.sets = []
+        for c in range(self.nsets):
+            self.sets.append(dict(attn_norm=(1.0 + g.normal((H,), 0.1)).to(torch.bfloat16), ffn_norm=(1.0 + g.normal((H,), 0.1)).to(torch.bfloat16),
+                                  xproj=g.normal((XR, H), 0.02, torch.bfloat16), router=g.normal((E, H), 0.05, torch.bfloat16),
+                                  qb=mat(NQ, QL), oproj=mat(H, NQ)))
+        self.lw = lw
+        self.dense_bytes = XR * H * 2 + E * H * 2 + mat_bytes(gen.fmt, NQ, QL) + mat_bytes(gen.fmt, H, NQ)
+        self.ch = LayerChain(M, H, XR, QL, NQ, E, gen.route_scale, lambda n: torch.zeros(n, dtype=torch.uint8, device="cuda"))
+        self.x0 = g.normal((M, H), 1.0, torch.bfloat16)
 
-    def time(self):
-        def run():
-            for l in range(self.layers):
-                self.layer(l)
-        self.xn[0].copy_(self.x0)
-        self.res.zero_()
+    def layer(self, l, fused):
+        W = dict(self.sets[l % self.nsets], moe=self.lw[l % self.gen.NSH], ws=self.ws)
+        if self.moe_only:  # the MoE half alone: router GEMV (+ add + norm) and the experts
+            ch, g = self.ch, self.gen
+            a, b = ch.res[ch.cur], ch.res[ch.cur ^ 1]
+            rt = [dict(fmt=abi.FMT_BF16, w=W["router"], n=g.E, y=ch.logits, ldy=g.E)]
+            if fused:
+                lib.add_norm_gemv(ch.yr, None, a, b, W["ffn_norm"], 1e-5, ch.xn, self.M, g.H, rt, abi.OUT_F32, splitk=4)
+            else:
+                lib.add_norm(ch.yr, None, self.M, g.H, a, b, W["ffn_norm"], 1e-5, ch.xn)
+                lib.gemv(ch.xn, g.H, self.M, g.H, rt, abi.OUT_F32, splitk=4)
+            ch.cur ^= 1
+            lib.moe_decode(W["moe"], ch.xn, None, None, self.M, W["ws"], ch.yr, ch.ys, logits=ch.logits, route_scale=g.route_scale, ysum=True, up=self.up)
+            return
+        self.ch.layer(W, fused=fused, up=self.up)
+
+    def _reset(self):
+        self.ch.cur = 0
+        self.ch.res[0].copy_(self.x0.view(torch.uint8).reshape(-1))
+        self.ch.yr.zero_()
+
+    def time(self, fused=True):
+        self._reset()
         for l in range(4):
-            self.layer(l)
+            self.layer(l, fused)
         torch.cuda.synchronize()
-        self.xn[0].copy_(self.x0)
-        self.res.zero_()
+        self._reset()
         gr = torch.cuda.CUDAGraph()
         with torch.cuda.graph(gr):
-            run()
+            for l in range(self.layers):
+                self.layer(l, fused)
         gr.replay()
         torch.cuda.synchronize()
-        self.xn[0].copy_(self.x0)
-        self.res.zero_()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        gr.replay()
-        e1.record()
-        torch.cuda.synchronize()
+        sec, lo, hi = time_graph(gr)
         lib.decode_status(self.lw[0], self.ws)
-        finite = bool(torch.isfinite(self.xn[self.layers & 1].float()).all())
-        return dict(workload=self.gen.name.replace("decode", "layer_chain"), M=self.M, layers=self.layers,
-                    launches_per_layer=["k_gemv_sk (router logits, f32, K over 4)", "k_decode / k_decode_mfma (+ its ordered sum)", "k_add_norm"],
-                    us_per_layer=e0.elapsed_time(e1) * 1e3 / self.layers, outputs_finite=finite)
+        finite = bool(torch.isfinite(self.ch.yr.view(torch.float32)).all())
+        us = sec * 1e6 / self.layers
+        moe_bytes = self.gen.layer_bytes(self.gen.topk * self.M if self.M == 1 else self.gen.topk)  # (M = 1: eight experts + shared)
+        total = moe_bytes + (self.gen.E * self.gen.H * 2 if self.moe_only else self.dense_bytes)
+        names = (["k_gemv_sk (router logits, add + norm in its prologue)" if fused else "k_add_norm, k_gemv_sk (router logits)", "k_decode / k_decode_mfma (+ its ordered sum)"]
+                 if self.moe_only else
+                 ["k_add_norm", "k_gemv_sk (x-projection)", "k_gemv (q_b)", "k_gemv (o_proj)",
+                  "k_gemv_sk (router logits%s)" % (", add + norm in its prologue" if fused else "; k_add_norm before it"), "k_decode / k_decode_mfma (+ its ordered sum)"])
+        return dict(workload=self.gen.name.replace("decode", "moe_half_chain" if self.moe_only else "layer_chain"), M=self.M, layers=self.layers, fused_add_norm=fused,
+                    launches_per_layer=names, us_per_layer=us, us_per_layer_min=lo * 1e6 / self.layers, us_per_layer_max=hi * 1e6 / self.layers,
+                    bytes_per_layer=total, hbm_frac=total / (us * 1e-6) / HBM_PEAK, outputs_finite=finite)
+
+
+def launch_floors(reps=64):
+    """what a graph node costs with nothing in it: an empty kernel, and one wavefront doing two dependent loads and a store"""
+    buf = torch.zeros(1 << 16, dtype=torch.uint8, device="cuda")
+    sink = torch.zeros(16, dtype=torch.uint8, device="cuda")
+    out = {}
+    for name, kind in (("empty_kernel_us", 0), ("two_dependent_loads_us", 1)):
+        lib.launch_floor(kind, buf, sink)
+        torch.cuda.synchronize()
+        gr = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(gr):
+            for _ in range(reps):
+                lib.launch_floor(kind, buf, sink)
+        gr.replay()
+        out[name] = time_graph(gr)[0] * 1e6 / reps
+    return out
 
 
 def gemv_bench(reps=64):
     """the two dense GEMV configurations: FP8 [2048 x 4096] at 1 row, INT4 [1536 x 6144] at 1, 2, 4, 6 rows, and the router's
     logits (BF16 [E x H], f32 out, 1 row), each with K unsplit and split over 2 and 4 waves; weights rotate over copies that
-    exceed the caches"""
+    exceed the caches; beside them what an empty graph node and a node of two dependent memory round trips cost"""
     out = []
-    g = torch.Generator(device="cuda")
-    g.manual_seed(7)
+    g = Seeded(7)
+    floors = launch_floors(reps)
     for name, fmt, N, K, rows, kind in (("dense_fp8_gemv_2048x4096", abi.FMT_FP8, 2048, 4096, (1,), abi.OUT_BF16),
                                         ("dense_int4_gemv_1536x6144", abi.FMT_INT4, 1536, 6144, (1, 2, 4, 6), abi.OUT_BF16),
                                         ("router_bf16_gemv_256x4096", abi.FMT_BF16, 256, 4096, (1,), abi.OUT_F32),
@@ -466,10 +515,10 @@ def gemv_bench(reps=64):
         copies = max(8, int(600e6 // per))
         mats = []
         for c in range(copies):
-            w = torch.randn(N, K, generator=g, device="cuda") * 0.02
+            w = g.normal((N, K), 0.02)
             mats.append(fp8_quantize_gpu(w) if fmt == abi.FMT_FP8 else int4_quantize_gpu(w) if fmt == abi.FMT_INT4 else (w.to(torch.bfloat16), None))
         for M in rows:
-            x = torch.randn(M, K, generator=g, device="cuda").to(torch.bfloat16)
+            x = g.normal((M, K), 1.0, torch.bfloat16)
             y = torch.zeros(M, N, dtype=torch.float32 if kind == abi.OUT_F32 else torch.bfloat16, device="cuda")
             for sk in (1, 2, 4):
                 def one(c):
@@ -484,15 +533,9 @@ def gemv_bench(reps=64):
                     for c in range(reps):
                         one(c)
                 gr.replay()
-                torch.cuda.synchronize()
-                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                e0.record()
-                gr.replay()
-                e1.record()
-                torch.cuda.synchronize()
-                us = e0.elapsed_time(e1) * 1e3 / reps
+                us = time_graph(gr)[0] * 1e6 / reps
                 b = per + M * K * 2 + M * N * y.element_size()
-                out.append(dict(workload=name, M=M, splitk=sk, us_per_call=us, bytes=b, hbm_frac=b / (us * 1e-6) / HBM_PEAK))
+                out.append(dict(workload=name, M=M, splitk=sk, us_per_call=us, bytes=b, hbm_frac=b / (us * 1e-6) / HBM_PEAK, floors=floors))
     return out
 
 
@@ -503,9 +546,9 @@ class PrefillBench:
 
     def __init__(self, gen, T, zipf_s=1.1, seed=4321):
         self.gen, self.T = gen, T
-        g = torch.Generator(device="cuda")
+        g = torch.Generator(device="cuda")   # (the Zipf draw: torch's multinomial)
         g.manual_seed(seed)
-        self.x = torch.randn(T, gen.H, generator=g, device="cuda").to(torch.bfloat16)
+        self.x = Seeded(seed).normal((T, gen.H), 1.0, torch.bfloat16)
         rank = torch.randperm(gen.E, generator=g, device="cuda").to(torch.float32) + 1.0
         p = rank.pow(-zipf_s)
         self.idx = torch.multinomial(p.expand(T, gen.E), gen.topk, replacement=False, generator=g).to(torch.int32).contiguous()
@@ -521,7 +564,7 @@ class PrefillBench:
     def run(self, phases=31, shared=True):
         lib.moe_prefill(self.layer, self.x, self.idx, self.w, self.T, self.ws, self.yr, self.ys, shared=shared, phases=phases)
 
-    def time(self, phases=31, shared=True, reps=8, samples=3):
+    def time(self, phases=31, shared=True, reps=8, samples=7):
         """Seconds per call: `reps` calls back to back between two events (a model's layers follow each other the same
         way; a lone launch after an idle gap runs at a lower clock), the median of `samples` such runs."""
         self.run(phases, shared)

@@ -12,8 +12,10 @@ runner's:
     experts        routing, shared expert and yr += ys fused                                         model.cu:334-343
     add + norm     the next layer's attention norm                                                   model.cu:346-352
 
-fused = True runs each add + norm as the prologue of the GEMV that reads it (dsgx_add_norm_gemv): five launches a layer
-(six with the MFMA variant's ordered sum) instead of seven; the bits are the same."""
+fused = True runs the add + norm in front of the router as the prologue of the router's GEMV (dsgx_add_norm_gemv): six
+launches a layer (seven with the MFMA variant's ordered sum) instead of seven (eight); the bits are the same. fuse_xproj does
+the same for the x-projection: right for the bits, but that GEMV has ten times the router's workgroups, each of which would
+redo the rows' norm, and the layer gets slower (measured: +4 us at hidden 4096, +10 us at 6144), so it is off by default."""
 from . import abi, lib
 
 
@@ -31,7 +33,7 @@ class LayerChain:
         self.ys = alloc(M * H * 4)
         self.cur = 0
 
-    def layer(self, W, fused=True, up=-1, stream=None, tap=None):
+    def layer(self, W, fused=True, up=-1, stream=None, tap=None, fuse_xproj=False):
         """W: dict(attn_norm, ffn_norm bf16 [H]; xproj bf16 [XR][H]; qb, oproj: dict(fmt, w, s, zp) [NQ][QL], [H][NQ]; router bf16
         [E][H]; moe: a dsgx_layer_w; ws: its decode workspace). Reads res[cur] and yr, leaves the new residual in res[cur].
         tap(name): called after each stage (tests read the stage's buffers then)."""
@@ -39,7 +41,7 @@ class LayerChain:
         a, b = self.res[self.cur], self.res[self.cur ^ 1]
         tap = tap or (lambda name: None)
         xp = [dict(fmt=abi.FMT_BF16, w=W["xproj"], n=XR, y=self.xg, ldy=XR)]
-        if fused:
+        if fused and fuse_xproj:
             lib.add_norm_gemv(self.yr, None, a, b, W["attn_norm"], 1e-5, None, M, H, xp, abi.OUT_BF16, splitk=4, stream=stream)
         else:
             lib.add_norm(self.yr, None, M, H, a, b, W["attn_norm"], 1e-5, self.xn, stream=stream)

@@ -160,7 +160,7 @@ def test_chained_layers_against_the_oracle_chain(fmt, shared, scale):
                                       ("logits", ch.logits, np.float32, (M, E)), ("yr", ch.yr, np.float32, (M, H))):
                     got[name + "." + k] = gpu.host(t, dt, shp)
             yr_prev, res_prev = gpu.host(ch.yr, np.float32, (M, H)), gpu.host(ch.res[ch.cur], np.uint16, (M, H))
-            ch.layer(d, fused=fused, up=0 if fmt == abi.FMT_FP8 else 1, tap=None if fused else tap)
+            ch.layer(d, fused=fused, up=0 if fmt == abi.FMT_FP8 else 1, tap=None if fused else tap, fuse_xproj=fused)
             if fused:
                 continue
             # (2) stage by stage, the oracle fed with the GPU's own inputs
