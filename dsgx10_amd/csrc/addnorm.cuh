@@ -34,6 +34,11 @@ __device__ __forceinline__ void add_norm_row(const NormIn& a, int row, int H, fl
   const size_t base = (size_t)row * H + (size_t)tid * per;
   float hv[64];
   float ss = 0.f;
+  // the norm's weights are fetched with the row's other inputs: one memory round trip for the call, not two
+  u32x4_t wq[8];
+#pragma unroll
+  for (int i = 0; i < 64; i += 8)
+    if (want_xn && i < per) wq[i >> 3] = *reinterpret_cast<const DSGX_GLOBAL u32x4_t*>((uintptr_t)(a.w + (size_t)tid * per + i));
 #pragma unroll
   for (int i = 0; i < 64; i += 8) {
     if (i >= per) break;
@@ -64,11 +69,11 @@ __device__ __forceinline__ void add_norm_row(const NormIn& a, int row, int H, fl
 #pragma unroll
   for (int i = 0; i < 64; i += 8) {
     if (i >= per) break;
-    const u32x4_t wq = *reinterpret_cast<const DSGX_GLOBAL u32x4_t*>((uintptr_t)(a.w + (size_t)tid * per + i));
+    const u32x4_t wv4 = wq[i >> 3];
     uint32_t o[4];
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
-      const float wv = bf16_bits_to_f32(j & 1 ? wq[j >> 1] >> 16 : wq[j >> 1] & 0xFFFFu);
+      const float wv = bf16_bits_to_f32(j & 1 ? wv4[j >> 1] >> 16 : wv4[j >> 1] & 0xFFFFu);
       const uint32_t b = f32_to_bf16_bits(__fmul_rn(wv, bf16_round(__fmul_rn(hv[i + j], rstd))));
       if (j & 1) o[j >> 1] |= b << 16;
       else o[j >> 1] = b;

@@ -251,8 +251,8 @@ int launch_gemv_rb(const GemvArgs& a, hipStream_t st) {
     if (a.splitk == 2) return launch_gemv_sk<FMT, M, 2>(a, st);
     return launch_gemv_sk<FMT, M, 4>(a, st);
   }
-  // few rows: two rows a wavefront so that the whole chip streams
-  if (a.total_rows / 4 < 4 * num_cus_cached()) return launch_gemv<FMT, M, 2>(a, st);
+  // few rows: two rows a wavefront so that every wavefront of the launch (two workgroups of four a CU) has rows to stream
+  if (a.total_rows / 4 < 2 * 8 * num_cus_cached()) return launch_gemv<FMT, M, 2>(a, st);
   return launch_gemv<FMT, M, 4>(a, st);
 }
 template <int FMT>
