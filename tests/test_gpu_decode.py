@@ -115,6 +115,22 @@ def test_decode_fused_routing_and_ysum():
     assert np.array_equal(yr, b_yr + ysin) and np.array_equal(ys, ysin)
 
 
+def test_default_variant_is_the_named_one_per_row_count():
+    """up = -1 (the library's default) picks a variant per call: FP8 layers the vector kernels at one row and variant 1
+    from two rows on, INT4 layers variant 1 at every row count. A row's bits under the default therefore depend on the
+    batch it is decoded in; under a named variant they do not (test_decode_rows, test_decode_mfma_variant). This pins
+    which named variant the default is, so that a caller who needs batch invariance knows what to name."""
+    for case, pick in ((CASES[0], lambda M: 0 if M == 1 else 1), (CASES[2], lambda M: 1)):
+        fmt, H, I, E, topk, NS, shared, scale = case
+        hl, dl = _layer(fmt, H, I, E, topk, NS, shared)
+        x, logits, idx, w = rows_and_routing(77, 4, H, E, topk, scale)
+        for M in (1, 2, 4):
+            yr, ys, _ = gpu.decode_layer(dl, x[:M], idx[:M], w[:M], M, up=-1)
+            yn, sn, _ = gpu.decode_layer(dl, x[:M], idx[:M], w[:M], M, up=pick(M))
+            assert np.array_equal(yr.view(np.uint32), yn.view(np.uint32)), (fmt, M)
+            assert np.array_equal(ys.view(np.uint32), sn.view(np.uint32)), (fmt, M)
+
+
 def test_decode_two_launch_variant_equals_default_and_flag_clear():
     """down variant 1 (gate/up and down as two launches) gives the default's bits (one persistent kernel with a grid
     barrier); the barrier's error flag in the workspace stays 0"""
