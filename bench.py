@@ -74,6 +74,61 @@ def prefill_extra(gen, T, name, peak, check=True):
     return d
 
 
+def dsk_prefill_extra(T=8192, check=True):
+    """DeepSeek's prefill MoE chunk (dsgx_dsk_moe_prefill): T rows, top-6 of 256 MXFP4 experts (Zipf(1.1)) + the FP8 shared expert,
+    on the block-scaled e4m3 / e2m1 MFMA (peak 5 PFLOP/s: the wider operand sets the rate); phases: 1 bucketing, 2 shared
+    expert, 4 gate/up, 8 down, 16 combine"""
+    from benchdata import DskPrefillBench
+    import torch
+    pb = DskPrefillBench(T)
+    peak = 5.0e15
+    t_routed, t_all = pb.time(1 | 4 | 8 | 16), pb.time(31)
+    picked = int((torch.bincount(pb.idx.reshape(-1).long(), minlength=pb.E) > 0).sum())
+    d = dict(workload=pb.name, T=T, zipf_s=1.1, ms_routed=t_routed * 1e3, ms_with_shared=t_all * 1e3, tflops_routed=pb.flops_routed / t_routed / 1e12,
+             tflops_with_shared=(pb.flops_routed + pb.flops_shared) / t_all / 1e12, mfma_peak_tflops=peak / 1e12, mfma_frac=pb.flops_routed / t_routed / peak,
+             phases_ms={n: pb.time(ph) * 1e3 for n, ph in (("bucket", 1), ("shared", 2), ("up", 4), ("down", 8), ("combine", 16))},
+             algorithmic_bytes_routed=picked * pb.expert_bytes + T * pb.H * (1 + 4) + T * pb.H // 32)
+    d["hbm_bound_ms"] = d["algorithmic_bytes_routed"] / (HBM_PEAK_GBS * 1e9) * 1e3
+    d["mfma_bound_ms"] = pb.flops_routed / peak * 1e3
+    d["hbm_frac"] = d["hbm_bound_ms"] / d["ms_routed"]
+    d["bound"] = "hbm" if d["hbm_bound_ms"] > d["mfma_bound_ms"] else "mfma"
+    log("  %s T=%d: routed %.3f ms (%.0f TFLOP/s, %.1f%% of %.1f PFLOP/s; %.2f GB of weights and rows at least: %.1f%% of 8 TB/s), with shared %.3f ms; phases %s" %
+        (pb.name, T, d["ms_routed"], d["tflops_routed"], 100 * d["mfma_frac"], peak / 1e15, d["algorithmic_bytes_routed"] / 1e9, 100 * d["hbm_frac"],
+         d["ms_with_shared"], {k: round(v, 3) for k, v in d["phases_ms"].items()}))
+    if check:
+        d["gpu_vs_oracle"] = dsk_prefill_check_rows(pb)
+        log("  %s: rows %s against the oracle's chain: max-abs %.2e, rel-L2 %.2e" % (pb.name, d["gpu_vs_oracle"]["rows"], d["gpu_vs_oracle"]["max_abs_err"], d["gpu_vs_oracle"]["rel_l2"]))
+    del pb
+    return d
+
+
+def dsk_prefill_check_rows(pb, rows=(0, 4097, 8191)):
+    """Part of the CPU leg: a few rows of the chunk just timed against the C++ oracle's chain (each picked expert and the shared
+    one: gate/up, clamped SwiGLU times the routing weight, h quantised per 32, w2, rounded to bf16; summed in expert-id order)"""
+    import torch
+    from tests import orc   # the oracle: test infrastructure, used here as the checker only
+    pb.run(31)
+    torch.cuda.synchronize()
+    rows = [t for t in rows if t < pb.T] or [0]
+    host = lambda t: t.cpu().numpy()
+    sh = tuple(orc.fp8e_dequant(host(pb.t["sh_w" + n]), host(pb.t["sh_s" + n])) for n in ("1", "3", "2"))
+    worst = dict(rows=rows, max_abs_err=0.0, rel_l2=0.0, oracle="C++ oracle (DeepSeek's expert arithmetic, f32 sums)")
+    for t in rows:
+        xd = orc.dequant_act_ue8m0(host(pb.xq[t:t + 1]), host(pb.xs[t:t + 1]))
+        ref = np.zeros(pb.H, np.float32)
+        idx, w = host(pb.idx[t]), host(pb.w[t])
+        for e in sorted(int(v) for v in idx):
+            w1, w3, w2 = (orc.mxfp4_dequant(host(pb.t["w" + n][e]), host(pb.t["s" + n][e])) for n in ("1", "3", "2"))
+            up = orc.dsk_up(w1, w3, xd, np.array([w[list(idx).index(e)]], np.float32), want_range=False)
+            ref = ref + orc.bf16_to_f32(orc.dsk_down(w2, up["h32"])["outb"][0])
+        up = orc.dsk_up(sh[0], sh[1], xd, None, want_range=False)
+        ref = ref + orc.bf16_to_f32(orc.dsk_down(sh[2], up["h32"])["outb"][0])
+        got = host(pb.y[t])
+        worst["max_abs_err"] = max(worst["max_abs_err"], float(np.abs(got - ref).max()))
+        worst["rel_l2"] = max(worst["rel_l2"], float(np.linalg.norm(got - ref) / max(np.linalg.norm(ref), 1e-30)))
+    return worst
+
+
 def chain_entries(gen, layers=96):
     """the layer chains of one format at one row: the MoE half alone (router GEMV + experts + add + norm) and the whole chain
     with the dense projections, each with the add + norms as launches of their own and fused into the GEMVs that read them"""
@@ -146,7 +201,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=64)
     ap.add_argument("--no-extra", action="store_true", help="only the headline workload")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
-    ap.add_argument("--workload", default="fp8_m1", help="headline workload: fp8_m1 | int4_m1; fp8_prefill | int4_prefill time only that prefill chunk; gemv only the dense GEMVs; chain only the layer chains; dsk only the MXFP4 layer")
+    ap.add_argument("--workload", default="fp8_m1", help="headline workload: fp8_m1 | int4_m1; fp8_prefill | int4_prefill time only that prefill chunk; gemv only the dense GEMVs; chain only the layer chains; dsk only the MXFP4 layer's decode steps; dsk_prefill only its prefill chunk")
     ap.add_argument("--variant", default="vector", choices=("vector", "mfma"),
                     help="the headline's decode kernels (dsgx_decode_cfg::up = 0 | 1); --no-extra then runs nothing else")
     args = ap.parse_args()
@@ -237,6 +292,15 @@ def main():
                                        "frac": ds[0]["hbm_frac"], "traffic": None},
                           "cpu_baseline": None, "extra": ds, "wall_s": round(time.time() - t_start, 1)}))
         return
+    if args.workload == "dsk_prefill":
+        d = dsk_prefill_extra(8192, check=not args.no_cpu)
+        print(json.dumps({"metric": "ms_per_prefill_chunk", "value": d["ms_routed"], "unit": "ms", "n_gpus": 1, "steps": 8, "warmup": 1, "ms_per_step": d["ms_routed"],
+                          "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "e2m1 / e4m3 x e4m3 with ue8m0 scales, f32 sums (block-scaled MFMA)",
+                          "data": "synthetic", "config": {"workload": d["workload"], "T": d["T"]},
+                          "roofline": {"bound": "mfma", "achieved": d["tflops_routed"], "peak": d["mfma_peak_tflops"], "unit": "TFLOP/s", "frac": d["mfma_frac"],
+                                       "traffic": None, "hbm_frac": d["hbm_frac"]},
+                          "cpu_baseline": None, "extra": [d], "wall_s": round(time.time() - t_start, 1)}))
+        return
     if args.workload == "chain":
         # only the layer chains (router GEMV -> experts -> add + norm, 128 layers a graph), FP8 then INT4
         from benchdata import ChainBench
@@ -304,6 +368,9 @@ def main():
             log("  %s M=%d: %.2f us/layer (%.1f%% of 8 TB/s)" % (d["workload"], M, d["us_per_layer"], 100 * d["hbm_frac"]))
             extra.append(d)
         del dg
+        import torch
+        torch.cuda.empty_cache()
+        extra.append(dsk_prefill_extra(8192, check=not args.no_cpu))
         extra += gemv_bench()
 
     out = {

@@ -539,6 +539,61 @@ def gemv_bench(reps=64):
     return out
 
 
+class DskPrefillBench:
+    """One prefill chunk of T rows through dsgx_dsk_moe_prefill (dsk::moe_prefill, ds41f-4xgx10-switchless/engine/kernels/
+    dsk.h:268-295) at DeepSeek's unsharded layer shape: hidden 5120, intermediate 2304 (the reference's 576 a rank x 4), 256 MXFP4
+    experts stacked by id, top-6 drawn from a Zipf(s) popularity with uniform weights, one FP8 shared expert; random e2m1
+    codes and scale bytes, rows N(0, 1.5) quantised per 32 (ue8m0) as the reference's act_quant does."""
+    name = "dsk_mxfp4_moe_prefill"
+    H, I, E, topk = 5120, 2304, 256, 6
+
+    def __init__(self, T, zipf_s=1.1, seed=4321):
+        H, I, E, topk = self.H, self.I, self.E, self.topk
+        self.T = T
+        g = torch.Generator(device="cuda")
+        g.manual_seed(seed)
+        rnd = lambda shape, lo, hi: torch.randint(lo, hi, shape, generator=g, device="cuda", dtype=torch.uint8)
+        self.t = {}
+        for n, (N, K) in (("1", (I, H)), ("3", (I, H)), ("2", (H, I))):
+            self.t["w" + n], self.t["s" + n] = rnd((E, N, K // 2), 0, 256), rnd((E, N, K // 32), 114, 120)
+            self.t["sh_w" + n] = (torch.randn(N, K, generator=g, device="cuda") * 40.0).clamp(-448, 448).to(torch.float8_e4m3fn).view(torch.uint8)
+            self.t["sh_s" + n] = rnd((N // 32, K // 32), 110, 116)
+        self.weights = abi.DskWeights(*[self.t[k].data_ptr() for k in ("w1", "s1", "w3", "s3", "w2", "s2", "sh_w1", "sh_s1", "sh_w3", "sh_s3", "sh_w2", "sh_s2")],
+                                      H, I, E, topk)
+        x = Seeded(seed).normal((T, H), 1.5)
+        blk = x.view(T, H // 32, 32)
+        v = blk.abs().amax(-1).clamp_min(1e-4) * torch.tensor(1.0 / 448.0, device="cuda")
+        bits = v.view(torch.int32)
+        e = ((bits >> 23) & 0xFF) + ((bits & 0x7FFFFF) != 0).to(torch.int32)
+        self.xs = e.to(torch.uint8).contiguous()
+        self.xq = (blk * torch.ldexp(torch.ones_like(v), (127 - e).float())[..., None]).clamp(-448, 448).to(torch.float8_e4m3fn).view(torch.uint8).reshape(T, H).contiguous()
+        rank = torch.randperm(E, generator=g, device="cuda").to(torch.float32) + 1.0
+        self.idx = torch.multinomial(rank.pow(-zipf_s).expand(T, E), topk, replacement=False, generator=g).to(torch.int32).contiguous()
+        self.w = torch.full((T, topk), 1.0 / topk, dtype=torch.float32, device="cuda")
+        self.ws = torch.empty(lib.dsk_prefill_ws_bytes(H, I, E, topk, T), dtype=torch.uint8, device="cuda")
+        self.y = torch.zeros(T, H, dtype=torch.float32, device="cuda")
+        self.flops_routed = 2.0 * T * topk * 3 * I * H
+        self.flops_shared = 2.0 * T * 3 * I * H
+        self.expert_bytes = 3 * (I * H // 2 + I * H // 32)
+
+    def run(self, phases=31):
+        lib.dsk_moe_prefill(self.weights, self.xq, self.xs, self.idx, self.w, self.T, self.ws, self.y, phases=phases)
+
+    def time(self, phases=31, reps=8, samples=7):
+        self.run(phases)
+        torch.cuda.synchronize()
+        ts = []
+        for _ in range(samples):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(reps):
+                self.run(phases)
+            e1.record()
+            torch.cuda.synchronize()
+            ts.append(e0.elapsed_time(e1) * 1e-3 / reps)
+        return float(np.median(ts))
+
+
 class PrefillBench:
     """One prefill chunk of T rows over a generated FP8 layer: each row picks top-k distinct experts drawn from a
     Zipf(s) popularity over a seeded permutation of the experts, uniform weights 1/top-k (the reference's

@@ -34,6 +34,14 @@ class DskWeights(C.Structure):
                [(n, C.c_int32) for n in ("H", "I", "E", "topk")]
 
 
+class DskPrefillCfg(C.Structure):
+    _fields_ = [("swiglu_limit", C.c_float), ("phases", C.c_int32)]
+
+
+class DskPrefillView(C.Structure):
+    _fields_ = [(n, C.c_void_p) for n in ("rpos", "re", "off", "perm", "h", "hsh", "d", "dsh", "hq", "hs")]
+
+
 class DecodeCfg(C.Structure):
     _fields_ = [("up", C.c_int32), ("down", C.c_int32), ("parts", C.c_int32), ("ysum", C.c_int32),
                 ("logits", C.c_void_p), ("bias", C.c_void_p), ("route_scale", C.c_float), ("score_fn", C.c_int32),
@@ -66,4 +74,5 @@ SYMBOLS = [
     "dsgx_decode_ws_bytes", "dsgx_decode_ws_flag_offset", "dsgx_decode_status", "dsgx_moe_decode", "dsgx_moe_decode_noalloc", "dsgx_finalize", "dsgx_add_norm", "dsgx_dsk_cfg_default", "dsgx_dsk_moe", "dsgx_dsk_ws_bytes", "dsgx_dsk_moe_stacked", "dsgx_prefill_cfg_default", "dsgx_prefill_ws_bytes",
     "dsgx_moe_prefill", "dsgx_prefill_view_get", "dsgx_gemv", "dsgx_dequant_int4", "dsgx_probe_dequant_int4", "dsgx_probe_mfma_fp8",
     "dsgx_widen_fp8", "dsgx_act_quant", "dsgx_last_error", "dsgx_version", "dsgx_stream_read", "dsgx_stream_read_cfg", "dsgx_stream_copy", "dsgx_add_norm_gemv", "dsgx_fill_normal", "dsgx_launch_floor",
+    "dsgx_dsk_prefill_cfg_default", "dsgx_dsk_prefill_ws_bytes", "dsgx_dsk_moe_prefill", "dsgx_dsk_prefill_view_get", "dsgx_probe_mfma_scaled",
 ]

@@ -19,6 +19,7 @@
 #include "abi_internal.h"
 #include "common.cuh"
 #include "pf_gemm_fp8.cuh"
+#include "pf_gemm_mx.cuh"
 
 #ifdef DSGX_TRACE
 extern "C" unsigned long long* dsgx_trace_buf();
@@ -71,7 +72,7 @@ __global__ void __launch_bounds__(64) k_probe_mfma_fp8(const uint8_t* __restrict
 constexpr int kTile = 128;  // rows of a tile (token positions) and weight rows a workgroup
 constexpr int kRowBlock = 128;  // token rows a workgroup of the bucketing kernels
 struct PfLayout {
-  size_t cnt, off, ntiles, tile_e, tile_m0, perm, pickpos, rpos, re, rk, xq, xs, h, hq, hs, hsh, hshq, hshs, d, bcnt, boff, bmask, total;
+  size_t cnt, off, ntiles, tile_e, tile_m0, perm, pickpos, posw, rpos, re, rk, xq, xs, h, hq, hs, hsh, hshq, hshs, d, bcnt, boff, bmask, total;
   size_t nbig, big_e, big_m0, nsmall, small_e, small_m0;  // the FP8 kernels' lists: 256-position tiles, and the experts' remainders
   size_t nmix, mix_e, mix_m0;                             // ... and the two merged into the order the kernels run them in
   int P, max_tiles, max_big;
@@ -89,7 +90,7 @@ PfLayout pf_layout(const dsgx_layer_w* L, int T) {
   o.nbig = take(4), o.big_e = take((size_t)o.max_big * 4), o.big_m0 = take((size_t)o.max_big * 4);
   o.nsmall = take(4), o.small_e = take(E * 4), o.small_m0 = take(E * 4);
   o.nmix = take(4), o.mix_e = take((size_t)(o.max_big + E) * 4), o.mix_m0 = take((size_t)(o.max_big + E) * 4);
-  o.perm = take(P * 4), o.pickpos = take(P * 4), o.rpos = take(P * 4), o.re = take(P * 4), o.rk = take(P * 4);
+  o.perm = take(P * 4), o.pickpos = take(P * 4), o.posw = take(P * 4), o.rpos = take(P * 4), o.re = take(P * 4), o.rk = take(P * 4);
   o.xq = take((size_t)T * H), o.xs = take((size_t)T * (H / 128) * 4);
   o.h = take(P * I * 2), o.hq = take(P * I), o.hs = take(P * (I / 128) * 4);
   o.hsh = take((size_t)T * I * 2), o.hshq = take((size_t)T * I), o.hshs = take((size_t)T * (I / 128) * 4);
@@ -183,7 +184,7 @@ __global__ void __launch_bounds__(256) k_pf_place(const int* __restrict__ idx, c
                                                   const int* __restrict__ off, const int* __restrict__ boff,
                                                   const uint32_t* __restrict__ bmask, const dsgx_mat_desc* __restrict__ desc,
                                                   int* __restrict__ perm, int* __restrict__ pickpos, int* __restrict__ rpos,
-                                                  int* __restrict__ re, float* __restrict__ rk) {
+                                                  int* __restrict__ re, float* __restrict__ rk, float* __restrict__ posw) {
   __shared__ uint32_t mask[DSGX_MAX_EXPERTS * 4];
   __shared__ int base[DSGX_MAX_EXPERTS];
   const int b = blockIdx.x, t0 = b * kRowBlock, rows = min(kRowBlock, T - t0);
@@ -203,7 +204,9 @@ __global__ void __launch_bounds__(256) k_pf_place(const int* __restrict__ idx, c
     int rank = 0;
     for (int j = 0; j < topk; ++j) rank += idx[(size_t)t * topk + j] < e;
     const size_t o = (size_t)t * topk + rank;
-    re[o] = e, rpos[o] = pos, rk[o] = __fmul_rn(desc[(size_t)e * 3 + 2].s2, w[(size_t)t * topk + k]);
+    const float wv = w[(size_t)t * topk + k];
+    re[o] = e, rpos[o] = pos, rk[o] = desc ? __fmul_rn(desc[(size_t)e * 3 + 2].s2, wv) : wv;
+    if (posw) posw[pos] = wv;  // (DeepSeek's layers apply the routing weight to h, position by position)
   }
 }
 
@@ -550,6 +553,50 @@ __global__ void __launch_bounds__(256) k_pf_combine(const float* __restrict__ d,
   *reinterpret_cast<float4*>(yr + (size_t)t * H + n) = a;
 }
 
+// DeepSeek's combine (ds41f engine/kernels/moe.cu:974-981): y[t] = the f32 sum, in expert-id order, of the picks' outputs
+// (each already rounded to bf16 by the down GEMM), then the shared expert's; eight columns a thread
+__global__ void __launch_bounds__(256) k_pfmx_combine(const uint16_t* __restrict__ d, const uint16_t* __restrict__ dsh, const int* __restrict__ rpos,
+                                                      int T, int H, int topk, float* __restrict__ y) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int per = H / 8;
+  if (i >= (size_t)T * per) return;
+  const int t = (int)(i / per), n = (int)(i % per) * 8;
+  float a[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  auto add = [&](const uint16_t* row) {
+    const u32x4_t v = *reinterpret_cast<const u32x4_t*>(row + n);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) a[2 * j] = __fadd_rn(a[2 * j], bf16_bits_to_f32(v[j] & 0xFFFFu)), a[2 * j + 1] = __fadd_rn(a[2 * j + 1], bf16_bits_to_f32(v[j] >> 16));
+  };
+  for (int r = 0; r < topk; ++r) add(d + (size_t)rpos[t * topk + r] * H);
+  if (dsh) add(dsh + (size_t)t * H);
+  float4* o = reinterpret_cast<float4*>(y + (size_t)t * H + n);
+  o[0] = make_float4(a[0], a[1], a[2], a[3]), o[1] = make_float4(a[4], a[5], a[6], a[7]);
+}
+
+// one v_mfma_scale_f32_16x16x128_f8f6f4: A [16 rows][128 k] as e2m1 pairs (64 bytes a row) or e4m3, B [16][128] e4m3, a
+// ue8m0 byte per row and 32 k for each (SA, SB [16][4]); out[a row][b row]. Operands as the kernels of pf_gemm_mx.cuh
+// hand them over: an 8-bit row's bytes 16 part ... and 64 + 16 part ..., a 4-bit row's bytes 16 part ..., scale byte `part`.
+template <int CBSZ>
+__global__ void __launch_bounds__(64) k_probe_mfma_scaled(const uint8_t* __restrict__ A, const uint8_t* __restrict__ SA, const uint8_t* __restrict__ B,
+                                                          const uint8_t* __restrict__ SB, float* __restrict__ out) {
+  const int l = threadIdx.x, row = l % 16, part = l / 16;
+  pf8::v8i_t a = {0, 0, 0, 0, 0, 0, 0, 0}, b;
+  if (CBSZ == 4) {
+    const uint4 lo = *reinterpret_cast<const uint4*>(A + row * 64 + part * 16);
+    a = pf8::v8i_t{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, 0, 0, 0, 0};
+  } else {
+    const uint4 lo = *reinterpret_cast<const uint4*>(A + row * 128 + part * 16), hi = *reinterpret_cast<const uint4*>(A + row * 128 + 64 + part * 16);
+    a = pf8::v8i_t{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
+  }
+  {
+    const uint4 lo = *reinterpret_cast<const uint4*>(B + row * 128 + part * 16), hi = *reinterpret_cast<const uint4*>(B + row * 128 + 64 + part * 16);
+    b = pf8::v8i_t{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
+  }
+  const pf8::v4f_t c = pfmx::mfma_mx<CBSZ>(a, b, pf8::v4f_t{0.f, 0.f, 0.f, 0.f}, SA[row * 4 + part], SB[row * 4 + part]);
+#pragma unroll
+  for (int q = 0; q < 4; ++q) out[(4 * part + q) * 16 + row] = c[q];
+}
+
 bool layer_has_fp8_shared(const dsgx_layer_w* L) { return L->sh.g && L->sh.u && L->sh.d && L->sh.gs && L->sh.us && L->sh.ds; }
 
 }  // namespace
@@ -623,7 +670,7 @@ int dsgx_moe_prefill(const dsgx_layer_w* L, const uint16_t* x, const int* idx, c
                        I32(o.nmix), I32(o.mix_e), I32(o.mix_m0)};
     hipLaunchKernelGGL(k_pf_scan, dim3(1), dim3(DSGX_MAX_EXPERTS), 0, st, I32(o.bcnt), NB, E, I32(o.boff), I32(o.cnt), I32(o.off), tl);
     hipLaunchKernelGGL(k_pf_place, dim3(NB), dim3(256), 0, st, idx, w, T, topk, E, I32(o.off), I32(o.boff), bmask, L->desc, I32(o.perm),
-                       I32(o.pickpos), I32(o.rpos), I32(o.re), F32(o.rk));
+                       I32(o.pickpos), I32(o.rpos), I32(o.re), F32(o.rk), (float*)nullptr);
     DSGX_HIP(hipGetLastError());
   }
   if (i4 || !cfg.act_fp8) {
@@ -734,6 +781,141 @@ int dsgx_prefill_view_get(const dsgx_layer_w* L, void* ws, int T, dsgx_prefill_v
   out->hsh = reinterpret_cast<const uint16_t*>(W + o.hsh);
   out->off = reinterpret_cast<const int*>(W + o.off);
   out->perm = reinterpret_cast<const int*>(W + o.perm);
+  return DSGX_OK;
+}
+
+int dsgx_probe_mfma_scaled(const void* A, const void* SA, const void* B, const void* SB, int a_fp4, float* out, void* stream) {
+  if (!A || !SA || !B || !SB || !out) return fail(DSGX_EINVAL, "probe_mfma_scaled: null argument");
+  const uint8_t *a = (const uint8_t*)A, *sa = (const uint8_t*)SA, *b = (const uint8_t*)B, *sb = (const uint8_t*)SB;
+  if (a_fp4) hipLaunchKernelGGL(k_probe_mfma_scaled<4>, dim3(1), dim3(64), 0, (hipStream_t)stream, a, sa, b, sb, out);
+  else hipLaunchKernelGGL(k_probe_mfma_scaled<0>, dim3(1), dim3(64), 0, (hipStream_t)stream, a, sa, b, sb, out);
+  DSGX_HIP(hipGetLastError());
+  return DSGX_OK;
+}
+
+// ---- DeepSeek's prefill MoE (dsk::moe_prefill, ds41f-4xgx10-switchless/engine/kernels/dsk.h:268-295, prefill.cu:1605-1675) ----
+void dsgx_dsk_prefill_cfg_default(dsgx_dsk_prefill_cfg* c) {
+  if (!c) return;
+  c->swiglu_limit = 10.f;
+  c->phases = 31;
+}
+static int dsk_prefill_check(const dsgx_dsk_weights* W, int T, const char* who, dsgx_layer_w* shape) {
+  if (!W) return fail(DSGX_EINVAL, "%s: null weights", who);
+  if (T < 1 || T > DSGX_MAX_CHUNK) return fail(DSGX_EINVAL, "%s: T %d (1..%d)", who, T, DSGX_MAX_CHUNK);
+  if (W->H < 256 || W->H % 256 || W->I < 128 || W->I % 128 || W->H > 16384 || W->I > 16384)
+    return fail(DSGX_EINVAL, "%s: H %d (a multiple of 256), I %d (a multiple of 128), both up to 16384", who, W->H, W->I);
+  if (W->E < 1 || W->E > DSGX_MAX_EXPERTS || W->topk < 1 || W->topk > DSGX_MAX_TOPK || W->topk > W->E)
+    return fail(DSGX_EINVAL, "%s: E %d, top-k %d", who, W->E, W->topk);
+  *shape = dsgx_layer_w{};
+  shape->H = W->H, shape->I = W->I, shape->E = W->E, shape->topk = W->topk, shape->fmt = DSGX_FMT_MXFP4_G32;
+  return DSGX_OK;
+}
+size_t dsgx_dsk_prefill_ws_bytes(int H, int I, int E, int topk, int T) {
+  dsgx_dsk_weights w{};
+  w.H = H, w.I = I, w.E = E, w.topk = topk;
+  dsgx_layer_w shape;
+  if (dsk_prefill_check(&w, T, "dsk_prefill_ws_bytes", &shape)) return 0;
+  return pf_layout(&shape, T).total;
+}
+
+int dsgx_dsk_moe_prefill(const dsgx_dsk_weights* Wt, const uint8_t* xq, const uint8_t* xs, int T, const int* idx, const float* w, void* ws,
+                         float* y, void* stream, const dsgx_dsk_prefill_cfg* cfg_in) {
+  dsgx_layer_w shape;
+  if (int rc = dsk_prefill_check(Wt, T, "dsk_moe_prefill", &shape)) return rc;
+  dsgx_dsk_prefill_cfg cfg;
+  dsgx_dsk_prefill_cfg_default(&cfg);
+  if (cfg_in) cfg = *cfg_in;
+  if (!xq || !xs || !idx || !w || !ws || !y) return fail(DSGX_EINVAL, "dsk_moe_prefill: null xq, xs, idx, w, ws or y");
+  if (!Wt->w1 || !Wt->s1 || !Wt->w3 || !Wt->s3 || !Wt->w2 || !Wt->s2) return fail(DSGX_EINVAL, "dsk_moe_prefill: null expert tensor");
+  const bool shared = Wt->sh_w1 != nullptr;
+  if (shared && (!Wt->sh_s1 || !Wt->sh_w3 || !Wt->sh_s3 || !Wt->sh_w2 || !Wt->sh_s2)) return fail(DSGX_EINVAL, "dsk_moe_prefill: shared expert tensors missing");
+  for (const void* p : {(const void*)xq, (const void*)Wt->w1, (const void*)Wt->w3, (const void*)Wt->w2, (const void*)Wt->sh_w1, (const void*)Wt->sh_w3, (const void*)Wt->sh_w2})
+    if ((uintptr_t)p % 16) return fail(DSGX_EINVAL, "dsk_moe_prefill: xq and the weight tensors must be 16-byte aligned");
+  for (const void* p : {(const void*)xs, (const void*)Wt->s1, (const void*)Wt->s3, (const void*)Wt->s2, (const void*)Wt->sh_s1, (const void*)Wt->sh_s3, (const void*)Wt->sh_s2})
+    if ((uintptr_t)p % 4) return fail(DSGX_EINVAL, "dsk_moe_prefill: the scale tensors must be 4-byte aligned");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const PfLayout o = pf_layout(&shape, T);
+  uint8_t* W = static_cast<uint8_t*>(ws);
+  auto I32 = [&](size_t off) { return reinterpret_cast<int*>(W + off); };
+  auto F32 = [&](size_t off) { return reinterpret_cast<float*>(W + off); };
+  auto U16 = [&](size_t off) { return reinterpret_cast<uint16_t*>(W + off); };
+  const int H = Wt->H, I = Wt->I, E = Wt->E, topk = Wt->topk, P = o.P;
+  constexpr int F4 = DSGX_FMT_MXFP4_G32, F8 = DSGX_FMT_FP8_B32E;
+  constexpr int kLdsMix = pfmx::Shape<1, F4>::kLds > pfmx::Shape<2, F4>::kLds ? pfmx::Shape<1, F4>::kLds : pfmx::Shape<2, F4>::kLds;
+  constexpr int kLdsSh = pfmx::Shape<2, F8>::kLds;
+  void (*k_up)(pfmx::Args) = pfmx::k_gemm_mixed<true, F4>;
+  void (*k_dn)(pfmx::Args) = pfmx::k_gemm_mixed<false, F4>;
+  void (*k_sup)(pfmx::Args) = pfmx::k_gemm<true, F8>;
+  void (*k_sdn)(pfmx::Args) = pfmx::k_gemm<false, F8>;
+  for (const void* k : {(const void*)k_up, (const void*)k_dn})
+    if (int rc = allow_dynamic_lds(k, kLdsMix)) return rc;
+  for (const void* k : {(const void*)k_sup, (const void*)k_sdn})
+    if (int rc = allow_dynamic_lds(k, kLdsSh)) return rc;
+  const int NSU = I / (pf8::kWgRows / 2), NSD = H / pf8::kWgRows;
+  uint16_t* dsh = U16(o.d + align256((size_t)P * H * 2));  // the shared expert's outputs behind the picks', both bf16
+  // phases (dsk::MoePCfg, dsk.h:278-282): 1 bucketing, 2 shared expert, 4 routed up, 8 routed down, 16 combine
+  if (cfg.phases & 1) {
+    const int NB = (T + kRowBlock - 1) / kRowBlock;
+    uint32_t* bmask = reinterpret_cast<uint32_t*>(W + o.bmask);
+    hipLaunchKernelGGL(k_pf_mask, dim3(NB), dim3(256), 0, st, idx, T, topk, E, I32(o.bcnt), bmask);
+    const TileLists tl{I32(o.ntiles), I32(o.tile_e), I32(o.tile_m0), I32(o.nbig), I32(o.big_e), I32(o.big_m0), I32(o.nsmall), I32(o.small_e), I32(o.small_m0),
+                       I32(o.nmix), I32(o.mix_e), I32(o.mix_m0)};
+    hipLaunchKernelGGL(k_pf_scan, dim3(1), dim3(DSGX_MAX_EXPERTS), 0, st, I32(o.bcnt), NB, E, I32(o.boff), I32(o.cnt), I32(o.off), tl);
+    hipLaunchKernelGGL(k_pf_place, dim3(NB), dim3(256), 0, st, idx, w, T, topk, E, I32(o.off), I32(o.boff), bmask, (const dsgx_mat_desc*)nullptr, I32(o.perm),
+                       I32(o.pickpos), I32(o.rpos), I32(o.re), F32(o.rk), F32(o.posw));
+    DSGX_HIP(hipGetLastError());
+  }
+  pfmx::Args g{};
+  g.H = H, g.I = I, g.limit = cfg.swiglu_limit;
+  if ((cfg.phases & 2) && shared) {
+    const int tiles = (T + 255) / 256;
+    g.tile_e = g.tile_m0 = g.ntiles = g.off = nullptr, g.nrows = T, g.gather = nullptr, g.posw = nullptr, g.wstride = g.sstride = 0;
+    g.aq = xq, g.as = xs, g.wa = Wt->sh_w1, g.sa = Wt->sh_s1, g.wb = Wt->sh_w3, g.sb = Wt->sh_s3;
+    g.h = U16(o.hsh), g.hq = W + o.hshq, g.hs = W + o.hshs, g.d = nullptr;
+    hipLaunchKernelGGL(k_sup, dim3(pf8::grid_of(tiles, NSU)), dim3(pf8::kThreads), kLdsSh, st, g);
+    g.aq = W + o.hshq, g.as = W + o.hshs, g.wa = Wt->sh_w2, g.sa = Wt->sh_s2, g.wb = g.sb = nullptr;
+    g.h = nullptr, g.hq = g.hs = nullptr, g.d = dsh;
+    hipLaunchKernelGGL(k_sdn, dim3(pf8::grid_of(tiles, NSD)), dim3(pf8::kThreads), kLdsSh, st, g);
+    DSGX_HIP(hipGetLastError());
+  }
+  g.tile_e = I32(o.mix_e), g.tile_m0 = I32(o.mix_m0), g.ntiles = I32(o.nmix), g.off = I32(o.off), g.nrows = P;
+  if (cfg.phases & 4) {
+    g.aq = xq, g.as = xs, g.gather = I32(o.perm), g.posw = F32(o.posw);
+    g.wa = Wt->w1, g.sa = Wt->s1, g.wb = Wt->w3, g.sb = Wt->s3, g.wstride = (size_t)I * H / 2, g.sstride = (size_t)I * H / 32;
+    g.h = U16(o.h), g.hq = W + o.hq, g.hs = W + o.hs, g.d = nullptr;
+    hipLaunchKernelGGL(k_up, dim3(pf8::grid_of(o.max_big + E, NSU)), dim3(pf8::kThreads), kLdsMix, st, g);
+    DSGX_HIP(hipGetLastError());
+  }
+  if (cfg.phases & 8) {
+    g.aq = W + o.hq, g.as = W + o.hs, g.gather = nullptr, g.posw = nullptr;
+    g.wa = Wt->w2, g.sa = Wt->s2, g.wb = g.sb = nullptr, g.wstride = (size_t)I * H / 2, g.sstride = (size_t)I * H / 32;
+    g.h = nullptr, g.hq = g.hs = nullptr, g.d = U16(o.d);
+    hipLaunchKernelGGL(k_dn, dim3(pf8::grid_of(o.max_big + E, NSD)), dim3(pf8::kThreads), kLdsMix, st, g);
+    DSGX_HIP(hipGetLastError());
+  }
+  if (cfg.phases & 16) {
+    const size_t n = (size_t)T * (H / 8);
+    hipLaunchKernelGGL(k_pfmx_combine, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, U16(o.d), shared ? dsh : (const uint16_t*)nullptr, I32(o.rpos), T, H, topk, y);
+    DSGX_HIP(hipGetLastError());
+  }
+  return DSGX_OK;
+}
+
+int dsgx_dsk_prefill_view_get(const dsgx_dsk_weights* Wt, void* ws, int T, dsgx_dsk_prefill_view* out) {
+  dsgx_layer_w shape;
+  if (int rc = dsk_prefill_check(Wt, T, "dsk_prefill_view", &shape)) return rc;
+  if (!ws || !out) return fail(DSGX_EINVAL, "dsk_prefill_view: null ws or out");
+  const PfLayout o = pf_layout(&shape, T);
+  uint8_t* W = static_cast<uint8_t*>(ws);
+  out->rpos = reinterpret_cast<const int*>(W + o.rpos);
+  out->re = reinterpret_cast<const int*>(W + o.re);
+  out->off = reinterpret_cast<const int*>(W + o.off);
+  out->perm = reinterpret_cast<const int*>(W + o.perm);
+  out->h = reinterpret_cast<const uint16_t*>(W + o.h);
+  out->hsh = reinterpret_cast<const uint16_t*>(W + o.hsh);
+  out->hq = W + o.hq, out->hs = W + o.hs;
+  out->d = reinterpret_cast<const uint16_t*>(W + o.d);
+  out->dsh = reinterpret_cast<const uint16_t*>(W + o.d + align256((size_t)o.P * Wt->H * 2));
   return DSGX_OK;
 }
 

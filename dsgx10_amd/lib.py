@@ -61,6 +61,12 @@ def lib():
         L.dsgx_dsk_ws_bytes.argtypes = [C.c_int, C.c_int]
         L.dsgx_dsk_moe_stacked.argtypes = [C.POINTER(abi.DskWeights), C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
                                            C.c_void_p, C.POINTER(abi.DskCfg), C.c_void_p, C.c_void_p]
+        L.dsgx_dsk_prefill_ws_bytes.restype = C.c_size_t
+        L.dsgx_dsk_prefill_ws_bytes.argtypes = [C.c_int, C.c_int, C.c_int, C.c_int, C.c_int]
+        L.dsgx_dsk_moe_prefill.argtypes = [C.POINTER(abi.DskWeights), C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
+                                           C.c_void_p, C.POINTER(abi.DskPrefillCfg)]
+        L.dsgx_dsk_prefill_view_get.argtypes = [C.POINTER(abi.DskWeights), C.c_void_p, C.c_int, C.POINTER(abi.DskPrefillView)]
+        L.dsgx_probe_mfma_scaled.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p]
         L.dsgx_add_norm_gemv.argtypes = [C.POINTER(abi.NormIn), C.c_int, C.c_int, C.POINTER(abi.GemvSeg), C.c_int, C.c_int, C.c_int, C.c_void_p]
         L.dsgx_fill_normal.argtypes = [C.c_uint64, C.c_uint64, C.c_size_t, C.c_double, C.c_void_p, C.c_int, C.c_void_p]
         L.dsgx_launch_floor.argtypes = [C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]
@@ -135,6 +141,26 @@ def dsk_moe_stacked(weights, xq, xs, idx, w, M, ws, y, stream=None, limit=10.0, 
     cfg = abi.DskCfg(limit, _ptr(logits), _ptr(bias), route_scale, parts)
     _check(lib().dsgx_dsk_moe_stacked(C.byref(weights), _ptr(xq), _ptr(xs), M, _ptr(idx), _ptr(w), _ptr(ws), _ptr(y), _stream(stream),
                                       C.byref(cfg), _ptr(idx_out), _ptr(wts_out)))
+
+
+def dsk_prefill_ws_bytes(H, I, E, topk, T):
+    return lib().dsgx_dsk_prefill_ws_bytes(H, I, E, topk, T)
+
+
+def dsk_moe_prefill(weights, xq, xs, idx, w, T, ws, y, stream=None, limit=10.0, phases=31):
+    """dsk::moe_prefill: a chunk of T quantised rows through the MXFP4 experts (abi.DskWeights) on the block-scaled MFMA"""
+    cfg = abi.DskPrefillCfg(limit, phases)
+    _check(lib().dsgx_dsk_moe_prefill(C.byref(weights), _ptr(xq), _ptr(xs), T, _ptr(idx), _ptr(w), _ptr(ws), _ptr(y), _stream(stream), C.byref(cfg)))
+
+
+def dsk_prefill_view(weights, ws, T):
+    v = abi.DskPrefillView()
+    _check(lib().dsgx_dsk_prefill_view_get(C.byref(weights), _ptr(ws), T, C.byref(v)))
+    return v
+
+
+def probe_mfma_scaled(A, SA, B, SB, a_fp4, out, stream=None):
+    _check(lib().dsgx_probe_mfma_scaled(_ptr(A), _ptr(SA), _ptr(B), _ptr(SB), int(a_fp4), _ptr(out), _stream(stream)))
 
 
 def decode_status(layer_w, ws, stream=None):

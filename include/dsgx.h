@@ -205,6 +205,33 @@ DSGX_API size_t dsgx_dsk_ws_bytes(int H, int I);
 DSGX_API int dsgx_dsk_moe_stacked(const dsgx_dsk_weights* W, const uint8_t* xq, const uint8_t* xs, int M, const int* idx, const float* w,
                                   void* ws, float* y, void* stream, const dsgx_dsk_cfg* cfg, int* idx_out, float* wts_out);
 
+/* DeepSeek's prefill MoE: dsk::moe_prefill (ds41f-4xgx10-switchless/engine/kernels/dsk.h:268-295, prefill.cu:1605-1675) for a
+   chunk of T rows given as act_quant(x) (xq e4m3 [T][H], xs ue8m0 [T][H/32]) with the router's idx, w [T][topk]: picks
+   bucketed by expert, grouped GEMMs on v_mfma_scale_f32_16x16x128_f8f6f4 (e2m1 / e4m3 weights, e4m3 rows and both ue8m0
+   scale tensors go to the instruction as stored), dsgx_dsk_moe's arithmetic per expert (clamped SwiGLU times the routing
+   weight, h quantised per 32, each pick's output rounded to bf16), then per row the f32 sum in expert-id order, the shared
+   expert last: y f32 [T][H]. The sums inside a dot product are the matrix unit's (block-scaled, 128 k an instruction),
+   not the decode kernels' bf16-MFMA sums: a row's y agrees with dsgx_dsk_moe_stacked's to the tolerance both are tested
+   at, not bit for bit. phases as dsk::MoePCfg: 1 bucketing, 2 shared expert, 4 routed gate/up, 8 routed down, 16 combine.
+   ws: dsgx_dsk_prefill_ws_bytes(...) bytes, no initialisation needed. H a multiple of 256, I of 128, T <= DSGX_MAX_CHUNK. */
+typedef struct dsgx_dsk_prefill_cfg {
+  float swiglu_limit;  /* 10 */
+  int32_t phases;      /* 31 */
+} dsgx_dsk_prefill_cfg;
+DSGX_API void dsgx_dsk_prefill_cfg_default(dsgx_dsk_prefill_cfg* cfg);
+DSGX_API size_t dsgx_dsk_prefill_ws_bytes(int H, int I, int E, int topk, int T);
+DSGX_API int dsgx_dsk_moe_prefill(const dsgx_dsk_weights* W, const uint8_t* xq, const uint8_t* xs, int T, const int* idx, const float* w,
+                                  void* ws, float* y, void* stream, const dsgx_dsk_prefill_cfg* cfg);
+/* The workspace's intermediates after a call: device pointers into ws (bucket positions as dsgx_prefill_view). h: bf16
+   [position][I] before its quantisation, hq / hs: as the down GEMM reads it (e4m3, ue8m0 [position][I/32]); d: each pick's
+   output bf16 [position][H]; hsh / dsh: the shared expert's h [T][I] and output [T][H]. */
+typedef struct dsgx_dsk_prefill_view {
+  const int *rpos, *re, *off, *perm;
+  const uint16_t *h, *hsh, *d, *dsh;
+  const uint8_t *hq, *hs;
+} dsgx_dsk_prefill_view;
+DSGX_API int dsgx_dsk_prefill_view_get(const dsgx_dsk_weights* W, void* ws, int T, dsgx_dsk_prefill_view* out);
+
 /* The residual add after the expert step and the next layer's RMSNorm, the local half of the reference's
    comm::glm::allreduce_add_norm / allreduce2_add_norm (engine/comm/glmcoll.h:34-62; the norm: engine/attn/prep.cu:12-66),
    M rows of H (a multiple of 2048, up to 16384):
@@ -298,6 +325,10 @@ DSGX_API int dsgx_act_quant(const uint16_t* x, int T, int K, uint8_t* q, float* 
    load them (pins the layouts in a test). form 0: v_mfma_f32_32x32x64_f8f6f4 over A [32][64], B [32][64];
    form 1: v_mfma_f32_16x16x128_f8f6f4 over A [16][128], B [16][128] (four registers a lane). */
 DSGX_API int dsgx_probe_mfma_fp8(const void* A, const void* B, float* raw, int form, void* stream);
+/* Probe: one v_mfma_scale_f32_16x16x128_f8f6f4. A [16][128 k]: e2m1 pairs (a_fp4 = 1: 64 bytes a row, the low nibble the even
+   k) or e4m3 codes; B [16][128] e4m3; SA, SB [16][4]: the ue8m0 byte of each row's four groups of 32 k. out f32 [16][16]:
+   out[i][j] = sum over k of A[i][k] 2^(SA[i][k/32] - 127) B[j][k] 2^(SB[j][k/32] - 127), as the matrix unit adds it. */
+DSGX_API int dsgx_probe_mfma_scaled(const void* A, const void* SA, const void* B, const void* SB, int a_fp4, float* out, void* stream);
 
 /* ---- misc ---------------------------------------------------------------------------------------------------- */
 DSGX_API const char* dsgx_last_error(void);

@@ -11,8 +11,11 @@
 //    values here, set once with dsk::set_shape (default: the whole layer on one GPU, hidden 5120, intermediate 2304,
 //    256 routed experts, top-6); moe_workspace_bytes() and moe() read them.
 //  - The 1-bit scale code (ScaleCode, dsk.h:181-198) is accepted and must be empty: scales are read as stored.
-//  - moe_prefill on MXFP4 layers runs the chunk through the decode operator sixteen rows at a time: the bits the reference
-//    promises ("the same result as moe()", dsk.h:284-286), not yet a grouped GEMM.
+//  - moe_prefill is grouped GEMMs on the block-scaled matrix instruction (dsgx_dsk_moe_prefill). The reference promises
+//    "the same result as moe()" (dsk.h:284-286) because its two paths share one MMA; here the chunk's dot products are
+//    summed by the block-scaled MFMA and moe()'s by the bf16 MFMA, so a row's y agrees between the two to the tolerance both
+//    are tested at (relative L2 ~1e-3), not bit for bit. moe_prefill_rows() is moe() over the chunk sixteen rows at a
+//    time for a caller that needs moe()'s bits.
 // The FP8 e4m3 / 128 x 128 block-scaled configuration (bf16 rows, a dsgx_layer_w) is served by the overloads at the end.
 #pragma once
 #include <cstddef>
@@ -110,20 +113,31 @@ inline void moe_routed(const uint8_t* xq, const uint8_t* xs, int M, const float*
   DSGX_DIE_ON(dsgx_dsk_moe_stacked(&c, xq, xs, M, nullptr, nullptr, ws, y, st, &d, idx_out, wts_out));
 }
 
-// dsk.h:284-295. The chunk goes through moe() sixteen rows at a time: ws needs moe()'s workspace only.
+// dsk.h:268-295: picks bucketed by expert, grouped GEMMs, each pick's output rounded to bf16, then per row summed in
+// expert-id order in fp32, shared expert last. ws: moe_prefill_workspace_bytes(M, E) bytes, no initialisation needed.
 struct MoePCfg {
-  int phases = 31;
-  void* side = nullptr;   // accepted, unused
+  int phases = 31;        // 1 bucketing, 2 shared expert, 4 routed up, 8 routed down, 16 combine
+  void* side = nullptr;   // accepted, unused: the shared expert runs on st
   int col0 = 0, cols = 0; // must be 0: all columns
 };
 inline size_t moe_prefill_workspace_bytes(int M, int E) {
-  (void)M, (void)E;
-  return moe_workspace_bytes();
+  const Shape& s = shape();
+  const size_t a = dsgx_dsk_prefill_ws_bytes(s.dim, s.inter, E, s.topk, M), b = moe_workspace_bytes();
+  return a > b ? a : b;  // (so that moe_prefill_rows can use the same buffer)
 }
 inline void moe_prefill(const uint8_t* xq, const uint8_t* xs, int M, const int* idx, const float* wts, int E, const MoeWeights& w, void* ws,
                         float* y, void* st, MoePCfg cfg = MoePCfg{}) {
   if (E != shape().experts) die("dsk::moe_prefill: E %d for a layer of %d experts (dsk::set_shape)", E, shape().experts);
-  if (cfg.phases != 31 || cfg.col0 || cfg.cols) die("dsk::moe_prefill: phases %d, columns [%d, +%d): the whole step only", cfg.phases, cfg.col0, cfg.cols);
+  if (cfg.col0 || cfg.cols) die("dsk::moe_prefill: columns [%d, +%d): all columns only", cfg.col0, cfg.cols);
+  const dsgx_dsk_weights c = detail::c_weights(w, "dsk::moe_prefill");
+  dsgx_dsk_prefill_cfg p;
+  dsgx_dsk_prefill_cfg_default(&p);
+  p.phases = cfg.phases;
+  DSGX_DIE_ON(dsgx_dsk_moe_prefill(&c, xq, xs, M, idx, wts, ws, y, st, &p));
+}
+// moe() over a chunk, sixteen rows at a time: moe()'s bits for every row. ws: moe_workspace_bytes(), ZEROED once.
+inline void moe_prefill_rows(const uint8_t* xq, const uint8_t* xs, int M, const int* idx, const float* wts, const MoeWeights& w, void* ws,
+                             float* y, void* st) {
   const Shape& s = shape();
   for (int m0 = 0; m0 < M; m0 += kMaxRows) {
     const int m = M - m0 < kMaxRows ? M - m0 : kMaxRows;

@@ -1,6 +1,6 @@
 // Test program: drives include/dsk/dsk.h on the GPU the way the reference's runner calls its DeepSeek MoE operators
 // (ds41f-4xgx10-switchless/engine/kernels/dsk.h:171-241, 284-295): tile_fp4 / tile_fp8 at load time, experts stacked by id
-// in MoeWeights, then router_topk -> moe, moe_routed with idx_out / wts_out, and moe_prefill over the same rows. Inputs are
+// in MoeWeights, then router_topk -> moe, moe_routed with idx_out / wts_out, moe_prefill (the grouped GEMMs) and moe_prefill_rows (moe() sixteen rows at a time) over the same rows. Inputs are
 // raw files written by tests/test_gpu_mirror.py; outputs go back as raw files and the test compares them bit for bit with
 // the ctypes binding of the C ABI on a pooled layer of the same weights.
 //   mirror_run_dsk <dir> <H> <I> <E> <M> <route scale> <shared 0|1>
@@ -103,6 +103,8 @@ int main(int argc, char** argv) {
   dsk::moe_routed(xq, xs, M, logits, bias, E, scale, w, ws, y2, dsk::MoeCfg{}, st, idx2, wts2);
   void* pws = dalloc<uint8_t>(dsk::moe_prefill_workspace_bytes(M, E), 0);
   dsk::moe_prefill(xq, xs, M, idx, wts, E, w, pws, y3, st);
+  float* y4 = dalloc<float>((size_t)M * H * 4, 0xFF);
+  dsk::moe_prefill_rows(xq, xs, M, idx, wts, w, ws, y4, st);
   HIPOK(hipStreamSynchronize(st));
   dump(dir + "o_idx.bin", idx, (size_t)M * dsk::kTopK * 4);
   dump(dir + "o_w.bin", wts, (size_t)M * dsk::kTopK * 4);
@@ -111,6 +113,7 @@ int main(int argc, char** argv) {
   dump(dir + "o_y.bin", y, (size_t)M * H * 4);
   dump(dir + "o_y2.bin", y2, (size_t)M * H * 4);
   dump(dir + "o_y3.bin", y3, (size_t)M * H * 4);
+  dump(dir + "o_y4.bin", y4, (size_t)M * H * 4);
   std::printf("CHECK mirror_run_dsk ok  ws %zu bytes\n", dsk::moe_workspace_bytes());
   return 0;
 }

@@ -78,9 +78,10 @@ def test_cpp_mirrors_give_the_c_abi_bits(fmt, shared, scale, up):
 @pytest.mark.parametrize("H,I,E,M,shared", [(1024, 512, 16, 3, True), (2048, 768, 32, 12, True), (1024, 256, 8, 16, False)])
 def test_dsk_mirror_gives_the_c_abi_bits(H, I, E, M, shared):
     """include/dsk/dsk.h with the reference's own argument lists (tests/mirror_run_dsk.cpp): experts stacked by id after
-    tile_fp4 / tile_fp8, router_topk -> moe, moe_routed with idx_out / wts_out, moe_prefill; against dsgx_route and dsgx_dsk_moe
-    on a pooled layer of the same weights (whose parity with the oracle tests/test_gpu_dsk.py holds), bit for bit. 12 and 16 rows
-    take two passes of the kernels."""
+    tile_fp4 / tile_fp8, router_topk -> moe, moe_routed with idx_out / wts_out, moe_prefill_rows; against dsgx_route and
+    dsgx_dsk_moe on a pooled layer of the same weights (whose parity with the oracle tests/test_gpu_dsk.py holds), bit for bit;
+    moe_prefill against dsgx_dsk_moe_prefill on the same stacked tensors (parity: tests/test_gpu_dsk_prefill.py), bit for bit.
+    12 and 16 rows take two passes of the decode kernels."""
     from tests.test_gpu_dsk import _layer
     exe = os.path.join(ROOT, "tests", "mirror_run_dsk")
     assert os.path.exists(exe), "tests/mirror_run_dsk is not built (python -m dsgx10_amd.build)"
@@ -99,10 +100,16 @@ def test_dsk_mirror_gives_the_c_abi_bits(H, I, E, M, shared):
             if shared:
                 put("sh_w" + n, hl.shared_fp8[j][0]), put("sh_s" + n, hl.shared_fp8[j][1])
         put("xq", xq), put("xs", xs), put("logits", logits), put("bias", bias)
+        stacks = {}
+        for j, n in enumerate(("1", "3", "2")):
+            stacks["w" + n] = gpu.dev(np.stack([hl.experts[int(hl.emap[e])][j][0] for e in range(E)]))
+            stacks["s" + n] = gpu.dev(np.stack([hl.experts[int(hl.emap[e])][j][1] for e in range(E)]))
+            if shared:
+                stacks["sh_w" + n], stacks["sh_s" + n] = gpu.dev(hl.shared_fp8[j][0]), gpu.dev(hl.shared_fp8[j][1])
         r = subprocess.run([exe, d, str(H), str(I), str(E), str(M), repr(scale), str(int(shared))], capture_output=True, text=True, timeout=120)
         assert r.returncode == 0 and "CHECK mirror_run_dsk ok" in r.stdout, r.stdout + r.stderr
         got = {n: np.fromfile(os.path.join(d, "o_%s.bin" % n), dt) for n, dt in
-               (("idx", np.int32), ("w", np.uint32), ("idx2", np.int32), ("w2", np.uint32), ("y", np.uint32), ("y2", np.uint32), ("y3", np.uint32))}
+               (("idx", np.int32), ("w", np.uint32), ("idx2", np.int32), ("w2", np.uint32), ("y", np.uint32), ("y2", np.uint32), ("y3", np.uint32), ("y4", np.uint32))}
     idx, w = orc.route(logits, bias, topk, scale, score_fn=1)
     for k in ("idx", "idx2"):
         assert np.array_equal(got[k], idx.reshape(-1)), k
@@ -113,5 +120,13 @@ def test_dsk_mirror_gives_the_c_abi_bits(H, I, E, M, shared):
     lib.dsk_moe(dl.w, gpu.dev(xq), gpu.dev(xs), gpu.dev(idx), gpu.dev(w), M, ws, y, ys)
     want = gpu.host(y, np.uint32, (-1,))
     assert np.isfinite(want.view(np.float32)).all()
-    for k in ("y", "y2", "y3"):
+    for k in ("y", "y2", "y4"):
         assert np.array_equal(got[k], want), (k, int((got[k] != want).sum()))
+    ptr = lambda k: stacks[k].data_ptr() if k in stacks else None
+    dw = abi.DskWeights(*[ptr(k) for k in ("w1", "s1", "w3", "s3", "w2", "s2", "sh_w1", "sh_s1", "sh_w3", "sh_s3", "sh_w2", "sh_s2")], H, I, E, topk)
+    pws, yp = gpu.empty(lib.dsk_prefill_ws_bytes(H, I, E, topk, M), 0xEE), gpu.empty(M * H * 4, 0xFF)
+    lib.dsk_moe_prefill(dw, gpu.dev(xq), gpu.dev(xs), gpu.dev(idx), gpu.dev(w), M, pws, yp)
+    wantp = gpu.host(yp, np.uint32, (-1,))
+    assert np.array_equal(got["y3"], wantp), int((got["y3"] != wantp).sum())
+    rel = np.linalg.norm(wantp.view(np.float32) - want.view(np.float32)) / np.linalg.norm(want.view(np.float32))
+    assert rel <= 5e-3, rel  # the two operators agree to their tolerance
