@@ -847,6 +847,16 @@ int dsgx_dsk_moe_prefill(const dsgx_dsk_weights* Wt, const uint8_t* xq, const ui
   void (*k_dn)(pfmx::Args) = pfmx::k_gemm_mixed<false, F4>;
   void (*k_sup)(pfmx::Args) = pfmx::k_gemm<true, F8>;
   void (*k_sdn)(pfmx::Args) = pfmx::k_gemm<false, F8>;
+#ifdef DSGX_PF_DIAG
+  {  // diagnostic build: DSGX_PF_DIAG=<bits> switches parts of the kernels off (wrong results; for timing only)
+    const char* dv = std::getenv("DSGX_PF_DIAG");
+    switch (dv ? std::atoi(dv) : 0) {
+#define DSGX_DIAG_CASE(n) case n: k_up = pfmx::k_gemm_mixed<true, F4, n>, k_dn = pfmx::k_gemm_mixed<false, F4, n>, k_sup = pfmx::k_gemm<true, F8, n>, k_sdn = pfmx::k_gemm<false, F8, n>; break;
+      DSGX_DIAG_CASE(1) DSGX_DIAG_CASE(4) DSGX_DIAG_CASE(8) DSGX_DIAG_CASE(32) DSGX_DIAG_CASE(64) DSGX_DIAG_CASE(128) DSGX_DIAG_CASE(256) DSGX_DIAG_CASE(384) DSGX_DIAG_CASE(512) DSGX_DIAG_CASE(1024) DSGX_DIAG_CASE(513) DSGX_DIAG_CASE(1025) DSGX_DIAG_CASE(1152) DSGX_DIAG_CASE(1280) DSGX_DIAG_CASE(1408) DSGX_DIAG_CASE(1032) DSGX_DIAG_CASE(1088) DSGX_DIAG_CASE(1056)
+#undef DSGX_DIAG_CASE
+    }
+  }
+#endif
   for (const void* k : {(const void*)k_up, (const void*)k_dn})
     if (int rc = allow_dynamic_lds(k, kLdsMix)) return rc;
   for (const void* k : {(const void*)k_sup, (const void*)k_sdn})
@@ -879,18 +889,21 @@ int dsgx_dsk_moe_prefill(const dsgx_dsk_weights* Wt, const uint8_t* xq, const ui
     DSGX_HIP(hipGetLastError());
   }
   g.tile_e = I32(o.mix_e), g.tile_m0 = I32(o.mix_m0), g.ntiles = I32(o.nmix), g.off = I32(o.off), g.nrows = P;
+  auto launch = [&](bool up) {
+    hipLaunchKernelGGL(up ? k_up : k_dn, dim3(pf8::grid_of(o.max_big + E, up ? NSU : NSD)), dim3(pf8::kThreads), kLdsMix, st, g);
+  };
   if (cfg.phases & 4) {
     g.aq = xq, g.as = xs, g.gather = I32(o.perm), g.posw = F32(o.posw);
     g.wa = Wt->w1, g.sa = Wt->s1, g.wb = Wt->w3, g.sb = Wt->s3, g.wstride = (size_t)I * H / 2, g.sstride = (size_t)I * H / 32;
     g.h = U16(o.h), g.hq = W + o.hq, g.hs = W + o.hs, g.d = nullptr;
-    hipLaunchKernelGGL(k_up, dim3(pf8::grid_of(o.max_big + E, NSU)), dim3(pf8::kThreads), kLdsMix, st, g);
+    launch(true);
     DSGX_HIP(hipGetLastError());
   }
   if (cfg.phases & 8) {
     g.aq = W + o.hq, g.as = W + o.hs, g.gather = nullptr, g.posw = nullptr;
     g.wa = Wt->w2, g.sa = Wt->s2, g.wb = g.sb = nullptr, g.wstride = (size_t)I * H / 2, g.sstride = (size_t)I * H / 32;
     g.h = nullptr, g.hq = g.hs = nullptr, g.d = U16(o.d);
-    hipLaunchKernelGGL(k_dn, dim3(pf8::grid_of(o.max_big + E, NSD)), dim3(pf8::kThreads), kLdsMix, st, g);
+    launch(false);
     DSGX_HIP(hipGetLastError());
   }
   if (cfg.phases & 16) {

@@ -64,20 +64,28 @@ struct Args {
 };
 
 __device__ __forceinline__ int sw4(int r) { return (r >> 2) & 3; }
+// 128-byte rows (activations, e4m3 weights) lie in LDS in pf_gemm_fp8.cuh's layout, whose fragment reads (a lane's two
+// neighbouring slots 2 part, 2 part + 1, swizzled by row) run without bank conflicts; what differs is WHICH 16 bytes of the
+// row a slot holds: the block-scaled instruction wants bytes 16 part ... and 64 + 16 part ... in a lane, so logical piece
+// x holds the row's piece x / 2 + 4 (x % 2). (Reading pieces part and 4 + part of rows stored in natural order instead
+// costs every second LDS cycle to bank conflicts - measured.)
+__device__ __forceinline__ int pc8(int x) { return (x >> 1) + 4 * (x & 1); }
 
 template <int CBSZ>
 __device__ __forceinline__ v4f_t mfma_mx(v8i_t a, v8i_t b, v4f_t c, int sa, int sb) {
   return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, c, CBSZ, 0, 0, sa, 0, sb);
 }
 
-template <bool UP, int WP, int WF>
+// DIAG (diagnostic builds only; results are then wrong): 1 no loads after the first stages, 4 no workgroup barrier in the
+// loop, 8 no MFMAs, 16 no fragment reads after the first turn, 32 two blocks only, 64 no epilogue
+template <bool UP, int WP, int WF, int DIAG = 0>
 __device__ __forceinline__ void gemm_tile(const Args& g, uint8_t* smem, int e, int m0, int mend, int ns) {
   using S = Shape<WP, WF>;
   constexpr bool F4 = S::F4;
   constexpr int CBSZ = F4 ? 4 : 0;
   const int K = UP ? g.H : g.I, KB = K / 128, G = K / 32;
   if (mend > m0 + S::kPos) mend = m0 + S::kPos;
-  const size_t eo = e < 0 ? 0 : (size_t)e;
+  const size_t eo = (e < 0 || (DIAG & 128)) ? 0 : (size_t)e;  // (diagnostic 128: every tile reads expert 0's weights)
   const uint8_t *wa = g.wa + eo * g.wstride, *sa = g.sa + eo * g.sstride;
   const uint8_t *wb = UP ? g.wb + eo * g.wstride : wa, *sb = UP ? g.sb + eo * g.sstride : sa;
   const int tid = threadIdx.x, lane = tid & 63, wave = uni(tid >> 6), r16 = lane & 15, part = lane >> 4;
@@ -111,7 +119,7 @@ __device__ __forceinline__ void gemm_tile(const Args& g, uint8_t* smem, int e, i
 #pragma unroll
       for (int hh = 0; hh < 2; ++hh) {
         const int r = 8 * hh + (lane >> 3);
-        pw[t][hh] = wbase + (size_t)(row + r) * K + 16 * ((lane & 7) ^ swz(r));
+        pw[t][hh] = wbase + (size_t)(row + r) * K + 16 * pc8((lane & 7) ^ swz(r));
       }
     }
     if (((lane >> 4) & 1) == t) pws = sbase + (size_t)(F4 ? row + r16 : (row + r16) / 32) * G;
@@ -125,7 +133,7 @@ __device__ __forceinline__ void gemm_tile(const Args& g, uint8_t* smem, int e, i
       const int r = 8 * hh + lr;
       int pos = m0 + 16 * (WP * wave + t) + r;
       if (pos >= mend) pos = mend - 1;
-      px[t][hh] = g.aq + (size_t)(g.gather ? g.gather[pos] : pos) * K + 16 * (lq ^ swz(r));
+      px[t][hh] = g.aq + (size_t)((DIAG & 256) ? pos & 255 : g.gather ? g.gather[pos] : pos) * K + 16 * pc8(lq ^ swz(r));  // (diagnostic 256: 256 hot rows)
     }
   const uint8_t* pxs;  // lanes 0 .. 16 WP - 1: the scale word of position 16 WP wave + lane
   {
@@ -134,25 +142,32 @@ __device__ __forceinline__ void gemm_tile(const Args& g, uint8_t* smem, int e, i
     pxs = g.as + (size_t)(g.gather ? g.gather[pos] : pos) * G;
   }
   const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)smem;
-  auto issue = [&](int kb) {
+  // load number i (0 .. kLoads - 1) of block kb: the two scale words, the activations (L2 hits mostly), the weights last: a
+  // wave's loads return in issue order, so a load that waits for HBM holds back every later one of its wave and the
+  // cache's miss slots with them (weights first: 7% slower, measured). A turn issues them one at a time between its MFMAs (issue_some), so that the
+  // texture unit works through a block's 50 KB while the matrix unit runs instead of in front of it: issued together after
+  // the barrier they cost every wave the time the unit takes to accept them all (measured: a third of a turn).
+  constexpr int kLW = F4 ? 2 : 4;
+  auto issue_one = [&](int kb, int i) {
     const int kc = kb < KB ? kb : KB - 1;
     const uint32_t st = lds0 + (uint32_t)(kb % S::kStages) * S::kStageBytes;
     const uint32_t wbase = st + (uint32_t)wave * (2 * 16 * S::kRowB), xbase = st + S::kStageW + (uint32_t)wave * (2048 * WP);
-#pragma unroll
-    for (int t = 0; t < 2; ++t) {
-      if (F4) {
-        dma16(pw[t][0] + (size_t)kc * 64, uni(wbase + t * 1024));
-      } else {
-#pragma unroll
-        for (int hh = 0; hh < 2; ++hh) dma16(pw[t][hh] + (size_t)kc * 128, uni(wbase + t * 2048 + hh * 1024));
-      }
+    if (i == 0) {
+      if (lane < 16 * WP) dma4(reinterpret_cast<const float*>(pxs + 4 * kc), uni(st + S::kStageW + S::kStageX + S::kStageWS + (uint32_t)wave * (64 * WP)));
+    } else if (i == 1) {
+      if (lane < 32) dma4(reinterpret_cast<const float*>(pws + 4 * kc), uni(st + S::kStageW + S::kStageX + (uint32_t)wave * 128));
+    } else if (i < 2 + 2 * WP) {
+      const int q = i - 2;
+      dma16(px[q >> 1][q & 1] + (size_t)kc * 128, uni(xbase + (q >> 1) * 2048 + (q & 1) * 1024));
+    } else {
+      const int q = i - 2 - 2 * WP;
+      if (F4) dma16(pw[q][0] + (size_t)kc * 64, uni(wbase + q * 1024));
+      else dma16(pw[q >> 1][q & 1] + (size_t)kc * 128, uni(wbase + (q >> 1) * 2048 + (q & 1) * 1024));
     }
+  };
+  auto issue = [&](int kb) {
 #pragma unroll
-    for (int t = 0; t < WP; ++t)
-#pragma unroll
-      for (int hh = 0; hh < 2; ++hh) dma16(px[t][hh] + (size_t)kc * 128, uni(xbase + t * 2048 + hh * 1024));
-    if (lane < 32) dma4(reinterpret_cast<const float*>(pws + 4 * kc), uni(st + S::kStageW + S::kStageX + (uint32_t)wave * 128));
-    if (lane < 16 * WP) dma4(reinterpret_cast<const float*>(pxs + 4 * kc), uni(st + S::kStageW + S::kStageX + S::kStageWS + (uint32_t)wave * (64 * WP)));
+    for (int i = 0; i < S::kLoads; ++i) issue_one(kb, i);
   };
 #pragma unroll
   for (int s = 0; s + 1 < S::kStages; ++s) issue(s);
@@ -160,10 +175,10 @@ __device__ __forceinline__ void gemm_tile(const Args& g, uint8_t* smem, int e, i
   // fragment reads. The instruction numbers an 8-bit operand's k as 64 h + 16 part + i (h: the lane's first or second four
   // registers, i: the byte) and a 4-bit operand's as 32 part + i, and takes the scale of k block g = k / 32 from the lanes
   // of part g (measured with one-hot operands): so activations and e4m3 weights give lane (row r16, part) the 16-byte
-  // pieces part and 4 + part of its row's 128 bytes, e2m1 weights piece part of the row's 64, and every operand's scale
-  // byte `part` of the row's four goes to the lanes of that part.
-  const int rd0 = (r16 >> 3) * 1024 + (r16 & 7) * 128 + (part ^ swz(r16)) * 16;
-  const int rd1 = (r16 >> 3) * 1024 + (r16 & 7) * 128 + ((4 + part) ^ swz(r16)) * 16;
+  // pieces part and 4 + part of its row's 128 bytes (LDS slots 2 part and 2 part + 1, see pc8), e2m1 weights piece part of
+  // the row's 64, and every operand's scale byte `part` of the row's four goes to the lanes of that part.
+  const int rd0 = (r16 >> 3) * 1024 + (r16 & 7) * 128 + ((2 * part) ^ swz(r16)) * 16;
+  const int rd1 = (r16 >> 3) * 1024 + (r16 & 7) * 128 + ((2 * part + 1) ^ swz(r16)) * 16;
   const int rd4 = r16 * 64 + (part ^ sw4(r16)) * 16;
   auto frag8 = [&](const uint8_t* t) {
     const u32x4_t lo = *reinterpret_cast<const u32x4_t*>(t + rd0), hi = *reinterpret_cast<const u32x4_t*>(t + rd1);
@@ -173,7 +188,8 @@ __device__ __forceinline__ void gemm_tile(const Args& g, uint8_t* smem, int e, i
     const u32x4_t lo = *reinterpret_cast<const u32x4_t*>(t + rd4);
     return v8i_t{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, 0, 0, 0, 0};
   };
-  const int rds = r16 * 4 + part;  // the lane's scale byte within a 16-row (16-position) tile's 64 bytes
+  const int rds = r16 * 4;         // the lane's row's scale word within a 16-row (16-position) tile's 64 bytes; its byte: `part`
+  const int rsh = 8 * part;
 
   v4f_t acc[S::RA][8];
 #pragma unroll
@@ -183,12 +199,19 @@ __device__ __forceinline__ void gemm_tile(const Args& g, uint8_t* smem, int e, i
 
   auto run = [&](auto nj_c) {
     constexpr int NJ = decltype(nj_c)::value;
-    for (int kb = 0; kb < KB; ++kb) {
+    for (int kb = 0; kb < ((DIAG & 32) ? 2 : KB); ++kb) {
       wait_loads<(S::kStages - 2) * S::kLoads>();
-      __syncthreads();
-      issue(kb + S::kStages - 1);
+      if (!(DIAG & 4)) __syncthreads();
+      if (!(DIAG & 1) && NJ == 0) issue(kb + S::kStages - 1);
       if (NJ == 0) continue;
-      const uint8_t* st = smem + (size_t)(kb % S::kStages) * S::kStageBytes;
+      // loads i with i * NJ / kLoads == j go out after the fragment reads of 16-position tile j
+      auto issue_some = [&](int j) {
+        if (DIAG & 1) return;
+#pragma unroll
+        for (int i = 0; i < S::kLoads; ++i)
+          if (i * (NJ > 0 ? NJ : 1) / S::kLoads == j) issue_one(kb + S::kStages - 1, i);
+      };
+      const uint8_t* st = smem + (size_t)(((DIAG & 16) ? 0 : kb) % S::kStages) * S::kStageBytes;
       const uint8_t* W = st + S::RA * rg * (16 * S::kRowB);
       const uint8_t* X = st + S::kStageW + pg * 2048;
       const uint8_t* WS = st + S::kStageW + S::kStageX + S::RA * rg * 64 + rds;
@@ -198,14 +221,18 @@ __device__ __forceinline__ void gemm_tile(const Args& g, uint8_t* smem, int e, i
 #pragma unroll
       for (int t = 0; t < S::RA; ++t) {
         fa[t] = F4 ? frag4(W + t * 1024) : frag8(W + t * 2048);
-        fs[t] = WS[t * 64];
+        fs[t] = (*reinterpret_cast<const uint32_t*>(WS + t * 64) >> rsh) & 0xFFu;
       }
 #pragma unroll
       for (int j = 0; j < NJ; ++j) {
         const v8i_t fb = frag8(X + j * (2048 * WP));
-        const int xsb = XS[j * (64 * WP)];
+        const int xsb = (*reinterpret_cast<const uint32_t*>(XS + j * (64 * WP)) >> rsh) & 0xFFu;
+        issue_some(j);
 #pragma unroll
-        for (int t = 0; t < S::RA; ++t) acc[t][j] = mfma_mx<CBSZ>(fa[t], fb, acc[t][j], fs[t], xsb);
+        for (int t = 0; t < S::RA; ++t) {
+          if (DIAG & 8) acc[t][j][0] += __builtin_bit_cast(float, fa[t][0] ^ fb[1] ^ fs[t] ^ xsb), acc[t][j][2] += __builtin_bit_cast(float, fa[t][3] ^ fb[6]);
+          else acc[t][j] = mfma_mx<CBSZ>(fa[t], fb, acc[t][j], fs[t], xsb);
+        }
       }
     }
   };
@@ -222,6 +249,15 @@ __device__ __forceinline__ void gemm_tile(const Args& g, uint8_t* smem, int e, i
   }
   wait_loads<0>();
   __syncthreads();
+  if (DIAG & 64) {
+    float sum = 0.f;
+#pragma unroll
+    for (int t = 0; t < S::RA; ++t)
+#pragma unroll
+      for (int j = 0; j < 8; ++j) sum += acc[t][j][0] + acc[t][j][1] + acc[t][j][2] + acc[t][j][3];
+    if (sum == 12345.678f) reinterpret_cast<float*>(UP ? (void*)g.h : (void*)g.d)[tid] = sum;
+    return;
+  }
 
   // register q of lane l is weight row 4 (l / 16) + q of the 16-row tile, position l % 16 of the 16 positions
   if (UP) {
@@ -307,7 +343,7 @@ __device__ __forceinline__ void gemm_tile(const Args& g, uint8_t* smem, int e, i
 }
 
 // The shared expert (tile_e null: tiles of 256 rows over [0, nrows)).
-template <bool UP, int WF>
+template <bool UP, int WF, int DIAG = 0>
 __global__ void __launch_bounds__(kThreads) k_gemm(Args g) {
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
   const int NS = UP ? g.I / (kWgRows / 2) : g.H / kWgRows;
@@ -316,10 +352,10 @@ __global__ void __launch_bounds__(kThreads) k_gemm(Args g) {
   if (ns >= NS) return;
   const int m0 = tile * Shape<2, WF>::kPos, mend = g.nrows;
   if (m0 >= mend) return;
-  gemm_tile<UP, 2, WF>(g, smem, -1, m0, mend, ns);
+  gemm_tile<UP, 2, WF, DIAG>(g, smem, -1, m0, mend, ns);
 }
 // The routed experts' list of both tile shapes (bit 30 of tile_e: a 256-position tile), an expert's tiles next to each other.
-template <bool UP, int WF>
+template <bool UP, int WF, int DIAG = 0>
 __global__ void __launch_bounds__(kThreads) k_gemm_mixed(Args g) {
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
   const int NS = UP ? g.I / (kWgRows / 2) : g.H / kWgRows;
@@ -328,8 +364,10 @@ __global__ void __launch_bounds__(kThreads) k_gemm_mixed(Args g) {
   if (ns >= NS || tile >= *g.ntiles) return;
   const int te = g.tile_e[tile], e = te & 0xFFFF;
   const int m0 = g.off[e] + g.tile_m0[tile], mend = g.off[e + 1];
-  if (te >> 30) gemm_tile<UP, 2, WF>(g, smem, e, m0, mend, ns);
-  else gemm_tile<UP, 1, WF>(g, smem, e, m0, mend, ns);
+  if ((DIAG & 512) && !(te >> 30)) return;  // (diagnostic: the 256-position tiles only / the remainders only)
+  if ((DIAG & 1024) && (te >> 30)) return;
+  if (te >> 30) gemm_tile<UP, 2, WF, DIAG>(g, smem, e, m0, mend, ns);
+  else gemm_tile<UP, 1, WF, DIAG>(g, smem, e, m0, mend, ns);
 }
 
 }  // namespace pfmx
