@@ -97,14 +97,18 @@ def dsk_prefill_extra(T=8192, check=True):
          d["ms_with_shared"], {k: round(v, 3) for k, v in d["phases_ms"].items()}))
     if check:
         d["gpu_vs_oracle"] = dsk_prefill_check_rows(pb)
-        log("  %s: rows %s against the oracle's chain: max-abs %.2e, rel-L2 %.2e" % (pb.name, d["gpu_vs_oracle"]["rows"], d["gpu_vs_oracle"]["max_abs_err"], d["gpu_vs_oracle"]["rel_l2"]))
+        log("  %s: rows %s against the oracle's chain (the matrix unit's sums): max-abs %.2e, rel-L2 %.2e; against the oracle with sequential f32 sums: rel-L2 %.2e" %
+            (pb.name, d["gpu_vs_oracle"]["rows"], d["gpu_vs_oracle"]["max_abs_err"], d["gpu_vs_oracle"]["rel_l2"], d["gpu_vs_oracle"]["vs_sequential_f32_sums_rel_l2"]))
     del pb
     return d
 
 
 def dsk_prefill_check_rows(pb, rows=(0, 4097, 8191)):
     """Part of the CPU leg: a few rows of the chunk just timed against the C++ oracle's chain (each picked expert and the shared
-    one: gate/up, clamped SwiGLU times the routing weight, h quantised per 32, w2, rounded to bf16; summed in expert-id order)"""
+    one: gate/up, clamped SwiGLU times the routing weight, h quantised per 32, w2, rounded to bf16; summed in expert-id order),
+    with every dot product added as the block-scaled MFMA adds it (the rule pinned by tests/golden/mfma_scaled_k128.npz), and,
+    beside it, with sequential f32 sums (two correct evaluations of the contract: their distance is what h's 3-bit-mantissa
+    quantisation makes of sums that differ in the last bits)"""
     import torch
     from tests import orc   # the oracle: test infrastructure, used here as the checker only
     pb.run(31)
@@ -112,20 +116,31 @@ def dsk_prefill_check_rows(pb, rows=(0, 4097, 8191)):
     rows = [t for t in rows if t < pb.T] or [0]
     host = lambda t: t.cpu().numpy()
     sh = tuple(orc.fp8e_dequant(host(pb.t["sh_w" + n]), host(pb.t["sh_s" + n])) for n in ("1", "3", "2"))
-    worst = dict(rows=rows, max_abs_err=0.0, rel_l2=0.0, oracle="C++ oracle (DeepSeek's expert arithmetic, f32 sums)")
+    worst = dict(rows=rows, max_abs_err=0.0, rel_l2=0.0, vs_sequential_f32_sums_rel_l2=0.0, vs_sequential_f32_sums_max_abs=0.0,
+                 oracle="C++ oracle, DeepSeek's expert arithmetic with every dot product added as the block-scaled MFMA adds it")
     for t in rows:
-        xd = orc.dequant_act_ue8m0(host(pb.xq[t:t + 1]), host(pb.xs[t:t + 1]))
-        ref = np.zeros(pb.H, np.float32)
+        xq, xs = host(pb.xq[t:t + 1]), host(pb.xs[t:t + 1])
+        xd = orc.dequant_act_ue8m0(xq, xs)
+        ref, seq = np.zeros(pb.H, np.float32), np.zeros(pb.H, np.float32)
         idx, w = host(pb.idx[t]), host(pb.w[t])
         for e in sorted(int(v) for v in idx):
-            w1, w3, w2 = (orc.mxfp4_dequant(host(pb.t["w" + n][e]), host(pb.t["s" + n][e])) for n in ("1", "3", "2"))
-            up = orc.dsk_up(w1, w3, xd, np.array([w[list(idx).index(e)]], np.float32), want_range=False)
-            ref = ref + orc.bf16_to_f32(orc.dsk_down(w2, up["h32"])["outb"][0])
+            raw = [(host(pb.t["w" + n][e]), host(pb.t["s" + n][e])) for n in ("1", "3", "2")]
+            rw = np.array([w[list(idx).index(e)]], np.float32)
+            hm = orc.dsk_up_mx(raw[0][0], raw[0][1], raw[1][0], raw[1][1], 1, xq, xs, rw)
+            ref = ref + orc.bf16_to_f32(orc.dsk_down_mx(raw[2][0], raw[2][1], 1, hm)["outb"][0])
+            w1, w3, w2 = (orc.mxfp4_dequant(*r) for r in raw)
+            up = orc.dsk_up(w1, w3, xd, rw, want_range=False)
+            seq = seq + orc.bf16_to_f32(orc.dsk_down(w2, up["h32"])["outb"][0])
+        rawsh = [(host(pb.t["sh_w" + n]), host(pb.t["sh_s" + n])) for n in ("1", "3", "2")]
+        hm = orc.dsk_up_mx(rawsh[0][0], rawsh[0][1], rawsh[1][0], rawsh[1][1], 0, xq, xs, None)
+        ref = ref + orc.bf16_to_f32(orc.dsk_down_mx(rawsh[2][0], rawsh[2][1], 0, hm)["outb"][0])
         up = orc.dsk_up(sh[0], sh[1], xd, None, want_range=False)
-        ref = ref + orc.bf16_to_f32(orc.dsk_down(sh[2], up["h32"])["outb"][0])
+        seq = seq + orc.bf16_to_f32(orc.dsk_down(sh[2], up["h32"])["outb"][0])
         got = host(pb.y[t])
         worst["max_abs_err"] = max(worst["max_abs_err"], float(np.abs(got - ref).max()))
         worst["rel_l2"] = max(worst["rel_l2"], float(np.linalg.norm(got - ref) / max(np.linalg.norm(ref), 1e-30)))
+        worst["vs_sequential_f32_sums_max_abs"] = max(worst["vs_sequential_f32_sums_max_abs"], float(np.abs(got - seq).max()))
+        worst["vs_sequential_f32_sums_rel_l2"] = max(worst["vs_sequential_f32_sums_rel_l2"], float(np.linalg.norm(got - seq) / max(np.linalg.norm(seq), 1e-30)))
     return worst
 
 

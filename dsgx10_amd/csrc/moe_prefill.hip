@@ -578,7 +578,7 @@ __global__ void __launch_bounds__(256) k_pfmx_combine(const uint16_t* __restrict
 // hand them over: an 8-bit row's bytes 16 part ... and 64 + 16 part ..., a 4-bit row's bytes 16 part ..., scale byte `part`.
 template <int CBSZ>
 __global__ void __launch_bounds__(64) k_probe_mfma_scaled(const uint8_t* __restrict__ A, const uint8_t* __restrict__ SA, const uint8_t* __restrict__ B,
-                                                          const uint8_t* __restrict__ SB, float* __restrict__ out) {
+                                                          const uint8_t* __restrict__ SB, const float* __restrict__ C, float* __restrict__ out) {
   const int l = threadIdx.x, row = l % 16, part = l / 16;
   pf8::v8i_t a = {0, 0, 0, 0, 0, 0, 0, 0}, b;
   if (CBSZ == 4) {
@@ -592,7 +592,12 @@ __global__ void __launch_bounds__(64) k_probe_mfma_scaled(const uint8_t* __restr
     const uint4 lo = *reinterpret_cast<const uint4*>(B + row * 128 + part * 16), hi = *reinterpret_cast<const uint4*>(B + row * 128 + 64 + part * 16);
     b = pf8::v8i_t{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
   }
-  const pf8::v4f_t c = pfmx::mfma_mx<CBSZ>(a, b, pf8::v4f_t{0.f, 0.f, 0.f, 0.f}, SA[row * 4 + part], SB[row * 4 + part]);
+  pf8::v4f_t c = {0.f, 0.f, 0.f, 0.f};
+  if (C) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q) c[q] = C[(4 * part + q) * 16 + row];
+  }
+  c = pfmx::mfma_mx<CBSZ>(a, b, c, SA[row * 4 + part], SB[row * 4 + part]);
 #pragma unroll
   for (int q = 0; q < 4; ++q) out[(4 * part + q) * 16 + row] = c[q];
 }
@@ -784,11 +789,11 @@ int dsgx_prefill_view_get(const dsgx_layer_w* L, void* ws, int T, dsgx_prefill_v
   return DSGX_OK;
 }
 
-int dsgx_probe_mfma_scaled(const void* A, const void* SA, const void* B, const void* SB, int a_fp4, float* out, void* stream) {
+int dsgx_probe_mfma_scaled(const void* A, const void* SA, const void* B, const void* SB, int a_fp4, const float* C, float* out, void* stream) {
   if (!A || !SA || !B || !SB || !out) return fail(DSGX_EINVAL, "probe_mfma_scaled: null argument");
   const uint8_t *a = (const uint8_t*)A, *sa = (const uint8_t*)SA, *b = (const uint8_t*)B, *sb = (const uint8_t*)SB;
-  if (a_fp4) hipLaunchKernelGGL(k_probe_mfma_scaled<4>, dim3(1), dim3(64), 0, (hipStream_t)stream, a, sa, b, sb, out);
-  else hipLaunchKernelGGL(k_probe_mfma_scaled<0>, dim3(1), dim3(64), 0, (hipStream_t)stream, a, sa, b, sb, out);
+  if (a_fp4) hipLaunchKernelGGL(k_probe_mfma_scaled<4>, dim3(1), dim3(64), 0, (hipStream_t)stream, a, sa, b, sb, C, out);
+  else hipLaunchKernelGGL(k_probe_mfma_scaled<0>, dim3(1), dim3(64), 0, (hipStream_t)stream, a, sa, b, sb, C, out);
   DSGX_HIP(hipGetLastError());
   return DSGX_OK;
 }

@@ -327,8 +327,10 @@ DSGX_API int dsgx_act_quant(const uint16_t* x, int T, int K, uint8_t* q, float* 
 DSGX_API int dsgx_probe_mfma_fp8(const void* A, const void* B, float* raw, int form, void* stream);
 /* Probe: one v_mfma_scale_f32_16x16x128_f8f6f4. A [16][128 k]: e2m1 pairs (a_fp4 = 1: 64 bytes a row, the low nibble the even
    k) or e4m3 codes; B [16][128] e4m3; SA, SB [16][4]: the ue8m0 byte of each row's four groups of 32 k. out f32 [16][16]:
-   out[i][j] = sum over k of A[i][k] 2^(SA[i][k/32] - 127) B[j][k] 2^(SB[j][k/32] - 127), as the matrix unit adds it. */
-DSGX_API int dsgx_probe_mfma_scaled(const void* A, const void* SA, const void* B, const void* SB, int a_fp4, float* out, void* stream);
+   out[i][j] = C[i][j] (null: 0) + sum over k of A[i][k] 2^(SA[i][k/32] - 127) B[j][k] 2^(SB[j][k/32] - 127), as the matrix unit
+   adds it. */
+DSGX_API int dsgx_probe_mfma_scaled(const void* A, const void* SA, const void* B, const void* SB, int a_fp4, const float* C, float* out,
+                                    void* stream);
 
 /* ---- misc ---------------------------------------------------------------------------------------------------- */
 DSGX_API const char* dsgx_last_error(void);

@@ -355,6 +355,28 @@ def dsk_down(w2, hpre):
     return o
 
 
+def dsk_up_mx(w1, s1, w3, s3, a_fp4, xq, xs, rw=None, limit=10.0):
+    """DeepSeek's gate/up with every dot product added as the block-scaled MFMA adds it: weights as stored (e2m1 pairs [I][H/2]
+    with ue8m0 [I][H/32], or e4m3 [I][H] with ue8m0 [I/32][H/32]), rows e4m3 [M][H] + ue8m0 [M][H/32] -> h bf16 bits [M][I]"""
+    w1, s1, w3, s3, xq, xs = (np.ascontiguousarray(v, np.uint8) for v in (w1, s1, w3, s3, xq, xs))
+    M, H = xq.shape
+    I = w1.shape[0]
+    r = None if rw is None else np.ascontiguousarray(rw, np.float32)
+    h = np.empty((M, I), np.uint16)
+    lib().orc_dsk_up_mx(_p(w1), _p(s1), _p(w3), _p(s3), int(a_fp4), _p(xq), _p(xs), M, H, I, _p(r), C.c_float(limit), _p(h))
+    return h
+
+
+def dsk_down_mx(w2, s2, a_fp4, hpre):
+    """w2 as stored ([H][I/2] e2m1 or [H][I] e4m3), hpre bf16 bits [M][I] -> dict hq, hs (h as the GEMM reads it), outb (bf16 bits [M][H])"""
+    w2, s2, hpre = np.ascontiguousarray(w2, np.uint8), np.ascontiguousarray(s2, np.uint8), np.ascontiguousarray(hpre, np.uint16)
+    M, I = hpre.shape
+    H = w2.shape[0]
+    o = dict(hq=np.empty((M, I), np.uint8), hs=np.empty((M, I // 32), np.uint8), outb=np.empty((M, H), np.uint16))
+    lib().orc_dsk_down_mx(_p(w2), _p(s2), int(a_fp4), _p(hpre), M, H, I, _p(o["hq"]), _p(o["hs"]), _p(o["outb"]))
+    return o
+
+
 def mfma_fp8_k128(a, b):
     """the oracle's statement of gfx950's v_mfma_f32_16x16x128_f8f6f4 block sum: e4m3 codes a [R][128], b [S][128] in
     register order -> f32 [R][S]"""
@@ -364,6 +386,20 @@ def mfma_fp8_k128(a, b):
     for i in range(a.shape[0]):
         for j in range(b.shape[0]):
             out[i, j] = lib().orc_mfma_fp8_k128(C.c_void_p(a[i].ctypes.data), C.c_void_p(b[j].ctypes.data))
+    return out
+
+
+def mfma_scaled_k128(a, sa, a_fp4, b, sb, acc=None):
+    """the oracle's statement of gfx950's v_mfma_scale_f32_16x16x128_f8f6f4: a [R][64] e2m1 pairs (a_fp4) or [R][128] e4m3 codes,
+    b e4m3 [S][128], sa [R][4], sb [S][4] ue8m0 bytes, acc f32 [R][S] (None: zeros), all in k order as stored -> f32 [R][S]"""
+    a, b, sa, sb = (np.ascontiguousarray(v, np.uint8) for v in (a, b, sa, sb))
+    f = lib().orc_mfma_scaled_k128
+    f.restype = C.c_float
+    f.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_float]
+    out = np.empty((a.shape[0], b.shape[0]), np.float32)
+    for i in range(a.shape[0]):
+        for j in range(b.shape[0]):
+            out[i, j] = f(a[i].ctypes.data, sa[i].ctypes.data, int(a_fp4), b[j].ctypes.data, sb[j].ctypes.data, 0.0 if acc is None else float(acc[i, j]))
     return out
 
 

@@ -8,7 +8,10 @@ kernel's own inputs, then y):
   h's quantisation (codes and scale bytes) equal to the oracle's act_quant of the GPU's own h, bit for bit;
   each pick's w2 output (bf16) from the GPU's own h within 1e-4 sum|terms| + one bf16 step of the f64 sums;
   y equal, bit for bit, to the f32 fold of the GPU's own outputs in expert-id order with the shared expert last;
-  y against the oracle's chain at max-abs 2e-2 / rel-L2 3e-3, and against the decode operator on the same rows."""
+  y against the oracle's chain at max-abs 2e-2 / rel-L2 3e-3, and against the decode operator on the same rows;
+  and, bit for bit, against the oracle variant that adds every dot product as the matrix instruction does (orc_dsk_up_mx /
+  orc_dsk_down_mx over the rule of tests/golden/mfma_scaled_k128.npz): each pick's w2 output from the GPU's own h equal in
+  every bit, h equal but for the rare value where expf() on the two sides rounds apart."""
 import ctypes as C
 
 import numpy as np
@@ -51,6 +54,9 @@ def test_scaled_mfma_is_the_dequantised_product():
             assert np.all(err <= 1e-4 * mag + 1e-30), (a_fp4, trial, float((err / np.maximum(mag, 1e-30)).max()))
             if trial == 3:
                 assert np.array_equal(got.astype(np.float32), want.astype(np.float32)), (a_fp4, "sparse")
+            # and, on these fresh operands, bit for bit what the oracle's statement of the instruction's summation gives
+            rule = orc.mfma_scaled_k128(a, sa, a_fp4, b, sb)
+            assert np.array_equal(rule.view(np.uint32), got.astype(np.float32).view(np.uint32)), (a_fp4, trial, int((rule != got.astype(np.float32)).sum()))
 
 
 class Stacked:
@@ -75,6 +81,10 @@ class Stacked:
         self.w = abi.DskWeights(p("w1"), p("s1"), p("w3"), p("s3"), p("w2"), p("s2"), p("sh_w1"), p("sh_s1"), p("sh_w3"), p("sh_s3"), p("sh_w2"), p("sh_s2"),
                                 H, I, E, topk)
         self._deq = {}
+
+    def raw(self, e):
+        """the stored tensors ((w1, s1), (w3, s3), (w2, s2)) of expert id e (-1: the shared expert) and whether they are e2m1"""
+        return (self.shared, 0) if e < 0 else (self.experts[int(self.emap[e])], 1)
 
     def deq(self, e):
         """dequantised (w1, w3, w2) of expert id e (-1: the shared expert)"""
@@ -117,7 +127,7 @@ def check_chunk(L, x, idx, w, rows, got, note="", e2e=3e-3):
             e, pos = got["re"][t][r], got["rpos"][t][r]
             assert got["off"][e] <= pos < got["off"][e + 1] and got["perm"][pos] == t
     assert np.all(np.diff(got["perm"][got["off"][3]:got["off"][4]]) > 0)
-    nh = nbad = 0
+    nh = nbad = nbad_mx = ny = nybad = 0
     ref = np.zeros((len(rows), H), np.float64)
     worst_d = 0.0
     for i, t in enumerate(rows):
@@ -132,10 +142,20 @@ def check_chunk(L, x, idx, w, rows, got, note="", e2e=3e-3):
             assert np.all(hf >= up["lo"][0] - 1e-30) and np.all(hf <= up["hi"][0] + 1e-30), (t, e, note)
             nbad += int((hg != up["h64"][0]).sum())
             nh += I
+            # the oracle that adds every dot product as the matrix instruction does (its rule: tests/golden/mfma_scaled_k128.npz):
+            # h equal but for the rare value where the two exponential routines round apart, everything after it bit for bit
+            (r1, r3, r2), f4 = L.raw(e)
+            hm = orc.dsk_up_mx(r1[0], r1[1], r3[0], r3[1], f4, xq[t:t + 1], xs[t:t + 1], rw)[0]
+            nbad_mx += int((hg != hm).sum())
+            dm = orc.dsk_down_mx(r2[0], r2[1], f4, hg[None, :])
+            chain = orc.dsk_down_mx(r2[0], r2[1], f4, hm[None, :])["outb"][0]
             own = orc.dsk_down(w2, hg[None, :])
             if e >= 0:  # the quantisation of h as the down GEMM read it
                 assert np.array_equal(got["hq"][pos], own["hq"][0]) and np.array_equal(got["hs"][pos], own["hs"][0]), (t, e)
             dg = (got["dsh"] if e < 0 else got["d"])[pos]
+            assert np.array_equal(dg, dm["outb"][0]), (t, e, "w2 from the GPU's own h: the matrix unit's sums", int((dg != dm["outb"][0]).sum()))
+            ny += H
+            nybad += int((dg != chain).sum())
             err = np.abs(orc.bf16_to_f32(dg).astype(np.float64) - own["out64"][0])
             tol = 1e-4 * own["mag"][0] + np.abs(own["out64"][0]) * 2.0 ** -8
             assert np.all(err <= tol), (t, e, float((err / tol).max()))
@@ -147,6 +167,10 @@ def check_chunk(L, x, idx, w, rows, got, note="", e2e=3e-3):
     rl2 = np.linalg.norm(y - ref) / max(np.linalg.norm(ref), 1e-30)
     print("dsk prefill %s H=%d I=%d T=%d: %d rows checked, h equal %.2f%%, w2 worst %.2f of its tolerance, end-to-end rel-L2 %.2e max-abs %.2e (|y| max %.2f)"
           % (note, H, I, T, len(rows), 100 - 100.0 * nbad / nh, worst_d, rl2, np.abs(y - ref).max(), np.abs(ref).max()))
+    print("  against the oracle with the matrix unit's sums: h differs in %d of %d values, the picks' outputs from the oracle's own h in %d of %d"
+          % (nbad_mx, nh, nybad, ny))
+    assert nbad_mx <= 2e-4 * nh + 1, (nbad_mx, nh)
+    assert nybad <= 2e-3 * ny + 8, (nybad, ny)
     assert nbad <= 0.015 * nh, (nbad, nh)
     assert np.abs(y - ref).max() <= 2e-2 + 2.0 ** -7 * np.abs(ref).max()
     assert rl2 <= e2e

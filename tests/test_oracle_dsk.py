@@ -96,3 +96,35 @@ def test_expert_against_the_reference_vectors():
             assert (y_late == yref).mean() < 0.9
             noclamp = orc.dsk_up(w1, w3, xd, rw, limit=1e30, want_range=False)
             assert np.any(noclamp["h32"] != up["h32"])
+
+
+def test_matrix_unit_variant_stays_inside_the_contract():
+    """orc_dsk_up_mx / orc_dsk_down_mx (every dot product added as gfx950's block-scaled MFMA adds it; the rule itself is pinned
+    by tests/golden/mfma_scaled_k128.npz) against orc_dsk_up / orc_dsk_down (pinned above by the reference's vectors): h inside
+    the range of the reference's sum tolerance and mostly equal, outputs within one bf16 step; the shared expert's form too"""
+    rng = np.random.default_rng(9)
+    H, I, M = 512, 256, 3
+    x = orc.normal_bf16(9, 1, (M, H), 1.5)
+    xq, xs = orc.act_quant_ue8m0(x)
+    xd = orc.dequant_act_ue8m0(xq, xs)
+    rw = np.array([0.3, 1.1, 0.7], np.float32)
+
+    def fp4(N, K, lo, hi):
+        codes = rng.integers(0, 16, (N, K), dtype=np.uint8)
+        return (codes[:, 0::2] | (codes[:, 1::2] << 4)).astype(np.uint8), rng.integers(lo, hi, (N, K // 32), dtype=np.uint8)
+
+    def fp8(N, K, lo, hi):
+        return orc.f32_to_e4m3(np.clip(rng.standard_normal((N, K)).astype(np.float32) * 40.0, -448, 448)), rng.integers(lo, hi, (N // 32, K // 32), dtype=np.uint8)
+    for f4, mk, deq, r in ((1, fp4, orc.mxfp4_dequant, rw), (0, fp8, orc.fp8e_dequant, None)):
+        (w1, s1), (w3, s3), (w2, s2) = mk(I, H, 116, 121), mk(I, H, 116, 121), mk(H, I, 118, 123)
+        up = orc.dsk_up(deq(w1, s1), deq(w3, s3), xd, r, sum_tol=1e-4)
+        hm = orc.dsk_up_mx(w1, s1, w3, s3, f4, xq, xs, r)
+        hf = orc.bf16_to_f32(hm)
+        assert np.all(hf >= up["lo"]) and np.all(hf <= up["hi"])
+        assert (hm == up["h32"]).mean() >= 0.97, (hm == up["h32"]).mean()
+        dn = orc.dsk_down(deq(w2, s2), hm)
+        dm = orc.dsk_down_mx(w2, s2, f4, hm)
+        assert np.array_equal(dm["hq"], dn["hq"]) and np.array_equal(dm["hs"], dn["hs"])
+        err = np.abs(orc.bf16_to_f32(dm["outb"]).astype(np.float64) - dn["out64"])
+        assert np.all(err <= 1e-4 * dn["mag"] + np.abs(dn["out64"]) * 2.0 ** -8)
+        assert (dm["outb"] == dn["outb"]).mean() >= 0.97
