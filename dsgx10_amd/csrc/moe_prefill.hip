@@ -20,6 +20,7 @@
 #include "common.cuh"
 #include "pf_gemm_fp8.cuh"
 #include "pf_gemm_mx.cuh"
+#include "pf_gemm_i4.cuh"
 
 #ifdef DSGX_TRACE
 extern "C" unsigned long long* dsgx_trace_buf();
@@ -691,13 +692,26 @@ int dsgx_moe_prefill(const dsgx_layer_w* L, const uint16_t* x, const int* idx, c
     Gemm16Args q{};
     q.L = *L;
     q.tile_e = I32(o.tile_e), q.tile_m0 = I32(o.tile_m0), q.ntiles = I32(o.ntiles), q.off = I32(o.off), q.nrows = P;
+    // INT4 experts: the LDS-staged kernels of pf_gemm_i4.cuh (DSGX_PF_I4_OLD=1: the register-ring kernel they replaced, same bits)
+    const char* old4 = std::getenv("DSGX_PF_I4_OLD");
+    const bool new4 = i4 && !(old4 && old4[0] == '1');
+    pfi4::Args q4{};
+    if (new4) {
+      for (const void* k : {(const void*)pfi4::k_gemm<true>, (const void*)pfi4::k_gemm<false>})
+        if (int rc = allow_dynamic_lds(k, pfi4::kLds)) return rc;
+      q4.L = *L, q4.tile_e = I32(o.tile_e), q4.tile_m0 = I32(o.tile_m0), q4.ntiles = I32(o.ntiles), q4.off = I32(o.off);
+    }
     if (cfg.phases & 2) {
       q.x = x, q.gather = I32(o.perm), q.h = reinterpret_cast<uint16_t*>(W + o.h), q.d = nullptr;
-      hipLaunchKernelGGL(k_up, dim3(pf_grid(o.max_tiles, I / (kWgRows / 2))), dim3(kGemmThreads), lds16, st, q);
+      q4.x = q.x, q4.gather = q.gather, q4.h = q.h, q4.d = nullptr;
+      if (new4) hipLaunchKernelGGL(pfi4::k_gemm<true>, dim3(pf8::grid_of(o.max_tiles, I / (kWgRows / 2))), dim3(pf8::kThreads), pfi4::kLds, st, q4);
+      else hipLaunchKernelGGL(k_up, dim3(pf_grid(o.max_tiles, I / (kWgRows / 2))), dim3(kGemmThreads), lds16, st, q);
     }
     if (cfg.phases & 4) {
       q.x = reinterpret_cast<const uint16_t*>(W + o.h), q.gather = nullptr, q.h = nullptr, q.d = F32(o.d);
-      hipLaunchKernelGGL(k_dn, dim3(pf_grid(o.max_tiles, H / kWgRows)), dim3(kGemmThreads), lds16, st, q);
+      q4.x = q.x, q4.gather = nullptr, q4.h = nullptr, q4.d = q.d;
+      if (new4) hipLaunchKernelGGL(pfi4::k_gemm<false>, dim3(pf8::grid_of(o.max_tiles, H / kWgRows)), dim3(pf8::kThreads), pfi4::kLds, st, q4);
+      else hipLaunchKernelGGL(k_dn, dim3(pf_grid(o.max_tiles, H / kWgRows)), dim3(kGemmThreads), lds16, st, q);
     }
     if (cfg.phases & 8) {
       const size_t n = (size_t)T * (H / 4);

@@ -147,7 +147,6 @@ __device__ __forceinline__ void gemm_tile(const Args& g, uint8_t* smem, int e, i
   // cache's miss slots with them (weights first: 7% slower, measured). A turn issues them one at a time between its MFMAs (issue_some), so that the
   // texture unit works through a block's 50 KB while the matrix unit runs instead of in front of it: issued together after
   // the barrier they cost every wave the time the unit takes to accept them all (measured: a third of a turn).
-  constexpr int kLW = F4 ? 2 : 4;
   auto issue_one = [&](int kb, int i) {
     const int kc = kb < KB ? kb : KB - 1;
     const uint32_t st = lds0 + (uint32_t)(kb % S::kStages) * S::kStageBytes;

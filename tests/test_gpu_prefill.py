@@ -248,6 +248,27 @@ def test_prefill_int4_against_oracle(H, I, E, topk, T, shared):
     _rows_are_decode_rows(abi.FMT_INT4, H, I, E, topk, T, shared, seed=6)
 
 
+def test_prefill_int4_lds_staged_kernels_give_the_register_ring_kernels_bits():
+    """the INT4 experts' grouped GEMMs (pf_gemm_i4.cuh: both operands staged in LDS by DMA, weights decoded a turn ahead) add
+    in the k order of the kernel they replaced (k_pf_gemm16: register ring, kept behind DSGX_PF_I4_OLD=1): yr, ys and h equal
+    bit for bit, on a chunk with full and ragged tiles"""
+    import os
+    H, I, E, topk, T = 512, 256, 4, 2, 300
+    hl = helpers.make_layer(abi.FMT_INT4, H, I, E, topk, 4, seed=9, shared="bf16")
+    x, _, idx, w = helpers.rows_and_routing(17, T, H, E, topk, 2.5)
+    outs = []
+    for old in ("0", "1"):
+        os.environ["DSGX_PF_I4_OLD"] = old
+        try:
+            yr, ys, ws, dl = _prefill(hl, x, idx, w, T)
+            v = lib.prefill_view(dl.w, ws, T)
+            outs.append((yr.view(np.uint32), ys.view(np.uint32), gpu.host(gpu.view(ws, v.h, T * topk * I * 2), np.uint16, (-1,))))
+        finally:
+            os.environ.pop("DSGX_PF_I4_OLD", None)
+    for a, b in zip(*outs):
+        assert np.array_equal(a, b)
+
+
 @pytest.mark.parametrize("H,I,E,topk,T,shared", [(512, 256, 8, 2, 150, "fp8"), (1024, 128, 16, 4, 37, None)])
 def test_prefill_fp8_bf16_activations_against_oracle(H, I, E, topk, T, shared):
     """FP8 weights under the engine's own prefill contract (prefill.cu:337-352: bf16 activations, per 128-k block the sum
