@@ -603,6 +603,22 @@ __global__ void __launch_bounds__(64) k_probe_mfma_scaled(const uint8_t* __restr
   for (int q = 0; q < 4; ++q) out[(4 * part + q) * 16 + row] = c[q];
 }
 
+// one v_mfma_f32_16x16x32_bf16: A [16][32], B [16][32] bf16 bits (a lane of part p holds k = 8 p .. 8 p + 7 of its row), C [16][16]
+__global__ void __launch_bounds__(64) k_probe_mfma_bf16(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B, const float* __restrict__ C,
+                                                        float* __restrict__ out) {
+  typedef __bf16 v8bf_t __attribute__((ext_vector_type(8)));
+  const int l = threadIdx.x, row = l % 16, part = l / 16;
+  const uint4 a = *reinterpret_cast<const uint4*>(A + row * 32 + part * 8), b = *reinterpret_cast<const uint4*>(B + row * 32 + part * 8);
+  pf8::v4f_t c = {0.f, 0.f, 0.f, 0.f};
+  if (C) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q) c[q] = C[(4 * part + q) * 16 + row];
+  }
+  c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf_t, a), __builtin_bit_cast(v8bf_t, b), c, 0, 0, 0);
+#pragma unroll
+  for (int q = 0; q < 4; ++q) out[(4 * part + q) * 16 + row] = c[q];
+}
+
 bool layer_has_fp8_shared(const dsgx_layer_w* L) { return L->sh.g && L->sh.u && L->sh.d && L->sh.gs && L->sh.us && L->sh.ds; }
 
 }  // namespace
@@ -800,6 +816,13 @@ int dsgx_prefill_view_get(const dsgx_layer_w* L, void* ws, int T, dsgx_prefill_v
   out->hsh = reinterpret_cast<const uint16_t*>(W + o.hsh);
   out->off = reinterpret_cast<const int*>(W + o.off);
   out->perm = reinterpret_cast<const int*>(W + o.perm);
+  return DSGX_OK;
+}
+
+int dsgx_probe_mfma_bf16(const void* A, const void* B, const float* C, float* out, void* stream) {
+  if (!A || !B || !out) return fail(DSGX_EINVAL, "probe_mfma_bf16: null argument");
+  hipLaunchKernelGGL(k_probe_mfma_bf16, dim3(1), dim3(64), 0, (hipStream_t)stream, (const uint16_t*)A, (const uint16_t*)B, C, out);
+  DSGX_HIP(hipGetLastError());
   return DSGX_OK;
 }
 

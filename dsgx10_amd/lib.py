@@ -67,6 +67,7 @@ def lib():
                                            C.c_void_p, C.POINTER(abi.DskPrefillCfg)]
         L.dsgx_dsk_prefill_view_get.argtypes = [C.POINTER(abi.DskWeights), C.c_void_p, C.c_int, C.POINTER(abi.DskPrefillView)]
         L.dsgx_probe_mfma_scaled.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]
+        L.dsgx_probe_mfma_bf16.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]
         L.dsgx_add_norm_gemv.argtypes = [C.POINTER(abi.NormIn), C.c_int, C.c_int, C.POINTER(abi.GemvSeg), C.c_int, C.c_int, C.c_int, C.c_void_p]
         L.dsgx_fill_normal.argtypes = [C.c_uint64, C.c_uint64, C.c_size_t, C.c_double, C.c_void_p, C.c_int, C.c_void_p]
         L.dsgx_launch_floor.argtypes = [C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]
@@ -157,6 +158,10 @@ def dsk_prefill_view(weights, ws, T):
     v = abi.DskPrefillView()
     _check(lib().dsgx_dsk_prefill_view_get(C.byref(weights), _ptr(ws), T, C.byref(v)))
     return v
+
+
+def probe_mfma_bf16(A, B, out, stream=None, acc=None):
+    _check(lib().dsgx_probe_mfma_bf16(_ptr(A), _ptr(B), _ptr(acc), _ptr(out), _stream(stream)))
 
 
 def probe_mfma_scaled(A, SA, B, SB, a_fp4, out, stream=None, acc=None):

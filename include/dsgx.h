@@ -331,6 +331,9 @@ DSGX_API int dsgx_probe_mfma_fp8(const void* A, const void* B, float* raw, int f
    adds it. */
 DSGX_API int dsgx_probe_mfma_scaled(const void* A, const void* SA, const void* B, const void* SB, int a_fp4, const float* C, float* out,
                                     void* stream);
+/* Probe: one v_mfma_f32_16x16x32_bf16 (the decode kernels' variant 1 and the bf16-activation prefill GEMMs): A, B bf16 bits
+   [16][32], C f32 [16][16] or null; out[i][j] = C[i][j] + sum over k of A[i][k] B[j][k] as the matrix unit adds it. */
+DSGX_API int dsgx_probe_mfma_bf16(const void* A, const void* B, const float* C, float* out, void* stream);
 
 /* ---- misc ---------------------------------------------------------------------------------------------------- */
 DSGX_API const char* dsgx_last_error(void);

@@ -176,3 +176,22 @@ def test_stream_read_and_copy_run():
     lib.stream_read(a, a.numel(), sink)
     lib.stream_copy(a, b, a.numel())
     assert np.array_equal(gpu.host(b, np.uint32, (-1,)), np.arange(1 << 20, dtype=np.uint32))
+
+
+def test_bf16_mfma_probe_is_the_f32_product_sum():
+    """one v_mfma_f32_16x16x32_bf16 (the instruction of decode variant 1 and of the bf16-activation prefill GEMMs), operands as the
+    kernels hand them over (a lane of part p holds k = 8 p .. 8 p + 7 of its row), with an accumulator going in: within 1e-6 of
+    the sum of |terms| of the f64 result (the unit adds in f32-like precision; its exact order of adds is not restated in the
+    oracle: these paths' parity is the reference's tolerance parity)"""
+    rng = np.random.default_rng(4)
+    for trial in range(4):
+        a = orc.f32_to_bf16((rng.standard_normal((16, 32)) * 2.0 ** rng.integers(-3, 4, (16, 32))).astype(np.float32))
+        b = orc.f32_to_bf16(rng.standard_normal((16, 32)).astype(np.float32))
+        c = (rng.standard_normal((16, 16)) * 3).astype(np.float32) if trial % 2 else None
+        out = gpu.empty(16 * 16 * 4, 0xFF)
+        lib.probe_mfma_bf16(gpu.dev(a), gpu.dev(b), out, acc=None if c is None else gpu.dev(c))
+        got = gpu.host(out, np.float32, (16, 16)).astype(np.float64)
+        av, bv = orc.bf16_to_f32(a).astype(np.float64), orc.bf16_to_f32(b).astype(np.float64)
+        want = av @ bv.T + (0 if c is None else c.astype(np.float64))
+        mag = np.abs(av) @ np.abs(bv).T + (0 if c is None else np.abs(c).astype(np.float64))
+        assert np.all(np.abs(got - want) <= 1e-6 * mag), float((np.abs(got - want) / mag).max())
