@@ -1,0 +1,78 @@
+"""Writes tests/golden/mfma_bf16_k32.npz: operands and results of gfx950's v_mfma_f32_16x16x32_bf16, the instruction the
+bf16-activation prefill GEMMs and the MFMA decode kernels run on. RUN ON THE GPU: it calls the library's own probe
+(dsgx_probe_mfma_bf16), nothing of the reference. The CPU tests check the oracle's statement of how the instruction adds its
+32 products (orc_mfma_bf16_k32) against these vectors bit for bit.
+
+    python tests/golden/make_mfma_bf16_vectors.py [out.npz]
+
+Per case c: a[c], b[c] bf16 bit patterns [16][32] in the instruction's k order (a lane of part p holds k = 8 p .. 8 p + 7),
+acc[c] f32 [16][16] (the accumulator going in; zeros in every third case), d[c] f32 [16][16]: d[i][j] = acc[i][j] + sum over k
+of a[i][k] b[j][k] as the instruction adds it.
+Cases: standard normals times 2^r, r uniform in +-0, 2, 6, 12, 20 (the wider, the more of a sum is lost to alignment);
+sparse rows; accumulators of 1e-3 to 1e3 times a standard normal; rows shaped like the kernels' operands (INT4 weights
+(u - z) s against activations); operands with bf16 subnormals; and two crafted cases that sit on the edge of the
+accumulator adder's width (the last two)."""
+import os
+import sys
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+sys.path.insert(0, ROOT)
+
+
+def main(out):
+    from dsgx10_amd import lib
+    from tests import gpu, orc
+
+    rng = np.random.default_rng(23)
+    A, B, ACC, D = [], [], [], []
+
+    def run(a, b, acc):
+        o = gpu.empty(16 * 16 * 4, 0xFF)
+        lib.probe_mfma_bf16(gpu.dev(a), gpu.dev(b), o, acc=None if acc is None else gpu.dev(acc))
+        A.append(a), B.append(b), ACC.append(np.zeros((16, 16), np.float32) if acc is None else acc), D.append(gpu.host(o, np.float32, (16, 16)))
+
+    for trial in range(30):
+        style = trial % 6
+        spread = (0, 2, 6, 12, 20, 0)[style]
+
+        def mk():
+            v = rng.standard_normal((16, 32)) * 2.0 ** rng.integers(-spread, spread + 1, (16, 32))
+            if style == 4:
+                v = np.where(rng.random((16, 32)) < 0.2, v, 0)
+            return orc.f32_to_bf16(v.astype(np.float32))
+
+        a, b = mk(), mk()
+        if style == 5:  # INT4 weights: (u - z) s with one s and z a row
+            u = rng.integers(0, 16, (16, 32)) - rng.integers(0, 16, (16, 1))
+            a = orc.f32_to_bf16((u * orc.bf16_to_f32(orc.f32_to_bf16((rng.random((16, 1)) * 0.02 + 0.002).astype(np.float32)))).astype(np.float32))
+        acc = None if trial % 3 == 0 else (rng.standard_normal((16, 16)) * 10.0 ** rng.integers(-3, 4)).astype(np.float32)
+        run(a, b, acc)
+    # bf16 subnormals (exponent field 0) against large normal values: the products are ordinary f32 magnitudes
+    for trial in range(3):
+        a = rng.integers(1, 128, (16, 32)).astype(np.uint16) | (rng.integers(0, 2, (16, 32)).astype(np.uint16) << 15)
+        if trial:  # mixed with small normal values
+            small = orc.f32_to_bf16((rng.standard_normal((16, 32)) * 2.0 ** -124).astype(np.float32))
+            a = np.where(rng.random((16, 32)) < 0.5, a, small).astype(np.uint16)
+        b = orc.f32_to_bf16((rng.standard_normal((16, 32)) * 2.0 ** 120).astype(np.float32))
+        acc = None if trial == 0 else (rng.standard_normal((16, 16)) * 1e-3).astype(np.float32)
+        run(a, b, acc)
+    # crafted: the accumulator adder's width and rounding. Row i of a pairs with row i of b (its result is d[i][i]): the
+    # accumulator is 2^30 (or 2^30 + 2^29): its ulp is 128; one group adds (or subtracts) 2^6 - half an ulp - and 2^p,
+    # p = 5 .. -6: the result moves by a whole ulp exactly while 2^p still reaches the adder
+    one = lambda v: int(orc.f32_to_bf16(np.array([v], np.float32))[0])
+    for sign, accv in ((1.0, 2.0 ** 30), (-1.0, 2.0 ** 30 + 2.0 ** 29)):
+        a, b = np.zeros((16, 32), np.uint16), np.zeros((16, 32), np.uint16)
+        acc = np.zeros((16, 16), np.float32)
+        for i in range(12):
+            a[i, 0], b[i, 0] = one(sign * 64.0), one(1.0)
+            a[i, 1], b[i, 1] = one(sign * 2.0 ** (5 - i)), one(1.0)
+            acc[i, i] = accv
+        run(a, b, acc)
+    np.savez_compressed(out, a=np.stack(A), b=np.stack(B), acc=np.stack(ACC), d=np.stack(D))
+    print("wrote", out, len(A), "cases")
+
+
+if __name__ == "__main__":
+    main(sys.argv[1] if len(sys.argv) > 1 else os.path.join(os.path.dirname(os.path.abspath(__file__)), "mfma_bf16_k32.npz"))

@@ -403,6 +403,20 @@ def mfma_scaled_k128(a, sa, a_fp4, b, sb, acc=None):
     return out
 
 
+def mfma_bf16_k32(a, b, acc=None):
+    """the oracle's statement of gfx950's v_mfma_f32_16x16x32_bf16: a bf16 bits [R][32], b [S][32] in the instruction's k order
+    (k = 8 part + i of a lane), acc f32 [R][S] (None: zeros) -> f32 [R][S]"""
+    a, b = (np.ascontiguousarray(v, np.uint16) for v in (a, b))
+    f = lib().orc_mfma_bf16_k32
+    f.restype = C.c_float
+    f.argtypes = [C.c_void_p, C.c_void_p, C.c_float]
+    out = np.empty((a.shape[0], b.shape[0]), np.float32)
+    for i in range(a.shape[0]):
+        for j in range(b.shape[0]):
+            out[i, j] = f(a[i].ctypes.data, b[j].ctypes.data, 0.0 if acc is None else float(acc[i, j]))
+    return out
+
+
 def set_fp8_block_rule(rule):
     """0: a 128-k block's products are added sequentially in f32 (the contract as the reference's CPU stand-in states it);
     1: by the gfx950 matrix unit's rule (orc_mfma_fp8_k128) in the prefill kernels' k map"""
