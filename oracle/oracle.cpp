@@ -915,6 +915,82 @@ ORC void orc_moe_prefill_fp8_row_h_perturbed(const dsgx_layer_w* L, const dsgx_m
   }
 }
 
+// ---- prefill with bf16 activations, as the bf16 MFMA adds it ---------------------------------------------------------------
+// The altar-1 contract (A/engine/experts/prefill.cu:337-352, 772-831: a chunk row is a decode row) leaves the order of the f32
+// adds inside a dot product open; this restates the one the prefill kernels take, so that their outputs can be checked bit
+// for bit: a 128-k block is four v_mfma_f32_16x16x32_bf16 (j = 0 .. 3), whose accumulator runs through all of K (INT4, BF16)
+// or, for FP8 weights, starts from zero in every block and enters the row's sum as fmaf(S, block sum, acc). First k of the 8
+// products of lane part p in MFMA j of a block:
+static inline int pf16_k0(uint32_t fmt, int j, int p) {
+  if (fmt == DSGX_FMT_INT4_G32) return 32 * p + 8 * j;               // a lane holds one scale group
+  if (fmt == DSGX_FMT_FP8_B128) return 64 * (j >> 1) + 16 * p + 8 * (j & 1);  // a lane's 16 codes at 16 p and at 64 + 16 p
+  return 32 * j + 8 * p;                                             // BF16 weights as stored
+}
+// wrow: the row's weights as f32 (mat_row_raw: exact bf16 values; FP8 without its block scale), x: bf16 bits [K]
+static float pf16_dot(const Mat& m, int n, const float* wrow, const uint16_t* x) {
+  const float* sr = m.fmt == DSGX_FMT_FP8_B128 ? m.fs + (size_t)(n / 128) * (m.K / 128) : nullptr;
+  float acc = 0.f;
+  for (int kb = 0; kb < m.K / 128; ++kb) {
+    float c = sr ? 0.f : acc;
+    for (int j = 0; j < 4; ++j) {
+      uint16_t a[32], b[32];
+      for (int p = 0; p < 4; ++p) {
+        const int k0 = 128 * kb + pf16_k0(m.fmt, j, p);
+        for (int i = 0; i < 8; ++i) a[8 * p + i] = f2bf(wrow[k0 + i]), b[8 * p + i] = x[k0 + i];
+      }
+      c = mfma_bf16_block(c, a, b);
+    }
+    acc = sr ? fmaf(sr[kb], c, acc) : c;
+  }
+  return acc;
+}
+// One row of a chunk through the bf16-activation prefill (INT4 experts with a BF16 shared expert, or FP8 weights with bf16
+// activations): picks idx[topk], w[topk] of token row x bf16 [H]. h_out (optional) bf16 [topk in expert-id order (+ 1, the
+// shared expert's)][I]; yr f32 [H] = over the picks in expert-id order acc = fmaf(s2 w, d, acc); ys f32 [H] the shared
+// expert's sums (optional). Every bit as the kernels give it.
+ORC void orc_moe_prefill_b16_row_mfma(const dsgx_layer_w* L, const dsgx_mat_desc* desc, const uint16_t* x, const int* idx,
+                                      const float* w, uint16_t* h_out, float* yr, float* ys) {
+  const int H = L->H, I = L->I, topk = L->topk;
+  int ord[8];
+  for (int k = 0; k < topk; ++k) ord[k] = k;
+  std::sort(ord, ord + topk, [&](int a, int b) { return idx[a] < idx[b]; });
+  const bool shared = sh_fp8(L) || sh_b16(L);
+  std::vector<float> acc(H, 0.f), d(H);
+  std::vector<uint16_t> hb(I);
+  for (int s = 0; s < topk + (shared ? 1 : 0); ++s) {
+    const bool sh = s == topk, inter = sh && sh_b16(L);
+    const int e = sh ? -1 : idx[ord[s]];
+    const Mat G = sh ? shared_mat(L, 0) : expert_mat(L, desc, e, 0);
+    const Mat Uw = sh ? (inter ? G : shared_mat(L, 1)) : expert_mat(L, desc, e, 1);
+    const Mat Dn = sh ? shared_mat(L, 2) : expert_mat(L, desc, e, 2);
+#pragma omp parallel
+    {
+      std::vector<float> row(std::max(H, I));
+#pragma omp for schedule(static)
+      for (int c = 0; c < I; ++c) {
+        mat_row_raw(G, inter ? 2 * c : c, row.data());
+        const float g = pf16_dot(G, inter ? 2 * c : c, row.data(), x);
+        mat_row_raw(Uw, inter ? 2 * c + 1 : c, row.data());
+        const float u = pf16_dot(Uw, inter ? 2 * c + 1 : c, row.data(), x);
+        hb[c] = f2bf(silu_mul(bfr(g * G.s2), bfr(u * Uw.s2)));
+      }
+#pragma omp for schedule(static)
+      for (int n = 0; n < H; ++n) {
+        mat_row_raw(Dn, n, row.data());
+        d[n] = pf16_dot(Dn, n, row.data(), hb.data());
+      }
+    }
+    if (h_out) memcpy(h_out + (size_t)s * I, hb.data(), (size_t)I * 2);
+    if (sh) {
+      if (ys) memcpy(ys, d.data(), (size_t)H * 4);
+    } else {
+      const float k0 = Dn.s2 * w[ord[s]];
+      for (int n = 0; n < H; ++n) acc[n] = fmaf(k0, d[n], acc[n]);
+    }
+  }
+  memcpy(yr, acc.data(), (size_t)H * 4);
+}
+
 // The residual add and RMSNorm after the expert step: A/engine/comm/glmcoll.h:34-62 (allreduce_add_norm at one rank),
 // A/ref/glmref.py:225-228 (rms_norm), :269-276 (add_residual), A/engine/attn/prep.cu:26-34 (rstd and the two roundings).
 // res_out bf16 = the contract's h; xn from mean(h^2) summed in f64 (xn) and in f32 sequentially (xn32).

@@ -230,6 +230,18 @@ def moe_prefill_fp8_row(hl, xrow, idx, w, h_in=None):
     return out
 
 
+def moe_prefill_b16_row_mfma(hl, xrow, idx, w):
+    """one chunk row through the bf16-activation prefill with every sum added as the bf16 MFMA adds it in the kernels' k map:
+    dict(h bf16 [topk in expert-id order (+ 1, the shared expert's)][I], yr f32 [H], ys f32 [H])"""
+    xrow = np.ascontiguousarray(xrow, np.uint16)
+    idx = np.ascontiguousarray(idx, np.int32)
+    w = np.ascontiguousarray(w, np.float32)
+    out = dict(h=np.empty((hl.topk + (1 if hl.has_shared else 0), hl.I), np.uint16), yr=np.empty(hl.H, np.float32), ys=np.zeros(hl.H, np.float32))
+    Lw, desc = hl.host_layer_w()
+    lib().orc_moe_prefill_b16_row_mfma(C.byref(Lw), _p(desc), _p(xrow), _p(idx), _p(w), _p(out["h"]), _p(out["yr"]), _p(out["ys"]))
+    return out
+
+
 def moe_prefill_fp8_row_range(hl, xrow, idx, sum_tol):
     """(lo, hi) f32 [topk in expert-id order (+ 1)][I]: the values h may take when the gate and up sums move by
     sum_tol * their sums of |terms|"""

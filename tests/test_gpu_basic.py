@@ -181,8 +181,8 @@ def test_stream_read_and_copy_run():
 def test_bf16_mfma_probe_is_the_f32_product_sum():
     """one v_mfma_f32_16x16x32_bf16 (the instruction of decode variant 1 and of the bf16-activation prefill GEMMs), operands as the
     kernels hand them over (a lane of part p holds k = 8 p .. 8 p + 7 of its row), with an accumulator going in: within 1e-6 of
-    the sum of |terms| of the f64 result (the unit adds in f32-like precision; its exact order of adds is not restated in the
-    oracle: these paths' parity is the reference's tolerance parity)"""
+    the sum of |terms| of the f64 result, and equal bit for bit to the oracle's statement of how the unit adds (orc_mfma_bf16_k32,
+    pinned on the CPU by tests/golden/mfma_bf16_k32.npz) on these fresh operands"""
     rng = np.random.default_rng(4)
     for trial in range(4):
         a = orc.f32_to_bf16((rng.standard_normal((16, 32)) * 2.0 ** rng.integers(-3, 4, (16, 32))).astype(np.float32))
@@ -195,3 +195,5 @@ def test_bf16_mfma_probe_is_the_f32_product_sum():
         want = av @ bv.T + (0 if c is None else c.astype(np.float64))
         mag = np.abs(av) @ np.abs(bv).T + (0 if c is None else np.abs(c).astype(np.float64))
         assert np.all(np.abs(got - want) <= 1e-6 * mag), float((np.abs(got - want) / mag).max())
+        mine = gpu.host(out, np.float32, (16, 16))
+        assert np.array_equal(mine.view(np.uint32), orc.mfma_bf16_k32(a, b, c).view(np.uint32))

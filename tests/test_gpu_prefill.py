@@ -274,3 +274,31 @@ def test_prefill_fp8_bf16_activations_against_oracle(H, I, E, topk, T, shared):
     """FP8 weights under the engine's own prefill contract (prefill.cu:337-352: bf16 activations, per 128-k block the sum
     from zero, then fma(S, sum, acc)): act_fp8 = 0"""
     _rows_are_decode_rows(abi.FMT_FP8, H, I, E, topk, T, shared, seed=8, per_row=False, act_fp8=False)
+
+
+@pytest.mark.parametrize("fmt,H,I,E,topk,T,shared,kw", [
+    (abi.FMT_INT4, 512, 256, 8, 2, 150, "bf16", {}),
+    (abi.FMT_INT4, 256, 384, 4, 4, 300, None, {}),
+    (abi.FMT_FP8, 512, 256, 8, 2, 150, "fp8", dict(act_fp8=False)),
+    (abi.FMT_FP8, 1024, 128, 16, 4, 37, None, dict(act_fp8=False)),
+])
+def test_prefill_bf16_activations_every_bit_against_the_matrix_unit_oracle(fmt, H, I, E, topk, T, shared, kw):
+    """with the bf16 MFMA's order of adds restated in the oracle (pinned on the CPU by tests/golden/mfma_bf16_k32.npz) the
+    bf16-activation prefill is checked bit for bit: h of every pick and of the shared expert, yr, ys, on chunks with full
+    and ragged tiles (INT4 experts: pf_gemm_i4.cuh; the BF16 and FP8 matrices: k_pf_gemm16)"""
+    hl = helpers.make_layer(fmt, H, I, E, topk, min(E, 5), seed=21, shared=shared)
+    x, _, idx, w = helpers.rows_and_routing(29, T, H, E, topk, 2.5)
+    yr, ys, ws, dl = _prefill(hl, x, idx, w, T, **kw)
+    v = lib.prefill_view(dl.w, ws, T)
+    P = T * topk
+    rpos = gpu.host(gpu.view(ws, v.rpos, P * 4), np.int32, (T, topk))
+    hg = gpu.host(gpu.view(ws, v.h, P * I * 2), np.uint16, (P, I))
+    hsh = gpu.host(gpu.view(ws, v.hsh, T * I * 2), np.uint16, (T, I)) if shared else None
+    rows = list(range(T)) if T <= 40 else sorted(set(np.random.default_rng(1).integers(0, T, 24).tolist()) | {0, T - 1})
+    for t in rows:
+        o = orc.moe_prefill_b16_row_mfma(hl, x[t], idx[t], w[t])
+        mine = np.stack([hg[rpos[t, r]] for r in range(topk)] + ([hsh[t]] if shared else []))
+        assert np.array_equal(mine, o["h"]), (t, int((mine != o["h"]).sum()))
+        assert np.array_equal(yr[t].view(np.uint32), o["yr"].view(np.uint32)), (t, int((yr[t] != o["yr"]).sum()))
+        if shared:
+            assert np.array_equal(ys[t].view(np.uint32), o["ys"].view(np.uint32)), (t, int((ys[t] != o["ys"]).sum()))
