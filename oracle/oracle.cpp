@@ -359,6 +359,12 @@ static inline float mat_raw(const Mat& m, int n, int k) {
 static inline void mat_row_raw(const Mat& m, int n, float* out) {
   for (int k = 0; k < m.K; ++k) out[k] = mat_raw(m, n, k);
 }
+// 0 (the default): the f32 sum of a dot product in the contract's order (below). 1, 2: as the bf16 MFMA adds it in the prefill
+// kernels (1) or in the MFMA decode kernels (2): the contract leaves the order of the adds inside a dot product open, these
+// restate the kernels' own so that their outputs can be checked bit for bit (mfma_order_dot, further down).
+static int g_dot_rule = 0;
+ORC void orc_set_dot_rule(int rule) { g_dot_rule = rule; }
+static float mfma_order_dot(const Mat& m, int n, const float* wrow, const float* x, int rule);
 struct Dot { float f; double d, mag; };
 // f32 sums only (the timed CPU baseline): the f64 sums and sums of |terms| come back as 0
 static int g_f32_only = 0;
@@ -399,6 +405,7 @@ static inline Dot dot_row(const Mat& m, int n, const float* wrow, const float* x
       r.d += t; r.mag += fabs(t);
     }
   }
+  if (g_dot_rule) r.f = mfma_order_dot(m, n, wrow, x, g_dot_rule);
   return r;
 }
 // h = bf16(bf16(silu(g)) * u): A/engine/experts/decode.cu:110-113, tests/test_experts.cu:350
@@ -943,6 +950,50 @@ static float pf16_dot(const Mat& m, int n, const float* wrow, const uint16_t* x)
     acc = sr ? fmaf(sr[kb], c, acc) : c;
   }
   return acc;
+}
+// The MFMA decode kernels (dsgx_decode_cfg::up = 1): K is cut into ns equal slices (ns: the largest power of two up to 8 that
+// divides the steps of K and leaves a slice `minsteps` steps or more; a step = 128 bytes of a weight row), every slice is
+// summed from zero on the bf16 MFMA and the slices' sums are added in slice order. Inside a slice: FP8 per 128-k step the
+// four MFMAs from zero (lane part p of MFMA j: k = 32 j + 8 p ..), then acc = fmaf(S, sum, acc); INT4 a step of 256 k, eight
+// MFMAs (jj, j) on one accumulator, lane part p: k = 64 p + 32 jj + 8 j ..; BF16 a step of 64 k, two MFMAs, k = 32 jj + 8 p ...
+static float mf_decode_dot(const Mat& m, int n, const float* wrow, const float* x) {
+  const bool f8 = m.fmt == DSGX_FMT_FP8_B128, i4 = m.fmt == DSGX_FMT_INT4_G32;
+  const int stepk = f8 ? 128 : i4 ? 256 : 64, minsteps = f8 ? 4 : 8, steps_all = m.K / stepk;
+  int ns = 8;
+  while (ns > 1 && (steps_all % ns || steps_all / ns < minsteps)) ns >>= 1;
+  const int steps = steps_all / ns;
+  const float* sr = f8 ? m.fs + (size_t)(n / 128) * (m.K / 128) : nullptr;
+  auto block = [&](float c, int k0, int kp) {  // one MFMA: lane part p holds k0 + kp p + [0, 8)
+    uint16_t a[32], b[32];
+    for (int p = 0; p < 4; ++p)
+      for (int i = 0; i < 8; ++i) a[8 * p + i] = f2bf(wrow[k0 + kp * p + i]), b[8 * p + i] = f2bf(x[k0 + kp * p + i]);
+    return mfma_bf16_block(c, a, b);
+  };
+  float total = 0.f;
+  for (int w = 0; w < ns; ++w) {
+    float acc = 0.f;
+    for (int st = 0; st < steps; ++st) {
+      const int k0 = (w * steps + st) * stepk;
+      if (f8) {
+        float c = 0.f;
+        for (int j = 0; j < 4; ++j) c = block(c, k0 + 32 * j, 8);
+        acc = fmaf(sr[k0 / 128], c, acc);
+      } else if (i4) {
+        for (int jj = 0; jj < 2; ++jj)
+          for (int j = 0; j < 4; ++j) acc = block(acc, k0 + 32 * jj + 8 * j, 64);
+      } else {
+        for (int jj = 0; jj < 2; ++jj) acc = block(acc, k0 + 32 * jj, 8);
+      }
+    }
+    total = ns == 1 ? acc : total + acc;
+  }
+  return total;
+}
+static float mfma_order_dot(const Mat& m, int n, const float* wrow, const float* x, int rule) {
+  if (rule == 2) return mf_decode_dot(m, n, wrow, x);
+  std::vector<uint16_t> xb(m.K);
+  for (int k = 0; k < m.K; ++k) xb[k] = f2bf(x[k]);
+  return pf16_dot(m, n, wrow, xb.data());
 }
 // One row of a chunk through the bf16-activation prefill (INT4 experts with a BF16 shared expert, or FP8 weights with bf16
 // activations): picks idx[topk], w[topk] of token row x bf16 [H]. h_out (optional) bf16 [topk in expert-id order (+ 1, the

@@ -429,6 +429,12 @@ def mfma_bf16_k32(a, b, acc=None):
     return out
 
 
+def set_dot_rule(rule):
+    """how moe_up / moe_down / gemv add the f32 sum of a dot product: 0 in the contract's order (sequential), 1 as the bf16 MFMA
+    adds it in the prefill kernels, 2 as in the MFMA decode kernels (cfg.up = 1). Tests that set it put it back to 0."""
+    lib().orc_set_dot_rule(int(rule))
+
+
 def set_fp8_block_rule(rule):
     """0: a 128-k block's products are added sequentially in f32 (the contract as the reference's CPU stand-in states it);
     1: by the gfx950 matrix unit's rule (orc_mfma_fp8_k128) in the prefill kernels' k map"""

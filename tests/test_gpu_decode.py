@@ -227,6 +227,32 @@ def test_decode_mfma_variant(case):
     assert np.array_equal(yr_l.view(np.uint32), runs[8][0].view(np.uint32))
 
 
+@pytest.mark.parametrize("fmt,H,I,E,topk,shared,scale", [(abi.FMT_FP8, 2048, 1024, 32, 8, "fp8", 1.0), (abi.FMT_FP8, 1280, 768, 32, 8, None, 1.0),
+                                                       (abi.FMT_INT4, 2048, 2048, 168, 8, "bf16", 2.5), (abi.FMT_INT4, 6144, 512, 16, 4, None, 2.5),
+                                                       (abi.FMT_INT4, 2048, 2048, 32, 8, "fp8", 2.5)],
+                         ids=["fp8", "fp8-no-shared", "int4", "int4-I512-no-shared", "int4-fp8-shared"])
+def test_decode_mfma_variant_every_bit_against_the_matrix_unit_oracle(fmt, H, I, E, topk, shared, scale):
+    """with the bf16 MFMA's order of adds and the kernels' slicing of K restated in the oracle (orc.set_dot_rule(2); the
+    instruction's rule is pinned on the CPU by tests/golden/mfma_bf16_k32.npz) variant 1 is checked bit for bit: h of every
+    slot, yr from the GPU's own h and from the oracle's, ys; at 1, 3 and 8 rows"""
+    hl, dl = _layer(fmt, H, I, E, topk, 4, shared, seed=7)
+    x, _, idx, w = rows_and_routing(31, 8, H, E, topk, scale)
+    orc.set_dot_rule(2)
+    try:
+        for M in (1, 3, 8):
+            yr, ys, ws = gpu.decode_layer(dl, x[:M], idx[:M], w[:M], M, up=1)
+            uni = orc.union(idx[:M], E)
+            hg = gpu.h_of(ws, dl, M, len(uni))
+            up = orc.moe_up(hl, x[:M], uni)
+            assert np.array_equal(hg, up["h32"]), (M, int((hg != up["h32"]).sum()))
+            dn = orc.moe_down(hl, up["h32"], idx[:M], w[:M], uni)
+            assert np.array_equal(yr.view(np.uint32), dn["yr32"].view(np.uint32)), (M, int((yr != dn["yr32"]).sum()))
+            if hl.has_shared:
+                assert np.array_equal(ys.view(np.uint32), dn["ys32"].view(np.uint32)), (M, int((ys != dn["ys32"]).sum()))
+    finally:
+        orc.set_dot_rule(0)
+
+
 @pytest.mark.parametrize("fmt,H,I,E,shared,scale", [(abi.FMT_INT4, 6144, 512, 168, "bf16", 2.5), (abi.FMT_INT4, 2048, 2048, 32, "fp8", 2.5),
                                                    (abi.FMT_FP8, 1280, 768, 32, "fp8", 1.0)],
                          ids=["int4-per-rank-I512", "int4-fp8-shared", "fp8-H1280-I768"])
