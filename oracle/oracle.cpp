@@ -956,13 +956,13 @@ static float pf16_dot(const Mat& m, int n, const float* wrow, const uint16_t* x)
 // summed from zero on the bf16 MFMA and the slices' sums are added in slice order. Inside a slice: FP8 per 128-k step the
 // four MFMAs from zero (lane part p of MFMA j: k = 32 j + 8 p ..), then acc = fmaf(S, sum, acc); INT4 a step of 256 k, eight
 // MFMAs (jj, j) on one accumulator, lane part p: k = 64 p + 32 jj + 8 j ..; BF16 a step of 64 k, two MFMAs, k = 32 jj + 8 p ...
-static float mf_decode_dot(const Mat& m, int n, const float* wrow, const float* x) {
-  const bool f8 = m.fmt == DSGX_FMT_FP8_B128, i4 = m.fmt == DSGX_FMT_INT4_G32;
-  const int stepk = f8 ? 128 : i4 ? 256 : 64, minsteps = f8 ? 4 : 8, steps_all = m.K / stepk;
+// kind: 0 FP8 with 128 x 128 block scales sr (per step), 1 a scale group of 32 a lane (INT4, MXFP4), 2 BF16, 3 FP8 with the
+// scales already inside the bf16 values (DeepSeek's shared expert: the steps of kind 0, one accumulator through the slice)
+static float mf_decode_dot_raw(const float* wrow, const float* x, int K, int kind, const float* sr) {
+  const int stepk = kind == 1 ? 256 : kind == 2 ? 64 : 128, minsteps = (kind == 0 || kind == 3) ? 4 : 8, steps_all = K / stepk;
   int ns = 8;
   while (ns > 1 && (steps_all % ns || steps_all / ns < minsteps)) ns >>= 1;
   const int steps = steps_all / ns;
-  const float* sr = f8 ? m.fs + (size_t)(n / 128) * (m.K / 128) : nullptr;
   auto block = [&](float c, int k0, int kp) {  // one MFMA: lane part p holds k0 + kp p + [0, 8)
     uint16_t a[32], b[32];
     for (int p = 0; p < 4; ++p)
@@ -974,11 +974,13 @@ static float mf_decode_dot(const Mat& m, int n, const float* wrow, const float* 
     float acc = 0.f;
     for (int st = 0; st < steps; ++st) {
       const int k0 = (w * steps + st) * stepk;
-      if (f8) {
+      if (kind == 0) {
         float c = 0.f;
         for (int j = 0; j < 4; ++j) c = block(c, k0 + 32 * j, 8);
         acc = fmaf(sr[k0 / 128], c, acc);
-      } else if (i4) {
+      } else if (kind == 3) {
+        for (int j = 0; j < 4; ++j) acc = block(acc, k0 + 32 * j, 8);
+      } else if (kind == 1) {
         for (int jj = 0; jj < 2; ++jj)
           for (int j = 0; j < 4; ++j) acc = block(acc, k0 + 32 * jj + 8 * j, 64);
       } else {
@@ -988,6 +990,10 @@ static float mf_decode_dot(const Mat& m, int n, const float* wrow, const float* 
     total = ns == 1 ? acc : total + acc;
   }
   return total;
+}
+static float mf_decode_dot(const Mat& m, int n, const float* wrow, const float* x) {
+  const bool f8 = m.fmt == DSGX_FMT_FP8_B128;
+  return mf_decode_dot_raw(wrow, x, m.K, f8 ? 0 : m.fmt == DSGX_FMT_INT4_G32 ? 1 : 2, f8 ? m.fs + (size_t)(n / 128) * (m.K / 128) : nullptr);
 }
 static float mfma_order_dot(const Mat& m, int n, const float* wrow, const float* x, int rule) {
   if (rule == 2) return mf_decode_dot(m, n, wrow, x);
@@ -1126,6 +1132,10 @@ ORC void orc_fp8e_dequant(const uint8_t* w, const uint8_t* s, int N, int K, floa
 // (D/engine/kernels/moe.cu:519-528; model.py:841-850): gt = bf16(sum), up = bf16(sum), up clamped to +-limit, gt to <= limit,
 // h = gt / (1 + exp(-gt)) * up, routed: h = rw * h; hpre = bf16(h). h32: from f32 sums in k order; h64: from f64 sums;
 // lo / hi: the range when each sum moves by sum_tol * its sum of |terms|. rw null: the shared expert.
+// 0 (the default): the f32 sums of orc_dsk_up / orc_dsk_down in k order; 1, 3: as DeepSeek's decode kernels add them on the bf16
+// MFMA (mf_decode_dot_raw's kind: 1 the MXFP4 experts, 3 the shared expert), for checks of their outputs bit by bit
+static int g_dsk_dot_rule = 0;
+ORC void orc_set_dsk_dot_rule(int rule) { g_dsk_dot_rule = rule; }
 static inline float dsk_h(float gs, float us, float limit, const float* rw) {
   float gt = bfr(gs), up = bfr(us);
   up = std::min(std::max(up, -limit), limit);
@@ -1145,6 +1155,10 @@ ORC void orc_dsk_up(const float* w1, const float* w3, const float* xd, int M, in
         const float x = xd[(size_t)m * H + k], a = w1[(size_t)c * H + k], b = w3[(size_t)c * H + k];
         gf += a * x, uf += b * x;
         gd += (double)a * x, ud += (double)b * x, gm += fabs((double)a * x), um += fabs((double)b * x);
+      }
+      if (g_dsk_dot_rule) {
+        gf = mf_decode_dot_raw(w1 + (size_t)c * H, xd + (size_t)m * H, H, g_dsk_dot_rule, nullptr);
+        uf = mf_decode_dot_raw(w3 + (size_t)c * H, xd + (size_t)m * H, H, g_dsk_dot_rule, nullptr);
       }
       const size_t i = (size_t)m * I + c;
       const float* r = rw ? rw + m : nullptr;
@@ -1186,6 +1200,7 @@ ORC void orc_dsk_down(const float* w2, const uint16_t* hpre, int M, int H, int I
         const float w = w2[(size_t)n * I + k], h = hd[(size_t)m * I + k];
         f += w * h, d += (double)w * h, a += fabs((double)w * h);
       }
+      if (g_dsk_dot_rule) f = mf_decode_dot_raw(w2 + (size_t)n * I, hd.data() + (size_t)m * I, I, g_dsk_dot_rule, nullptr);
       const size_t i = (size_t)m * H + n;
       if (out32) out32[i] = f;
       if (out64) out64[i] = d;

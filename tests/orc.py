@@ -435,6 +435,12 @@ def set_dot_rule(rule):
     lib().orc_set_dot_rule(int(rule))
 
 
+def set_dsk_dot_rule(rule):
+    """how dsk_up / dsk_down add their f32 sums: 0 in k order, 1 / 3 as DeepSeek's decode kernels add them on the bf16 MFMA (1: the
+    MXFP4 experts, 3: the shared expert). Tests that set it put it back to 0."""
+    lib().orc_set_dsk_dot_rule(int(rule))
+
+
 def set_fp8_block_rule(rule):
     """0: a 128-k block's products are added sequentially in f32 (the contract as the reference's CPU stand-in states it);
     1: by the gfx950 matrix unit's rule (orc_mfma_fp8_k128) in the prefill kernels' k map"""

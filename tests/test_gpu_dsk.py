@@ -97,6 +97,52 @@ def test_dsk_moe_against_oracle(H, I, E, M, shared, fused):
     assert rl2 <= 3e-3
 
 
+@pytest.mark.parametrize("H,I,E,M,shared", [(1024, 512, 16, 1, True), (2048, 768, 32, 3, True), (1024, 256, 8, 8, False), (5120, 2304, 48, 2, True)])
+def test_dsk_moe_every_bit_against_the_matrix_unit_oracle(H, I, E, M, shared):
+    """with the bf16 MFMA's order of adds and the decode kernels' slicing of K restated in the oracle (orc.set_dsk_dot_rule;
+    the instruction's rule is pinned on the CPU by tests/golden/mfma_bf16_k32.npz) DeepSeek's decode layer is checked bit
+    for bit: h of every slot and row, the shared expert's output, and the fold y"""
+    topk = 6
+    hl = _layer(23, H, I, E, topk, 5, shared)
+    dl = hl.upload()
+    x = orc.normal_bf16(23, 1, (M, H), 1.5)
+    xq, xs = orc.act_quant_ue8m0(x)
+    xd = orc.dequant_act_ue8m0(xq, xs)
+    idx, w = orc.route(orc.normal_f32(23, 2, (M, E), 1.0), orc.normal_f32(23, 3, (E,), 0.2), topk, 1.5, score_fn=1)
+    ws = gpu.empty(lib.decode_ws_bytes(dl.w), 0)
+    y, ys = gpu.empty(M * H * 4, 0xFF), gpu.empty(M * H * 4, 0xFF)
+    lib.dsk_moe(dl.w, gpu.dev(xq), gpu.dev(xs), gpu.dev(idx), gpu.dev(w), M, ws, y, ys)
+    lib.decode_status(dl.w, ws)
+    y, ys = gpu.host(y, np.float32, (M, H)), gpu.host(ys, np.float32, (M, H))
+    uni = orc.union(idx, E)
+    hg = gpu.h_of(ws, dl, M, len(uni))
+    want = np.zeros((M, H), np.float32)
+    try:
+        for u, e in enumerate(uni):
+            ex = hl.experts[int(hl.emap[int(e)])]
+            w1, w3, w2 = (orc.mxfp4_dequant(*p) for p in ex)
+            rw = np.array([w[m][list(idx[m]).index(e)] if e in idx[m] else 0.0 for m in range(M)], np.float32)
+            orc.set_dsk_dot_rule(1)
+            up = orc.dsk_up(w1, w3, xd, rw)
+            assert np.array_equal(hg[u], up["h32"]), (u, int((hg[u] != up["h32"]).sum()))
+            dn = orc.dsk_down(w2, up["h32"])
+            for m in range(M):
+                if e in idx[m]:
+                    want[m] = want[m] + orc.bf16_to_f32(dn["outb"][m])
+        if shared:
+            orc.set_dsk_dot_rule(3)
+            w1, w3, w2 = (orc.fp8e_dequant(*p) for p in hl.shared_fp8)
+            up = orc.dsk_up(w1, w3, xd, None)
+            assert np.array_equal(hg[len(uni)], up["h32"]), int((hg[len(uni)] != up["h32"]).sum())
+            dn = orc.dsk_down(w2, up["h32"])
+            sh = orc.bf16_to_f32(dn["outb"])
+            assert np.array_equal(ys.view(np.uint32), sh.view(np.uint32)), int((ys != sh).sum())
+            want = want + sh
+    finally:
+        orc.set_dsk_dot_rule(0)
+    assert np.array_equal(y.view(np.uint32), want.view(np.uint32)), int((y != want).sum())
+
+
 @pytest.mark.parametrize("M", [12, 16])
 def test_dsk_moe_nine_to_sixteen_rows(M):
     """9-16 rows run as two passes of the kernels built for eight (dsk.h:211-223's up16 / down16 range): every row's bits are
