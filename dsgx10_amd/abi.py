@@ -74,5 +74,5 @@ SYMBOLS = [
     "dsgx_decode_ws_bytes", "dsgx_decode_ws_flag_offset", "dsgx_decode_status", "dsgx_moe_decode", "dsgx_moe_decode_noalloc", "dsgx_finalize", "dsgx_add_norm", "dsgx_dsk_cfg_default", "dsgx_dsk_moe", "dsgx_dsk_ws_bytes", "dsgx_dsk_moe_stacked", "dsgx_prefill_cfg_default", "dsgx_prefill_ws_bytes",
     "dsgx_moe_prefill", "dsgx_prefill_view_get", "dsgx_gemv", "dsgx_dequant_int4", "dsgx_probe_dequant_int4", "dsgx_probe_mfma_fp8",
     "dsgx_widen_fp8", "dsgx_act_quant", "dsgx_last_error", "dsgx_version", "dsgx_stream_read", "dsgx_stream_read_cfg", "dsgx_stream_copy", "dsgx_add_norm_gemv", "dsgx_fill_normal", "dsgx_launch_floor",
-    "dsgx_dsk_prefill_cfg_default", "dsgx_dsk_prefill_ws_bytes", "dsgx_dsk_moe_prefill", "dsgx_dsk_prefill_view_get", "dsgx_probe_mfma_scaled", "dsgx_probe_mfma_bf16",
+    "dsgx_dsk_prefill_cfg_default", "dsgx_dsk_prefill_ws_bytes", "dsgx_dsk_moe_prefill", "dsgx_dsk_prefill_view_get", "dsgx_probe_mfma_scaled", "dsgx_probe_mfma_bf16", "dsgx_probe_dot2_bf16",
 ]

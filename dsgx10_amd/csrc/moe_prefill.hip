@@ -826,6 +826,19 @@ int dsgx_probe_mfma_bf16(const void* A, const void* B, const float* C, float* ou
   return DSGX_OK;
 }
 
+// one v_dot2_f32_bf16 a thread (the vector-unit kernels' multiply-add: common.cuh's dot2)
+__global__ void __launch_bounds__(256) k_probe_dot2(const uint32_t* __restrict__ a, const uint32_t* __restrict__ b, const float* __restrict__ c,
+                                                    float* __restrict__ out, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) out[i] = dot2(a[i], b[i], c[i]);
+}
+int dsgx_probe_dot2_bf16(const void* a, const void* b, const float* c, float* out, int n, void* stream) {
+  if (!a || !b || !c || !out || n <= 0) return fail(DSGX_EINVAL, "probe_dot2_bf16: null argument or n <= 0");
+  hipLaunchKernelGGL(k_probe_dot2, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, (hipStream_t)stream, (const uint32_t*)a, (const uint32_t*)b, c, out, n);
+  DSGX_HIP(hipGetLastError());
+  return DSGX_OK;
+}
+
 int dsgx_probe_mfma_scaled(const void* A, const void* SA, const void* B, const void* SB, int a_fp4, const float* C, float* out, void* stream) {
   if (!A || !SA || !B || !SB || !out) return fail(DSGX_EINVAL, "probe_mfma_scaled: null argument");
   const uint8_t *a = (const uint8_t*)A, *sa = (const uint8_t*)SA, *b = (const uint8_t*)B, *sb = (const uint8_t*)SB;

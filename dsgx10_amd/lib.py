@@ -68,6 +68,7 @@ def lib():
         L.dsgx_dsk_prefill_view_get.argtypes = [C.POINTER(abi.DskWeights), C.c_void_p, C.c_int, C.POINTER(abi.DskPrefillView)]
         L.dsgx_probe_mfma_scaled.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]
         L.dsgx_probe_mfma_bf16.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]
+        L.dsgx_probe_dot2_bf16.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p]
         L.dsgx_add_norm_gemv.argtypes = [C.POINTER(abi.NormIn), C.c_int, C.c_int, C.POINTER(abi.GemvSeg), C.c_int, C.c_int, C.c_int, C.c_void_p]
         L.dsgx_fill_normal.argtypes = [C.c_uint64, C.c_uint64, C.c_size_t, C.c_double, C.c_void_p, C.c_int, C.c_void_p]
         L.dsgx_launch_floor.argtypes = [C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]
@@ -162,6 +163,11 @@ def dsk_prefill_view(weights, ws, T):
 
 def probe_mfma_bf16(A, B, out, stream=None, acc=None):
     _check(lib().dsgx_probe_mfma_bf16(_ptr(A), _ptr(B), _ptr(acc), _ptr(out), _stream(stream)))
+
+
+def probe_dot2_bf16(a, b, c, out, n, stream=None):
+    """out[i] = c[i] + a[i].lo b[i].lo + a[i].hi b[i].hi by v_dot2_f32_bf16 (a, b packed bf16 pairs, c, out f32; device tensors)"""
+    _check(lib().dsgx_probe_dot2_bf16(_ptr(a), _ptr(b), _ptr(c), _ptr(out), int(n), _stream(stream)))
 
 
 def probe_mfma_scaled(A, SA, B, SB, a_fp4, out, stream=None, acc=None):

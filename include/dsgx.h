@@ -334,6 +334,9 @@ DSGX_API int dsgx_probe_mfma_scaled(const void* A, const void* SA, const void* B
 /* Probe: one v_mfma_f32_16x16x32_bf16 (the decode kernels' variant 1 and the bf16-activation prefill GEMMs): A, B bf16 bits
    [16][32], C f32 [16][16] or null; out[i][j] = C[i][j] + sum over k of A[i][k] B[j][k] as the matrix unit adds it. */
 DSGX_API int dsgx_probe_mfma_bf16(const void* A, const void* B, const float* C, float* out, void* stream);
+/* Probe: n times v_dot2_f32_bf16, the multiply-add of the vector-unit kernels (decode variant 0, the dense GEMV): a, b packed
+   bf16 pairs [n] (the low half first), c f32 [n]; out[i] = c[i] + a[i].lo b[i].lo + a[i].hi b[i].hi as the instruction adds it. */
+DSGX_API int dsgx_probe_dot2_bf16(const void* a, const void* b, const float* c, float* out, int n, void* stream);
 
 /* ---- misc ---------------------------------------------------------------------------------------------------- */
 DSGX_API const char* dsgx_last_error(void);

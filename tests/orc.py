@@ -429,9 +429,19 @@ def mfma_bf16_k32(a, b, acc=None):
     return out
 
 
+def dot2_bf16(a, b, c):
+    """the oracle's statement of v_dot2_f32_bf16: a, b packed bf16 pairs (uint32 [n]), c f32 [n] -> f32 [n]"""
+    a, b, c = np.ascontiguousarray(a, np.uint32), np.ascontiguousarray(b, np.uint32), np.ascontiguousarray(c, np.float32)
+    f = lib().orc_dot2_bf16
+    f.restype = C.c_float
+    f.argtypes = [C.c_uint32, C.c_uint32, C.c_float]
+    return np.array([f(int(a[i]), int(b[i]), float(c[i])) for i in range(a.size)], np.float32)
+
+
 def set_dot_rule(rule):
     """how moe_up / moe_down / gemv add the f32 sum of a dot product: 0 in the contract's order (sequential), 1 as the bf16 MFMA
-    adds it in the prefill kernels, 2 as in the MFMA decode kernels (cfg.up = 1). Tests that set it put it back to 0."""
+    adds it in the prefill kernels, 2 as in the MFMA decode kernels (cfg.up = 1), 3 as in the vector-unit decode kernels (cfg.up = 0)
+    and the dense GEMV. Tests that set it put it back to 0."""
     lib().orc_set_dot_rule(int(rule))
 
 

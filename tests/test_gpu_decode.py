@@ -253,6 +253,32 @@ def test_decode_mfma_variant_every_bit_against_the_matrix_unit_oracle(fmt, H, I,
         orc.set_dot_rule(0)
 
 
+@pytest.mark.parametrize("fmt,H,I,E,topk,shared,scale", [(abi.FMT_FP8, 2048, 1024, 32, 8, "fp8", 1.0), (abi.FMT_FP8, 1024, 2048, 256, 8, None, 1.0),
+                                                       (abi.FMT_INT4, 2048, 2048, 168, 8, "bf16", 2.5), (abi.FMT_INT4, 4096, 2048, 16, 4, None, 2.5),
+                                                       (abi.FMT_BF16, 1024, 512, 16, 4, None, 2.5)],
+                         ids=["fp8", "fp8-no-shared", "int4", "int4-no-shared", "bf16"])
+def test_decode_vector_variant_every_bit_against_the_oracle(fmt, H, I, E, topk, shared, scale):
+    """with v_dot2_f32_bf16's rule (pinned on the CPU by tests/golden/dot2_bf16.npz), the lanes' split of K and the cross-lane
+    tree restated in the oracle (orc.set_dot_rule(3)) variant 0 is checked bit for bit: h of every slot, yr, ys; at 1, 2, 5 and
+    8 rows (the one-launch kernel and, where the step's h does not fit LDS, the slot-partitioned down phase)"""
+    hl, dl = _layer(fmt, H, I, E, topk, 4, shared, seed=7)
+    x, _, idx, w = rows_and_routing(37, 8, H, E, topk, scale)
+    orc.set_dot_rule(3)
+    try:
+        for M in (1, 2, 5, 8):
+            yr, ys, ws = gpu.decode_layer(dl, x[:M], idx[:M], w[:M], M, up=0)
+            uni = orc.union(idx[:M], E)
+            hg = gpu.h_of(ws, dl, M, len(uni))
+            up = orc.moe_up(hl, x[:M], uni)
+            assert np.array_equal(hg, up["h32"]), (M, int((hg != up["h32"]).sum()))
+            dn = orc.moe_down(hl, up["h32"], idx[:M], w[:M], uni)
+            assert np.array_equal(yr.view(np.uint32), dn["yr32"].view(np.uint32)), (M, int((yr != dn["yr32"]).sum()))
+            if hl.has_shared:
+                assert np.array_equal(ys.view(np.uint32), dn["ys32"].view(np.uint32)), (M, int((ys != dn["ys32"]).sum()))
+    finally:
+        orc.set_dot_rule(0)
+
+
 @pytest.mark.parametrize("fmt,H,I,E,shared,scale", [(abi.FMT_INT4, 6144, 512, 168, "bf16", 2.5), (abi.FMT_INT4, 2048, 2048, 32, "fp8", 2.5),
                                                    (abi.FMT_FP8, 1280, 768, 32, "fp8", 1.0)],
                          ids=["int4-per-rank-I512", "int4-fp8-shared", "fp8-H1280-I768"])
