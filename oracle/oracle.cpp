@@ -360,7 +360,7 @@ static inline void mat_row_raw(const Mat& m, int n, float* out) {
   for (int k = 0; k < m.K; ++k) out[k] = mat_raw(m, n, k);
 }
 // 0 (the default): the f32 sum of a dot product in the contract's order (below). 1, 2: as the bf16 MFMA adds it in the prefill
-// kernels (1) or in the MFMA decode kernels (2); 3: as the vector-unit decode kernels and the dense GEMV add it: the contract leaves the order of the adds inside a dot product open, these
+// kernels (1) or in the MFMA decode kernels (2); 3: as the vector-unit decode kernels add it, 4: as the dense GEMV does (orc_set_gemv_splitk): the contract leaves the order of the adds inside a dot product open, these
 // restate the kernels' own so that their outputs can be checked bit for bit (mfma_order_dot, further down).
 static int g_dot_rule = 0;
 ORC void orc_set_dot_rule(int rule) { g_dot_rule = rule; }
@@ -1015,19 +1015,19 @@ static inline float dot2_bf16(float c, uint16_t a0, uint16_t b0, uint16_t a1, ui
   return mfma_add_unit(c, S, Eg - 24);
 }
 ORC float orc_dot2_bf16(uint32_t a, uint32_t b, float c) { return dot2_bf16(c, (uint16_t)a, (uint16_t)b, (uint16_t)(a >> 16), (uint16_t)(b >> 16)); }
-// The vector-unit decode kernels (dsgx_decode_cfg::up = 0) and the dense GEMV: K is cut into segments of 64 KL values (KL = 16
+// The vector-unit decode kernels (dsgx_decode_cfg::up = 0): K is cut into segments of 64 KL values (KL = 16
 // FP8, 32 INT4, 8 BF16), lane l of the wave holds k = seg 64 KL + l KL .. of every segment and chains its products two at a
 // time through v_dot2_f32_bf16, segment after segment (FP8: a lane's 16 values of a segment from zero, then
 // acc = fmaf(S, sum, acc) with the block scale of those k); the 64 lanes' sums are then added in a fixed tree: lanes l and
 // l + 32, then l and l + 16, then within the sixteen i and 15 - i, i and 7 - i, i and i ^ 2, i and i ^ 1.
-static float vec_decode_dot(const Mat& m, int n, const float* wrow, const float* x) {
+// the 64 lanes' sums over the segments seg0, seg0 + step, ...
+static void vec_lane_sums(const Mat& m, int n, const float* wrow, const float* x, int seg0, int step, float (&v)[64]) {
   const bool f8 = m.fmt == DSGX_FMT_FP8_B128;
   const int KL = f8 ? 16 : m.fmt == DSGX_FMT_INT4_G32 ? 32 : 8, SEGK = 64 * KL, nseg = (m.K + SEGK - 1) / SEGK;
   const float* sr = f8 ? m.fs + (size_t)(n / 128) * (m.K / 128) : nullptr;
-  float v[64];
   for (int l = 0; l < 64; ++l) {
     float acc = 0.f;
-    for (int seg = 0; seg < nseg; ++seg) {
+    for (int seg = seg0; seg < nseg; seg += step) {
       const int k0 = seg * SEGK + l * KL;
       if (k0 >= m.K) continue;
       float p = f8 ? 0.f : acc;
@@ -1036,15 +1036,40 @@ static float vec_decode_dot(const Mat& m, int n, const float* wrow, const float*
     }
     v[l] = acc;
   }
+}
+static float vec_decode_dot(const Mat& m, int n, const float* wrow, const float* x) {
+  float v[64];
+  vec_lane_sums(m, n, wrow, x, 0, 1, v);
   float u[16], t3[8], t4[4];
   for (int l = 0; l < 16; ++l) u[l] = (v[l] + v[l + 32]) + (v[l + 16] + v[l + 48]);
   for (int i = 0; i < 8; ++i) t3[i] = u[i] + u[15 - i];
   for (int i = 0; i < 4; ++i) t4[i] = t3[i] + t3[7 - i];
   return (t4[0] + t4[2]) + (t4[1] + t4[3]);
 }
+// The dense GEMV (dsgx_gemv, dsgx_add_norm_gemv): the same lanes, added by another tree - within a row of sixteen lanes the
+// quads ((v0 + v1) + (v2 + v3)), two quads, two eights, then rows 0 + 1 and 2 + 3, then those two; with split-K (splitk 2 or
+// 4 on a matrix of up to 8192 rows) wave w of the SK sums the segments w, w + SK, ... and the waves' sums are added in order.
+static int g_gemv_splitk = 1;
+ORC void orc_set_gemv_splitk(int sk) { g_gemv_splitk = sk; }
+static float vec_gemv_dot(const Mat& m, int n, const float* wrow, const float* x) {
+  float total = 0.f;
+  for (int w = 0; w < g_gemv_splitk; ++w) {
+    float v[64], row[4];
+    vec_lane_sums(m, n, wrow, x, w, g_gemv_splitk, v);
+    for (int r = 0; r < 4; ++r) {
+      float q[4];
+      for (int j = 0; j < 4; ++j) q[j] = (v[16 * r + 4 * j] + v[16 * r + 4 * j + 1]) + (v[16 * r + 4 * j + 2] + v[16 * r + 4 * j + 3]);
+      row[r] = (q[0] + q[1]) + (q[2] + q[3]);
+    }
+    const float s = (row[0] + row[1]) + (row[2] + row[3]);
+    total = w == 0 ? s : total + s;
+  }
+  return total;
+}
 static float mfma_order_dot(const Mat& m, int n, const float* wrow, const float* x, int rule) {
   if (rule == 2) return mf_decode_dot(m, n, wrow, x);
   if (rule == 3) return vec_decode_dot(m, n, wrow, x);
+  if (rule == 4) return vec_gemv_dot(m, n, wrow, x);
   std::vector<uint16_t> xb(m.K);
   for (int k = 0; k < m.K; ++k) xb[k] = f2bf(x[k]);
   return pf16_dot(m, n, wrow, xb.data());

@@ -438,11 +438,13 @@ def dot2_bf16(a, b, c):
     return np.array([f(int(a[i]), int(b[i]), float(c[i])) for i in range(a.size)], np.float32)
 
 
-def set_dot_rule(rule):
+def set_dot_rule(rule, splitk=1):
     """how moe_up / moe_down / gemv add the f32 sum of a dot product: 0 in the contract's order (sequential), 1 as the bf16 MFMA
-    adds it in the prefill kernels, 2 as in the MFMA decode kernels (cfg.up = 1), 3 as in the vector-unit decode kernels (cfg.up = 0)
-    and the dense GEMV. Tests that set it put it back to 0."""
+    adds it in the prefill kernels, 2 as in the MFMA decode kernels (cfg.up = 1), 3 as in the vector-unit decode kernels (cfg.up = 0),
+    4 as in the dense GEMV (splitk: the split of K the call asked for, where the kernel honours it: up to 8192 rows).
+    Tests that set it put it back to 0."""
     lib().orc_set_dot_rule(int(rule))
+    lib().orc_set_gemv_splitk(int(splitk))
 
 
 def set_dsk_dot_rule(rule):

@@ -171,6 +171,36 @@ def test_split_k(case, sk):
         assert np.abs(orc.bf16_to_f32(got) - orc.bf16_to_f32(o["y16"])).max() <= 2e-2
 
 
+@pytest.mark.parametrize("sk", [1, 2, 4])
+@pytest.mark.parametrize("case", ["router168", "fp8_cfg1", "int4_cfg2", "int4_tail", "swiglu"])
+def test_gemv_every_bit_against_the_oracle(case, sk):
+    """with v_dot2_f32_bf16's rule (pinned on the CPU by tests/golden/dot2_bf16.npz), the lanes' split of K, the wave's tree
+    and the split-K order restated in the oracle (orc.set_dot_rule(4, splitk)) the dense GEMV is checked bit for bit:
+    f32 sums, bf16 outputs, SwiGLU outputs, a partial last segment"""
+    fmt, N, K, M, kind = {
+        "router168": (abi.FMT_BF16, 168, 6144, 4, abi.OUT_F32),
+        "fp8_cfg1": (abi.FMT_FP8, 2048, 4096, 1, abi.OUT_BF16),
+        "int4_cfg2": (abi.FMT_INT4, 1536, 6144, 6, abi.OUT_BF16),
+        "int4_tail": (abi.FMT_INT4, 72, 1280, 3, abi.OUT_F32),
+        "swiglu": (abi.FMT_BF16, 512, 2048, 2, abi.OUT_SWIGLU),
+    }[case]
+    x = orc.normal_bf16(13, 1, (M, K), 1.0)
+    if fmt == abi.FMT_FP8:
+        parts = quant_fp8(13, 2, N, K)
+    elif fmt == abi.FMT_INT4:
+        parts = quant_int4(13, 2, N, K)
+    else:
+        parts = (orc.normal_bf16(13, 2, (N, K), 0.05),)
+    got = _run(x, fmt, parts, N, K, kind, splitk=sk)
+    orc.set_dot_rule(4, sk)
+    try:
+        o = _oracle(x, fmt, parts, N, K, kind)
+    finally:
+        orc.set_dot_rule(0)
+    want = o["yf"] if kind == abi.OUT_F32 else o["y16"]
+    assert np.array_equal(got.view(np.uint32 if kind == abi.OUT_F32 else np.uint16), want.view(np.uint32 if kind == abi.OUT_F32 else np.uint16)), int((got != want).sum())
+
+
 @pytest.mark.parametrize("H", [2048, 4096, 6144])
 @pytest.mark.parametrize("mode", ["contract", "round2", "two_partials"])
 def test_add_norm(H, mode):
