@@ -177,7 +177,7 @@ def prefill_check_rows(pb, nrows=4):
     for t in (int(np.nonzero((idx_h == hot).any(1))[0][-1]), int(np.nonzero((idx_h == cold).any(1))[0][0]), 0, T - 1, T // 2, T // 3):
         if t not in rows and len(rows) < nrows:
             rows.append(t)
-    worst = dict(rows=rows, max_abs_err=0.0, rel_l2=0.0, oracle="C++ oracle; FP8 activations: each 128-k block added by the e4m3 MFMA's rule" if gen.fmt == abi.FMT_FP8 else "C++ oracle (decode contract row by row)")
+    worst = dict(rows=rows, max_abs_err=0.0, rel_l2=0.0, oracle="C++ oracle; FP8 activations: each 128-k block added by the e4m3 MFMA's rule" if gen.fmt == abi.FMT_FP8 else "C++ oracle; a chunk row is a decode row, each sum added by the bf16 MFMA's rule in the kernels' k order")
     for t in rows:
         experts = sorted(int(e) for e in idx_h[t])
         hl = gen.host_sublayer(experts, 0)
@@ -199,10 +199,17 @@ def prefill_check_rows(pb, nrows=4):
                                                                float(np.sqrt(((got - r).astype(np.float64) ** 2).sum() / max((r.astype(np.float64) ** 2).sum(), 1e-300))))
                 worst["vs_sequential_block_sums_max_abs"] = max(worst.get("vs_sequential_block_sums_max_abs", 0.0), float(np.abs(got - r).max()))
         else:
+            # every sum added as the bf16 MFMA adds it in the kernels' k order (pinned by tests/golden/mfma_bf16_k32.npz) ...
+            o = orc.moe_prefill_b16_row_mfma(hl, x[0], li, w[0])
+            ref = [o["yr"], o["ys"]]
+            # ... and the decode contract's sequential f32 sums
             uni = np.arange(len(experts), dtype=np.int32)
             up = orc.moe_up(hl, x, uni, want_range=False)
             dn = orc.moe_down(hl, up["h32"], li[None, :], w, uni)
-            ref = [dn["yr32"][0], dn["ys32"][0]]
+            for got, r in zip((pb.yr[t].cpu().numpy(), pb.ys[t].cpu().numpy()), (dn["yr32"][0], dn["ys32"][0])):
+                worst["vs_sequential_block_sums_rel_l2"] = max(worst.get("vs_sequential_block_sums_rel_l2", 0.0),
+                                                               float(np.sqrt(((got - r).astype(np.float64) ** 2).sum() / max((r.astype(np.float64) ** 2).sum(), 1e-300))))
+                worst["vs_sequential_block_sums_max_abs"] = max(worst.get("vs_sequential_block_sums_max_abs", 0.0), float(np.abs(got - r).max()))
         for got, r in zip((pb.yr[t].cpu().numpy(), pb.ys[t].cpu().numpy()), ref):
             worst["max_abs_err"] = max(worst["max_abs_err"], float(np.abs(got - r).max()))
             worst["rel_l2"] = max(worst["rel_l2"], float(np.sqrt(((got - r).astype(np.float64) ** 2).sum() / max((r.astype(np.float64) ** 2).sum(), 1e-300))))
@@ -271,6 +278,16 @@ def main():
         par = {"yr": err(d["yr"], dn["yr32"])}
         if hl.has_shared:
             par["ys"] = err(d["ys"], dn["ys32"])
+        # the same step with every dot product added in the kernels' own order (the oracle's restatement of v_dot2_f32_bf16 /
+        # the bf16 MFMA, the lanes' split of K and the reduction tree): the outputs then agree bit for bit
+        orc.set_dot_rule(2 if getattr(b, "up", 0) == 1 else 3)
+        try:
+            up2 = orc.moe_up(hl, d["x"], uni, want_range=False)
+            dn2 = orc.moe_down(hl, up2["h32"], d["idx"], d["w"], uni)
+        finally:
+            orc.set_dot_rule(0)
+        par["bits_equal_in_kernel_order"] = bool(np.array_equal(d["yr"].view(np.uint32), dn2["yr32"].view(np.uint32)) and
+                                                 (not hl.has_shared or np.array_equal(d["ys"].view(np.uint32), dn2["ys32"].view(np.uint32))))
         return dict(value=float(np.mean(ts[1:]) * 1e6), unit="us", cores=orc.threads(), kind="port",
                     sample="step 0 of the same workload (M=%d, %d routed experts + shared), %d repetitions after one warm-up, "
                            "C++ oracle, OpenMP, f32 sums" % (b.M, len(d["experts"]), len(ts) - 1),
