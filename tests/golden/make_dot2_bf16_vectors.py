@@ -6,7 +6,8 @@ reference. The CPU tests check the oracle's statement of the instruction (orc_do
 
 a, b: packed bf16 pairs (uint32, the low half first), c f32, d f32 = c + a.lo b.lo + a.hi b.hi as the instruction adds it.
 Cases: standard normals times 2^r, r uniform in +-0, 2, 6, 12, 20, with c of comparable or far smaller / larger size and
-zero in a tenth of the cases; operands with bf16 subnormals; zero operands; and crafted cases on the edge of the adder's width
+zero in a tenth of the cases; operands with bf16 subnormals; zero operands; c just above a power of two with products that
+take the result below it; and crafted cases on the edge of the adder's width
 (c = 2^30 whose ulp is 128, one product 2^6 - half an ulp - and the other 2^p, p = 5 .. -6) and on a sum that carries out of
 c's binade (c = 2 - 2^e + 2^-23, the products 2^e and 2^p, p = -26 .. -33)."""
 import os
@@ -37,6 +38,11 @@ def main(out):
     a = rng.integers(1, 128, (n, 2)).astype(np.uint16) | (rng.integers(0, 2, (n, 2)).astype(np.uint16) << 15)
     b = orc.f32_to_bf16((rng.standard_normal((n, 2)) * 2.0 ** 120).astype(np.float32))
     A.append(pack(a)), B.append(pack(b)), Cc.append((rng.standard_normal(n) * 1e-3).astype(np.float32))
+    # cancellation: c just above a power of two, products of either sign
+    a = orc.f32_to_bf16((rng.standard_normal((n, 2)) * 0.05).astype(np.float32))
+    b = orc.f32_to_bf16(rng.standard_normal((n, 2)).astype(np.float32))
+    c = (np.where(rng.random(n) < 0.5, 1.0, -1.0) * 2.0 ** rng.integers(-2, 4, n) * (1.0 + rng.random(n) * 0.01)).astype(np.float32)
+    A.append(pack(a)), B.append(pack(b)), Cc.append(c)
     # the adder's width
     one = lambda v: int(orc.f32_to_bf16(np.array([v], np.float32))[0])
     a, b, c = np.zeros((n, 2), np.uint16), np.zeros((n, 2), np.uint16), np.zeros(n, np.float32)

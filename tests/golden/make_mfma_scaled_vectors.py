@@ -12,7 +12,7 @@ zeros in every third case), d[c] f32 [16][16]: d[i][j] = acc[i][j] + sum over k 
 2^(sb[j][k/32] - 127) as the instruction adds it, k as stored.
 Cases: operands shaped like quantised rows and weights with unit scales; uniformly random codes; scale bytes spread over
 +-3, +-6 and +-10 around 127; sparse rows; accumulators of 1e-3 to 1e3 times a standard normal; two crafted cases that
-sit on the edge of the accumulator adder's width, and two whose sums carry out of the accumulator's binade (the last two)."""
+sit on the edge of the accumulator adder's width, six with accumulators just above a power of two, and two whose sums carry out of the accumulator's binade (the last two)."""
 import os
 import sys
 
@@ -73,6 +73,17 @@ def main(out):
             a[i, 0], b[i, 0] = code(sign), code(1.0)
             a[i, 8], b[i, 8] = code(sign * 2.0 ** e1), code(2.0 ** (e - e1))
             acc[i, i] = accv
+        o = gpu.empty(16 * 16 * 4, 0xFF)
+        lib.probe_mfma_scaled(gpu.dev(a), gpu.dev(sa), gpu.dev(b), gpu.dev(sb), 0, o, acc=gpu.dev(acc))
+        fp4s.append(0), A.append(a), B.append(b), SA.append(sa), SB.append(sb), ACC.append(acc), D.append(gpu.host(o, np.float32, (16, 16)))
+    # cancellation: accumulators just above a power of two against small sums of either sign (results that fall below it)
+    for trial in range(6):
+        a = e4m3_of(rng.standard_normal((16, 128)) * (2.0, 6.0, 1.0)[trial % 3])
+        b = e4m3_of(rng.standard_normal((16, 128)) * 4.0)
+        if trial % 2:
+            a[:, 16 * (1 + trial):] = 0
+        sa, sb = np.full((16, 4), 127 - 6, np.uint8), np.full((16, 4), 127 - 4, np.uint8)
+        acc = (np.where(rng.random((16, 16)) < 0.5, 1.0, -1.0) * 2.0 ** rng.integers(-2, 4, (16, 16)) * (1.0 + rng.random((16, 16)) * (0.002, 0.02)[trial % 2])).astype(np.float32)
         o = gpu.empty(16 * 16 * 4, 0xFF)
         lib.probe_mfma_scaled(gpu.dev(a), gpu.dev(sa), gpu.dev(b), gpu.dev(sb), 0, o, acc=gpu.dev(acc))
         fp4s.append(0), A.append(a), B.append(b), SA.append(sa), SB.append(sb), ACC.append(acc), D.append(gpu.host(o, np.float32, (16, 16)))

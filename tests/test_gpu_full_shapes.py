@@ -173,6 +173,13 @@ def test_prefill_int4_chunk_at_the_benchmark_shape():
             assert err <= 2e-3, (t, k, err)
             row_l2.append(helpers.rel_l2(got[t], full[k][0]))
         ref_yr.append(full["yr32"][0]), ref_ys.append(full["ys32"][0]), got_yr.append(yr[t]), got_ys.append(ys[t])
+    # and with every sum added as the bf16 MFMA adds it in the kernels' k order (the instruction's rule is pinned on the CPU by
+    # tests/golden/mfma_bf16_k32.npz): bit for bit, h of every pick and of the shared expert, yr, ys
+    for t in rows[:8]:
+        o = orc.moe_prefill_b16_row_mfma(hl, x[t], idx[t], w[t])
+        mine = np.concatenate([_h_rows(ws, v.h, T * topk, I, rpos[t]), _h_rows(ws, v.hsh, T, I, [t])])
+        assert np.array_equal(mine, o["h"]), (t, int((mine != o["h"]).sum()))
+        assert np.array_equal(yr[t].view(np.uint32), o["yr"].view(np.uint32)) and np.array_equal(ys[t].view(np.uint32), o["ys"].view(np.uint32)), t
     print("int4 prefill T=2048: %d rows sampled, h bit-equal %.3f%%, worst row error %.2e of the row's max, per-row rel-L2 median %.2e max %.2e, "
           "sampled rows together rel-L2 routed %.2e shared %.2e, max-abs %.2e"
           % (len(rows), 100.0 * exact / total, worst_row, np.median(row_l2), np.max(row_l2), helpers.rel_l2(np.stack(got_yr), np.stack(ref_yr)),
@@ -202,6 +209,20 @@ def test_decode_layers_at_the_benchmark_shapes(fmt, H, I, E, shared, scale, NS):
         outs = {}
         for up in (0, 1):
             outs[up] = _check_step(hl, dl, x, idx, w, M, up=up)
+            if M == 1:
+                # with every dot product added in the kernel's own order (orc.set_dot_rule: v_dot2_f32_bf16 and the lanes'
+                # tree, or the bf16 MFMA and its K slices; the instructions' rules are pinned on the CPU by tests/golden/
+                # dot2_bf16.npz and mfma_bf16_k32.npz): h, yr and ys bit for bit
+                uni = orc.union(idx[:M], E)
+                orc.set_dot_rule(3 if up == 0 else 2)
+                try:
+                    upk = orc.moe_up(hl, x[:M], uni, want_range=False)
+                    dnk = orc.moe_down(hl, upk["h32"], idx[:M], w[:M], uni)
+                finally:
+                    orc.set_dot_rule(0)
+                assert np.array_equal(outs[up][2], upk["h32"]), (up, int((outs[up][2] != upk["h32"]).sum()))
+                assert np.array_equal(outs[up][0].view(np.uint32), dnk["yr32"].view(np.uint32)), up
+                assert np.array_equal(outs[up][1].view(np.uint32), dnk["ys32"].view(np.uint32)), up
         yr_a, ys_a, _ = gpu.decode_layer(dl, x[:M], None, None, M, logits=gpu.dev(logits[:M]), route_scale=scale, up=-1)
         pick = 1 if fmt == abi.FMT_INT4 or M >= 2 else 0   # the library's table
         assert np.array_equal(yr_a.view(np.uint32), outs[pick][0].view(np.uint32)), (M, "auto variant / fused routing")
