@@ -49,7 +49,7 @@ class DecodeCfg(C.Structure):
 
 
 class PrefillCfg(C.Structure):
-    _fields_ = [("shared", C.c_int32), ("phases", C.c_int32), ("act_fp8", C.c_int32), ("fast_act", C.c_int32)]
+    _fields_ = [("shared", C.c_int32), ("phases", C.c_int32), ("act_fp8", C.c_int32), ("fast_act", C.c_int32), ("tile_order", C.c_int32)]
 
 
 class PrefillView(C.Structure):

@@ -45,7 +45,9 @@ def _compile(src, force, extra=(), suffix=""):
 
 
 def build(jobs=None, force=False, extra=(), suffix=""):
-    """extra / suffix: a diagnostic variant (e.g. extra=["-DDSGX_TRACE"], suffix="_trace" -> libdsgx_trace.so)"""
+    """extra / suffix: a diagnostic variant (e.g. extra=["-DDSGX_TRACE"], suffix="_trace" -> libdsgx_trace.so; DSGX_TRACE:
+    the decode kernels' phase stamps, DSGX_PF_TRACE: the FP8 prefill GEMM's, eight wall-clock stamps a workgroup into the
+    buffer whose address DSGX_PF_TRACE_PTR names; DSGX_LIB=libdsgx_trace.so loads the variant)"""
     srcs = [s for s in SOURCES if os.path.exists(os.path.join(CSRC, s))]
     jobs = jobs or min(len(srcs), os.cpu_count() or 4)
     so = SO.replace(".so", suffix + ".so")
@@ -82,4 +84,4 @@ if __name__ == "__main__":
     ap.add_argument("--force", action="store_true")
     ap.add_argument("--trace", action="store_true", help="the diagnostic variant libdsgx_trace.so (phase time stamps)")
     a = ap.parse_args()
-    print(build(a.j, a.force, ["-DDSGX_TRACE"], "_trace") if a.trace else build(a.j, a.force))
+    print(build(a.j, a.force, ["-DDSGX_TRACE", "-DDSGX_PF_TRACE"], "_trace") if a.trace else build(a.j, a.force))

@@ -70,12 +70,14 @@ __global__ void __launch_bounds__(64) k_probe_mfma_fp8(const uint8_t* __restrict
 }
 
 // ---- the workspace -------------------------------------------------------------------------------------------------------
+constexpr int kDefaultTileOrder = 0;  // dsgx_prefill_cfg::tile_order = -1
 constexpr int kTile = 128;  // rows of a tile (token positions) and weight rows a workgroup
 constexpr int kRowBlock = 128;  // token rows a workgroup of the bucketing kernels
 struct PfLayout {
   size_t cnt, off, ntiles, tile_e, tile_m0, perm, pickpos, posw, rpos, re, rk, xq, xs, h, hq, hs, hsh, hshq, hshs, d, bcnt, boff, bmask, total;
   size_t nbig, big_e, big_m0, nsmall, small_e, small_m0;  // the FP8 kernels' lists: 256-position tiles, and the experts' remainders
-  size_t nmix, mix_e, mix_m0;                             // ... and the two merged into the order the kernels run them in
+  size_t nmix, mix_e, mix_m0;                             // ... and the two merged, in expert order
+  size_t ord_e, ord_m0;                                   // ... and merged with the experts by falling count, remainders spread evenly
   int P, max_tiles, max_big;
 };
 PfLayout pf_layout(const dsgx_layer_w* L, int T) {
@@ -91,6 +93,7 @@ PfLayout pf_layout(const dsgx_layer_w* L, int T) {
   o.nbig = take(4), o.big_e = take((size_t)o.max_big * 4), o.big_m0 = take((size_t)o.max_big * 4);
   o.nsmall = take(4), o.small_e = take(E * 4), o.small_m0 = take(E * 4);
   o.nmix = take(4), o.mix_e = take((size_t)(o.max_big + E) * 4), o.mix_m0 = take((size_t)(o.max_big + E) * 4);
+  o.ord_e = take((size_t)(o.max_big + E) * 4), o.ord_m0 = take((size_t)(o.max_big + E) * 4);
   o.perm = take(P * 4), o.pickpos = take(P * 4), o.posw = take(P * 4), o.rpos = take(P * 4), o.re = take(P * 4), o.rk = take(P * 4);
   o.xq = take((size_t)T * H), o.xs = take((size_t)T * (H / 128) * 4);
   o.h = take(P * I * 2), o.hq = take(P * I), o.hs = take(P * (I / 128) * 4);
@@ -136,9 +139,10 @@ struct TileLists {
   int *nbig, *big_e, *big_m0;         // 256-position tiles
   int *nsmall, *small_e, *small_m0;   // the remainders of up to 128 positions
   int *nmix, *mix_e, *mix_m0;         // both, in expert order (expert | 1 << 30 for a 256-position tile)
+  int *ord_e, *ord_m0;                // both (nmix of them), the experts by falling count (see k_pf_scan)
 };
 __global__ void __launch_bounds__(DSGX_MAX_EXPERTS) k_pf_scan(const int* __restrict__ bcnt, int NB, int E, int* __restrict__ boff,
-                                                              int* __restrict__ cnt, int* __restrict__ off, TileLists tl) {
+                                                              int* __restrict__ cnt, int* __restrict__ off, TileLists tl, int order) {
   __shared__ int sa[DSGX_MAX_EXPERTS], sb[DSGX_MAX_EXPERTS], sc[DSGX_MAX_EXPERTS], sd[DSGX_MAX_EXPERTS];
   const int e = threadIdx.x;
   int c = 0;
@@ -178,8 +182,58 @@ __global__ void __launch_bounds__(DSGX_MAX_EXPERTS) k_pf_scan(const int* __restr
     const int p0 = (sc[e] - nbig) + (sd[e] - nsmall);
     for (int i = 0; i < nbig; ++i) tl.mix_e[p0 + i] = e | (1 << 30), tl.mix_m0[p0 + i] = i * 256;
     if (nsmall) tl.mix_e[p0 + nbig] = e, tl.mix_m0[p0 + nbig] = (c / 256) * 256;
+    if (!order) {  // (the second list is always a valid one: a later call may name it whatever this call was told)
+      for (int i = 0; i < nbig; ++i) tl.ord_e[p0 + i] = e | (1 << 30), tl.ord_m0[p0 + i] = i * 256;
+      if (nsmall) tl.ord_e[p0 + nbig] = e, tl.ord_m0[p0 + nbig] = (c / 256) * 256;
+    }
   }
   if (e == 0) *tl.nmix = nb + nsm;
+  // The same tiles in the order of the reference's prefill_tuning tord (ds41f-4xgx10-switchless/engine/kernels/prefill.cu:
+  // 658-668: the most-picked experts' tiles with those of the least-picked between them): the experts by falling count
+  // (ties by id), their 256-position tiles as one list B and their remainders as one list S, merged so that both lists
+  // run out together (B's tile k at key (k + 1/2) / |B|, S's tile j at (j + 1/2) / |S|, by rising key, B first on a tie).
+  // A 256-position tile is bound by the matrix unit and a remainder by the weight stream, so at any time the chip runs
+  // a mix of the two. The order of the sums does not depend on the list's order.
+  if (!order) return;  // (the same for every thread)
+  __syncthreads();
+  sa[e] = e < E ? c : -1;
+  __syncthreads();
+  int rank = 0, rank2 = 0;  // by falling count; by falling remainder (order 2's list of remainders)
+  {
+    const int ce = e < E ? c : -1, re = (e < E && nsmall) ? rem : -1;
+    for (int j = 0; j < DSGX_MAX_EXPERTS; ++j) {
+      const int cj = sa[j];
+      const int rj = (cj >= 0 && cj % 256 > 0 && cj % 256 <= 128) ? cj % 256 : -1;
+      rank += (cj > ce) || (cj == ce && j < e);
+      rank2 += (rj > re) || (rj == re && j < e);
+    }
+  }
+  __syncthreads();
+  sb[rank] = e < E ? nbig : 0, sd[order == 2 ? rank2 : rank] = e < E ? nsmall : 0;
+  __syncthreads();
+  for (int d = 1; d < DSGX_MAX_EXPERTS; d <<= 1) {  // inclusive scans in rank order
+    const int vb = e >= d ? sb[e - d] : 0, vd = e >= d ? sd[e - d] : 0;
+    __syncthreads();
+    sb[e] += vb, sd[e] += vd;
+    __syncthreads();
+  }
+  if (e < E) {
+    const long long NB_ = nb, NS_ = nsm;
+    const int k0 = sb[rank] - nbig, j0 = sd[order == 2 ? rank2 : rank] - nsmall;
+    for (int i = 0; i < nbig; ++i) {
+      const long long k = k0 + i;
+      long long before = NS_ ? ((2 * k + 1) * NS_ + NB_ - 1) / (2 * NB_) : 0;  // S tiles of a key below this one's
+      if (before > NS_) before = NS_;
+      if (order == 2) before = 0;  // every 256-position tile before every remainder
+      tl.ord_e[k + before] = e | (1 << 30), tl.ord_m0[k + before] = i * 256;
+    }
+    if (nsmall) {
+      const long long j = j0;
+      long long before = NB_ ? ((2 * j + 1) * NB_ + NS_) / (2 * NS_) : 0;      // B tiles of a key up to this one's
+      if (before > NB_ || order == 2) before = NB_;
+      tl.ord_e[j + before] = e, tl.ord_m0[j + before] = (c / 256) * 256;
+    }
+  }
 }
 __global__ void __launch_bounds__(256) k_pf_place(const int* __restrict__ idx, const float* __restrict__ w, int T, int topk, int E,
                                                   const int* __restrict__ off, const int* __restrict__ boff,
@@ -645,6 +699,7 @@ void dsgx_prefill_cfg_default(dsgx_prefill_cfg* c) {
   c->phases = 31;
   c->act_fp8 = 1;
   c->fast_act = 0;
+  c->tile_order = -1;
 }
 
 static int prefill_check(const dsgx_layer_w* L, int T, const char* who) {
@@ -683,14 +738,17 @@ int dsgx_moe_prefill(const dsgx_layer_w* L, const uint16_t* x, const int* idx, c
   auto I32 = [&](size_t off) { return reinterpret_cast<int*>(W + off); };
   auto F32 = [&](size_t off) { return reinterpret_cast<float*>(W + off); };
   const int H = L->H, I = L->I, E = L->E, topk = L->topk, P = o.P;
+  int order = cfg.tile_order < 0 ? kDefaultTileOrder : cfg.tile_order;
+  if (order > 2) return fail(DSGX_EINVAL, "moe_prefill: tile_order %d (-1, 0, 1, 2)", cfg.tile_order);
+  if (i4 || !cfg.act_fp8) order = 0;  // (the bf16-activation kernels walk the 128-position list)
 
   if (cfg.phases & 1) {
     const int NB = (T + kRowBlock - 1) / kRowBlock;
     uint32_t* bmask = reinterpret_cast<uint32_t*>(W + o.bmask);
     hipLaunchKernelGGL(k_pf_mask, dim3(NB), dim3(256), 0, st, idx, T, topk, E, I32(o.bcnt), bmask);
     const TileLists tl{I32(o.ntiles), I32(o.tile_e), I32(o.tile_m0), I32(o.nbig), I32(o.big_e), I32(o.big_m0), I32(o.nsmall), I32(o.small_e), I32(o.small_m0),
-                       I32(o.nmix), I32(o.mix_e), I32(o.mix_m0)};
-    hipLaunchKernelGGL(k_pf_scan, dim3(1), dim3(DSGX_MAX_EXPERTS), 0, st, I32(o.bcnt), NB, E, I32(o.boff), I32(o.cnt), I32(o.off), tl);
+                       I32(o.nmix), I32(o.mix_e), I32(o.mix_m0), I32(o.ord_e), I32(o.ord_m0)};
+    hipLaunchKernelGGL(k_pf_scan, dim3(1), dim3(DSGX_MAX_EXPERTS), 0, st, I32(o.bcnt), NB, E, I32(o.boff), I32(o.cnt), I32(o.off), tl, order);
     hipLaunchKernelGGL(k_pf_place, dim3(NB), dim3(256), 0, st, idx, w, T, topk, E, I32(o.off), I32(o.boff), bmask, L->desc, I32(o.perm),
                        I32(o.pickpos), I32(o.rpos), I32(o.re), F32(o.rk), (float*)nullptr);
     DSGX_HIP(hipGetLastError());
@@ -770,8 +828,12 @@ int dsgx_moe_prefill(const dsgx_layer_w* L, const uint16_t* x, const int* idx, c
   pf8::Args g{};
   g.L = *L;
   g.fast_act = cfg.fast_act;
+#ifdef DSGX_PF_TRACE
+  if (const char* tp = std::getenv("DSGX_PF_TRACE_PTR")) g.trace = reinterpret_cast<unsigned long long*>(std::strtoull(tp, nullptr, 0));
+#endif
   const int NSU = I / (pf8::kWgRows / 2), NSD = H / pf8::kWgRows;
-  g.tile_e = I32(o.mix_e), g.tile_m0 = I32(o.mix_m0), g.ntiles = I32(o.nmix), g.off = I32(o.off), g.nrows = P;
+  const bool mixed = order >= 1;
+  g.tile_e = I32(mixed ? o.ord_e : o.mix_e), g.tile_m0 = I32(mixed ? o.ord_m0 : o.mix_m0), g.ntiles = I32(o.nmix), g.off = I32(o.off), g.nrows = P;
   if (cfg.phases & (2 | 16)) {
     if (int rc = dsgx_act_quant(x, T, H, W + o.xq, F32(o.xs), stream)) return rc;
   }
@@ -924,8 +986,8 @@ int dsgx_dsk_moe_prefill(const dsgx_dsk_weights* Wt, const uint8_t* xq, const ui
     uint32_t* bmask = reinterpret_cast<uint32_t*>(W + o.bmask);
     hipLaunchKernelGGL(k_pf_mask, dim3(NB), dim3(256), 0, st, idx, T, topk, E, I32(o.bcnt), bmask);
     const TileLists tl{I32(o.ntiles), I32(o.tile_e), I32(o.tile_m0), I32(o.nbig), I32(o.big_e), I32(o.big_m0), I32(o.nsmall), I32(o.small_e), I32(o.small_m0),
-                       I32(o.nmix), I32(o.mix_e), I32(o.mix_m0)};
-    hipLaunchKernelGGL(k_pf_scan, dim3(1), dim3(DSGX_MAX_EXPERTS), 0, st, I32(o.bcnt), NB, E, I32(o.boff), I32(o.cnt), I32(o.off), tl);
+                       I32(o.nmix), I32(o.mix_e), I32(o.mix_m0), I32(o.ord_e), I32(o.ord_m0)};
+    hipLaunchKernelGGL(k_pf_scan, dim3(1), dim3(DSGX_MAX_EXPERTS), 0, st, I32(o.bcnt), NB, E, I32(o.boff), I32(o.cnt), I32(o.off), tl, 0);
     hipLaunchKernelGGL(k_pf_place, dim3(NB), dim3(256), 0, st, idx, w, T, topk, E, I32(o.off), I32(o.boff), bmask, (const dsgx_mat_desc*)nullptr, I32(o.perm),
                        I32(o.pickpos), I32(o.rpos), I32(o.re), F32(o.rk), F32(o.posw));
     DSGX_HIP(hipGetLastError());

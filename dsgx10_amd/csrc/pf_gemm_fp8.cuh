@@ -74,7 +74,15 @@ struct Args {
   uint8_t* hq;         // UP: h quantised, e4m3 [position][I]
   float* hs;           // UP: its scales [position][I / 128]
   float* d;            // DOWN: f32 [position][H]
+#ifdef DSGX_PF_TRACE
+  unsigned long long* trace;  // (diagnostic build: thread 0's wall-clock stamps, 8 a workgroup)
+#endif
 };
+#ifdef DSGX_PF_TRACE
+#define PF_STAMP(g, k) do { if ((g).trace && threadIdx.x == 0) (g).trace[(size_t)blockIdx.x * 8 + (k)] = wall_clock64(); } while (0)
+#else
+#define PF_STAMP(g, k) do { } while (0)
+#endif
 
 // Workgroup -> (position tile, group of weight rows): blocks of kMapTiles consecutive tiles x kMapNs row groups get 32
 // consecutive workgroup numbers of ONE XCD (numbers x, x + 8, x + 16, ...), so that what they share (a tile's
@@ -207,7 +215,9 @@ __device__ __forceinline__ void gemm_tile(const Args& g, uint8_t* smem, int e, i
     wsa_l = swa[kc], wsb_l = swb[kc];
     asm volatile("" : "+v"(wsa_l), "+v"(wsb_l));  // (uses that make the compiler place its wait here)
   };
+  PF_STAMP(g, 2);
   load_ws(0);
+  PF_STAMP(g, 3);
 #pragma unroll
   for (int s = 0; s + 1 < S::kStages; ++s) issue(s);
 
@@ -232,6 +242,7 @@ __device__ __forceinline__ void gemm_tile(const Args& g, uint8_t* smem, int e, i
       // everyone is done reading the stage of block kb - 1, which the loads of block kb + kStages - 1 now overwrite
       wait_loads<(S::kStages - 2) * S::kLoads>();
       if (!(DIAG & 4)) __syncthreads();
+      if (kb == 0) PF_STAMP(g, 4);
       if (!(DIAG & 1)) issue(kb + S::kStages - 1);
       if (NJ == 0) continue;
       const float wsa = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, wsa_l), kb & 63));
@@ -277,6 +288,7 @@ __device__ __forceinline__ void gemm_tile(const Args& g, uint8_t* smem, int e, i
   }
   wait_loads<0>();   // the trailing loads into unused stages: nothing may still be landing in LDS from here on
   __syncthreads();   // ... in any wave's part of it: the epilogues reuse the stages
+  PF_STAMP(g, 5);
   if (DIAG & 64) {   // (diagnostic: no epilogue; one store keeps the sums alive)
     float sum = 0.f;
 #pragma unroll
@@ -364,6 +376,7 @@ __device__ __forceinline__ void gemm_tile(const Args& g, uint8_t* smem, int e, i
       }
     }
   }
+  PF_STAMP(g, 6);
 }
 
 // The shared expert (tile_e null: tiles of Shape<WP>::kPos rows over [0, nrows)) or one list of tiles of one shape.
@@ -391,10 +404,15 @@ __global__ void __launch_bounds__(kThreads) k_gemm_mixed(Args g) {
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
   const int NS = UP ? g.L.I / (kWgRows / 2) : g.L.H / kWgRows;
   int tile, ns;
+  PF_STAMP(g, 0);
   task_of<false>(NS, tile, ns);
   if (ns >= NS || tile >= *g.ntiles) return;
   const int te = g.tile_e[tile], e = te & 0xFFFF;
   const int m0 = g.off[e] + g.tile_m0[tile], mend = g.off[e + 1];
+  if (m0 >= 0) PF_STAMP(g, 1);
+#ifdef DSGX_PF_TRACE
+  if (g.trace && threadIdx.x == 0) g.trace[(size_t)blockIdx.x * 8 + 7] = ((te >> 30) ? 0x10000 : 0) | min(mend - m0, (te >> 30) ? 256 : 128);
+#endif
   if (te >> 30) gemm_tile<UP, 2, DIAG>(g, smem, e, m0, mend, ns);
   else gemm_tile<UP, 1, DIAG>(g, smem, e, m0, mend, ns);
 }

@@ -195,8 +195,8 @@ def prefill_ws_bytes(layer_w, T):
     return lib().dsgx_prefill_ws_bytes(C.byref(layer_w), T)
 
 
-def moe_prefill(layer_w, x, idx, w, T, ws, yr, ys, stream=None, shared=True, phases=31, act_fp8=True, fast_act=False):
-    cfg = abi.PrefillCfg(int(shared), phases, int(act_fp8), int(fast_act))
+def moe_prefill(layer_w, x, idx, w, T, ws, yr, ys, stream=None, shared=True, phases=31, act_fp8=True, fast_act=False, tile_order=-1):
+    cfg = abi.PrefillCfg(int(shared), phases, int(act_fp8), int(fast_act), int(tile_order))
     _check(lib().dsgx_moe_prefill(C.byref(layer_w), _ptr(x), _ptr(idx), _ptr(w), T, _ptr(ws), _ptr(yr), _ptr(ys),
                                   _stream(stream), C.byref(cfg)))
 

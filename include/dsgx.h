@@ -254,6 +254,14 @@ typedef struct dsgx_prefill_cfg {
                        and the reference compute it (engine/experts/decode.cu:110-113); 1: the hardware's exponential and
                        reciprocal (each within 1 ulp; h then differs from the exact form's in about one value in 10^4, by one
                        bf16 step), for callers that trade that for the epilogue's time */
+  int32_t tile_order; /* FP8 activations only: the order in which the grouped GEMMs walk the tiles (the reference's
+                       prefill_tuning tord, ds41f-4xgx10-switchless/engine/kernels/dsk.h:252, prefill.cu:658-668). 0: by
+                       expert id, an expert's tiles next to each other; 1: the experts by falling count, their
+                       256-position tiles and the remainders merged evenly (tiles bound by the matrix unit beside tiles
+                       bound by the weight stream); 2: every 256-position tile first, then the remainders by falling
+                       size; -1 (the default): the library's choice (0: on MI355X 1 and 2 measured no faster). The
+                       results do not depend on it; a call that runs later phases alone names the same order as the
+                       call that ran the bucketing (any order finds a valid list). */
 } dsgx_prefill_cfg;
 DSGX_API void dsgx_prefill_cfg_default(dsgx_prefill_cfg* cfg);
 DSGX_API size_t dsgx_prefill_ws_bytes(const dsgx_layer_w* L, int T);

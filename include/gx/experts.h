@@ -133,6 +133,7 @@ struct PrefillCfg {
   void* side = nullptr;     // accepted, unused
   bool act_fp8 = true;      // FP8 layers: e4m3 activations on the fp8 MFMA (see dsgx_prefill_cfg)
   bool fast_act = false;    // ... with SwiGLU by the hardware's exp2 / rcp (see dsgx_prefill_cfg)
+  int tile_order = -1;      // ... and the order the grouped GEMMs walk the tiles in (see dsgx_prefill_cfg; the same bits in any)
 };
 inline size_t prefill_ws_bytes(const LayerW& L, int T) { const dsgx_layer_w c = L.c(); return dsgx_prefill_ws_bytes(&c, T); }
 inline size_t prefill_ws_bytes(int T) { return prefill_ws_bytes(LayerW(), T); }  // the reference's form (experts.h:180)
@@ -142,7 +143,7 @@ inline void moe_prefill_phases(const LayerW& L, const uint16_t* x, const int* id
   const dsgx_layer_w c = L.c();
   dsgx_prefill_cfg p;
   dsgx_prefill_cfg_default(&p);
-  p.shared = cfg.shared, p.phases = phases, p.act_fp8 = cfg.act_fp8, p.fast_act = cfg.fast_act;
+  p.shared = cfg.shared, p.phases = phases, p.act_fp8 = cfg.act_fp8, p.fast_act = cfg.fast_act, p.tile_order = cfg.tile_order;
   DSGX_DIE_ON(dsgx_moe_prefill(&c, x, idx, w, T, ws, yr, ys, st, &p));
 }
 inline void moe_prefill(const LayerW& L, const uint16_t* x, const int* idx, const float* w, int T, void* ws, float* yr, float* ys,

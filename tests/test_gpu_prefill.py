@@ -190,6 +190,38 @@ def test_prefill_rows_do_not_depend_on_the_chunk():
     assert np.array_equal(yr[50:60], yr2) and np.array_equal(ys[50:60], ys2)
 
 
+def test_prefill_tile_order_does_not_change_a_bit():
+    """dsgx_prefill_cfg::tile_order (the reference's prefill_tuning tord, ds41f engine/kernels/dsk.h:252) only changes which
+    workgroup takes which tile: experts of 0, a few, 128, 129, 256 and several hundred rows (remainders, 256-position
+    tiles and both), every order, the same yr, ys and workspace views as the order by expert id"""
+    H, I, E, topk, T = 256, 256, 12, 2, 900
+    hl = helpers.make_layer(abi.FMT_FP8, H, I, E, topk, 5, seed=9, shared="fp8")
+    x, _, _, w = helpers.rows_and_routing(21, T, H, E, topk, 1.0)
+    # rows an expert: 0, 1, 17, 128, 129, 256, 257, 300, 421, ... (pairs (a, b), a < b, dealt so that the counts come out)
+    want = [0, 1, 17, 128, 129, 256, 257, 300, 421, 291, 0, 0]
+    want[10] = (2 * T - sum(want)) // 2
+    want[11] = 2 * T - sum(want)
+    left = list(want)
+    idx = np.zeros((T, topk), np.int32)
+    for t in range(T):
+        a = int(np.argmax(left))
+        left[a] -= 1
+        b = int(np.argmax([v if j != a else -1 for j, v in enumerate(left)]))
+        left[b] -= 1
+        idx[t] = (a, b)
+    assert min(left) == 0 and max(left) == 0 and (idx[:, 0] != idx[:, 1]).all()
+    ref = None
+    for order in (0, 1, 2, -1):
+        yr, ys, ws, dl = _prefill(hl, x, idx, w, T, tile_order=order)
+        got = (yr.view(np.uint32), ys.view(np.uint32))
+        if ref is None:
+            ref = got
+            assert np.isfinite(yr).all() and np.isfinite(ys).all() and np.abs(yr).max() > 0
+        assert np.array_equal(ref[0], got[0]) and np.array_equal(ref[1], got[1]), order
+    with pytest.raises(lib.DsgxError):
+        _prefill(hl, x, idx, w, T, tile_order=3)
+
+
 def test_prefill_argument_errors():
     hl = helpers.make_layer(abi.FMT_BF16, 512, 256, 8, 2, 4, seed=1)
     dl = hl.upload()
