@@ -86,8 +86,10 @@ struct Args {
 
 // Workgroup -> (position tile, group of weight rows): blocks of kMapTiles consecutive tiles x kMapNs row groups get 32
 // consecutive workgroup numbers of ONE XCD (numbers x, x + 8, x + 16, ...), so that what they share (a tile's
-// activations, an expert's weights) is fetched into that XCD's L2 once.
-constexpr int kMapTiles = 4, kMapNs = 8, kXcds = 8;
+// activations, an expert's weights) is fetched into that XCD's L2 once. 8 tiles x 4 row groups measured best at the
+// benchmark's chunk (routed 2.83 ms against 2.875 with 4 x 8, 2.85 with 16 x 2, 2.97 with 2 x 16 or 32 x 1: what pays
+// is an expert's weights shared between its neighbouring tiles, more than a tile's activations between row groups).
+constexpr int kMapTiles = 8, kMapNs = 4, kXcds = 8;
 __host__ __device__ inline unsigned grid_of(int tiles, int NS) {
   const int blocks = ((tiles + kMapTiles - 1) / kMapTiles) * ((NS + kMapNs - 1) / kMapNs);
   return (unsigned)((blocks + kXcds - 1) / kXcds) * kXcds * (kMapTiles * kMapNs);
@@ -188,6 +190,11 @@ __device__ __forceinline__ void gemm_tile(const Args& g, uint8_t* smem, int e, i
   }
   // (the dynamic segment's address inside LDS: the pointer in the LDS address space is that 32-bit offset)
   const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)smem;
+  // the 16-position tiles this wave brings that hold rows: a ragged tile's other slots are neither fetched nor read (a
+  // remainder of a few rows otherwise spends a third of its loads on them; gate/up 1.6% and down 0.8% faster at the
+  // benchmark's chunk; the same change in the INT4 and MXFP4 kernels, whose loads sit between their MFMAs, gained nothing
+  // and is not in them). A wave's loads a turn are then 4, or 4 + 2 nx + 1, which its waits count.
+  const int nx = uni(min(WP, max(0, nmt - WP * wave)));
   auto issue = [&](int kb) {  // block kb (clamped: past the end the last block again, into a stage nobody reads) -> its stage
     const int kc = kb < KB ? kb : KB - 1;
     const uint32_t st = lds0 + (uint32_t)(kb % S::kStages) * S::kStageBytes;
@@ -197,10 +204,12 @@ __device__ __forceinline__ void gemm_tile(const Args& g, uint8_t* smem, int e, i
 #pragma unroll
       for (int hh = 0; hh < 2; ++hh) dma16(pw[t][hh] + (size_t)kc * 128, uni(wbase + t * 2048 + hh * 1024));
 #pragma unroll
-    for (int t = 0; t < WP; ++t)
+    for (int t = 0; t < WP; ++t) {
+      if (t >= nx) break;  // (a ragged tile: nobody reads the 16-position tiles past its end)
 #pragma unroll
       for (int hh = 0; hh < 2; ++hh) dma16(px[t][hh] + (size_t)kc * 128, uni(xbase + t * 2048 + hh * 1024));
-    if (lane < 16 * WP) dma4(pxs + kc, uni(st + S::kStageW + S::kStageX + (uint32_t)wave * (64 * WP)));
+    }
+    if (nx > 0 && lane < 16 * WP) dma4(pxs + kc, uni(st + S::kStageW + S::kStageX + (uint32_t)wave * (64 * WP)));
   };
   // The wave's weight scales: lane l holds those of block l; one value
   // a 16-row tile pair (UP: gate and up; DOWN: all of a wave's rows lie in one 128-row block). They are loaded with
@@ -240,7 +249,10 @@ __device__ __forceinline__ void gemm_tile(const Args& g, uint8_t* smem, int e, i
     for (int kb = 0; kb < ((DIAG & 32) ? 2 : KB); ++kb) {
       // this wave's loads of block kb have landed (later blocks may be in flight); after the barrier everyone's have, and
       // everyone is done reading the stage of block kb - 1, which the loads of block kb + kStages - 1 now overwrite
-      wait_loads<(S::kStages - 2) * S::kLoads>();
+      if (S::kStages == 2) wait_loads<0>();
+      else if (nx == WP) wait_loads<(S::kStages - 2) * S::kLoads>();
+      else if (nx == 0) wait_loads<(S::kStages - 2) * 4>();
+      else wait_loads<(S::kStages - 2) * (5 + 2 * (WP - 1))>();  // (WP 2 with one live tile; two stages wait for all anyway)
       if (!(DIAG & 4)) __syncthreads();
       if (kb == 0) PF_STAMP(g, 4);
       if (!(DIAG & 1)) issue(kb + S::kStages - 1);
