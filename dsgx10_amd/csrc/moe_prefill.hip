@@ -592,7 +592,9 @@ __global__ void __launch_bounds__(kGemmThreads) k_pf_gemm16(Gemm16Args g) {
   }
 }
 
-// yr[t][n] over the row's picks in expert-id order: acc = fma(s2 * w, d, acc); four columns a thread
+// yr[t][n] over the row's picks in expert-id order: acc = fma(s2 * w, d, acc); four columns a thread. TOPK > 0: the picks'
+// loads are all issued before the first add (the adds keep their order); 0: any top-k, one pick after the other
+template <int TOPK>
 __global__ void __launch_bounds__(256) k_pf_combine(const float* __restrict__ d, const int* __restrict__ rpos, const float* __restrict__ rk,
                                                     int T, int H, int topk, float* __restrict__ yr) {
   const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -600,16 +602,36 @@ __global__ void __launch_bounds__(256) k_pf_combine(const float* __restrict__ d,
   if (i >= (size_t)T * per) return;
   const int t = (int)(i / per), n = (int)(i % per) * 4;
   float4 a = make_float4(0.f, 0.f, 0.f, 0.f);
-  for (int r = 0; r < topk; ++r) {
-    const float k = rk[t * topk + r];
-    const float4 v = *reinterpret_cast<const float4*>(d + (size_t)rpos[t * topk + r] * H + n);
-    a.x = fmaf(k, v.x, a.x), a.y = fmaf(k, v.y, a.y), a.z = fmaf(k, v.z, a.z), a.w = fmaf(k, v.w, a.w);
+  if (TOPK > 0) {
+    float k[TOPK > 0 ? TOPK : 1];
+    pf8::v4f_t v[TOPK > 0 ? TOPK : 1];
+#pragma unroll
+    for (int r = 0; r < TOPK; ++r) {
+      k[r] = rk[t * TOPK + r];
+      v[r] = __builtin_nontemporal_load(reinterpret_cast<const pf8::v4f_t*>(d + (size_t)rpos[t * TOPK + r] * H + n));
+    }
+#pragma unroll
+    for (int r = 0; r < TOPK; ++r) a.x = fmaf(k[r], v[r][0], a.x), a.y = fmaf(k[r], v[r][1], a.y), a.z = fmaf(k[r], v[r][2], a.z), a.w = fmaf(k[r], v[r][3], a.w);
+  } else {
+    for (int r = 0; r < topk; ++r) {
+      const float k = rk[t * topk + r];
+      const float4 v = *reinterpret_cast<const float4*>(d + (size_t)rpos[t * topk + r] * H + n);
+      a.x = fmaf(k, v.x, a.x), a.y = fmaf(k, v.y, a.y), a.z = fmaf(k, v.z, a.z), a.w = fmaf(k, v.w, a.w);
+    }
   }
   *reinterpret_cast<float4*>(yr + (size_t)t * H + n) = a;
 }
+static void launch_pf_combine(const float* d, const int* rpos, const float* rk, int T, int H, int topk, float* yr, hipStream_t st) {
+  const size_t n = (size_t)T * (H / 4);
+  const dim3 grid((unsigned)((n + 255) / 256)), block(256);
+  if (topk == 8) hipLaunchKernelGGL(k_pf_combine<8>, grid, block, 0, st, d, rpos, rk, T, H, topk, yr);
+  else hipLaunchKernelGGL(k_pf_combine<0>, grid, block, 0, st, d, rpos, rk, T, H, topk, yr);
+}
 
 // DeepSeek's combine (ds41f engine/kernels/moe.cu:974-981): y[t] = the f32 sum, in expert-id order, of the picks' outputs
-// (each already rounded to bf16 by the down GEMM), then the shared expert's; eight columns a thread
+// (each already rounded to bf16 by the down GEMM), then the shared expert's; eight columns a thread. TOPK > 0: every
+// row is requested before the first add (the adds keep their order); 0: any top-k, one row after the other
+template <int TOPK>
 __global__ void __launch_bounds__(256) k_pfmx_combine(const uint16_t* __restrict__ d, const uint16_t* __restrict__ dsh, const int* __restrict__ rpos,
                                                       int T, int H, int topk, float* __restrict__ y) {
   const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -617,13 +639,22 @@ __global__ void __launch_bounds__(256) k_pfmx_combine(const uint16_t* __restrict
   if (i >= (size_t)T * per) return;
   const int t = (int)(i / per), n = (int)(i % per) * 8;
   float a[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-  auto add = [&](const uint16_t* row) {
-    const u32x4_t v = *reinterpret_cast<const u32x4_t*>(row + n);
+  auto add = [&](const u32x4_t v) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) a[2 * j] = __fadd_rn(a[2 * j], bf16_bits_to_f32(v[j] & 0xFFFFu)), a[2 * j + 1] = __fadd_rn(a[2 * j + 1], bf16_bits_to_f32(v[j] >> 16));
   };
-  for (int r = 0; r < topk; ++r) add(d + (size_t)rpos[t * topk + r] * H);
-  if (dsh) add(dsh + (size_t)t * H);
+  if (TOPK > 0) {
+    u32x4_t v[TOPK > 0 ? TOPK + 1 : 1];
+#pragma unroll
+    for (int r = 0; r < TOPK; ++r) v[r] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(d + (size_t)rpos[t * TOPK + r] * H + n));
+    if (dsh) v[TOPK] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(dsh + (size_t)t * H + n));
+#pragma unroll
+    for (int r = 0; r < TOPK; ++r) add(v[r]);
+    if (dsh) add(v[TOPK]);
+  } else {
+    for (int r = 0; r < topk; ++r) add(*reinterpret_cast<const u32x4_t*>(d + (size_t)rpos[t * topk + r] * H + n));
+    if (dsh) add(*reinterpret_cast<const u32x4_t*>(dsh + (size_t)t * H + n));
+  }
   float4* o = reinterpret_cast<float4*>(y + (size_t)t * H + n);
   o[0] = make_float4(a[0], a[1], a[2], a[3]), o[1] = make_float4(a[4], a[5], a[6], a[7]);
 }
@@ -788,8 +819,7 @@ int dsgx_moe_prefill(const dsgx_layer_w* L, const uint16_t* x, const int* idx, c
       else hipLaunchKernelGGL(k_dn, dim3(pf_grid(o.max_tiles, H / kWgRows)), dim3(kGemmThreads), lds16, st, q);
     }
     if (cfg.phases & 8) {
-      const size_t n = (size_t)T * (H / 4);
-      hipLaunchKernelGGL(k_pf_combine, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, F32(o.d), I32(o.rpos), F32(o.rk), T, H, topk, yr);
+      launch_pf_combine(F32(o.d), I32(o.rpos), F32(o.rk), T, H, topk, yr, st);
     }
     if ((cfg.phases & 16) && shared) {
       const int tiles = (T + kTile - 1) / kTile;
@@ -850,8 +880,7 @@ int dsgx_moe_prefill(const dsgx_layer_w* L, const uint16_t* x, const int* idx, c
     DSGX_HIP(hipGetLastError());
   }
   if (cfg.phases & 8) {
-    const size_t n = (size_t)T * (H / 4);
-    hipLaunchKernelGGL(k_pf_combine, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, F32(o.d), I32(o.rpos), F32(o.rk), T, H, topk, yr);
+    launch_pf_combine(F32(o.d), I32(o.rpos), F32(o.rk), T, H, topk, yr, st);
     DSGX_HIP(hipGetLastError());
   }
   if ((cfg.phases & 16) && shared) {
@@ -1025,7 +1054,11 @@ int dsgx_dsk_moe_prefill(const dsgx_dsk_weights* Wt, const uint8_t* xq, const ui
   }
   if (cfg.phases & 16) {
     const size_t n = (size_t)T * (H / 8);
-    hipLaunchKernelGGL(k_pfmx_combine, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, U16(o.d), shared ? dsh : (const uint16_t*)nullptr, I32(o.rpos), T, H, topk, y);
+    const dim3 grid((unsigned)((n + 255) / 256)), block(256);
+    const uint16_t* sh = shared ? dsh : (const uint16_t*)nullptr;
+    if (topk == 6) hipLaunchKernelGGL(k_pfmx_combine<6>, grid, block, 0, st, U16(o.d), sh, I32(o.rpos), T, H, topk, y);
+    else if (topk == 8) hipLaunchKernelGGL(k_pfmx_combine<8>, grid, block, 0, st, U16(o.d), sh, I32(o.rpos), T, H, topk, y);
+    else hipLaunchKernelGGL(k_pfmx_combine<0>, grid, block, 0, st, U16(o.d), sh, I32(o.rpos), T, H, topk, y);
     DSGX_HIP(hipGetLastError());
   }
   return DSGX_OK;
