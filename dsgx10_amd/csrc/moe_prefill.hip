@@ -845,7 +845,7 @@ int dsgx_moe_prefill(const dsgx_layer_w* L, const uint16_t* x, const int* idx, c
     const char* dv = std::getenv("DSGX_PF_DIAG");
     switch (dv ? std::atoi(dv) : 0) {
 #define DSGX_DIAG_CASE(n) case n: k_up = pf8::k_gemm_mixed<true, n>, k_dn = pf8::k_gemm_mixed<false, n>, k_up2 = pf8::k_gemm<true, 2, n>, k_dn2 = pf8::k_gemm<false, 2, n>; break;
-      DSGX_DIAG_CASE(1) DSGX_DIAG_CASE(2) DSGX_DIAG_CASE(4) DSGX_DIAG_CASE(8) DSGX_DIAG_CASE(16) DSGX_DIAG_CASE(3) DSGX_DIAG_CASE(9) DSGX_DIAG_CASE(25) DSGX_DIAG_CASE(32) DSGX_DIAG_CASE(64)
+      DSGX_DIAG_CASE(1) DSGX_DIAG_CASE(2) DSGX_DIAG_CASE(4) DSGX_DIAG_CASE(8) DSGX_DIAG_CASE(16) DSGX_DIAG_CASE(3) DSGX_DIAG_CASE(9) DSGX_DIAG_CASE(25) DSGX_DIAG_CASE(32) DSGX_DIAG_CASE(64) DSGX_DIAG_CASE(128) DSGX_DIAG_CASE(256) DSGX_DIAG_CASE(384)
 #undef DSGX_DIAG_CASE
     }
   }

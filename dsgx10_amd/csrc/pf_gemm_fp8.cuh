@@ -122,7 +122,7 @@ __device__ __forceinline__ int swz(int r) { return (r & 7) ^ (r >> 3); }
 
 // DIAG (diagnostic builds only; results are then wrong): 1 no loads after the first stages, 2 the MFMAs accumulate by
 // themselves (no scaled adds on the vector unit), 4 no workgroup barrier in the loop, 8 no MFMAs, 16 no fragment reads
-// after the first turn
+// after the first turn, 128 the weight loads / 256 the activation loads re-read block 0 (cached) after the first stages
 // one tile: expert e (-1: the shared expert), rows [m0, mend) of the activations' positions, row group ns
 template <bool UP, int WP, int DIAG>
 __device__ __forceinline__ void gemm_tile(const Args& g, uint8_t* smem, int e, int m0, int mend, int ns) {
@@ -202,12 +202,12 @@ __device__ __forceinline__ void gemm_tile(const Args& g, uint8_t* smem, int e, i
 #pragma unroll
     for (int t = 0; t < 2; ++t)
 #pragma unroll
-      for (int hh = 0; hh < 2; ++hh) dma16(pw[t][hh] + (size_t)kc * 128, uni(wbase + t * 2048 + hh * 1024));
+      for (int hh = 0; hh < 2; ++hh) dma16(pw[t][hh] + (size_t)(((DIAG & 128) && kb >= S::kStages) ? 0 : kc) * 128, uni(wbase + t * 2048 + hh * 1024));
 #pragma unroll
     for (int t = 0; t < WP; ++t) {
       if (t >= nx) break;  // (a ragged tile: nobody reads the 16-position tiles past its end)
 #pragma unroll
-      for (int hh = 0; hh < 2; ++hh) dma16(px[t][hh] + (size_t)kc * 128, uni(xbase + t * 2048 + hh * 1024));
+      for (int hh = 0; hh < 2; ++hh) dma16(px[t][hh] + (size_t)(((DIAG & 256) && kb >= S::kStages) ? 0 : kc) * 128, uni(xbase + t * 2048 + hh * 1024));
     }
     if (nx > 0 && lane < 16 * WP) dma4(pxs + kc, uni(st + S::kStageW + S::kStageX + (uint32_t)wave * (64 * WP)));
   };
