@@ -31,15 +31,24 @@ using pf8::v4f_t;
 using pf8::wait_loads;
 typedef __bf16 v8bf_t __attribute__((ext_vector_type(8)));
 
-constexpr int kPos = 128;                    // positions of a tile
 constexpr int kStageW = kWgRows * 64;        // 16 KiB of nibbles
-constexpr int kStageX = kPos * 256;          // 32 KiB of bf16
 constexpr int kStageS = kWgRows * 8;         // four bf16 scales a row
 constexpr int kStageZ = (kWgRows / 8) * 16;  // four zero-point words a group of eight rows
-constexpr int kStageBytes = kStageW + kStageX + kStageS + kStageZ;  // 51,712
-constexpr int kStages = 3;
+// A tile's shape by its positions: 128 (three stages), or 64 for the tiles that hold no more rows (four stages). What a
+// turn waits for is the trip to HBM of a block's 18.5 KB of weights, scales and zero points, not their rate (9 GB/s a CU):
+// with three stages a block has one turn to land (it is decoded a turn ahead), with four it has two. Most tiles of a
+// chunk of 2048 rows are such tiles (the median bucket holds 34 rows).
+template <int POS>
+struct Shape {
+  static constexpr int kPos = POS;
+  static constexpr int kSub = POS / 16;                  // its 16-position tiles: waves 0 .. kSub - 1 bring one each
+  static constexpr int kStageX = POS * 256;              // bf16 rows of the block
+  static constexpr int kStageBytes = kStageW + kStageX + kStageS + kStageZ;  // 51,712 | 35,328
+  static constexpr int kStages = POS == 128 ? 3 : 4;
+  static constexpr int kLds = kStages * kStageBytes;     // (the epilogues reuse it: UP POS x 256 B, DOWN 8 x 2 KiB)
+};
 constexpr int kLoads = 2 + 4 + 1 + 1;        // a wave's loads a turn: two weight tiles, one activation tile (four pieces of 4 rows), scales, zero points
-constexpr int kLds = kStages * kStageBytes;  // (the epilogues reuse it: UP 128 x 256 B, DOWN 8 x 2 KiB)
+constexpr int kLds = Shape<128>::kLds > Shape<64>::kLds ? Shape<128>::kLds : Shape<64>::kLds;
 
 struct Args {
   const uint16_t* x;   // activations bf16 [rows][K]
@@ -55,8 +64,10 @@ struct Args {
 
 __device__ __forceinline__ int sw4(int r) { return (r >> 2) & 3; }
 
-template <bool UP>
+template <bool UP, int POS>
 __device__ __forceinline__ void gemm_tile(const Args& g, uint8_t* smem, int e, int m0, int mend, int ns) {
+  using S = Shape<POS>;
+  constexpr int kPos = S::kPos, kStageX = S::kStageX, kStageBytes = S::kStageBytes, kStages = S::kStages;
   const int K = UP ? g.L.H : g.L.I, N = UP ? g.L.I : g.L.H, KB = K / 128, G = K / 32;
   if (mend > m0 + kPos) mend = m0 + kPos;
   const dsgx_mat_desc* dsc = g.L.desc + (size_t)e * 3;
@@ -71,7 +82,8 @@ __device__ __forceinline__ void gemm_tile(const Args& g, uint8_t* smem, int e, i
     base = (UP && t) ? mb : ma;
     return UP ? c0 + 16 * wave : r0 + 32 * wave + 16 * t;
   };
-  const int nmt = uni(min(8, (mend - m0 + 15) / 16));
+  const int nmt = uni(min(S::kSub, (mend - m0 + 15) / 16));
+  const bool brings_x = wave < S::kSub;  // (a wave's loads a turn: kLoads, or kLoads - 4)
 
   // ---- what this lane fetches ----
   const uint8_t* pw[2];   // weights: row lane / 4 of tile t, piece (lane % 4) ^ sw4(row)
@@ -111,7 +123,7 @@ __device__ __forceinline__ void gemm_tile(const Args& g, uint8_t* smem, int e, i
     } else if (i == 1) {
       if (lane < 16) dma4(reinterpret_cast<const float*>(pzp + (size_t)kc * 16), uni(st + kStageW + kStageX + kStageS + (uint32_t)wave * 64));
     } else if (i < 6) {
-      dma16(px[i - 2] + (size_t)kc * 256, uni(st + kStageW + (uint32_t)wave * 4096 + (i - 2) * 1024));
+      if (brings_x) dma16(px[i - 2] + (size_t)kc * 256, uni(st + kStageW + (uint32_t)wave * 4096 + (i - 2) * 1024));
     } else {
       dma16(pw[i - 6] + (size_t)kc * 64, uni(st + (uint32_t)wave * 2048 + (i - 6) * 1024));
     }
@@ -139,7 +151,8 @@ __device__ __forceinline__ void gemm_tile(const Args& g, uint8_t* smem, int e, i
   // A block's weights are decoded a turn ahead, a piece (one MFMA's fragment) at a time between the MFMAs of the turn before:
   // the decode is vector-unit work and the MFMAs run beside it. (Decoded in front of its own MFMAs it stood in their way: both
   // waves of a SIMD reach it together behind the barrier: 1.39 -> 1.1 ms for gate/up.) Turn kb therefore needs block kb + 1
-  // landed: it waits for every load issued so far, and issues block kb + 2's.
+  // landed: with three stages it waits for every load issued so far and issues block kb + 2's; with four, block kb + 2 may
+  // still be in flight and it issues block kb + 3's.
   u32x4_t raw[2];
   float sc[2], nzs[2];
   auto open_block = [&](int kb) {  // the lane's raw words, scale and -(zero point * scale) of the wave's two tiles of block kb
@@ -160,13 +173,17 @@ __device__ __forceinline__ void gemm_tile(const Args& g, uint8_t* smem, int e, i
   auto run = [&](auto nj_c) {
     constexpr int NJ = decltype(nj_c)::value;
     u32x4_t fa[2][4], fn[2][4];
-    wait_loads<kLoads>();  // block 0 (block 1 may be in flight)
+    // block 0 has landed (the later ones of the first stages may be in flight)
+    if (brings_x) wait_loads<(kStages - 2) * kLoads>();
+    else wait_loads<(kStages - 2) * (kLoads - 4)>();
     __syncthreads();
     open_block(0);
 #pragma unroll
     for (int pc = 0; pc < 8; ++pc) piece(fa, pc);
     auto turn = [&](int kb, u32x4_t (&fa)[2][4], u32x4_t (&fn)[2][4]) {
-      wait_loads<0>();
+      // block kb + 1 has landed (four stages: block kb + 2 may be in flight)
+      if (brings_x) wait_loads<(kStages - 3) * kLoads>();
+      else wait_loads<(kStages - 3) * (kLoads - 4)>();
       __syncthreads();
       open_block(kb + 1);
       const uint8_t* X = smem + (size_t)(kb % kStages) * kStageBytes + kStageW;
@@ -198,11 +215,19 @@ __device__ __forceinline__ void gemm_tile(const Args& g, uint8_t* smem, int e, i
     case 1: run(std::integral_constant<int, 1>{}); break;
     case 2: run(std::integral_constant<int, 2>{}); break;
     case 3: run(std::integral_constant<int, 3>{}); break;
-    case 4: run(std::integral_constant<int, 4>{}); break;
-    case 5: run(std::integral_constant<int, 5>{}); break;
-    case 6: run(std::integral_constant<int, 6>{}); break;
-    case 7: run(std::integral_constant<int, 7>{}); break;
-    default: run(std::integral_constant<int, 8>{}); break;
+    default:
+      if constexpr (S::kSub == 4) {
+        run(std::integral_constant<int, 4>{});
+      } else {
+        switch (nmt) {
+          case 4: run(std::integral_constant<int, 4>{}); break;
+          case 5: run(std::integral_constant<int, 5>{}); break;
+          case 6: run(std::integral_constant<int, 6>{}); break;
+          case 7: run(std::integral_constant<int, 7>{}); break;
+          default: run(std::integral_constant<int, 8>{}); break;
+        }
+      }
+      break;
   }
   wait_loads<0>();
   __syncthreads();
@@ -264,7 +289,9 @@ __global__ void __launch_bounds__(kThreads) k_gemm(Args g) {
   pf8::task_of<false>(NS, tile, ns);
   if (ns >= NS || tile >= *g.ntiles) return;
   const int e = g.tile_e[tile];
-  gemm_tile<UP>(g, smem, e, g.off[e] + g.tile_m0[tile], g.off[e + 1], ns);
+  const int m0 = g.off[e] + g.tile_m0[tile], mend = g.off[e + 1];
+  if (mend - m0 <= 64) gemm_tile<UP, 64>(g, smem, e, m0, mend, ns);
+  else gemm_tile<UP, 128>(g, smem, e, m0, mend, ns);
 }
 
 }  // namespace pfi4
