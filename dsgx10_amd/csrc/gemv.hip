@@ -53,7 +53,10 @@ __global__ void __launch_bounds__(256) k_gemv(GemvArgs a) {
   extern __shared__ uint4 xs[];
   __shared__ float red[4];
   const int lane = threadIdx.x & 63;
-  const int gw = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6), GW = gridDim.x * (blockDim.x >> 6);
+  // (the wave's number is the same in every lane: said so, which keeps the row cursors and the segment's descriptor on the
+  // scalar unit - read from a vector register they came through vector loads of the kernel's arguments, which a wave's
+  // weight loads then queued behind, one ring entry after the other)
+  const int gw = uni(blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)), GW = gridDim.x * (blockDim.x >> 6);
   const int nbatch = a.total_rows / RB;
   const int nmine = gw < nbatch ? (nbatch - gw + GW - 1) / GW : 0;
   const int nsteps = nmine * a.nsegk;
@@ -147,7 +150,7 @@ __global__ void __launch_bounds__(256) k_gemv_sk(GemvArgs a) {
   extern __shared__ uint4 xs[];
   __shared__ float part[4][RB * M];
   __shared__ float red[4];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63, wave = uni(threadIdx.x >> 6);  // (uniform: the segment's descriptor stays on the scalar unit)
   constexpr int GPW = 4 / SK;  // batches a workgroup
   const int grp = wave / SK, slice = wave % SK;
   const int nbatch = a.total_rows / RB;
