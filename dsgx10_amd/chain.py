@@ -42,11 +42,12 @@ class LayerChain:
         tap = tap or (lambda name: None)
         xp = [dict(fmt=abi.FMT_BF16, w=W["xproj"], n=XR, y=self.xg, ldy=XR)]
         if fused and fuse_xproj:
-            lib.add_norm_gemv(self.yr, None, a, b, W["attn_norm"], 1e-5, None, M, H, xp, abi.OUT_BF16, splitk=4, stream=stream)
+            lib.add_norm_gemv(self.yr, None, a, b, W["attn_norm"], 1e-5, None, M, H, xp, abi.OUT_BF16, splitk=2, stream=stream)
         else:
             lib.add_norm(self.yr, None, M, H, a, b, W["attn_norm"], 1e-5, self.xn, stream=stream)
             tap("norm1")
-            lib.gemv(self.xn, H, M, H, xp, abi.OUT_BF16, splitk=4, stream=stream)
+            # (K over 2 waves: 7.2 / 9.1 us for the two layers' shapes against 8.7 / 11.2 over 4 and 8.0 / 10.1 unsplit, measured)
+            lib.gemv(self.xn, H, M, H, xp, abi.OUT_BF16, splitk=2, stream=stream)
         tap("xproj")
         lib.gemv(self.xg, XR, M, QL, [dict(W["qb"], n=NQ, y=self.q, ldy=NQ)], abi.OUT_BF16, stream=stream)
         tap("qb")
