@@ -83,16 +83,26 @@ __global__ void __launch_bounds__(256) k_gemv(GemvArgs a) {
     dummy = a.sg[si].m.w + (size_t)(row - a.sg[si].row0) * FmtT<FMT>::row_bytes(a.K);
   }
   int lt = 0, lj = 0, lseg = 0;  // the load cursor: step, batch number of this wave, segment
+  // the matrix of the batch under the load cursor and the batch's first row in it: fetched from the kernel's arguments when
+  // the cursor enters a batch, not at every step (scalar loads, but each is a wait in front of the step's weight loads)
+  MatDev lm;
+  int lrow = 0;
+  auto enter = [&]() {
+    const int row = lt < nsteps ? (gw + lj * GW) * RB : 0;
+    int si;
+    locate(row, si);
+    lm = a.sg[si].m, lrow = row - a.sg[si].row0;
+  };
+  enter();
   auto load = [&](Raw (&r)[RB]) {
     const bool ok = lt < nsteps;
     ++lt;
-    const int row = ok ? (gw + lj * GW) * RB : 0;
-    int si;
-    locate(row, si);
 #pragma unroll
-    for (int i = 0; i < RB; ++i)
-      load_raw<FMT, true>(r[i], a.sg[si].m, row - a.sg[si].row0 + i, lseg, lane, a.K, acc[i][0], ok ? nullptr : dummy);
-    if (ok && ++lseg == a.nsegk) lseg = 0, ++lj;
+    for (int i = 0; i < RB; ++i) load_raw<FMT, true>(r[i], lm, lrow + i, lseg, lane, a.K, acc[i][0], ok ? nullptr : dummy);
+    if (ok && ++lseg == a.nsegk) {
+      lseg = 0, ++lj;
+      enter();
+    }
   };
   int cj = 0, cseg = 0;
   auto compute = [&](const Raw (&raw)[RB]) {
