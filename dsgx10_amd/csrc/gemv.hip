@@ -78,20 +78,25 @@ __global__ void __launch_bounds__(256) k_gemv(GemvArgs a) {
   const uint8_t* dummy;
   {
     const int row = min(gw * RB, a.total_rows - 1);
-    int si;
-    locate(row, si);
+    int si = 0;
+    if (a.nsegs > 1) locate(row, si);
     dummy = a.sg[si].m.w + (size_t)(row - a.sg[si].row0) * FmtT<FMT>::row_bytes(a.K);
   }
   int lt = 0, lj = 0, lseg = 0;  // the load cursor: step, batch number of this wave, segment
   // the matrix of the batch under the load cursor and the batch's first row in it: fetched from the kernel's arguments when
   // the cursor enters a batch, not at every step (scalar loads, but each is a wait in front of the step's weight loads)
-  MatDev lm;
+  // (a call with one segment, the common one, fetches once: every later fetch would be two dependent scalar round trips)
+  MatDev lm = a.sg[0].m;
   int lrow = 0;
   auto enter = [&]() {
     const int row = lt < nsteps ? (gw + lj * GW) * RB : 0;
-    int si;
-    locate(row, si);
-    lm = a.sg[si].m, lrow = row - a.sg[si].row0;
+    int row0 = 0;
+    if (a.nsegs > 1) {
+      int si;
+      locate(row, si);
+      lm = a.sg[si].m, row0 = a.sg[si].row0;
+    }
+    lrow = row - row0;
   };
   enter();
   auto load = [&](Raw (&r)[RB]) {
@@ -123,8 +128,8 @@ __global__ void __launch_bounds__(256) k_gemv(GemvArgs a) {
         if (lane == (i ^ 1) * M + m) mine2 = v;  // the pair's other row (SwiGLU)
       }
     if (lane >= RB * M) return;
-    int si;
-    locate(row, si);
+    int si = 0;
+    if (a.nsegs > 1) locate(row, si);
     const GemvSegDev& sg = a.sg[si];
     const int r = lane / M, m = lane % M, n = row - sg.row0 + r;
     if (a.out == DSGX_OUT_BF16) {
