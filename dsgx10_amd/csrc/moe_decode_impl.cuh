@@ -209,6 +209,48 @@ __device__ __forceinline__ void resolve(Step<M>& S, const DecodeArgs& a, int rw,
   const int lane = threadIdx.x & 63, E = a.L.E, topk = a.L.topk, ne = M * topk;
   const int H = a.L.H, I = a.L.I, nsh = SHFMT != 0 ? 1 : 0;
   __builtin_amdgcn_s_setprio(3);
+  // the routed slot of expert e, its place r among the step's experts
+  auto make_slot = [&](int e, int r) {
+    Slot t;
+    auto ref = [&](int which, int N, int K) {
+      if (a.stk_w[0]) return MatRef{a.stk_w[which] + (size_t)e * a.stk_wb[which], a.stk_s[which] + (size_t)e * a.stk_sb[which], 1.f, 0};
+      const uint4 d = S.dtab[e * 3 + which];
+      return mat_ref<FMT>(a.L.pool + (((uint64_t)d.y << 32) | d.x), N, K, __uint_as_float(d.z));
+    };
+    t.g = ref(0, I, H), t.u = ref(1, I, H), t.d = ref(2, H, I);
+    t.hslot = r, t.shared = 0;
+    S.slots[nsh + r] = t;
+  };
+  if constexpr (M == 1) {
+    // One row: its picks are the step's experts, and a pick's slot is the number of picks with a lower id - counted in
+    // registers, without the tables' round trips through LDS. (Picks handed in by the caller that name an expert twice
+    // take the general path below.)
+    int id = 0;
+    float w = 0.f;
+    if (a.logits) route_row(R.lg, R.bs, E, topk, a.route_scale, a.score_fn, lane, id, w);
+    else if (lane < topk) id = a.idx[lane], w = a.w[lane];
+    int r = 0;
+    bool twice = false;
+#pragma unroll
+    for (int j = 0; j < DSGX_MAX_TOPK; ++j) {
+      const int ej = __builtin_amdgcn_readlane(id, j);
+      if (j < topk) r += ej < id ? 1 : 0, twice |= ej == id && j != lane;
+    }
+    if (__ballot(twice && lane < topk) == 0) {
+      DSGX_MARKW(9);
+      if (lane < topk) {
+        if (a.idx_out && blockIdx.x == 0) a.idx_out[lane] = id, a.wts_out[lane] = w;
+        S.wslot[r][0] = w;
+        make_slot(id, r);
+      }
+      if (lane == 0) S.n = topk;
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+      if (lane == 0) __hip_atomic_store(&S.ready, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+      __builtin_amdgcn_s_setprio(0);
+      DSGX_MARKW(2);
+      return;
+    }
+  }
   int mine = 0;
   for (int row = rw; row < M; row += nr, ++mine) {
     int id = 0;
@@ -252,16 +294,7 @@ __device__ __forceinline__ void resolve(Step<M>& S, const DecodeArgs& a, int rw,
       r += __popc(mk[j] & below);
     }
     S.wslot[r][i / topk] = S.rw[i];
-    // the routed slot (rows that picked the same expert write the same values)
-    Slot t;
-    auto ref = [&](int which, int N, int K) {
-      if (a.stk_w[0]) return MatRef{a.stk_w[which] + (size_t)e * a.stk_wb[which], a.stk_s[which] + (size_t)e * a.stk_sb[which], 1.f, 0};
-      const uint4 d = S.dtab[e * 3 + which];
-      return mat_ref<FMT>(a.L.pool + (((uint64_t)d.y << 32) | d.x), N, K, __uint_as_float(d.z));
-    };
-    t.g = ref(0, I, H), t.u = ref(1, I, H), t.d = ref(2, H, I);
-    t.hslot = r, t.shared = 0;
-    S.slots[nsh + r] = t;
+    make_slot(e, r);  // (rows that picked the same expert write the same values)
   }
   if (lane == 0) {
     int n = 0;
